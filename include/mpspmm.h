@@ -1,0 +1,257 @@
+/*
+ * mpspmm.h -- C ABI of the MI355X (gfx950) MergePath-SpMM library.
+ *
+ * The reference (cag-uconn/MergePath-SpMM) has no library interface: each
+ * program is one translation unit whose main() parses a .csr file, builds the
+ * schedule on the host and launches a kernel.  The entry points below are the
+ * seams of those programs, one per step, so that a host program -- the C++
+ * drivers shipped beside this library, or any FFI -- can replace the step it
+ * names.  Each declaration cites the reference lines it stands in for.
+ *
+ * Conventions
+ *   - Every function returns an int status: MPS_OK (0) or an mps_status
+ *     value; HIP runtime failures return MPS_ERR_HIP + hipError_t.  Nothing
+ *     throws and nothing calls exit().
+ *   - "d_" arguments are device pointers, everything else is host memory.
+ *   - The caller owns every buffer, including workspaces; unless a comment
+ *     says otherwise the library allocates no device memory.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Calls are asynchronous with respect to the host; the caller
+ *     synchronises.
+ *   - Indices are 32-bit (as in the reference); n_rows + 1 + nnz must fit in
+ *     an int.  The sparse matrix is square: column ids index the n_rows rows
+ *     of the dense input (src/MergePathSpMM.cu:459-460).
+ *   - Dense matrices are row-major, K columns, no padding.
+ *   - fp16 data is IEEE binary16 passed as uint16_t bit patterns.
+ *   - Y is overwritten (Y = A * X); results do not depend on what Y held and
+ *     repeated calls give identical bits (merge-path and row-wise kernels).
+ *   - d_col_idx, d_val, d_X and d_Y must be 16-byte aligned.
+ */
+#ifndef MPSPMM_H
+#define MPSPMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mps_status {
+    MPS_OK = 0,
+    MPS_ERR_INVALID_ARG = 1,  /* null pointer, negative size, cost <= 0 ...      */
+    MPS_ERR_UNSUPPORTED = 2,  /* sizes beyond 32-bit indexing, K out of range     */
+    MPS_ERR_WORKSPACE = 3,    /* workspace missing or too small                   */
+    MPS_ERR_ALIGNMENT = 4,    /* a device pointer is not 16-byte aligned          */
+    MPS_ERR_IO = 5,           /* file cannot be opened / read / written           */
+    MPS_ERR_FORMAT = 6,       /* malformed .csr text or generator spec            */
+    MPS_ERR_TPW = 7,          /* threads_per_wave beyond what one wave can hold   */
+    MPS_ERR_INVALID_CSR = 8,  /* device-side validation found a bad row_ptr/col   */
+    MPS_ERR_HIP = 1000        /* + hipError_t                                     */
+} mps_status;
+
+/* Human-readable text for a status value (static storage). */
+const char *mps_status_string(int status);
+
+/* Library version, "major.minor.patch". */
+const char *mps_version(void);
+
+/* ------------------------------------------------------------------------ */
+/* Host side: sizes and schedule arithmetic                                  */
+/* ------------------------------------------------------------------------ */
+
+/* cost -> number of merge-path partitions.
+ * Replaces src/MergePathSpMM.cu:138-139:
+ *   P = (n_rows + 1 + nnz - 1) / cost;  if (P < 1024) P = 1024.
+ * cost <= 0 is rejected (the reference divides by it). */
+int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out);
+
+/* Merge items per partition, src/MergePathSpMM.cu:327-328:
+ *   ceil((n_rows + 1 + nnz) / P). */
+int mps_items_per_partition(int n_rows, int nnz, int P, int *ipt_out);
+
+/* Largest threads_per_wave (partitions walked side by side by one 64-lane
+ * wavefront) for feature width K and element size elem_bytes (4 = fp32,
+ * 2 = fp16).  Stands in for WARP_SIZE / dimension at
+ * src/MergePathSpMM.cu:224-228: a partition occupies K / (16 / elem_bytes)
+ * lanes (one 16-byte load per lane), at least 4. */
+int mps_max_threads_per_wave(int K, int elem_bytes, int *tpw_out);
+
+/* ------------------------------------------------------------------------ */
+/* Host side: .csr text files                                                */
+/* ------------------------------------------------------------------------ */
+
+/* Two-line comma-separated text: line 1 = row_ptr (n_rows + 1 integers),
+ * line 2 = col_idx (nnz integers); every integer may be followed by ','.
+ * Written by scripts/fetch_dataset.py:14-21 and scripts/npz_to_csr.py:21-28,
+ * read by src/MergePathSpMM.cu:126-173.
+ *
+ * mps_csr_read_header: pass 1 of the reference reader (:131-137): n_rows is
+ * the number of cells of line 1 minus one, nnz its last cell. */
+int mps_csr_read_header(const char *path, int *n_rows_out, int *nnz_out);
+
+/* Pass 2 (:147-173): fill row_ptr[n_rows + 1] and col_idx[nnz] (host memory,
+ * sized from mps_csr_read_header).  MPS_ERR_FORMAT when a cell is not an
+ * integer, line 2 does not hold exactly nnz cells, row_ptr is not
+ * non-decreasing from 0, or a column id is outside [0, n_rows). */
+int mps_csr_read(const char *path, int n_rows, int nnz, int *row_ptr, int *col_idx);
+
+/* Writer with the byte layout of scripts/npz_to_csr.py:21-28 (each element
+ * followed by ',', one '\n' between the lines, none at the end). */
+int mps_csr_write(const char *path, int n_rows, const int *row_ptr, const int *col_idx);
+
+/* ------------------------------------------------------------------------ */
+/* Host side: seeded synthetic graphs and fills                              */
+/* ------------------------------------------------------------------------ */
+
+/* The reference ships no data (README.md:18-25 points at a download); these
+ * generators make the benchmark graphs reproducibly from a spec string:
+ *   "er:n=4096,deg=8"                          Erdos-Renyi G(n, deg/n), directed, no self-loops
+ *   "chunglu:n=232965,nnz=114600000,gamma=2.1,dmax=20000[,sorted=1]"
+ *                                              Chung-Lu, expected degrees ~ shifted power law
+ *   "blockdiag:blocks=1178,min=100,max=600,deg=5"
+ *                                              disjoint random-geometric blocks
+ *   "rmat:scale=20,ef=16,a=0.57,b=0.19,c=0.19" R-MAT, duplicates removed
+ * Column ids are sorted and distinct within every row.  The result depends
+ * only on (spec, seed), not on the number of host threads.
+ * The graph is held by an opaque handle owned by the library. */
+typedef struct mps_graph mps_graph;
+int mps_graph_generate(const char *spec, uint64_t seed, mps_graph **graph_out);
+int mps_graph_from_csr_file(const char *path, mps_graph **graph_out);
+int mps_graph_dims(const mps_graph *g, int *n_rows_out, int *nnz_out, int *max_degree_out);
+const int *mps_graph_row_ptr(const mps_graph *g); /* host, n_rows + 1 */
+const int *mps_graph_col_idx(const mps_graph *g); /* host, nnz        */
+void mps_graph_free(mps_graph *g);
+
+/* out[i] = lo + (hi - lo) * u(seed, i), u uniform in [0, 1) with 24 random
+ * bits; element i depends only on (seed, i).  Replaces the constant fill of
+ * src/MergePathSpMM.cu:180-182. */
+int mps_fill_uniform_f32(float *out, size_t n, uint64_t seed, float lo, float hi);
+/* Same with 11 random bits so that every value is exact in binary16. */
+int mps_fill_uniform_f16(uint16_t *out, size_t n, uint64_t seed, float lo, float hi);
+
+/* ------------------------------------------------------------------------ */
+/* Device side: validation                                                   */
+/* ------------------------------------------------------------------------ */
+
+/* Checks on the device that row_ptr starts at 0, is non-decreasing, ends at
+ * nnz, and that every column id lies in [0, n_cols).  Synchronises the
+ * stream and allocates a 4-byte device flag for the duration of the call.
+ * The reference performs no validation (src/MergePathSpMM.cu:147-173);
+ * the SpMM entry points below trust their inputs just the same, so callers
+ * holding untrusted data run this first. */
+int mps_csr_validate(const int *d_row_ptr, const int *d_col_idx, int n_rows, int n_cols,
+                     int nnz, void *stream);
+
+/* ------------------------------------------------------------------------ */
+/* Device side: merge-path partitioner                                       */
+/* ------------------------------------------------------------------------ */
+
+/* Path coordinates of the P + 1 partition boundaries.  Boundary i lies on
+ * diagonal min(ipt * i, n_rows + 1 + nnz), ipt = mps_items_per_partition.
+ * One thread per diagonal runs the binary search of MergePathSearch
+ * (src/MergePathSpMM.cu:280-297) over row_ptr[0..n_rows] against the nonzero
+ * index, with the diagonals of generate_mp_sched (:327-334); x counts
+ * row_ptr entries consumed (current row = x - 1), y nonzeros consumed.
+ * d_coord_x, d_coord_y: int[P + 1].  Bit-exact with the reference. */
+int mps_partition(const int *d_row_ptr, int n_rows, int nnz, int P, int *d_coord_x,
+                  int *d_coord_y, void *stream);
+
+/* The six per-partition arrays of generate_mp_sched
+ * (src/MergePathSpMM.cu:300-385), including its zero-means-none encoding,
+ * derived on the device from the coordinates of mps_partition.  Each output
+ * is int[P].  Provided for parity with the reference schedule; the SpMM
+ * kernels below consume the coordinates directly. */
+int mps_schedule_legacy(const int *d_row_ptr, int n_rows, int nnz, int P,
+                        const int *d_coord_x, const int *d_coord_y, int *d_feature_start,
+                        int *d_feature_start_num, int *d_feature_end, int *d_feature_end_num,
+                        int *d_start_row, int *d_end_row, void *stream);
+
+/* ------------------------------------------------------------------------ */
+/* Device side: merge-path SpMM                                              */
+/* ------------------------------------------------------------------------ */
+
+/* Bytes of device workspace mps_spmm_f32 / mps_spmm_f16 need for P
+ * partitions, width K and threads_per_wave tpw (0 = as many as fit).  The
+ * workspace holds one carry-out record per wavefront (the partial sums of
+ * the rows that cross its boundaries); it needs no initialisation. */
+int mps_spmm_workspace_bytes(int P, int K, int tpw, int elem_bytes, size_t *bytes_out);
+
+/* Y = A * X with A in CSR (row_ptr, col_idx, val), fp32.
+ * Replaces the launch loops and kernels spmm_merge_path / spmm_merge_path_64
+ * (src/MergePathSpMM.cu:223-264, :388-574) with explicit edge values in place
+ * of the degree product (:450,:459-460).
+ *   P, d_coord_x, d_coord_y  partition count and coordinates from mps_partition
+ *   tpw                      partitions per wavefront, 1..mps_max_threads_per_wave,
+ *                            or 0 for the maximum (argv[4] of the reference CLI, :122)
+ * Rows that lie inside one partition are stored once; rows that cross
+ * partition or wavefront boundaries are completed from carry-out records by
+ * a second small kernel -- no atomics, deterministic. */
+int mps_spmm_f32(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
+                 const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
+                 const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                 size_t workspace_bytes, void *stream);
+
+/* fp16 values and features, fp32 accumulation, fp16 result.
+ * Replaces src/MergePathSpMM_fp16.cu:224-265, :389-575 (which accumulates in
+ * half, :427-431,:460-461). */
+int mps_spmm_f16(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_val,
+                 const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K, int P,
+                 const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                 size_t workspace_bytes, void *stream);
+
+/* The same two entry points with the kernels selectable, for per-kernel
+ * timing: phases bit 0 = the main kernel, bit 1 = the carry-out fix-up. */
+#define MPS_PHASE_MAIN 1u
+#define MPS_PHASE_FIXUP 2u
+int mps_spmm_f32_phases(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
+                        const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
+                        const int *d_coord_x, const int *d_coord_y, int tpw,
+                        void *d_workspace, size_t workspace_bytes, unsigned phases,
+                        void *stream);
+int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_val,
+                        const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K, int P,
+                        const int *d_coord_x, const int *d_coord_y, int tpw,
+                        void *d_workspace, size_t workspace_bytes, unsigned phases,
+                        void *stream);
+
+/* ------------------------------------------------------------------------ */
+/* Device side: comparison kernels                                           */
+/* ------------------------------------------------------------------------ */
+
+/* Row-wise split: wavefront w owns rows [int(step * w), int(step * (w + 1)))
+ * with float step = (float)n_rows / num_waves, the arithmetic of
+ * src/row_wise.cu:211-213; the last wavefront also takes any rows the float
+ * rounding leaves over.  Replaces run_spmm_row_wise / spmm_row_wise
+ * (src/row_wise.cu:172-240).  Any K; no workspace; plain stores. */
+int mps_rowwise_spmm_f32(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
+                         const float *d_X, float *d_Y, int n_rows, int nnz, int K, int num_waves,
+                         void *stream);
+
+/* Row ranges of mps_rowwise_spmm_f32 (host arrays int[num_waves]). */
+int mps_rowwise_bounds(int n_rows, int num_waves, int *row_start, int *row_end);
+
+/* Nonzero splitting ("GNNAdvisor-opt"): every row is cut into groups of at
+ * most part_size nonzeros.
+ * mps_nzsplit_max_parts: upper bound for sizing (nnz / part_size + n_rows).
+ * mps_nzsplit_build: replaces calculate_part_num + build_part
+ *   (src/nz_splitting.cu:256-316) on the device: d_part_ptr[num_parts + 1]
+ *   (first nonzero of each group, then nnz), d_part2node[num_parts];
+ *   *num_parts_out is written on the host after the stream is synchronised.
+ *   d_scratch: int[n_rows + 1 + 2048] device scratch. */
+int mps_nzsplit_max_parts(int n_rows, int nnz, int part_size, int *max_parts_out);
+int mps_nzsplit_build(const int *d_row_ptr, int n_rows, int part_size, int *d_part_ptr,
+                      int *d_part2node, int max_parts, int *d_scratch, int *num_parts_out,
+                      void *stream);
+/* Replaces spmm_forward_cuda_kernel / _64 (src/nz_splitting.cu:212-240,
+ * :318-445): one group per lane-group, column ids staged in LDS, every group
+ * ends in fp32 atomic adds into Y, which this call zeroes first.  The order
+ * of the atomic adds, and with it the last bits of Y, varies run to run. */
+int mps_nzsplit_spmm_f32(const int *d_col_idx, const float *d_val, const float *d_X,
+                         float *d_Y, int n_rows, int nnz, int K, const int *d_part_ptr,
+                         const int *d_part2node, int num_parts, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MPSPMM_H */

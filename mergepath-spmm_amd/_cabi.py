@@ -1,0 +1,98 @@
+"""ctypes binding of libmpspmm.so (include/mpspmm.h).
+
+The library is the product; there is no Python or CPU fallback.  If the
+shared object has not been built, loading raises and every operation fails.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmpspmm.so")
+
+MPS_OK = 0
+MPS_ERR_INVALID_ARG = 1
+MPS_ERR_UNSUPPORTED = 2
+MPS_ERR_WORKSPACE = 3
+MPS_ERR_ALIGNMENT = 4
+MPS_ERR_IO = 5
+MPS_ERR_FORMAT = 6
+MPS_ERR_TPW = 7
+MPS_ERR_INVALID_CSR = 8
+MPS_ERR_HIP = 1000
+
+MPS_PHASE_MAIN = 1
+MPS_PHASE_FIXUP = 2
+
+c_int_p = ctypes.POINTER(ctypes.c_int)
+_vp, _i, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64
+
+# name -> (restype, argtypes); one entry per declaration in include/mpspmm.h
+PROTOTYPES = {
+    "mps_status_string": (ctypes.c_char_p, [_i]),
+    "mps_version": (ctypes.c_char_p, []),
+    "mps_num_partitions": (_i, [_i, _i, _i, c_int_p]),
+    "mps_items_per_partition": (_i, [_i, _i, _i, c_int_p]),
+    "mps_max_threads_per_wave": (_i, [_i, _i, c_int_p]),
+    "mps_csr_read_header": (_i, [ctypes.c_char_p, c_int_p, c_int_p]),
+    "mps_csr_read": (_i, [ctypes.c_char_p, _i, _i, _vp, _vp]),
+    "mps_csr_write": (_i, [ctypes.c_char_p, _i, _vp, _vp]),
+    "mps_graph_generate": (_i, [ctypes.c_char_p, _u64, ctypes.POINTER(_vp)]),
+    "mps_graph_from_csr_file": (_i, [ctypes.c_char_p, ctypes.POINTER(_vp)]),
+    "mps_graph_dims": (_i, [_vp, c_int_p, c_int_p, c_int_p]),
+    "mps_graph_row_ptr": (_vp, [_vp]),
+    "mps_graph_col_idx": (_vp, [_vp]),
+    "mps_graph_free": (None, [_vp]),
+    "mps_fill_uniform_f32": (_i, [_vp, _sz, _u64, ctypes.c_float, ctypes.c_float]),
+    "mps_fill_uniform_f16": (_i, [_vp, _sz, _u64, ctypes.c_float, ctypes.c_float]),
+    "mps_csr_validate": (_i, [_vp, _vp, _i, _i, _i, _vp]),
+    "mps_partition": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
+    "mps_schedule_legacy": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mps_spmm_workspace_bytes": (_i, [_i, _i, _i, _i, ctypes.POINTER(_sz)]),
+    "mps_spmm_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),
+    "mps_spmm_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),
+    "mps_spmm_f32_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
+                                 ctypes.c_uint, _vp]),
+    "mps_spmm_f16_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
+                                 ctypes.c_uint, _vp]),
+    "mps_rowwise_spmm_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "mps_rowwise_bounds": (_i, [_i, _i, _vp, _vp]),
+    "mps_nzsplit_max_parts": (_i, [_i, _i, _i, c_int_p]),
+    "mps_nzsplit_build": (_i, [_vp, _i, _i, _vp, _vp, _i, _vp, c_int_p, _vp]),
+    "mps_nzsplit_spmm_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp]),
+}
+
+
+class MpsError(RuntimeError):
+    """A C-ABI call returned a non-zero mps_status."""
+
+    def __init__(self, status, what=""):
+        self.status = int(status)
+        text = _lib.mps_status_string(self.status).decode() if _lib is not None else "?"
+        if self.status >= MPS_ERR_HIP:
+            text += " (hipError_t %d)" % (self.status - MPS_ERR_HIP)
+        super().__init__("%s: mps_status %d: %s" % (what or "libmpspmm", self.status, text))
+
+
+_lib = None
+
+
+def lib():
+    """The loaded shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libmpspmm.so is not built (%s): run `make -C mergepath-spmm_amd/csrc` or "
+                "__graft_entry__.build(); there is no fallback path" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status, what=""):
+    if status != MPS_OK:
+        raise MpsError(status, what)

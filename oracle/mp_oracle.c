@@ -1,0 +1,370 @@
+/*
+ * mp_oracle.c -- CPU restatement of the MergePath-SpMM reference algorithm.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library, the drivers or
+ * the Python package may link, load or call this file; it exists so that the
+ * tests (and the CPU-baseline leg of the benchmark) have an independent
+ * statement of what the reference computes.  Every function cites the
+ * reference lines (/root/reference/...) it follows.
+ *
+ * How each function is pinned (tests/test_oracle_*.py):
+ *   orc_num_partitions        integer formula, table of hand-computed values
+ *   orc_merge_path_search     literal loop; pinned against the closed form
+ *                             (lower bound of row_ptr[x]+x >= d), against a
+ *                             brute-force merge walk over every diagonal, and
+ *                             against three hand-worked coordinate lists
+ *   orc_generate_mp_sched     literal restatement; pinned by the tiling
+ *                             invariant (every nonzero covered at most once,
+ *                             the uncovered ones are exactly the
+ *                             zero-sentinel losses) and hand-worked cases
+ *   orc_spmm_f64 / _f16in     plain row loop; pinned by identity matrix,
+ *                             all-ones features, and scipy.sparse on fixtures
+ *   orc_spmm_mergepath_f32    reference kernel structure with explicit values;
+ *                             pinned against orc_spmm_f64
+ *   orc_rowwise_bounds        literal float arithmetic; hand-computed table
+ *   orc_build_part            literal restatement; tiling invariant
+ * The reference holds no tests, golden vectors or fixtures of its own, so
+ * parity with the reference itself is "parity unpinned" beyond these checks.
+ */
+#include <limits.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ---- src/MergePathSpMM.cu:138-139: cost -> number of partitions ---------- */
+int orc_num_partitions(int n_rows, int nnz, int cost)
+{
+    int node_act_num = n_rows + 1;
+    int num_threads = (node_act_num + nnz - 1) / cost;
+    if (num_threads < 1024) num_threads = 1024;
+    return num_threads;
+}
+
+/* ---- src/MergePathSpMM.cu:280-297: MergePathSearch ----------------------
+ * num_rows is the length of RP (= N+1, the whole row_ptr array, as the call
+ * sites at :333-334 pass NODE_ACT_NUM); NZ_INDICES[i] == i (:311-313) is
+ * materialised by the caller exactly as the reference does. */
+void orc_merge_path_search(int diagonal, const int *RP, const int *NZ_INDICES,
+                           int num_rows, int nnz, int *x_out, int *y_out)
+{
+    int x_min = diagonal - nnz > 0 ? diagonal - nnz : 0;
+    int x_max = diagonal < num_rows ? diagonal : num_rows;
+    while (x_min < x_max) {
+        int pivot = (x_min + x_max) >> 1;
+        if (RP[pivot] <= NZ_INDICES[diagonal - pivot - 1])
+            x_min = pivot + 1;
+        else
+            x_max = pivot;
+    }
+    *x_out = x_min < num_rows ? x_min : num_rows;
+    *y_out = diagonal - x_min;
+}
+
+/* Second, independent statement of the same split: the smallest x in
+ * [0, num_rows] with RP[x] + x >= diagonal (num_rows if there is none),
+ * found by a linear scan.  O(num_rows) per call: tiny inputs only. */
+void orc_merge_path_closed_form(int diagonal, const int *RP, int num_rows,
+                                int *x_out, int *y_out)
+{
+    int x = 0;
+    while (x < num_rows && (int64_t)RP[x] + x < diagonal) x++;
+    *x_out = x;
+    *y_out = diagonal - x;
+}
+
+/* Third statement: walk the merge of A = RP[0..num_rows) and B = 0..nnz-1
+ * one item at a time (take from A when A[x] <= B[y], else from B) and record
+ * the coordinate reached at every diagonal 0..num_rows+nnz. */
+void orc_merge_path_walk(const int *RP, int num_rows, int nnz, int *xs, int *ys)
+{
+    int x = 0, y = 0;
+    int total = num_rows + nnz;
+    for (int d = 0; d <= total; d++) {
+        xs[d] = x;
+        ys[d] = y;
+        if (d == total) break;
+        if (x < num_rows && (y >= nnz || RP[x] <= y))
+            x++;
+        else
+            y++;
+    }
+}
+
+/* Coordinates of the P+1 partition boundaries, diagonals chosen as in
+ * src/MergePathSpMM.cu:327-331. */
+void orc_partition_coords(const int *RP, int n_rows, int nnz, int P, int *xs, int *ys)
+{
+    int node_act_num = n_rows + 1;
+    int *nz = (int *)malloc(sizeof(int) * (size_t)(nnz > 0 ? nnz : 1));
+    for (int i = 0; i < nnz; i++) nz[i] = i;
+    int num_merge_items = node_act_num + nnz;
+    int items_per_thread = (num_merge_items + P - 1) / P;
+    for (int i = 0; i <= P; i++) {
+        int64_t d64 = (int64_t)items_per_thread * i;
+        int diagonal = d64 < num_merge_items ? (int)d64 : num_merge_items;
+        orc_merge_path_search(diagonal, RP, nz, node_act_num, nnz, &xs[i], &ys[i]);
+    }
+    free(nz);
+}
+
+/* ---- src/MergePathSpMM.cu:300-385: generate_mp_sched ---------------------
+ * Output order follows the arrays main() uploads (:209-220). */
+void orc_generate_mp_sched(const int *row_ptr, int n_rows, int nnz, int num_threads,
+                           int *feature_start_all, int *feature_start_num,
+                           int *feature_end_all, int *feature_end_num,
+                           int *start_row_all, int *end_row_all)
+{
+    int NODE_ACT_NUM = n_rows + 1;
+    int FEATURE_TOTAL = nnz;
+    int *NZ_INDICES = (int *)malloc(sizeof(int) * (size_t)(nnz > 0 ? nnz : 1));
+    for (int i = 0; i < FEATURE_TOTAL; i++) NZ_INDICES[i] = i;
+
+    for (int i = 0; i < num_threads; i++) {
+        int core_id = i;
+        int num_merge_items = NODE_ACT_NUM + FEATURE_TOTAL;
+        int items_per_thread = (num_merge_items + num_threads - 1) / num_threads;
+
+        int64_t d64 = (int64_t)items_per_thread * core_id;
+        int diagonal = d64 < num_merge_items ? (int)d64 : num_merge_items;
+        int diagonal_end = diagonal + items_per_thread < num_merge_items
+                               ? diagonal + items_per_thread : num_merge_items;
+
+        int cx, cy, ex, ey;
+        orc_merge_path_search(diagonal, row_ptr, NZ_INDICES, NODE_ACT_NUM, FEATURE_TOTAL, &cx, &cy);
+        orc_merge_path_search(diagonal_end, row_ptr, NZ_INDICES, NODE_ACT_NUM, FEATURE_TOTAL, &ex, &ey);
+
+        int start = cx - 1;
+        int end = ex - 1;
+        if (start < 0) start = 0;
+
+        int num_features = 0;
+        int feature_start = cy;
+        if (row_ptr[start] == feature_start) feature_start = 0;
+        if (core_id == 0) feature_start = 0;
+
+        int feature_end = ey;
+        if (row_ptr[end] == feature_end) feature_end = 0;
+
+        if (feature_start != 0) {
+            if (start == end && feature_end != 0) {
+                num_features = feature_end - feature_start;
+                feature_end = 0;
+            } else {
+                num_features = row_ptr[start + 1] - feature_start;
+            }
+        }
+        int num_features_end = 0;
+        if (feature_end != 0) {
+            num_features_end = feature_end - row_ptr[end];
+            feature_end = row_ptr[end];
+        }
+        feature_start_all[core_id] = feature_start;
+        feature_end_all[core_id] = feature_end;
+        feature_start_num[core_id] = num_features;
+        feature_end_num[core_id] = num_features_end;
+        start_row_all[core_id] = start;
+        end_row_all[core_id] = end;
+    }
+    free(NZ_INDICES);
+}
+
+/* ---- fp64 ground truth: Y = A * X, one row at a time ----------------------
+ * Explicit values replace the reference's on-the-fly degree product
+ * (src/MergePathSpMM.cu:450,459-460).  abs_out (optional) receives
+ * sum_j |a_ij * x_jk|, the scale the rounding-error bound is relative to. */
+void orc_spmm_f64(const int *row_ptr, const int *col_idx, const float *val,
+                  const float *X, int n_rows, int K, double *Y, double *abs_out)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int i = 0; i < n_rows; i++) {
+        double *y = Y + (size_t)i * K;
+        double *a = abs_out ? abs_out + (size_t)i * K : 0;
+        for (int k = 0; k < K; k++) { y[k] = 0.0; if (a) a[k] = 0.0; }
+        for (int e = row_ptr[i]; e < row_ptr[i + 1]; e++) {
+            double v = (double)val[e];
+            const float *x = X + (size_t)col_idx[e] * K;
+            for (int k = 0; k < K; k++) {
+                double t = v * (double)x[k];
+                y[k] += t;
+                if (a) a[k] += fabs(t);
+            }
+        }
+    }
+}
+
+/* IEEE binary16 bit pattern -> double (exact). */
+static double half_bits_to_double(uint16_t h)
+{
+    int sign = (h >> 15) & 1;
+    int exp = (h >> 10) & 0x1f;
+    int man = h & 0x3ff;
+    double v;
+    if (exp == 0)
+        v = ldexp((double)man, -24);
+    else if (exp == 31)
+        v = man ? NAN : INFINITY;
+    else
+        v = ldexp((double)(man | 0x400), exp - 25);
+    return sign ? -v : v;
+}
+
+double orc_half_to_double(uint16_t h) { return half_bits_to_double(h); }
+
+/* Same row loop for the fp16 variant (src/MergePathSpMM_fp16.cu:427-477 for
+ * structure): half values and features, result kept in fp64 (the comparison
+ * rounds the device's half output, not this). */
+void orc_spmm_f64_f16in(const int *row_ptr, const int *col_idx, const uint16_t *val,
+                        const uint16_t *X, int n_rows, int K, double *Y, double *abs_out)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int i = 0; i < n_rows; i++) {
+        double *y = Y + (size_t)i * K;
+        double *a = abs_out ? abs_out + (size_t)i * K : 0;
+        for (int k = 0; k < K; k++) { y[k] = 0.0; if (a) a[k] = 0.0; }
+        for (int e = row_ptr[i]; e < row_ptr[i + 1]; e++) {
+            double v = half_bits_to_double(val[e]);
+            const uint16_t *x = X + (size_t)col_idx[e] * K;
+            for (int k = 0; k < K; k++) {
+                double t = v * half_bits_to_double(x[k]);
+                y[k] += t;
+                if (a) a[k] += fabs(t);
+            }
+        }
+    }
+}
+
+/* ---- src/MergePathSpMM.cu:426-477 with explicit values --------------------
+ * The reference kernel's head / whole-rows / tail structure per partition,
+ * each running sum a sequential fp32 chain of rounded products (:441,:460,
+ * :474: the product is rounded by __fmaf_rn(a,b,0), then added).  Partial
+ * rows are combined in partition order instead of by atomicAdd_F (:54-59).
+ * Deliberately NOT reproduced: the zero-sentinel loss of a tail that starts
+ * at nonzero 0 (:366-369,:467) and the unit source weight of the tail
+ * (:468) -- with explicit values there is no source weight. */
+void orc_spmm_mergepath_f32(const int *row_ptr, const int *col_idx, const float *val,
+                            const float *X, int n_rows, int nnz, int K, int P, float *Y)
+{
+    int *xs = (int *)malloc(sizeof(int) * (size_t)(P + 1));
+    int *ys = (int *)malloc(sizeof(int) * (size_t)(P + 1));
+    orc_partition_coords(row_ptr, n_rows, nnz, P, xs, ys);
+    memset(Y, 0, sizeof(float) * (size_t)n_rows * K);
+    for (int p = 0; p < P; p++) {
+        int start = xs[p] - 1 < 0 ? 0 : xs[p] - 1;
+        int end = xs[p + 1] - 1;
+        int y = ys[p], y_end = ys[p + 1];
+        for (int row = start; row <= end && row < n_rows; row++) {
+            int lo = row_ptr[row] > y ? row_ptr[row] : y;
+            int hi = row_ptr[row + 1] < y_end ? row_ptr[row + 1] : y_end;
+            if (hi <= lo) continue;
+            for (int k = 0; k < K; k++) {
+                volatile float acc = 0.0f;
+                for (int e = lo; e < hi; e++) {
+                    volatile float prod = val[e] * X[(size_t)col_idx[e] * K + k];
+                    acc = acc + prod;
+                }
+                Y[(size_t)row * K + k] += acc;
+            }
+        }
+    }
+    free(xs);
+    free(ys);
+}
+
+/* ---- multithreaded fp32 CSR x dense: the timed CPU baseline ---------------
+ * Rows are cut into `threads` contiguous blocks of (nearly) equal nonzero
+ * count; the inner loop over K vectorises.  The reference has no CPU SpMM
+ * (its host code only builds the schedule), so this is a port of the same
+ * arithmetic, not of reference code. */
+void orc_spmm_f32_mt(const int *row_ptr, const int *col_idx, const float *val,
+                     const float *X, int n_rows, int K, float *Y, int threads)
+{
+    if (threads < 1) threads = 1;
+    int nnz = row_ptr[n_rows];
+    int *cut = (int *)malloc(sizeof(int) * (size_t)(threads + 1));
+    cut[0] = 0;
+    for (int t = 1; t < threads; t++) {
+        int64_t target = (int64_t)nnz * t / threads;
+        int lo = cut[t - 1], hi = n_rows;
+        while (lo < hi) {
+            int mid = lo + ((hi - lo) >> 1);
+            if (row_ptr[mid] < target) lo = mid + 1; else hi = mid;
+        }
+        cut[t] = lo;
+    }
+    cut[threads] = n_rows;
+#pragma omp parallel for num_threads(threads) schedule(static, 1)
+    for (int t = 0; t < threads; t++) {
+        for (int i = cut[t]; i < cut[t + 1]; i++) {
+            float *restrict y = Y + (size_t)i * K;
+            for (int k = 0; k < K; k++) y[k] = 0.0f;
+            for (int e = row_ptr[i]; e < row_ptr[i + 1]; e++) {
+                float v = val[e];
+                const float *restrict x = X + (size_t)col_idx[e] * K;
+                for (int k = 0; k < K; k++) y[k] += v * x[k];
+            }
+        }
+    }
+    free(cut);
+}
+
+int orc_max_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ---- src/row_wise.cu:211-213: row range of each warp ---------------------- */
+void orc_rowwise_bounds(int num_nodes, int num_warps, int *row_start, int *row_end)
+{
+    for (int warp_id = 0; warp_id < num_warps; warp_id++) {
+        float step = (float)num_nodes / num_warps;
+        row_start[warp_id] = (int)(step * warp_id);
+        row_end[warp_id] = (int)(step * (warp_id + 1));
+    }
+}
+
+/* ---- src/nz_splitting.cu:299-316: calculate_part_num ---------------------- */
+int orc_calculate_part_num(int partSize, const int *indptr, int num_nodes)
+{
+    int degree, thisNumParts, numParts = 0;
+    for (int i = 0; i < num_nodes; i++) {
+        degree = indptr[i + 1] - indptr[i];
+        if (degree % partSize == 0)
+            thisNumParts = degree / partSize;
+        else
+            thisNumParts = degree / partSize + 1;
+        numParts += thisNumParts;
+    }
+    return numParts;
+}
+
+/* ---- src/nz_splitting.cu:256-297: build_part ------------------------------
+ * partPtr has numParts+1 entries; the reference fills the last one only when
+ * the final row is non-empty (:292-293).  Here it is always set to
+ * indptr[num_nodes], which equals the reference's value whenever the
+ * reference defines it. */
+void orc_build_part(int partSize, const int *indptr, int num_nodes, int *partPtr, int *part2Node)
+{
+    int part_counter = 0;
+    for (int i = 0; i < num_nodes; i++) {
+        int degree = indptr[i + 1] - indptr[i];
+        int thisNumParts;
+        if (degree % partSize == 0)
+            thisNumParts = degree / partSize;
+        else
+            thisNumParts = degree / partSize + 1;
+        for (int pid = 0; pid < thisNumParts; pid++) {
+            int partBeg = indptr[i] + pid * partSize;
+            partPtr[part_counter] = partBeg;
+            part2Node[part_counter++] = i;
+        }
+    }
+    partPtr[part_counter] = indptr[num_nodes];
+}

@@ -1,0 +1,167 @@
+"""Merge-path SpMM on the GPU against the fp64 row loop of the oracle.
+
+Tolerances (stated by the task): fp32 within 1e-5 relative, 1e-6 absolute
+floor; fp16 within 2e-2 relative.  Where rows are long enough for their terms
+to cancel, "relative" is taken against sum_j |a_ij x_jk| (see gpu_util)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import check_fp32, make_csr, random_csr, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run_f32(pkg, dev, rp, ci, val, X, cost=None, P=None, tpw=0, poison=True):
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz, cost=cost, P=P)
+    out = torch.full_like(d_X, float("nan")) if poison else None
+    Y = pkg.spmm.spmm_merge_path(csr, d_X, sched, threads_per_wave=tpw, out=out)
+    torch.cuda.synchronize()
+    return Y.cpu().numpy(), sched
+
+
+def test_er_plumbing_config(pkg, orc, dev):
+    # BASELINE config 1: ER N=4096 deg 8, val U[0,1), X 4096x16 U[-1,1)
+    g = pkg.graphs
+    rp, ci, _ = g.generate(g.CONFIG_SPECS["er_4096"], seed=1)
+    n, K = rp.size - 1, 16
+    val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+    X = g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    for cost in (8, 32, 128):
+        Y, sched = run_f32(pkg, dev, rp, ci, val, X, cost=cost)
+        check_fp32(Y, ref, scale)
+    # the reference-structured fp32 walk of the oracle lands in the same place
+    Yo = orc.spmm_mergepath_f32(rp, ci, val, X, sched.P)
+    assert np.abs(Y - Yo).max() <= 1e-5
+
+
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 8, 12, 16, 20, 32, 48, 64, 100, 128, 256, 260, 512])
+def test_feature_widths(pkg, orc, dev, K):
+    rng = np.random.default_rng(K)
+    n = 500
+    rp, ci = random_csr(rng, n, 30, hub_rows=[(7, 400), (499, 333)])
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    for P in (1, 37, 1024):
+        Y, _ = run_f32(pkg, dev, rp, ci, val, X, P=P)
+        check_fp32(Y, ref, scale, rel_elem=False)
+
+
+def test_threads_per_wave(pkg, orc, dev):
+    rng = np.random.default_rng(5)
+    n, K = 700, 16
+    rp, ci = random_csr(rng, n, 40, hub_rows=[(0, 650)])
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    for tpw in (0, 1, 2, 3, 4, 7, 16):
+        Y, _ = run_f32(pkg, dev, rp, ci, val, X, cost=16, tpw=tpw)
+        check_fp32(Y, ref, scale, rel_elem=False)
+    with pytest.raises(pkg.MpsError) as e:
+        run_f32(pkg, dev, rp, ci, val, X, cost=16, tpw=17)
+    assert e.value.status == pkg._cabi.MPS_ERR_TPW
+
+
+def test_edge_shapes(pkg, orc, dev):
+    rng = np.random.default_rng(6)
+    K = 16
+    cases = {
+        # first row longer than a partition: the tail the reference's zero sentinel drops
+        "long_first_row": np.array([300, 0, 0, 1, 2, 0]),
+        "one_giant_row": np.array([0, 0, 5000, 0]),
+        "all_empty": np.zeros(50, dtype=np.int64),
+        "single_row": np.array([9]),
+        "partial_last_row": np.array([1, 1, 1, 1, 777]),
+        "single_nonzero": np.array([0, 1, 0]),
+    }
+    for name, deg in cases.items():
+        n = max(int(deg.size), int(deg.max()) if deg.size else 1, 1)
+        n = max(n, 16)
+        deg_full = np.zeros(n, dtype=np.int64)
+        deg_full[: deg.size] = deg
+        rp = np.concatenate([[0], np.cumsum(deg_full)]).astype(np.int32)
+        ci = np.concatenate([np.sort(rng.choice(n, size=int(d), replace=False)) for d in deg_full] +
+                            [np.zeros(0, dtype=np.int64)]).astype(np.int32)
+        val = rng.random(ci.size).astype(np.float32)
+        X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+        ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+        for P in (1, 2, 7, 64, 1024, n + 1 + int(rp[-1]) + 5):
+            Y, _ = run_f32(pkg, dev, rp, ci, val, X, P=P)
+            check_fp32(Y, ref, scale, rel_elem=False)
+            assert (Y[deg_full == 0] == 0).all(), name
+
+
+def test_closed_forms(pkg, dev):
+    n, K = 3000, 16
+    rng = np.random.default_rng(8)
+    # A = I  ->  Y = X exactly
+    rp = np.arange(n + 1, dtype=np.int32)
+    ci = np.arange(n, dtype=np.int32)
+    X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+    Y, _ = run_f32(pkg, dev, rp, ci, np.ones(n, dtype=np.float32), X, cost=16)
+    assert np.array_equal(Y, X)
+    # X = 1  ->  Y[i, :] = sum of row i's values
+    rp, ci = random_csr(rng, n, 64, hub_rows=[(100, 2500)])
+    val = rng.random(ci.size).astype(np.float32)
+    Y, _ = run_f32(pkg, dev, rp, ci, val, np.ones((n, K), dtype=np.float32), cost=32)
+    rows = np.add.reduceat(np.concatenate([val.astype(np.float64), [0.0]]), rp[:-1])
+    rows[np.diff(rp) == 0] = 0.0
+    assert np.abs(Y - rows[:, None]).max() <= 1e-5 * max(rows.max(), 1.0)
+    assert (Y == Y[:, :1]).all()
+
+
+def test_deterministic_and_overwrites(pkg, dev):
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=20000,nnz=2000000,gamma=2.1,dmax=4000", seed=3)
+    n, K = rp.size - 1, 16
+    val = g.fill_uniform_f32(ci.size, 1, 0.0, 1.0)
+    X = g.fill_uniform_f32(n * K, 2, -1.0, 1.0).reshape(n, K)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz, cost=64)
+    out = torch.full_like(d_X, float("nan"))
+    first = pkg.spmm.spmm_merge_path(csr, d_X, sched, out=out).clone()
+    for _ in range(3):  # repeat launches as the reference's loop does (:231-243): same bits every time
+        again = pkg.spmm.spmm_merge_path(csr, d_X, sched, out=out)
+        assert torch.equal(first, again)
+    assert torch.isfinite(first).all()
+
+
+def test_benchmark_graphs_reduced(pkg, orc, dev):
+    g = pkg.graphs
+    for spec, K, cost in (("blockdiag:blocks=1178,min=100,max=600,deg=5", 16, 32),
+                          ("rmat:scale=17,ef=16,a=0.57,b=0.19,c=0.19", 64, 128),
+                          ("chunglu:n=60000,nnz=12000000,gamma=2.1,dmax=8000", 16, 128)):
+        rp, ci, _ = g.generate(spec, seed=1)
+        n = rp.size - 1
+        val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+        X = g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)
+        ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+        Y, _ = run_f32(pkg, dev, rp, ci, val, X, cost=cost)
+        check_fp32(Y, ref, scale, rel_elem=False)
+
+
+def test_rejects_bad_arguments(pkg, dev):
+    rp = np.array([0, 2, 3, 4], dtype=np.int32)
+    ci = np.array([1, 2, 0, 1], dtype=np.int32)
+    val = np.ones(4, dtype=np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    X = torch.ones(3, 16, device=dev)
+    sched = pkg.spmm.generate_mp_sched(csr.row_ptr, 4, cost=4)
+    L, c = pkg._cabi.lib(), pkg._cabi
+    import ctypes
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    Y = torch.empty_like(X)
+    ws = sched.workspace(16, 0, 4)
+    base = [p(csr.row_ptr), p(csr.col_idx), p(csr.val), p(X), p(Y), 3, 4, 16, sched.P, p(sched.coord_x), p(sched.coord_y), 0]
+    assert L.mps_spmm_f32(*base, p(ws), 8, None) == c.MPS_ERR_WORKSPACE
+    assert L.mps_spmm_f32(*base, None, ws.numel(), None) == c.MPS_ERR_WORKSPACE
+    mis = base[:]
+    mis[3] = ctypes.c_void_p(X.data_ptr() + 4)
+    assert L.mps_spmm_f32(*mis, p(ws), ws.numel(), None) == c.MPS_ERR_ALIGNMENT
+    assert L.mps_spmm_f32(*base, p(ws), ws.numel(), None) == 0
+    torch.cuda.synchronize()

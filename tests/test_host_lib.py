@@ -1,0 +1,194 @@
+"""Host half of the C ABI, no GPU: exported symbols, schedule arithmetic,
+.csr text I/O, generators, fills."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "mpspmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b(mps_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_every_declared_symbol_is_exported(pkg):
+    names = declared_functions()
+    assert len(names) >= 25
+    handle = ctypes.CDLL(pkg._cabi.LIB_PATH)
+    for name in names:
+        assert hasattr(handle, name), name
+    assert sorted(pkg._cabi.PROTOTYPES) == names
+
+
+def test_status_strings(pkg):
+    L = pkg._cabi.lib()
+    assert L.mps_status_string(0) == b"ok"
+    seen = {L.mps_status_string(i) for i in range(0, 9)}
+    assert len(seen) == 9
+    assert b"HIP" in L.mps_status_string(1000 + 2)
+    assert re.match(rb"\d+\.\d+\.\d+", L.mps_version())
+
+
+def test_num_partitions_matches_oracle(pkg, orc):
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        n, nnz, cost = int(rng.integers(0, 10 ** 6)), int(rng.integers(0, 10 ** 8)), int(rng.integers(1, 4096))
+        assert pkg.graphs.num_partitions(n, nnz, cost) == orc.num_partitions(n, nnz, cost)
+    for bad in (0, -5):
+        with pytest.raises(pkg.MpsError) as e:
+            pkg.graphs.num_partitions(10, 10, bad)
+        assert e.value.status == pkg._cabi.MPS_ERR_INVALID_ARG
+    with pytest.raises(pkg.MpsError) as e:
+        pkg.graphs.num_partitions(2 ** 30, 2 ** 30 + 5, 16)
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+    assert pkg.graphs.items_per_partition(6, 15, 5) == 5
+
+
+def test_max_threads_per_wave(pkg):
+    table = {(16, 4): 16, (32, 4): 8, (64, 4): 4, (128, 4): 2, (256, 4): 1, (512, 4): 1, (8, 4): 8, (1, 4): 16,
+             (20, 4): 8, (17, 4): 2, (64, 2): 8, (32, 2): 16, (16, 2): 4, (128, 2): 4}
+    for (K, eb), want in table.items():
+        assert pkg.graphs.max_threads_per_wave(K, eb) == want, (K, eb)
+
+
+def test_rowwise_bounds_follow_reference_arithmetic(pkg, orc):
+    for n, w in ((10, 4), (7, 3), (3, 5), (232965, 4096), (1048576, 999), (5, 1)):
+        s, e = pkg.graphs.rowwise_bounds(n, w)
+        os_, oe = orc.rowwise_bounds(n, w)
+        assert np.array_equal(s, np.minimum(os_, n))
+        # the library differs from src/row_wise.cu:211-213 only in closing the last range at n_rows
+        assert np.array_equal(e[:-1], np.minimum(oe[:-1], n)) and e[-1] == n
+        assert s[0] == 0 and np.array_equal(s[1:], e[:-1])
+
+
+def test_csr_text_fixtures(pkg):
+    g = pkg.graphs
+    for name in ("tiny_trailing_comma.csr", "tiny_no_trailing_comma.csr"):
+        assert g.read_csr_header(os.path.join(GOLDEN, name)) == (3, 4)
+        rp, ci, md = g.read_csr(os.path.join(GOLDEN, name))
+        assert rp.tolist() == [0, 2, 3, 4] and ci.tolist() == [1, 2, 0, 1] and md == 2
+    rp, ci, md = g.read_csr(os.path.join(GOLDEN, "empty_rows_final_newline.csr"))
+    assert rp.tolist() == [0, 0, 2, 2, 2, 3] and ci.tolist() == [0, 4, 1]
+    rp, ci, md = g.read_csr(os.path.join(GOLDEN, "single_row.csr"))
+    assert rp.tolist() == [0, 1] and ci.tolist() == [0]
+    rp, ci, md = g.read_csr(os.path.join(GOLDEN, "single_row_dups.csr"))
+    assert rp.tolist() == [0, 3] and ci.tolist() == [0, 0, 0]
+    for name in ("bad_decreasing.csr", "bad_cell.csr", "bad_short_cols.csr"):
+        with pytest.raises(pkg.MpsError) as e:
+            g.read_csr(os.path.join(GOLDEN, name))
+        assert e.value.status == pkg._cabi.MPS_ERR_FORMAT, name
+    with pytest.raises(pkg.MpsError) as e:
+        g.read_csr(os.path.join(GOLDEN, "does_not_exist.csr"))
+    assert e.value.status == pkg._cabi.MPS_ERR_IO
+
+
+def test_csr_write_layout_and_round_trip(pkg, tmp_path):
+    g = pkg.graphs
+    rp, ci, _ = g.generate("er:n=300,deg=6", seed=3)
+    path = tmp_path / "g.csr"
+    g.write_csr(path, rp, ci)
+    text = path.read_text()
+    # byte layout of scripts/npz_to_csr.py:21-28
+    assert text == "".join("%d," % v for v in rp) + "\n" + "".join("%d," % v for v in ci)
+    rp2, ci2, _ = g.read_csr(path)
+    assert np.array_equal(rp, rp2) and np.array_equal(ci, ci2)
+    assert g.read_csr_header(path) == (300, ci.size)
+
+
+def rows_sorted_distinct(rp, ci):
+    d = np.diff(ci.astype(np.int64))
+    ok = np.ones(max(ci.size - 1, 0), dtype=bool)
+    ends = rp[1:-1] - 1
+    ends = ends[(ends >= 0) & (ends < ci.size - 1)]
+    ok[ends] = False
+    return bool((d[ok] > 0).all())
+
+
+def test_generators_shape_and_determinism(pkg):
+    g = pkg.graphs
+    rp, ci, md = g.generate(g.CONFIG_SPECS["er_4096"], seed=1)
+    n = rp.size - 1
+    assert n == 4096 and abs(ci.size / n - 8.0) < 0.3 and rows_sorted_distinct(rp, ci)
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    assert not (rows == ci).any()  # no self-loops
+    rp2, ci2, _ = g.generate(g.CONFIG_SPECS["er_4096"], seed=1)
+    assert np.array_equal(rp, rp2) and np.array_equal(ci, ci2)
+    rp3, ci3, _ = g.generate(g.CONFIG_SPECS["er_4096"], seed=2)
+    assert not np.array_equal(ci, ci3[: ci.size]) or ci.size != ci3.size
+
+    rp, ci, md = g.generate("chunglu:n=20000,nnz=800000,gamma=2.1,dmax=2000", seed=1)
+    assert rp.size - 1 == 20000 and abs(ci.size - 800000) < 0.02 * 800000
+    assert rows_sorted_distinct(rp, ci) and 1000 < md <= 2300 and ci.max() < 20000 and ci.min() >= 0
+    deg = np.diff(rp)
+    assert deg.max() > 20 * np.median(deg)  # heavy tail
+
+    rp, ci, md = g.generate("blockdiag:blocks=40,min=100,max=600,deg=5", seed=1)
+    n = rp.size - 1
+    assert 40 * 100 <= n <= 40 * 600 and abs(ci.size / n - 5.0) < 0.6 and rows_sorted_distinct(rp, ci)
+    A = set(zip(np.repeat(np.arange(n), np.diff(rp)).tolist(), ci.tolist()))
+    assert all((j, i) in A for (i, j) in list(A)[:2000])  # undirected
+
+    rp, ci, md = g.generate("rmat:scale=12,ef=16,a=0.57,b=0.19,c=0.19", seed=1)
+    assert rp.size - 1 == 4096 and 0.5 * 65536 < ci.size <= 65536 and rows_sorted_distinct(rp, ci)
+
+    for bad in ("nosuch:n=3", "er:n=abc", "er:n", "rmat:scale=40"):
+        with pytest.raises(pkg.MpsError) as e:
+            g.generate(bad, 1)
+        assert e.value.status == pkg._cabi.MPS_ERR_FORMAT, bad
+
+
+def test_generators_do_not_depend_on_thread_count(pkg):
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import __graft_entry__ as e, hashlib\n"
+        "g = e.load_package().graphs\n"
+        "h = hashlib.sha256()\n"
+        "for s in ('er:n=3000,deg=8', 'chunglu:n=5000,nnz=200000,gamma=2.1,dmax=800',\n"
+        "          'blockdiag:blocks=9,min=100,max=300,deg=5', 'rmat:scale=11,ef=8,a=0.57,b=0.19,c=0.19'):\n"
+        "    rp, ci, _ = g.generate(s, 5); h.update(rp.tobytes()); h.update(ci.tobytes())\n"
+        "h.update(g.fill_uniform_f32(100000, 3, -1.0, 1.0).tobytes())\n"
+        "print(h.hexdigest())\n" % ROOT)
+    digests = []
+    for threads in ("1", "5"):
+        env = dict(os.environ, MPS_HOST_THREADS=threads)
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True)
+        digests.append(out.stdout.strip())
+    assert digests[0] == digests[1] and len(digests[0]) == 64
+
+
+def test_fills(pkg):
+    g = pkg.graphs
+    v = g.fill_uniform_f32(200000, 11, 0.0, 1.0)
+    assert v.dtype == np.float32 and v.min() >= 0.0 and v.max() < 1.0 and abs(v.mean() - 0.5) < 0.01
+    x = g.fill_uniform_f32(200000, 13, -1.0, 1.0)
+    assert x.min() >= -1.0 and x.max() < 1.0 and abs(x.mean()) < 0.01
+    assert np.array_equal(v[:1000], g.fill_uniform_f32(1000, 11, 0.0, 1.0))  # element i depends on (seed, i) only
+    h = g.fill_uniform_f16(200000, 11, 0.0, 1.0)
+    assert h.dtype == np.float16 and h.min() >= 0 and h.max() < 1.0 and abs(float(h.astype(np.float32).mean()) - 0.5) < 0.01
+    hx = g.fill_uniform_f16(200000, 13, -1.0, 1.0)
+    assert hx.min() >= -1.0 and hx.max() < 1.0
+    assert len(np.unique(hx)) > 1500
+
+
+def test_device_entry_points_reject_bad_arguments_without_a_gpu(pkg):
+    # argument checks come before any HIP call, so these run on a CPU-only box
+    L, c = pkg._cabi.lib(), pkg._cabi
+    nb = ctypes.c_size_t()
+    assert L.mps_spmm_workspace_bytes(1024, 16, 0, 4, ctypes.byref(nb)) == 0
+    assert nb.value == 64 * 4 + 2 * 64 * 16 * 4
+    assert L.mps_spmm_workspace_bytes(1024, 16, 17, 4, ctypes.byref(nb)) == c.MPS_ERR_TPW
+    assert L.mps_spmm_workspace_bytes(1024, 16, 0, 3, ctypes.byref(nb)) == c.MPS_ERR_INVALID_ARG
+    assert L.mps_partition(None, 4, 4, 8, None, None, None) == c.MPS_ERR_INVALID_ARG
+    assert L.mps_spmm_f32(None, None, None, None, None, 4, 4, 16, 8, None, None, 0, None, 0, None) == c.MPS_ERR_INVALID_ARG
+    mp = ctypes.c_int()
+    assert L.mps_nzsplit_max_parts(10, 100, 8, ctypes.byref(mp)) == 0 and mp.value == 22
+    assert L.mps_nzsplit_max_parts(10, 100, 0, ctypes.byref(mp)) == c.MPS_ERR_INVALID_ARG
