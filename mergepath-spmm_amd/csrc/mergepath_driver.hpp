@@ -1,0 +1,99 @@
+// main() of MergePathSpMM and MergePathSpMM_fp16, templated on the element
+// type.  Command line of src/MergePathSpMM.cu:114-124:
+//   <input_file> <dimension> <cost> <threads_per_wave> <repeat>
+#ifndef MPS_MERGEPATH_DRIVER_HPP
+#define MPS_MERGEPATH_DRIVER_HPP
+
+#include "driver_common.hpp"
+
+namespace drv {
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr const char *name = "fp32";
+    static int fill(float *p, size_t n, uint64_t seed, float lo, float hi) { return mps_fill_uniform_f32(p, n, seed, lo, hi); }
+    static int spmm(const int *rp, const int *ci, const float *v, const float *X, float *Y, int n, int nnz, int K, int P,
+                    const int *cx, const int *cy, int tpw, void *ws, size_t wsb)
+    { return mps_spmm_f32(rp, ci, v, X, Y, n, nnz, K, P, cx, cy, tpw, ws, wsb, nullptr); }
+};
+template <> struct Elem<uint16_t> {
+    static constexpr const char *name = "fp16";
+    static int fill(uint16_t *p, size_t n, uint64_t seed, float lo, float hi) { return mps_fill_uniform_f16(p, n, seed, lo, hi); }
+    static int spmm(const int *rp, const int *ci, const uint16_t *v, const uint16_t *X, uint16_t *Y, int n, int nnz, int K,
+                    int P, const int *cx, const int *cy, int tpw, void *ws, size_t wsb)
+    { return mps_spmm_f16(rp, ci, v, X, Y, n, nnz, K, P, cx, cy, tpw, ws, wsb, nullptr); }
+};
+
+template <typename T>
+int mergepath_main(int argc, char **argv)
+{
+    Options opt;
+    std::vector<std::string> pos = split_args(argc, argv, opt);
+    if (pos.size() < 5) {
+        std::cout << "Usage: ./application <input_file> <dimension> <cost> <threads_per_wave> <repeat>" << std::endl;
+        std::exit(-1);
+    }
+    const int dimension = std::atoi(pos[1].c_str());
+    const int cost = parse_cost(pos[2]);
+    int threads_per_wave = std::atoi(pos[3].c_str());
+    const int repeats = std::atoi(pos[4].c_str());
+    if (dimension < 1) die("dimension must be positive");
+    if (cost < 0) die("cost must be positive");
+
+    Graph gr;
+    load_graph(pos[0], opt.seed, gr);
+    const int N = gr.n_rows, nnz = gr.nnz, K = dimension;
+
+    int max_tpw = 0;
+    mps_ok(mps_max_threads_per_wave(K, (int)sizeof(T), &max_tpw), "mps_max_threads_per_wave");
+    // "64" (or 0) asks for a full wavefront; otherwise the bound of src/MergePathSpMM.cu:224-228
+    if (threads_per_wave == 0 || threads_per_wave == 64) threads_per_wave = max_tpw;
+    if (threads_per_wave < 1 || threads_per_wave > max_tpw) {
+        std::cout << "Cannot process the given number of threads withing a warp." << std::endl;
+        std::cout << "Max threads per warp can be " << max_tpw << std::endl;
+        std::exit(-1);
+    }
+
+    int P = 0, ipt = 0;
+    mps_ok(mps_num_partitions(N, nnz, cost, &P), "mps_num_partitions");
+    mps_ok(mps_items_per_partition(N, nnz, P, &ipt), "mps_items_per_partition");
+
+    std::vector<T> h_val((size_t)nnz), h_X((size_t)N * K), h_Y((size_t)N * K);
+    mps_ok(Elem<T>::fill(h_val.data(), h_val.size(), kSeedVal, 0.0f, 1.0f), "fill val");
+    mps_ok(Elem<T>::fill(h_X.data(), h_X.size(), kSeedX, -1.0f, 1.0f), "fill X");
+
+    DevBuf<int> d_rp((size_t)N + 1), d_ci((size_t)nnz), d_cx((size_t)P + 1), d_cy((size_t)P + 1);
+    DevBuf<T> d_val((size_t)nnz), d_X((size_t)N * K), d_Y((size_t)N * K);
+    d_rp.upload(mps_graph_row_ptr(gr.g));
+    d_ci.upload(mps_graph_col_idx(gr.g));
+    d_val.upload(h_val.data());
+    d_X.upload(h_X.data());
+    mps_ok(mps_csr_validate(d_rp.p, d_ci.p, N, N, nnz, nullptr), "mps_csr_validate");
+
+    size_t ws_bytes = 0;
+    mps_ok(mps_spmm_workspace_bytes(P, K, threads_per_wave, (int)sizeof(T), &ws_bytes), "mps_spmm_workspace_bytes");
+    DevBuf<unsigned char> d_ws(ws_bytes);
+
+    // the schedule is built once, outside the repeat loop, as generate_mp_sched is (:192)
+    Timing plan = time_launches(1, 3, [&] { mps_ok(mps_partition(d_rp.p, N, nnz, P, d_cx.p, d_cy.p, nullptr), "mps_partition"); });
+
+    hip_ok(hipMemset(d_Y.p, 0xff, d_Y.n * sizeof(T)), "hipMemset");
+    Timing t = time_launches(opt.warmup, repeats, [&] {
+        mps_ok(Elem<T>::spmm(d_rp.p, d_ci.p, d_val.p, d_X.p, d_Y.p, N, nnz, K, P, d_cx.p, d_cy.p, threads_per_wave, d_ws.p,
+                             ws_bytes), "mps_spmm");
+    });
+    d_Y.download(h_Y.data());
+    double checksum = finish_output(h_Y, N, K, opt);
+
+    std::printf("partitions: %d (cost %d, %d merge items each), threads_per_wave %d, max row degree %d\n", P, cost, ipt,
+                threads_per_wave, gr.max_degree);
+    std::printf("partitioner: avg %.2f us per build (not in the launch time below)\n", plan.avg_us);
+    char extra[256];
+    std::snprintf(extra, sizeof extra, ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan_us\": %.3f", P, cost,
+                  threads_per_wave, plan.avg_us);
+    report("merge_path", Elem<T>::name, N, nnz, K, (int)sizeof(T), (int)sizeof(T), repeats, t, checksum, extra);
+    return 0;
+}
+
+}  // namespace drv
+#endif
