@@ -25,7 +25,8 @@
  *   - fp16 data is IEEE binary16 passed as uint16_t bit patterns.
  *   - Y is overwritten (Y = A * X); results do not depend on what Y held and
  *     repeated calls give identical bits (merge-path and row-wise kernels).
- *   - d_col_idx, d_val, d_X and d_Y must be 16-byte aligned.
+ *   - d_X, d_Y and workspaces must be 16-byte aligned; index and value
+ *     arrays need only their natural alignment.
  */
 #ifndef MPSPMM_H
 #define MPSPMM_H
@@ -47,6 +48,7 @@ typedef enum mps_status {
     MPS_ERR_FORMAT = 6,       /* malformed .csr text or generator spec            */
     MPS_ERR_TPW = 7,          /* threads_per_wave beyond what one wave can hold   */
     MPS_ERR_INVALID_CSR = 8,  /* device-side validation found a bad row_ptr/col   */
+    MPS_ERR_UNSORTED = 9,     /* tiling needs column ids sorted within every row  */
     MPS_ERR_HIP = 1000        /* + hipError_t                                     */
 } mps_status;
 
@@ -204,6 +206,7 @@ int mps_spmm_f16(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_v
  * timing: phases bit 0 = the main kernel, bit 1 = the carry-out fix-up. */
 #define MPS_PHASE_MAIN 1u
 #define MPS_PHASE_FIXUP 2u
+#define MPS_PHASE_REDUCE 4u /* tiled entry points only */
 int mps_spmm_f32_phases(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
                         const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
                         const int *d_coord_x, const int *d_coord_y, int tpw,
@@ -214,6 +217,67 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
                         const int *d_coord_x, const int *d_coord_y, int tpw,
                         void *d_workspace, size_t workspace_bytes, unsigned phases,
                         void *stream);
+
+/* ------------------------------------------------------------------------ */
+/* Device side: column-slab tiling of the merge-path SpMM                    */
+/* ------------------------------------------------------------------------ */
+
+/* The reference has no counterpart of this section.  Its kernels gather the
+ * dense rows straight from global memory (src/MergePathSpMM.cu:459-460); on
+ * MI355X those gathers are served by the 4 MiB L2 of the XCD a wavefront runs
+ * on, and a feature matrix larger than that is bound by L2 misses.  Tiling
+ * reorders the nonzeros once per matrix -- like the schedule, outside the
+ * repeat loop (:192) -- so that the running wavefronts gather from one slab
+ * of X at a time:
+ *   - columns are cut into num_slabs slabs of slab_cols columns;
+ *   - virtual row v = s * n_rows + r holds the nonzeros of row r whose
+ *     column lies in slab s; the nonzeros are stored in virtual-row order
+ *     (d_col_tiled, d_val_tiled) with row pointers d_vrow_ptr;
+ *   - the same merge-path partitioner and SpMM kernel run over the
+ *     num_slabs * n_rows virtual rows (call mps_num_partitions and
+ *     mps_partition with n_rows := num_slabs * n_rows and d_vrow_ptr), writing
+ *     fp32 partial rows into the workspace;
+ *   - a last kernel adds the num_slabs partial rows of every row in slab
+ *     order (deterministic) and writes Y.
+ *
+ * mps_tile_shape: slab count and width for an X of n_rows x K elements
+ *   (slab_bytes = 0: 2 MiB slabs).  num_slabs == 1 means tiling does not pay
+ *   (X fits in L2, or rows hold too few nonzeros per slab): use mps_spmm_f32.
+ * mps_tile_build: builds d_vrow_ptr[num_slabs * n_rows + 1], d_col_tiled[nnz]
+ *   and d_perm[nnz] (tiled position -> original nonzero index).  d_scratch:
+ *   int[num_slabs * n_rows + 2049].  Synchronises the stream; returns
+ *   MPS_ERR_UNSORTED when some row's column ids are not non-decreasing.
+ * mps_tile_gather_values: d_val_tiled[i] = d_val[d_perm[i]]; call again
+ *   whenever the values change. */
+int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,
+                   int *slab_cols_out);
+int mps_tile_build(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int num_slabs,
+                   int slab_cols, int *d_vrow_ptr, int *d_col_tiled, int *d_perm, int *d_scratch,
+                   void *stream);
+int mps_tile_gather_values(const void *d_val, const int *d_perm, int nnz, int elem_bytes,
+                           void *d_val_tiled, void *stream);
+/* Workspace = fp32 partial rows (num_slabs * n_rows * K) + carry-out records. */
+int mps_spmm_tiled_workspace_bytes(int n_rows, int num_slabs, int P, int K, int tpw, int elem_bytes,
+                                   size_t *bytes_out);
+/* Y = A * X from the tiled arrays.  P, d_coord_x, d_coord_y: partition of the
+ * virtual rows.  Same arithmetic and tolerance as mps_spmm_f32 / mps_spmm_f16
+ * (fp32 accumulation; the summation order differs). */
+int mps_spmm_tiled_f32(const int *d_vrow_ptr, const int *d_col_tiled, const float *d_val_tiled,
+                       const float *d_X, float *d_Y, int n_rows, int nnz, int K, int num_slabs, int P,
+                       const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                       size_t workspace_bytes, void *stream);
+int mps_spmm_tiled_f16(const int *d_vrow_ptr, const int *d_col_tiled, const uint16_t *d_val_tiled,
+                       const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K, int num_slabs,
+                       int P, const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                       size_t workspace_bytes, void *stream);
+int mps_spmm_tiled_f32_phases(const int *d_vrow_ptr, const int *d_col_tiled, const float *d_val_tiled,
+                              const float *d_X, float *d_Y, int n_rows, int nnz, int K, int num_slabs,
+                              int P, const int *d_coord_x, const int *d_coord_y, int tpw,
+                              void *d_workspace, size_t workspace_bytes, unsigned phases, void *stream);
+int mps_spmm_tiled_f16_phases(const int *d_vrow_ptr, const int *d_col_tiled, const uint16_t *d_val_tiled,
+                              const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K,
+                              int num_slabs, int P, const int *d_coord_x, const int *d_coord_y, int tpw,
+                              void *d_workspace, size_t workspace_bytes, unsigned phases, void *stream);
 
 /* ------------------------------------------------------------------------ */
 /* Device side: comparison kernels                                           */

@@ -18,10 +18,12 @@ MPS_ERR_IO = 5
 MPS_ERR_FORMAT = 6
 MPS_ERR_TPW = 7
 MPS_ERR_INVALID_CSR = 8
+MPS_ERR_UNSORTED = 9
 MPS_ERR_HIP = 1000
 
 MPS_PHASE_MAIN = 1
 MPS_PHASE_FIXUP = 2
+MPS_PHASE_REDUCE = 4
 
 c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp, _i, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64
@@ -54,6 +56,16 @@ PROTOTYPES = {
                                  ctypes.c_uint, _vp]),
     "mps_spmm_f16_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
                                  ctypes.c_uint, _vp]),
+    "mps_tile_shape": (_i, [_i, _i, _i, _i, _sz, c_int_p, c_int_p]),
+    "mps_tile_build": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "mps_tile_gather_values": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
+    "mps_spmm_tiled_workspace_bytes": (_i, [_i, _i, _i, _i, _i, _i, ctypes.POINTER(_sz)]),
+    "mps_spmm_tiled_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),
+    "mps_spmm_tiled_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),
+    "mps_spmm_tiled_f32_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
+                                       ctypes.c_uint, _vp]),
+    "mps_spmm_tiled_f16_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
+                                       ctypes.c_uint, _vp]),
     "mps_rowwise_spmm_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mps_rowwise_bounds": (_i, [_i, _i, _vp, _vp]),
     "mps_nzsplit_max_parts": (_i, [_i, _i, _i, c_int_p]),

@@ -634,11 +634,12 @@ const char *mps_status_string(int status)
     case MPS_ERR_INVALID_ARG: return "invalid argument";
     case MPS_ERR_UNSUPPORTED: return "unsupported size or shape";
     case MPS_ERR_WORKSPACE: return "workspace missing or too small";
-    case MPS_ERR_ALIGNMENT: return "device pointer not 16-byte aligned";
+    case MPS_ERR_ALIGNMENT: return "device pointer not sufficiently aligned";
     case MPS_ERR_IO: return "file cannot be opened, read or written";
     case MPS_ERR_FORMAT: return "malformed .csr text or generator spec";
     case MPS_ERR_TPW: return "threads_per_wave exceeds what one wavefront holds";
     case MPS_ERR_INVALID_CSR: return "CSR arrays failed validation";
+    case MPS_ERR_UNSORTED: return "column ids are not sorted within every row";
     default: break;
     }
     if (status >= MPS_ERR_HIP) return "HIP runtime error (status - 1000 is the hipError_t)";

@@ -6,17 +6,28 @@
 // K allows).  In the merge-path kernel every lane-group walks one partition
 // of the reference schedule (src/MergePathSpMM.cu:300-385): `cost` merge
 // items = row ends + nonzeros.  The group streams its col_idx / val run
-// through LDS in 16-nonzero windows (one coalesced 64-byte load per array per
-// window), gathers the 16 dense rows with 16-byte loads, and accumulates in
+// through LDS in 16-nonzero windows (one 64-byte load per array per window,
+// the next window prefetched into registers while the current one is
+// consumed), gathers the 16 dense rows with 16-byte loads, and accumulates in
 // fp32 registers.  Rows that end inside a partition after its first row end
 // are stored directly.  A group's first finished row and its unfinished last
 // row are partial: they are first combined across the groups of the
 // wavefront through LDS, and what still crosses the wavefront boundary is
 // written to a carry-out record that a second kernel folds in.  No atomics.
+//
+// Column-slab tiling.  The dense-row gathers are served by the L2 of the XCD
+// the wavefront runs on (4 MiB each); a feature matrix larger than that
+// misses to the fabric, whose request rate then bounds the kernel.  The tiled
+// entry points reorder the nonzeros slab-major (all rows of column slab 0,
+// then slab 1, ...), so that at any moment the running wavefronts gather from
+// one ~2 MiB slab of X, and run the same merge-path kernel over the resulting
+// num_slabs * n_rows "virtual rows"; a last kernel adds the per-slab partial
+// rows in slab order.
 #include <hip/hip_runtime.h>
 
 #include <climits>
 #include <cstdint>
+#include <cstdlib>
 
 #include "mpspmm.h"
 #include "mpspmm_internal.h"
@@ -34,6 +45,12 @@ constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kWindow = 16;  // nonzeros staged per lane-group per round
 
 using half_t = _Float16;
+typedef half_t half8_t __attribute__((ext_vector_type(8)));
+typedef half_t half4_t __attribute__((ext_vector_type(4)));
+// 4-byte aligned 16-byte vectors: windows start at any nonzero index
+typedef int int4u_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef float float4u_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef half_t half4u_t __attribute__((ext_vector_type(4), aligned(2)));
 
 // LDS traffic here is private to one wavefront (each wave owns its slice), and
 // a wave's LDS operations execute in order, so a compiler-level barrier is all
@@ -46,7 +63,7 @@ __device__ __forceinline__ void wave_lds_sync()
 }
 
 // ---------------------------------------------------------------------------
-// Per-(element type, vector width) access to the dense matrices.
+// Per-(element type, vector width) access to the dense input.
 // ---------------------------------------------------------------------------
 template <typename T, int VEC>
 struct XOps;
@@ -54,7 +71,6 @@ struct XOps;
 template <>
 struct XOps<float, 4> {
     using Raw = float4;
-    static __device__ __forceinline__ Raw zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
     static __device__ __forceinline__ void fma(float (&acc)[4], float v, const Raw &r)
     {
         acc[0] = __builtin_fmaf(v, r.x, acc[0]);
@@ -62,93 +78,126 @@ struct XOps<float, 4> {
         acc[2] = __builtin_fmaf(v, r.z, acc[2]);
         acc[3] = __builtin_fmaf(v, r.w, acc[3]);
     }
-    static __device__ __forceinline__ void store(float *p, const float (&acc)[4])
-    {
-        *reinterpret_cast<float4 *>(p) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    }
 };
 
 template <>
 struct XOps<float, 1> {
     using Raw = float;
-    static __device__ __forceinline__ Raw zero() { return 0.f; }
     static __device__ __forceinline__ void fma(float (&acc)[1], float v, const Raw &r)
     {
         acc[0] = __builtin_fmaf(v, r, acc[0]);
     }
-    static __device__ __forceinline__ void store(float *p, const float (&acc)[1]) { *p = acc[0]; }
 };
-
-typedef half_t half8_t __attribute__((ext_vector_type(8)));
 
 template <>
 struct XOps<half_t, 8> {
     using Raw = half8_t;
-    static __device__ __forceinline__ Raw zero() { return Raw{0, 0, 0, 0, 0, 0, 0, 0}; }
     static __device__ __forceinline__ void fma(float (&acc)[8], float v, const Raw &r)
     {
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(v, (float)r[i], acc[i]);
-    }
-    static __device__ __forceinline__ void store(half_t *p, const float (&acc)[8])
-    {
-        Raw o;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = (half_t)acc[i];
-        *reinterpret_cast<Raw *>(p) = o;
     }
 };
 
 template <>
 struct XOps<half_t, 1> {
     using Raw = half_t;
-    static __device__ __forceinline__ Raw zero() { return (half_t)0; }
     static __device__ __forceinline__ void fma(float (&acc)[1], float v, const Raw &r)
     {
         acc[0] = __builtin_fmaf(v, (float)r, acc[0]);
     }
-    static __device__ __forceinline__ void store(half_t *p, const float (&acc)[1]) { *p = (half_t)acc[0]; }
 };
 
-template <bool WIDE>
-struct OffT {
-    using type = unsigned;
-};
-template <>
-struct OffT<true> {
-    using type = size_t;
+// VEC accumulators -> VEC adjacent outputs (fp32 or fp16), one vector store
+// where the width allows.
+template <int VEC>
+__device__ __forceinline__ void store_acc(float *p, const float (&acc)[VEC])
+{
+    if constexpr (VEC % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4)
+            *reinterpret_cast<float4 *>(p + i) = make_float4(acc[i], acc[i + 1], acc[i + 2], acc[i + 3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) p[i] = acc[i];
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void store_acc(half_t *p, const float (&acc)[VEC])
+{
+    if constexpr (VEC == 8) {
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (half_t)acc[i];
+        *reinterpret_cast<half8_t *>(p) = o;
+    } else if constexpr (VEC == 4) {
+        half4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (half_t)acc[i];
+        *reinterpret_cast<half4_t *>(p) = o;
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) p[i] = (half_t)acc[i];
+    }
+}
+
+// Address of the VEC columns a lane owns in row `c` of X.  POW2: the row
+// pitch is a power of two and the matrix is below 4 GiB, so the byte offset
+// is one shift-or in 32 bits (the load then takes its base from SGPRs).
+template <typename T, int VEC, bool POW2>
+struct Gather {
+    using Raw = typename XOps<T, VEC>::Raw;
+    const char *xb;
+    size_t row_bytes;
+    unsigned col_byte;
+    int row_shift;
+    __device__ __forceinline__ Raw load(int c) const
+    {
+        if constexpr (POW2) {
+            unsigned off = ((unsigned)c << row_shift) | col_byte;
+            return *reinterpret_cast<const Raw *>(xb + off);
+        } else {
+            size_t off = (size_t)c * row_bytes + col_byte;
+            return *reinterpret_cast<const Raw *>(xb + off);
+        }
+    }
 };
 
-// Four consecutive values (16-byte aligned for fp32, 8-byte for fp16) -> fp32.
-__device__ __forceinline__ float4 load_val4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+// Four consecutive nonzeros of a window, as registers.
+struct Win {
+    int4 c;
+    float4 v;
+};
+
+__device__ __forceinline__ float4 load_val4(const float *p)
+{
+    float4u_t t = __builtin_nontemporal_load(reinterpret_cast<const float4u_t *>(p));
+    return make_float4(t[0], t[1], t[2], t[3]);
+}
 __device__ __forceinline__ float4 load_val4(const half_t *p)
 {
-    typedef half_t half4_t __attribute__((ext_vector_type(4)));
-    half4_t h = *reinterpret_cast<const half4_t *>(p);
+    half4u_t h = __builtin_nontemporal_load(reinterpret_cast<const half4u_t *>(p));
     return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
 }
 
-// Stage the window [wbase, wbase + 16) of a lane-group's col_idx / val run
-// into its LDS slot: lanes 0..3 of the group each move 4 nonzeros.
+// Nonzeros [i0, i0 + 4) of col_idx / val (those below nnz).  The sparse
+// stream is read once: non-temporal loads keep it from displacing X in L2.
 template <typename T>
-__device__ __forceinline__ void stage_window(const int *__restrict__ col_idx, const T *__restrict__ val,
-                                             int nnz, int wbase, int s, int *s_col, float *s_val)
+__device__ __forceinline__ Win load_win(const int *__restrict__ col_idx, const T *__restrict__ val, int nnz, int i0)
 {
-    if (s < 4) {
-        int i0 = wbase + 4 * s;
-        int4 c = make_int4(0, 0, 0, 0);
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (i0 + 3 < nnz) {
-            c = *reinterpret_cast<const int4 *>(col_idx + i0);
-            v = load_val4(val + i0);
-        } else {
-            if (i0 + 0 < nnz) { c.x = col_idx[i0 + 0]; v.x = (float)val[i0 + 0]; }
-            if (i0 + 1 < nnz) { c.y = col_idx[i0 + 1]; v.y = (float)val[i0 + 1]; }
-            if (i0 + 2 < nnz) { c.z = col_idx[i0 + 2]; v.z = (float)val[i0 + 2]; }
-        }
-        *reinterpret_cast<int4 *>(s_col + 4 * s) = c;
-        *reinterpret_cast<float4 *>(s_val + 4 * s) = v;
+    Win w;
+    w.c = make_int4(0, 0, 0, 0);
+    w.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i0 + 3 < nnz) {
+        int4u_t t = __builtin_nontemporal_load(reinterpret_cast<const int4u_t *>(col_idx + i0));
+        w.c = make_int4(t[0], t[1], t[2], t[3]);
+        w.v = load_val4(val + i0);
+    } else {
+        if (i0 + 0 < nnz) { w.c.x = col_idx[i0 + 0]; w.v.x = (float)val[i0 + 0]; }
+        if (i0 + 1 < nnz) { w.c.y = col_idx[i0 + 1]; w.v.y = (float)val[i0 + 1]; }
+        if (i0 + 2 < nnz) { w.c.z = col_idx[i0 + 2]; w.v.z = (float)val[i0 + 2]; }
     }
+    return w;
 }
 
 // ---------------------------------------------------------------------------
@@ -223,16 +272,15 @@ __global__ __launch_bounds__(256) void mp_schedule_legacy_kernel(
 // ---------------------------------------------------------------------------
 // Merge-path SpMM, main kernel.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, bool WIDE, int BATCH>
+template <typename T, typename TOut, int VEC, bool POW2, int BATCH>
 __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
-    const T *__restrict__ X, T *__restrict__ Y, const int *__restrict__ coord_x,
+    const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
     const int *__restrict__ coord_y, int nnz, int K, int P, int lanes_log2, int tpw, int num_waves,
-    int *__restrict__ ws_head_row, float *__restrict__ ws_head, float *__restrict__ ws_tail)
+    int row_shift, int *__restrict__ ws_head_row, float *__restrict__ ws_head, float *__restrict__ ws_tail)
 {
     using XO = XOps<T, VEC>;
     using Raw = typename XO::Raw;
-    using off_t_ = typename OffT<WIDE>::type;
     constexpr int kCombine = 64 * VEC;  // floats per wave for heads (and for tails)
     constexpr int kSlice = (2 * kCombine > 2 * 16 * kWindow) ? 2 * kCombine : 2 * 16 * kWindow;
     __shared__ float s_buf[kWavesPerBlock][kSlice];
@@ -249,9 +297,9 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
     const int KT = L * VEC;  // columns covered by one pass of the wave
     const int kcol = blockIdx.y * KT + s * VEC;
     const bool col_ok = kcol < K;
-    const off_t_ row_bytes = (off_t_)K * (off_t_)sizeof(T);
-    const off_t_ col_byte = (off_t_)kcol * (off_t_)sizeof(T);
-    const char *xb = reinterpret_cast<const char *>(X);
+    // lanes beyond K gather column 0 (a valid address) and never store
+    const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
+                                  col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
 
     int *s_col = reinterpret_cast<int *>(&s_buf[wib][0]) + g * kWindow;
     float *s_val = &s_buf[wib][16 * kWindow] + g * kWindow;
@@ -266,7 +314,10 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
         y_end = coord_y[p + 1];
     }
     // Row x - 1 is in progress; it ends where nonzero index row_ptr[x] begins.
-    int row_end = (x < x_end) ? row_ptr[x] : INT_MAX;
+    // The two row ends after it are loaded ahead, so that finishing a row does
+    // not wait on memory.
+    auto row_end_at = [&](int xx) { return (xx < x_end) ? row_ptr[xx] : INT_MAX; };
+    int row_end = row_end_at(x), row_end1 = row_end_at(x + 1), row_end2 = row_end_at(x + 2);
 
     float acc[VEC], head[VEC];
 #pragma unroll
@@ -280,17 +331,28 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
 #pragma unroll
             for (int i = 0; i < VEC; ++i) head[i] = acc[i];
         } else if (col_ok) {
-            XO::store(Y + (size_t)row * K + kcol, acc);
+            store_acc<VEC>(Y + (size_t)row * K + kcol, acc);
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
         ++x;
-        row_end = (x < x_end) ? row_ptr[x] : INT_MAX;
+        row_end = row_end1;
+        row_end1 = row_end2;
+        row_end2 = row_end_at(x + 2);
     };
 
-    int wbase = y_begin & ~3;
+    int wbase = y_begin;
+    Win pw;
+    pw.c = make_int4(0, 0, 0, 0);
+    pw.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (s < 4 && wbase < y_end) pw = load_win<T>(col_idx, val, nnz, wbase + 4 * s);
+
     while (__any(wbase < y_end)) {
-        if (wbase < y_end) stage_window<T>(col_idx, val, nnz, wbase, s, s_col, s_val);
+        const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
+        if (s < 4 && nvalid > 0) {
+            *reinterpret_cast<int4 *>(s_col + 4 * s) = pw.c;
+            *reinterpret_cast<float4 *>(s_val + 4 * s) = pw.v;
+        }
         wave_lds_sync();
 #pragma unroll
         for (int b = 0; b < kWindow; b += BATCH) {
@@ -303,16 +365,17 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
                 vals[j] = s_val[b + j];
             }
 #pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const int idx = wbase + b + j;
-                const bool ok = col_ok && idx >= y_begin && idx < y_end;
-                xr[j] = XO::zero();
-                if (ok) xr[j] = *reinterpret_cast<const Raw *>(xb + ((off_t_)cols[j] * row_bytes + col_byte));
+            for (int j = 0; j < BATCH; ++j)
+                if (b + j < nvalid) xr[j] = gx.load(cols[j]);
+            if (b == 0) {
+                // next window: in flight while this one is consumed
+                const int nb = wbase + kWindow;
+                if (s < 4 && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
             }
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
-                const int idx = wbase + b + j;
-                if (idx >= y_begin && idx < y_end) {
+                if (b + j < nvalid) {
+                    const int idx = wbase + b + j;
                     while (idx == row_end) emit();
                     XO::fma(acc, vals[j], xr[j]);
                 }
@@ -350,7 +413,7 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
                     if (kc == 0) ws_head_row[w] = hr;
                     first = false;
                 } else if (kc_ok) {
-                    Y[(size_t)hr * K + kc] = (T)v;
+                    Y[(size_t)hr * K + kc] = (TOut)v;
                 }
                 carry = t;
             } else {
@@ -365,11 +428,11 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
 // Carry-out fix-up: the first row that ends inside wavefront w also received
 // nonzeros from the wavefronts before it, back to (and including) the nearest
 // one that itself saw a row end.
-template <typename T>
+template <typename TOut>
 __global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ ws_head_row,
                                                         const float *__restrict__ ws_head,
                                                         const float *__restrict__ ws_tail,
-                                                        T *__restrict__ Y, int num_waves, int K)
+                                                        TOut *__restrict__ Y, int num_waves, int K)
 {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long w64 = idx / K;
@@ -401,7 +464,7 @@ __global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ w
         if (done) break;
         j -= 4;
     }
-    Y[(size_t)hr * K + k] = (T)sum;
+    Y[(size_t)hr * K + k] = (TOut)sum;
 }
 
 // ---------------------------------------------------------------------------
@@ -409,20 +472,25 @@ __global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ w
 // Wave-uniform control flow: every group of the wave runs the same number of
 // rounds, idle ones with an empty range.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, bool WIDE, int BATCH>
+template <typename T, int VEC, bool POW2, int BATCH>
 __device__ __forceinline__ void accumulate_range(const int *__restrict__ col_idx,
-                                                 const T *__restrict__ val, const char *xb, int nnz,
-                                                 int y_begin, int y_end, bool col_ok,
-                                                 typename OffT<WIDE>::type row_bytes,
-                                                 typename OffT<WIDE>::type col_byte, int s, int *s_col,
+                                                 const T *__restrict__ val, const Gather<T, VEC, POW2> &gx,
+                                                 int nnz, int y_begin, int y_end, int s, int *s_col,
                                                  float *s_val, float (&acc)[VEC])
 {
     using XO = XOps<T, VEC>;
     using Raw = typename XO::Raw;
-    using off_t_ = typename OffT<WIDE>::type;
-    int wbase = y_begin & ~3;
+    int wbase = y_begin;
+    Win pw;
+    pw.c = make_int4(0, 0, 0, 0);
+    pw.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (s < 4 && wbase < y_end) pw = load_win<T>(col_idx, val, nnz, wbase + 4 * s);
     while (__any(wbase < y_end)) {
-        if (wbase < y_end) stage_window<T>(col_idx, val, nnz, wbase, s, s_col, s_val);
+        const int nvalid = min(kWindow, y_end - wbase);
+        if (s < 4 && nvalid > 0) {
+            *reinterpret_cast<int4 *>(s_col + 4 * s) = pw.c;
+            *reinterpret_cast<float4 *>(s_val + 4 * s) = pw.v;
+        }
         wave_lds_sync();
 #pragma unroll
         for (int b = 0; b < kWindow; b += BATCH) {
@@ -435,17 +503,15 @@ __device__ __forceinline__ void accumulate_range(const int *__restrict__ col_idx
                 vals[j] = s_val[b + j];
             }
 #pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const int idx = wbase + b + j;
-                const bool ok = col_ok && idx >= y_begin && idx < y_end;
-                xr[j] = XO::zero();
-                if (ok) xr[j] = *reinterpret_cast<const Raw *>(xb + ((off_t_)cols[j] * row_bytes + col_byte));
+            for (int j = 0; j < BATCH; ++j)
+                if (b + j < nvalid) xr[j] = gx.load(cols[j]);
+            if (b == 0) {
+                const int nb = wbase + kWindow;
+                if (s < 4 && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
             }
 #pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const int idx = wbase + b + j;
-                if (idx >= y_begin && idx < y_end) XO::fma(acc, vals[j], xr[j]);
-            }
+            for (int j = 0; j < BATCH; ++j)
+                if (b + j < nvalid) XO::fma(acc, vals[j], xr[j]);
         }
         wbase += kWindow;
         wave_lds_sync();
@@ -455,14 +521,12 @@ __device__ __forceinline__ void accumulate_range(const int *__restrict__ col_idx
 // Row-wise comparison kernel (src/row_wise.cu:194-240): wavefront w owns the
 // rows [int(step * w), int(step * (w + 1))); its lane-groups take those rows
 // round-robin, one whole row per group, plain stores.
-template <typename T, int VEC, bool WIDE, int BATCH>
+template <typename T, int VEC, bool POW2, int BATCH>
 __global__ __launch_bounds__(kBlock) void rowwise_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
     const T *__restrict__ X, T *__restrict__ Y, int n_rows, int nnz, int K, int lanes_log2,
-    int num_waves, float step)
+    int num_waves, int row_shift, float step)
 {
-    using XO = XOps<T, VEC>;
-    using off_t_ = typename OffT<WIDE>::type;
     __shared__ float s_buf[kWavesPerBlock][2 * 16 * kWindow];
     const int wib = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -475,9 +539,8 @@ __global__ __launch_bounds__(kBlock) void rowwise_spmm_kernel(
     const int KT = L * VEC;
     const int kcol = blockIdx.y * KT + s * VEC;
     const bool col_ok = kcol < K;
-    const off_t_ row_bytes = (off_t_)K * (off_t_)sizeof(T);
-    const off_t_ col_byte = (off_t_)kcol * (off_t_)sizeof(T);
-    const char *xb = reinterpret_cast<const char *>(X);
+    const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
+                                  col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
     int *s_col = reinterpret_cast<int *>(&s_buf[wib][0]) + g * kWindow;
     float *s_val = &s_buf[wib][16 * kWindow] + g * kWindow;
 
@@ -495,21 +558,19 @@ __global__ __launch_bounds__(kBlock) void rowwise_spmm_kernel(
         float acc[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-        accumulate_range<T, VEC, WIDE, BATCH>(col_idx, val, xb, nnz, y_begin, y_end, col_ok, row_bytes,
-                                               col_byte, s, s_col, s_val, acc);
-        if (row_ok && col_ok) XO::store(Y + (size_t)row * K + kcol, acc);
+        accumulate_range<T, VEC, POW2, BATCH>(col_idx, val, gx, nnz, y_begin, y_end, s, s_col, s_val, acc);
+        if (row_ok && col_ok) store_acc<VEC>(Y + (size_t)row * K + kcol, acc);
     }
 }
 
 // Nonzero-splitting comparison kernel (src/nz_splitting.cu:318-445): one
 // group of at most part_size nonzeros per lane-group, ending in atomic adds.
-template <typename T, int VEC, bool WIDE, int BATCH>
+template <typename T, int VEC, bool POW2, int BATCH>
 __global__ __launch_bounds__(kBlock) void nzsplit_spmm_kernel(
     const int *__restrict__ col_idx, const T *__restrict__ val, const T *__restrict__ X,
-    float *__restrict__ Y, int nnz, int K, int lanes_log2, const int *__restrict__ part_ptr,
-    const int *__restrict__ part2node, int num_parts, int num_waves)
+    float *__restrict__ Y, int nnz, int K, int lanes_log2, int row_shift,
+    const int *__restrict__ part_ptr, const int *__restrict__ part2node, int num_parts, int num_waves)
 {
-    using off_t_ = typename OffT<WIDE>::type;
     __shared__ float s_buf[kWavesPerBlock][2 * 16 * kWindow];
     const int wib = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -522,9 +583,8 @@ __global__ __launch_bounds__(kBlock) void nzsplit_spmm_kernel(
     const int KT = L * VEC;
     const int kcol = blockIdx.y * KT + s * VEC;
     const bool col_ok = kcol < K;
-    const off_t_ row_bytes = (off_t_)K * (off_t_)sizeof(T);
-    const off_t_ col_byte = (off_t_)kcol * (off_t_)sizeof(T);
-    const char *xb = reinterpret_cast<const char *>(X);
+    const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
+                                  col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
     int *s_col = reinterpret_cast<int *>(&s_buf[wib][0]) + g * kWindow;
     float *s_val = &s_buf[wib][16 * kWindow] + g * kWindow;
 
@@ -539,8 +599,7 @@ __global__ __launch_bounds__(kBlock) void nzsplit_spmm_kernel(
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-    accumulate_range<T, VEC, WIDE, BATCH>(col_idx, val, xb, nnz, y_begin, y_end, col_ok, row_bytes,
-                                           col_byte, s, s_col, s_val, acc);
+    accumulate_range<T, VEC, POW2, BATCH>(col_idx, val, gx, nnz, y_begin, y_end, s, s_col, s_val, acc);
     if (part_ok && col_ok) {
         float *y = Y + (size_t)row * K + kcol;
 #pragma unroll
@@ -558,18 +617,10 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(float4 *__restrict__ p4,
 }
 
 // ---------------------------------------------------------------------------
-// nz-splitting plan (src/nz_splitting.cu:256-316) on the device.
+// Exclusive prefix sum of an int array, in place (three launches).
 // ---------------------------------------------------------------------------
 constexpr int kScanThreads = 1024;
 constexpr int kScanMaxBlocks = 2048;
-
-__device__ __forceinline__ int parts_of_row(const int *__restrict__ row_ptr, int r, int n_rows,
-                                            int part_size)
-{
-    if (r >= n_rows) return 0;
-    int degree = row_ptr[r + 1] - row_ptr[r];
-    return degree / part_size + (degree % part_size != 0);
-}
 
 // Inclusive scan of one value per thread across a 1024-thread block.
 __device__ __forceinline__ int block_inclusive_scan(int v, int *s_wave /*[16]*/, int &block_total)
@@ -593,30 +644,28 @@ __device__ __forceinline__ int block_inclusive_scan(int v, int *s_wave /*[16]*/,
     return v + wave_off;
 }
 
-// phase 1: per-segment sums; phase 3: exclusive offsets written to out[0..n].
+// PHASE 1: per-segment sums.  PHASE 3: exclusive offsets written back.
 template <int PHASE>
-__global__ __launch_bounds__(kScanThreads) void nzsplit_scan_kernel(const int *__restrict__ row_ptr,
-                                                                    int n_rows, int part_size,
-                                                                    int seg_len, int *__restrict__ sums,
-                                                                    int *__restrict__ out)
+__global__ __launch_bounds__(kScanThreads) void scan_segments_kernel(int *__restrict__ data, int n, int seg_len,
+                                                                     int *__restrict__ sums)
 {
     __shared__ int s_wave[kScanThreads / 64];
     const int seg_begin = blockIdx.x * seg_len;
-    const int seg_end = min(seg_begin + seg_len, n_rows + 1);
+    const int seg_end = min(seg_begin + seg_len, n);
     int running = (PHASE == 3) ? sums[blockIdx.x] : 0;
     for (int base = seg_begin; base < seg_end; base += kScanThreads) {
-        const int r = base + threadIdx.x;
-        int v = (r < seg_end) ? parts_of_row(row_ptr, r, n_rows, part_size) : 0;
+        const int i = base + threadIdx.x;
+        int v = (i < seg_end) ? data[i] : 0;
         int total;
         int incl = block_inclusive_scan(v, s_wave, total);
-        if (PHASE == 3 && r < seg_end) out[r] = running + incl - v;
+        if (PHASE == 3 && i < seg_end) data[i] = running + incl - v;
         running += total;
     }
     if (PHASE == 1 && threadIdx.x == 0) sums[blockIdx.x] = running;
 }
 
-// phase 2: exclusive scan of the (<= 2048) segment sums in place.
-__global__ __launch_bounds__(kScanThreads) void nzsplit_scan_sums_kernel(int *__restrict__ sums, int nseg)
+// PHASE 2: exclusive scan of the (<= 2048) segment sums in place.
+__global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(int *__restrict__ sums, int nseg)
 {
     __shared__ int s_wave[kScanThreads / 64];
     int running = 0;
@@ -628,6 +677,38 @@ __global__ __launch_bounds__(kScanThreads) void nzsplit_scan_sums_kernel(int *__
         if (i < nseg) sums[i] = running + incl - v;
         running += total;
     }
+}
+
+// data[0..n) -> exclusive prefix sums; sums: int[2048] scratch.
+int scan_exclusive_inplace(int *data, int n, int *sums, hipStream_t st)
+{
+    if (n <= 0) return MPS_OK;
+    int nseg = (n + kScanThreads - 1) / kScanThreads;
+    if (nseg > kScanMaxBlocks) nseg = kScanMaxBlocks;
+    int seg_len = (n + nseg - 1) / nseg;
+    seg_len = (seg_len + kScanThreads - 1) / kScanThreads * kScanThreads;
+    nseg = (n + seg_len - 1) / seg_len;
+    hipLaunchKernelGGL((scan_segments_kernel<1>), dim3(nseg), dim3(kScanThreads), 0, st, data, n, seg_len, sums);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, st, sums, nseg);
+    hipLaunchKernelGGL((scan_segments_kernel<3>), dim3(nseg), dim3(kScanThreads), 0, st, data, n, seg_len, sums);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// nz-splitting plan (src/nz_splitting.cu:256-316) on the device.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void nzsplit_count_kernel(const int *__restrict__ row_ptr, int n_rows,
+                                                             int part_size, int *__restrict__ counts)
+{
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r > n_rows) return;
+    int c = 0;
+    if (r < n_rows) {
+        int degree = row_ptr[r + 1] - row_ptr[r];
+        c = degree / part_size + (degree % part_size != 0);
+    }
+    counts[r] = c;
 }
 
 // One thread per group: find its row by binary search in the offsets.
@@ -649,6 +730,111 @@ __global__ __launch_bounds__(256) void nzsplit_fill_kernel(const int *__restrict
     const int pid = t - offsets[lo];
     part_ptr[t] = row_ptr[lo] + pid * part_size;
     part2node[t] = lo;
+}
+
+// ---------------------------------------------------------------------------
+// Column-slab tiling plan.
+// ---------------------------------------------------------------------------
+// first[s * n_rows + r] = index of the first nonzero of row r whose column is
+// >= s * slab_cols; counts[...] = number of nonzeros of row r in slab s.
+__global__ __launch_bounds__(256) void tile_count_kernel(const int *__restrict__ row_ptr,
+                                                          const int *__restrict__ col_idx, int n_rows,
+                                                          int num_slabs, int slab_cols, int *__restrict__ first,
+                                                          int *__restrict__ counts)
+{
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long nv = (long long)num_slabs * n_rows;
+    if (t == nv) counts[nv] = 0;
+    if (t >= nv) return;
+    const int s = (int)(t / n_rows);
+    const int r = (int)(t - (long long)s * n_rows);
+    const int b = row_ptr[r], e = row_ptr[r + 1];
+    auto lower = [&](long long key) {
+        int lo = b, hi = e;
+        while (lo < hi) {
+            int mid = lo + ((hi - lo) >> 1);
+            if (col_idx[mid] < key) lo = mid + 1; else hi = mid;
+        }
+        return lo;
+    };
+    const int f0 = lower((long long)s * slab_cols);
+    const int f1 = (s + 1 == num_slabs) ? e : lower((long long)(s + 1) * slab_cols);
+    first[t] = f0;
+    counts[t] = f1 - f0;
+}
+
+// Flags a row whose column ids decrease somewhere (tiling needs sorted rows).
+__global__ __launch_bounds__(256) void tile_sorted_check_kernel(const int *__restrict__ row_ptr,
+                                                                 const int *__restrict__ col_idx, int n_rows,
+                                                                 int nnz, int *__restrict__ bad)
+{
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e + 1 >= nnz) return;
+    if (col_idx[e] <= col_idx[e + 1]) return;
+    // a decrease is fine only where nonzero e + 1 starts a row
+    int lo = 0, hi = n_rows;  // largest r with row_ptr[r] <= e + 1
+    while (lo < hi) {
+        int mid = (lo + hi + 1) >> 1;
+        if (row_ptr[mid] <= e + 1) lo = mid; else hi = mid - 1;
+    }
+    if (row_ptr[lo] != e + 1) atomicOr(bad, 1);
+}
+
+// One thread per nonzero: its place in the slab-major order.
+__global__ __launch_bounds__(256) void tile_scatter_kernel(const int *__restrict__ row_ptr,
+                                                            const int *__restrict__ col_idx, int n_rows, int nnz,
+                                                            int num_slabs, int slab_cols,
+                                                            const int *__restrict__ first,
+                                                            const int *__restrict__ vrow_ptr,
+                                                            int *__restrict__ col_tiled, int *__restrict__ perm)
+{
+    const long long e64 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e64 >= nnz) return;
+    const int e = (int)e64;
+    int lo = 0, hi = n_rows;  // largest r with row_ptr[r] <= e  (the row that holds nonzero e)
+    while (lo < hi) {
+        int mid = (lo + hi + 1) >> 1;
+        if (row_ptr[mid] <= e) lo = mid; else hi = mid - 1;
+    }
+    const int c = col_idx[e];
+    int s = c / slab_cols;
+    if (s >= num_slabs) s = num_slabs - 1;
+    const long long v = (long long)s * n_rows + lo;
+    const int dst = vrow_ptr[v] + (e - first[v]);
+    col_tiled[dst] = c;
+    perm[dst] = e;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tile_gather_values_kernel(const T *__restrict__ val,
+                                                                  const int *__restrict__ perm, int nnz,
+                                                                  T *__restrict__ out)
+{
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nnz) out[i] = val[perm[i]];
+}
+
+// Y[r] = sum over slabs, in slab order, of the partial rows part[s * n_rows + r].
+template <typename TOut, int VEC>
+__global__ __launch_bounds__(256) void tile_reduce_kernel(const float *__restrict__ part, TOut *__restrict__ Y,
+                                                           int n_rows, int K, int num_slabs)
+{
+    const size_t per_slab = (size_t)n_rows * K;
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (i >= per_slab) return;
+    float acc[VEC];
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) acc[u] = 0.f;
+    for (int s = 0; s < num_slabs; ++s) {
+        const float *p = part + (size_t)s * per_slab + i;
+        if constexpr (VEC == 4) {
+            float4 t = *reinterpret_cast<const float4 *>(p);
+            acc[0] += t.x; acc[1] += t.y; acc[2] += t.z; acc[3] += t.w;
+        } else {
+            acc[0] += p[0];
+        }
+    }
+    store_acc<VEC>(Y + i, acc);
 }
 
 // ---------------------------------------------------------------------------
@@ -678,13 +864,24 @@ __global__ __launch_bounds__(256) void csr_validate_kernel(const int *__restrict
 // ---------------------------------------------------------------------------
 // Launch helpers
 // ---------------------------------------------------------------------------
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned_to(const void *p, unsigned a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// log2 of the row pitch in bytes when the fast addressing applies, else -1.
+int pow2_row_shift(int n_rows, int K, int elem_bytes)
+{
+    uint64_t rb = (uint64_t)K * elem_bytes;
+    if (rb & (rb - 1)) return -1;
+    if ((uint64_t)(n_rows > 0 ? n_rows : 1) * rb >= (1ull << 32)) return -1;
+    int sh = 0;
+    while ((1ull << sh) < rb) ++sh;
+    return sh;
+}
 
 struct SpmmShape {
     mps_lane_shape ls;
     int tpw;
     int num_waves;
-    bool wide;
+    int row_shift;  // >= 0: power-of-two pitch, 32-bit offsets
 };
 
 int make_spmm_shape(int n_rows, int K, int P, int tpw, int elem_bytes, SpmmShape &sh)
@@ -695,24 +892,31 @@ int make_spmm_shape(int n_rows, int K, int P, int tpw, int elem_bytes, SpmmShape
     if (tpw > sh.ls.groups) return MPS_ERR_TPW;
     sh.tpw = tpw;
     sh.num_waves = (P + tpw - 1) / tpw;
-    sh.wide = (uint64_t)(n_rows > 0 ? n_rows : 1) * (uint64_t)K * (uint64_t)elem_bytes >= (1ull << 32);
+    sh.row_shift = pow2_row_shift(n_rows, K, elem_bytes);
     return MPS_OK;
 }
 
-size_t workspace_bytes_for(int num_waves, int K)
+size_t carry_bytes_for(int num_waves, int K)
 {
     size_t rows = ((size_t)num_waves + 63) / 64 * 64;
     return rows * sizeof(int) + 2 * (size_t)num_waves * K * sizeof(float);
 }
 
-constexpr int kBatch = 8;
-
-template <typename T, int VEC>
-int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X, T *Y, int n_rows,
-                int nnz, int K, int P, const int *cx, const int *cy, const SpmmShape &sh, void *ws,
-                unsigned phases, hipStream_t st)
+// Gathers in flight per lane between waits: tuning knob, 8 or 16.
+int gather_batch()
 {
-    (void)n_rows;
+    static int b = [] {
+        const char *e = std::getenv("MPS_GATHER_BATCH");
+        int v = e ? std::atoi(e) : 0;
+        return v == 16 ? 16 : 8;
+    }();
+    return b;
+}
+
+template <typename T, typename TOut, int VEC>
+int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X, TOut *Y, int nnz, int K, int P,
+                const int *cx, const int *cy, const SpmmShape &sh, void *ws, unsigned phases, hipStream_t st)
+{
     const int W = sh.num_waves;
     size_t rows = ((size_t)W + 63) / 64 * 64;
     int *ws_head_row = static_cast<int *>(ws);
@@ -720,48 +924,112 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
     float *ws_tail = ws_head + (size_t)W * K;
     if (phases & MPS_PHASE_MAIN) {
         dim3 grid((W + kWavesPerBlock - 1) / kWavesPerBlock, sh.ls.col_tiles);
-        if (sh.wide)
-            hipLaunchKernelGGL((mp_spmm_kernel<T, VEC, true, kBatch>), grid, dim3(kBlock), 0, st, row_ptr,
-                               col_idx, val, X, Y, cx, cy, nnz, K, P, sh.ls.lanes_log2, sh.tpw, W,
-                               ws_head_row, ws_head, ws_tail);
-        else
-            hipLaunchKernelGGL((mp_spmm_kernel<T, VEC, false, kBatch>), grid, dim3(kBlock), 0, st, row_ptr,
-                               col_idx, val, X, Y, cx, cy, nnz, K, P, sh.ls.lanes_log2, sh.tpw, W,
-                               ws_head_row, ws_head, ws_tail);
+#define MPS_LAUNCH_MAIN(POW2, BATCH)                                                                        \
+    hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH>), grid, dim3(kBlock), 0, st, row_ptr,     \
+                       col_idx, val, X, Y, cx, cy, nnz, K, P, sh.ls.lanes_log2, sh.tpw, W, sh.row_shift,    \
+                       ws_head_row, ws_head, ws_tail)
+        if (sh.row_shift >= 0) {
+            if (gather_batch() == 16) MPS_LAUNCH_MAIN(true, 16); else MPS_LAUNCH_MAIN(true, 8);
+        } else {
+            MPS_LAUNCH_MAIN(false, 8);
+        }
+#undef MPS_LAUNCH_MAIN
         MPS_HIP_TRY(hipGetLastError());
     }
     if (phases & MPS_PHASE_FIXUP) {
         long long threads = (long long)W * K;
         unsigned blocks = (unsigned)((threads + 255) / 256);
-        hipLaunchKernelGGL((mp_fixup_kernel<T>), dim3(blocks), dim3(256), 0, st, ws_head_row, ws_head,
-                           ws_tail, Y, W, K);
+        hipLaunchKernelGGL((mp_fixup_kernel<TOut>), dim3(blocks), dim3(256), 0, st, ws_head_row, ws_head, ws_tail,
+                           Y, W, K);
         MPS_HIP_TRY(hipGetLastError());
     }
     return MPS_OK;
 }
 
+template <typename T, typename TOut>
+int launch_spmm_any(const int *row_ptr, const int *col_idx, const T *val, const T *X, TOut *Y, int nnz, int K,
+                    int P, const int *cx, const int *cy, const SpmmShape &sh, void *ws, unsigned phases,
+                    hipStream_t st)
+{
+    if (sh.ls.vec == 1)
+        return launch_spmm<T, TOut, 1>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, sh, ws, phases, st);
+    return launch_spmm<T, TOut, 16 / (int)sizeof(T)>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, sh, ws, phases,
+                                                     st);
+}
+
 template <typename T>
-int spmm_entry(const int *row_ptr, const int *col_idx, const T *val, const T *X, T *Y, int n_rows,
-               int nnz, int K, int P, const int *cx, const int *cy, int tpw, void *ws, size_t ws_bytes,
-               unsigned phases, void *stream)
+int check_spmm_args(const int *row_ptr, const int *col_idx, const T *val, const T *X, const void *Y, int n_rows,
+                    long long n_vrows, int nnz, int K, int P, const int *cx, const int *cy)
 {
     if (n_rows < 0 || nnz < 0 || K < 1 || P < 1) return MPS_ERR_INVALID_ARG;
     if (!row_ptr || !cx || !cy || (nnz > 0 && (!col_idx || !val))) return MPS_ERR_INVALID_ARG;
     if (n_rows > 0 && (!X || !Y)) return MPS_ERR_INVALID_ARG;
-    if ((long long)n_rows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
+    if (n_vrows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
     if ((long long)P > INT_MAX / 2) return MPS_ERR_UNSUPPORTED;
-    if (!aligned16(col_idx) || !aligned16(val) || !aligned16(X) || !aligned16(Y)) return MPS_ERR_ALIGNMENT;
-    SpmmShape sh;
-    int rc = make_spmm_shape(n_rows, K, P, tpw, (int)sizeof(T), sh);
+    if (!aligned_to(col_idx, 4) || !aligned_to(val, sizeof(T)) || !aligned_to(X, 16) || !aligned_to(Y, 16))
+        return MPS_ERR_ALIGNMENT;
+    return MPS_OK;
+}
+
+template <typename T>
+int spmm_entry(const int *row_ptr, const int *col_idx, const T *val, const T *X, T *Y, int n_rows, int nnz, int K,
+               int P, const int *cx, const int *cy, int tpw, void *ws, size_t ws_bytes, unsigned phases,
+               void *stream)
+{
+    int rc = check_spmm_args<T>(row_ptr, col_idx, val, X, Y, n_rows, n_rows, nnz, K, P, cx, cy);
     if (rc != MPS_OK) return rc;
-    if ((long long)sh.num_waves * K > (1ll << 40)) return MPS_ERR_UNSUPPORTED;
-    if (!ws || ws_bytes < workspace_bytes_for(sh.num_waves, K)) return MPS_ERR_WORKSPACE;
-    if (!aligned16(ws)) return MPS_ERR_ALIGNMENT;
+    SpmmShape sh;
+    rc = make_spmm_shape(n_rows, K, P, tpw, (int)sizeof(T), sh);
+    if (rc != MPS_OK) return rc;
+    if (!ws || ws_bytes < carry_bytes_for(sh.num_waves, K)) return MPS_ERR_WORKSPACE;
+    if (!aligned_to(ws, 16)) return MPS_ERR_ALIGNMENT;
+    return launch_spmm_any<T, T>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, sh, ws, phases,
+                                 static_cast<hipStream_t>(stream));
+}
+
+// Tiled: the main kernel writes fp32 partial rows for the num_slabs * n_rows
+// virtual rows; the reduce kernel produces Y.
+size_t tiled_part_bytes(int n_rows, int num_slabs, int K)
+{
+    size_t b = (size_t)num_slabs * (size_t)n_rows * K * sizeof(float);
+    return (b + 255) / 256 * 256;
+}
+
+template <typename T>
+int spmm_tiled_entry(const int *vrow_ptr, const int *col_t, const T *val_t, const T *X, T *Y, int n_rows, int nnz,
+                     int K, int num_slabs, int P, const int *cx, const int *cy, int tpw, void *ws, size_t ws_bytes,
+                     unsigned phases, void *stream)
+{
+    if (num_slabs < 1) return MPS_ERR_INVALID_ARG;
+    const long long n_vrows = (long long)num_slabs * n_rows;
+    int rc = check_spmm_args<T>(vrow_ptr, col_t, val_t, X, Y, n_rows, n_vrows, nnz, K, P, cx, cy);
+    if (rc != MPS_OK) return rc;
+    SpmmShape sh;
+    rc = make_spmm_shape(n_rows, K, P, tpw, (int)sizeof(T), sh);
+    if (rc != MPS_OK) return rc;
+    const size_t part_b = tiled_part_bytes(n_rows, num_slabs, K);
+    if (!ws || ws_bytes < part_b + carry_bytes_for(sh.num_waves, K)) return MPS_ERR_WORKSPACE;
+    if (!aligned_to(ws, 16)) return MPS_ERR_ALIGNMENT;
+    if (n_rows == 0) return MPS_OK;
+    float *part = static_cast<float *>(ws);
+    void *carry = static_cast<char *>(ws) + part_b;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (sh.ls.vec == 1)
-        return launch_spmm<T, 1>(row_ptr, col_idx, val, X, Y, n_rows, nnz, K, P, cx, cy, sh, ws, phases, st);
-    return launch_spmm<T, 16 / (int)sizeof(T)>(row_ptr, col_idx, val, X, Y, n_rows, nnz, K, P, cx, cy, sh,
-                                               ws, phases, st);
+    rc = launch_spmm_any<T, float>(vrow_ptr, col_t, val_t, X, part, nnz, K, P, cx, cy, sh, carry, phases, st);
+    if (rc != MPS_OK) return rc;
+    if (phases & MPS_PHASE_REDUCE) {
+        const size_t per_slab = (size_t)n_rows * K;
+        if (K % 4 == 0) {
+            unsigned blocks = (unsigned)((per_slab / 4 + 255) / 256);
+            hipLaunchKernelGGL((tile_reduce_kernel<T, 4>), dim3(blocks), dim3(256), 0, st, part, Y, n_rows, K,
+                               num_slabs);
+        } else {
+            unsigned blocks = (unsigned)((per_slab + 255) / 256);
+            hipLaunchKernelGGL((tile_reduce_kernel<T, 1>), dim3(blocks), dim3(256), 0, st, part, Y, n_rows, K,
+                               num_slabs);
+        }
+        MPS_HIP_TRY(hipGetLastError());
+    }
+    return MPS_OK;
 }
 
 }  // namespace
@@ -836,7 +1104,7 @@ int mps_spmm_workspace_bytes(int P, int K, int tpw, int elem_bytes, size_t *byte
     SpmmShape sh;
     int rc = make_spmm_shape(1, K, P, tpw, elem_bytes, sh);
     if (rc != MPS_OK) return rc;
-    *bytes_out = workspace_bytes_for(sh.num_waves, K);
+    *bytes_out = carry_bytes_for(sh.num_waves, K);
     return MPS_OK;
 }
 
@@ -877,6 +1145,146 @@ int mps_spmm_f16(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_v
                                MPS_PHASE_MAIN | MPS_PHASE_FIXUP, stream);
 }
 
+// ---- column-slab tiling ---------------------------------------------------
+
+int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,
+                   int *slab_cols_out)
+{
+    if (!num_slabs_out || !slab_cols_out || n_rows < 0 || nnz < 0 || K < 1) return MPS_ERR_INVALID_ARG;
+    if (elem_bytes != 4 && elem_bytes != 2) return MPS_ERR_INVALID_ARG;
+    if (slab_bytes == 0) slab_bytes = 2u << 20;
+    const uint64_t row_b = (uint64_t)K * elem_bytes;
+    const uint64_t x_bytes = (uint64_t)n_rows * row_b;
+    int slabs = 1, cols = n_rows > 0 ? n_rows : 1;
+    // Worth it when X overflows one XCD's L2 (4 MiB) and the nonzeros of a row
+    // inside one slab still form runs long enough to stream (>= 8 on average).
+    if (x_bytes > (3u << 20) && n_rows > 0) {
+        uint64_t want = (x_bytes + slab_bytes - 1) / slab_bytes;
+        if (want > 4096) want = 4096;
+        uint64_t per = ((uint64_t)n_rows + want - 1) / want;
+        per = (per + 63) / 64 * 64;
+        uint64_t s2 = ((uint64_t)n_rows + per - 1) / per;
+        if ((double)nnz / ((double)n_rows * (double)s2) >= 8.0 &&
+            (uint64_t)s2 * n_rows + 1 + (uint64_t)nnz <= (uint64_t)INT_MAX) {
+            slabs = (int)s2;
+            cols = (int)per;
+        }
+    }
+    *num_slabs_out = slabs;
+    *slab_cols_out = cols;
+    return MPS_OK;
+}
+
+int mps_tile_build(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int num_slabs,
+                   int slab_cols, int *d_vrow_ptr, int *d_col_tiled, int *d_perm, int *d_scratch, void *stream)
+{
+    if (!d_row_ptr || !d_vrow_ptr || !d_scratch || n_rows < 0 || nnz < 0) return MPS_ERR_INVALID_ARG;
+    if (num_slabs < 1 || slab_cols < 1) return MPS_ERR_INVALID_ARG;
+    if (nnz > 0 && (!d_col_idx || !d_col_tiled || !d_perm)) return MPS_ERR_INVALID_ARG;
+    if ((long long)num_slabs * slab_cols < n_rows) return MPS_ERR_INVALID_ARG;
+    const long long nv = (long long)num_slabs * n_rows;
+    if (nv + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int *first = d_scratch;           // [nv]
+    int *sums = d_scratch + nv;       // [2048]
+    int *bad = sums + kScanMaxBlocks; // [1]
+    int zero = 0, h_bad = 0;
+    MPS_HIP_TRY(hipMemcpyAsync(bad, &zero, sizeof(int), hipMemcpyHostToDevice, st));
+    if (nnz > 1) {
+        unsigned blocks = (unsigned)(((long long)nnz + 255) / 256);
+        hipLaunchKernelGGL(tile_sorted_check_kernel, dim3(blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n_rows,
+                           nnz, bad);
+    }
+    {
+        unsigned blocks = (unsigned)((nv + 1 + 255) / 256);
+        hipLaunchKernelGGL(tile_count_kernel, dim3(blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n_rows,
+                           num_slabs, slab_cols, first, d_vrow_ptr);
+    }
+    MPS_HIP_TRY(hipGetLastError());
+    int rc = scan_exclusive_inplace(d_vrow_ptr, (int)nv + 1, sums, st);
+    if (rc != MPS_OK) return rc;
+    if (nnz > 0) {
+        unsigned blocks = (unsigned)(((long long)nnz + 255) / 256);
+        hipLaunchKernelGGL(tile_scatter_kernel, dim3(blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n_rows, nnz,
+                           num_slabs, slab_cols, first, d_vrow_ptr, d_col_tiled, d_perm);
+        MPS_HIP_TRY(hipGetLastError());
+    }
+    MPS_HIP_TRY(hipMemcpyAsync(&h_bad, bad, sizeof(int), hipMemcpyDeviceToHost, st));
+    MPS_HIP_TRY(hipStreamSynchronize(st));
+    return h_bad ? MPS_ERR_UNSORTED : MPS_OK;
+}
+
+int mps_tile_gather_values(const void *d_val, const int *d_perm, int nnz, int elem_bytes, void *d_val_tiled,
+                           void *stream)
+{
+    if (nnz < 0 || (elem_bytes != 4 && elem_bytes != 2)) return MPS_ERR_INVALID_ARG;
+    if (nnz == 0) return MPS_OK;
+    if (!d_val || !d_perm || !d_val_tiled) return MPS_ERR_INVALID_ARG;
+    unsigned blocks = (unsigned)(((long long)nnz + 255) / 256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (elem_bytes == 4)
+        hipLaunchKernelGGL((tile_gather_values_kernel<float>), dim3(blocks), dim3(256), 0, st,
+                           static_cast<const float *>(d_val), d_perm, nnz, static_cast<float *>(d_val_tiled));
+    else
+        hipLaunchKernelGGL((tile_gather_values_kernel<half_t>), dim3(blocks), dim3(256), 0, st,
+                           static_cast<const half_t *>(d_val), d_perm, nnz, static_cast<half_t *>(d_val_tiled));
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+int mps_spmm_tiled_workspace_bytes(int n_rows, int num_slabs, int P, int K, int tpw, int elem_bytes,
+                                   size_t *bytes_out)
+{
+    if (!bytes_out || n_rows < 0 || num_slabs < 1 || (elem_bytes != 4 && elem_bytes != 2))
+        return MPS_ERR_INVALID_ARG;
+    SpmmShape sh;
+    int rc = make_spmm_shape(n_rows, K, P, tpw, elem_bytes, sh);
+    if (rc != MPS_OK) return rc;
+    *bytes_out = tiled_part_bytes(n_rows, num_slabs, K) + carry_bytes_for(sh.num_waves, K);
+    return MPS_OK;
+}
+
+int mps_spmm_tiled_f32_phases(const int *d_vrow_ptr, const int *d_col_tiled, const float *d_val_tiled,
+                              const float *d_X, float *d_Y, int n_rows, int nnz, int K, int num_slabs, int P,
+                              const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                              size_t workspace_bytes, unsigned phases, void *stream)
+{
+    return spmm_tiled_entry<float>(d_vrow_ptr, d_col_tiled, d_val_tiled, d_X, d_Y, n_rows, nnz, K, num_slabs, P,
+                                   d_coord_x, d_coord_y, tpw, d_workspace, workspace_bytes, phases, stream);
+}
+
+int mps_spmm_tiled_f32(const int *d_vrow_ptr, const int *d_col_tiled, const float *d_val_tiled, const float *d_X,
+                       float *d_Y, int n_rows, int nnz, int K, int num_slabs, int P, const int *d_coord_x,
+                       const int *d_coord_y, int tpw, void *d_workspace, size_t workspace_bytes, void *stream)
+{
+    return spmm_tiled_entry<float>(d_vrow_ptr, d_col_tiled, d_val_tiled, d_X, d_Y, n_rows, nnz, K, num_slabs, P,
+                                   d_coord_x, d_coord_y, tpw, d_workspace, workspace_bytes,
+                                   MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE, stream);
+}
+
+int mps_spmm_tiled_f16_phases(const int *d_vrow_ptr, const int *d_col_tiled, const uint16_t *d_val_tiled,
+                              const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K, int num_slabs,
+                              int P, const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                              size_t workspace_bytes, unsigned phases, void *stream)
+{
+    return spmm_tiled_entry<half_t>(d_vrow_ptr, d_col_tiled, reinterpret_cast<const half_t *>(d_val_tiled),
+                                    reinterpret_cast<const half_t *>(d_X), reinterpret_cast<half_t *>(d_Y), n_rows,
+                                    nnz, K, num_slabs, P, d_coord_x, d_coord_y, tpw, d_workspace, workspace_bytes,
+                                    phases, stream);
+}
+
+int mps_spmm_tiled_f16(const int *d_vrow_ptr, const int *d_col_tiled, const uint16_t *d_val_tiled,
+                       const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K, int num_slabs, int P,
+                       const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
+                       size_t workspace_bytes, void *stream)
+{
+    return mps_spmm_tiled_f16_phases(d_vrow_ptr, d_col_tiled, d_val_tiled, d_X, d_Y, n_rows, nnz, K, num_slabs, P,
+                                     d_coord_x, d_coord_y, tpw, d_workspace, workspace_bytes,
+                                     MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE, stream);
+}
+
+// ---- comparison kernels -----------------------------------------------------
+
 int mps_rowwise_bounds(int n_rows, int num_waves, int *row_start, int *row_end)
 {
     if (n_rows < 0 || num_waves < 1 || !row_start || !row_end) return MPS_ERR_INVALID_ARG;
@@ -900,20 +1308,19 @@ int mps_rowwise_spmm_f32(const int *d_row_ptr, const int *d_col_idx, const float
     if (n_rows < 0 || nnz < 0 || K < 1 || num_waves < 1 || !d_row_ptr) return MPS_ERR_INVALID_ARG;
     if (nnz > 0 && (!d_col_idx || !d_val)) return MPS_ERR_INVALID_ARG;
     if (n_rows > 0 && (!d_X || !d_Y)) return MPS_ERR_INVALID_ARG;
-    if (!aligned16(d_col_idx) || !aligned16(d_val) || !aligned16(d_X) || !aligned16(d_Y))
+    if (!aligned_to(d_col_idx, 4) || !aligned_to(d_val, 4) || !aligned_to(d_X, 16) || !aligned_to(d_Y, 16))
         return MPS_ERR_ALIGNMENT;
     if (n_rows == 0) return MPS_OK;
     mps_lane_shape ls = mps_make_lane_shape(K, 4);
-    bool wide = (uint64_t)n_rows * (uint64_t)K * 4ull >= (1ull << 32);
+    const int row_shift = pow2_row_shift(n_rows, K, 4);
     float step = (float)n_rows / (float)num_waves;
     dim3 grid((num_waves + kWavesPerBlock - 1) / kWavesPerBlock, ls.col_tiles);
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define MPS_LAUNCH_ROWWISE(VEC, WIDE)                                                                    \
-    hipLaunchKernelGGL((rowwise_spmm_kernel<float, VEC, WIDE, kBatch>), grid, dim3(kBlock), 0, st,       \
-                       d_row_ptr, d_col_idx, d_val, d_X, d_Y, n_rows, nnz, K, ls.lanes_log2, num_waves,   \
-                       step)
-    if (ls.vec == 4) { if (wide) MPS_LAUNCH_ROWWISE(4, true); else MPS_LAUNCH_ROWWISE(4, false); }
-    else { if (wide) MPS_LAUNCH_ROWWISE(1, true); else MPS_LAUNCH_ROWWISE(1, false); }
+#define MPS_LAUNCH_ROWWISE(VEC, POW2)                                                                     \
+    hipLaunchKernelGGL((rowwise_spmm_kernel<float, VEC, POW2, 8>), grid, dim3(kBlock), 0, st, d_row_ptr,  \
+                       d_col_idx, d_val, d_X, d_Y, n_rows, nnz, K, ls.lanes_log2, num_waves, row_shift, step)
+    if (ls.vec == 4) { if (row_shift >= 0) MPS_LAUNCH_ROWWISE(4, true); else MPS_LAUNCH_ROWWISE(4, false); }
+    else { if (row_shift >= 0) MPS_LAUNCH_ROWWISE(1, true); else MPS_LAUNCH_ROWWISE(1, false); }
 #undef MPS_LAUNCH_ROWWISE
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
@@ -935,19 +1342,13 @@ int mps_nzsplit_build(const int *d_row_ptr, int n_rows, int part_size, int *d_pa
     if (n_rows < 0 || part_size < 1 || max_parts < 0) return MPS_ERR_INVALID_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int n = n_rows + 1;
-    int nseg = (n + kScanThreads - 1) / kScanThreads;
-    if (nseg > kScanMaxBlocks) nseg = kScanMaxBlocks;
-    int seg_len = (n + nseg - 1) / nseg;
-    seg_len = (seg_len + kScanThreads - 1) / kScanThreads * kScanThreads;
-    nseg = (n + seg_len - 1) / seg_len;
-    int *offsets = d_scratch;          // [n_rows + 1]
-    int *sums = d_scratch + n;         // [<= 2048]
-    hipLaunchKernelGGL((nzsplit_scan_kernel<1>), dim3(nseg), dim3(kScanThreads), 0, st, d_row_ptr, n_rows,
-                       part_size, seg_len, sums, offsets);
-    hipLaunchKernelGGL(nzsplit_scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, st, sums, nseg);
-    hipLaunchKernelGGL((nzsplit_scan_kernel<3>), dim3(nseg), dim3(kScanThreads), 0, st, d_row_ptr, n_rows,
-                       part_size, seg_len, sums, offsets);
+    int *offsets = d_scratch;   // [n_rows + 1]
+    int *sums = d_scratch + n;  // [2048]
+    hipLaunchKernelGGL(nzsplit_count_kernel, dim3((n + 255) / 256), dim3(256), 0, st, d_row_ptr, n_rows, part_size,
+                       offsets);
     MPS_HIP_TRY(hipGetLastError());
+    int rc = scan_exclusive_inplace(offsets, n, sums, st);
+    if (rc != MPS_OK) return rc;
     unsigned blocks = (unsigned)(((long long)max_parts + 255) / 256);
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(nzsplit_fill_kernel, dim3(blocks), dim3(256), 0, st, d_row_ptr, offsets, n_rows,
@@ -968,7 +1369,7 @@ int mps_nzsplit_spmm_f32(const int *d_col_idx, const float *d_val, const float *
     if (n_rows < 0 || nnz < 0 || K < 1 || num_parts < 0) return MPS_ERR_INVALID_ARG;
     if (n_rows > 0 && (!d_X || !d_Y)) return MPS_ERR_INVALID_ARG;
     if (num_parts > 0 && (!d_part_ptr || !d_part2node || !d_col_idx || !d_val)) return MPS_ERR_INVALID_ARG;
-    if (!aligned16(d_col_idx) || !aligned16(d_val) || !aligned16(d_X) || !aligned16(d_Y))
+    if (!aligned_to(d_col_idx, 4) || !aligned_to(d_val, 4) || !aligned_to(d_X, 16) || !aligned_to(d_Y, 16))
         return MPS_ERR_ALIGNMENT;
     if (n_rows == 0) return MPS_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -983,15 +1384,15 @@ int mps_nzsplit_spmm_f32(const int *d_col_idx, const float *d_val, const float *
     MPS_HIP_TRY(hipGetLastError());
     if (num_parts == 0) return MPS_OK;
     mps_lane_shape ls = mps_make_lane_shape(K, 4);
-    bool wide = (uint64_t)n_rows * (uint64_t)K * 4ull >= (1ull << 32);
+    const int row_shift = pow2_row_shift(n_rows, K, 4);
     int num_waves = (num_parts + ls.groups - 1) / ls.groups;
     dim3 grid((num_waves + kWavesPerBlock - 1) / kWavesPerBlock, ls.col_tiles);
-#define MPS_LAUNCH_NZSPLIT(VEC, WIDE)                                                                  \
-    hipLaunchKernelGGL((nzsplit_spmm_kernel<float, VEC, WIDE, kBatch>), grid, dim3(kBlock), 0, st,     \
-                       d_col_idx, d_val, d_X, d_Y, nnz, K, ls.lanes_log2, d_part_ptr, d_part2node,     \
+#define MPS_LAUNCH_NZSPLIT(VEC, POW2)                                                                    \
+    hipLaunchKernelGGL((nzsplit_spmm_kernel<float, VEC, POW2, 8>), grid, dim3(kBlock), 0, st, d_col_idx, \
+                       d_val, d_X, d_Y, nnz, K, ls.lanes_log2, row_shift, d_part_ptr, d_part2node,       \
                        num_parts, num_waves)
-    if (ls.vec == 4) { if (wide) MPS_LAUNCH_NZSPLIT(4, true); else MPS_LAUNCH_NZSPLIT(4, false); }
-    else { if (wide) MPS_LAUNCH_NZSPLIT(1, true); else MPS_LAUNCH_NZSPLIT(1, false); }
+    if (ls.vec == 4) { if (row_shift >= 0) MPS_LAUNCH_NZSPLIT(4, true); else MPS_LAUNCH_NZSPLIT(4, false); }
+    else { if (row_shift >= 0) MPS_LAUNCH_NZSPLIT(1, true); else MPS_LAUNCH_NZSPLIT(1, false); }
 #undef MPS_LAUNCH_NZSPLIT
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;

@@ -125,6 +125,92 @@ def spmm_merge_path(csr, X, sched, threads_per_wave=0, out=None, phases=None):
     return Y
 
 
+class TiledCsr:
+    """Column-slab tiled copy of a CSR matrix plus the merge-path schedule over
+    its virtual rows (mps_tile_build; no counterpart in the reference)."""
+
+    def __init__(self, csr, num_slabs, slab_cols, vrow_ptr, col_tiled, perm, val_tiled):
+        self.n_rows, self.nnz = csr.n_rows, csr.nnz
+        self.num_slabs, self.slab_cols = num_slabs, slab_cols
+        self.vrow_ptr, self.col_tiled, self.perm, self.val_tiled = vrow_ptr, col_tiled, perm, val_tiled
+        self.sched = None
+        self._ws = {}
+
+    def set_values(self, val):
+        """Re-gather the tiled values after the caller changed val."""
+        eb = 4 if val.dtype == torch.float32 else 2
+        check(_cabi.lib().mps_tile_gather_values(_ptr(val), _ptr(self.perm), self.nnz, eb, _ptr(self.val_tiled),
+                                                 _stream()), "mps_tile_gather_values")
+
+    def workspace(self, K, tpw, elem_bytes):
+        key = (K, tpw, elem_bytes)
+        if key not in self._ws:
+            nbytes = ctypes.c_size_t()
+            check(_cabi.lib().mps_spmm_tiled_workspace_bytes(self.n_rows, self.num_slabs, self.sched.P, K, tpw,
+                                                             elem_bytes, ctypes.byref(nbytes)),
+                  "mps_spmm_tiled_workspace_bytes")
+            self._ws[key] = torch.empty(max(int(nbytes.value), 16), dtype=torch.uint8, device=self.vrow_ptr.device)
+        return self._ws[key]
+
+
+def tile_shape(n_rows, nnz, K, elem_bytes=4, slab_bytes=0):
+    ns, sc = ctypes.c_int(), ctypes.c_int()
+    check(_cabi.lib().mps_tile_shape(int(n_rows), int(nnz), int(K), int(elem_bytes), int(slab_bytes),
+                                     ctypes.byref(ns), ctypes.byref(sc)), "mps_tile_shape")
+    return ns.value, sc.value
+
+
+def build_tiles(csr, K, cost=None, slab_bytes=0, num_slabs=None, slab_cols=None):
+    """Tile csr for feature width K and build the schedule over the virtual rows.
+    Returns None when tiling does not pay for this shape (unless slabs are forced)."""
+    eb = 4 if csr.val.dtype == torch.float32 else 2
+    if num_slabs is None:
+        num_slabs, slab_cols = tile_shape(csr.n_rows, csr.nnz, K, eb, slab_bytes)
+        if num_slabs <= 1:
+            return None
+    dev = csr.row_ptr.device
+    nv = num_slabs * csr.n_rows
+    vrow_ptr = torch.empty(nv + 1, dtype=torch.int32, device=dev)
+    col_tiled = torch.empty(max(csr.nnz, 1), dtype=torch.int32, device=dev)
+    perm = torch.empty(max(csr.nnz, 1), dtype=torch.int32, device=dev)
+    scratch = torch.empty(nv + 2049, dtype=torch.int32, device=dev)
+    check(_cabi.lib().mps_tile_build(_ptr(csr.row_ptr), _ptr(csr.col_idx), csr.n_rows, csr.nnz, num_slabs, slab_cols,
+                                     _ptr(vrow_ptr), _ptr(col_tiled), _ptr(perm), _ptr(scratch), _stream()),
+          "mps_tile_build")
+    del scratch
+    val_tiled = torch.empty(max(csr.nnz, 1), dtype=csr.val.dtype, device=dev)
+    t = TiledCsr(csr, num_slabs, slab_cols, vrow_ptr, col_tiled, perm, val_tiled)
+    t.set_values(csr.val)
+    t.sched = generate_mp_sched(vrow_ptr, csr.nnz, cost=cost)
+    return t
+
+
+def spmm_merge_path_tiled(tiled, X, threads_per_wave=0, out=None, phases=None):
+    """Y = A @ X from the tiled arrays (mps_spmm_tiled_f32 / _f16)."""
+    dtype = X.dtype
+    if dtype not in (torch.float32, torch.float16) or tiled.val_tiled.dtype != dtype:
+        raise TypeError("X and val must both be float32 or both float16")
+    _need(X, dtype, "X")
+    if X.dim() != 2 or X.shape[0] != tiled.n_rows:
+        raise ValueError("X must be [n_rows, K]")
+    K = int(X.shape[1])
+    Y = out if out is not None else torch.empty_like(X)
+    eb = 4 if dtype == torch.float32 else 2
+    ws = tiled.workspace(K, threads_per_wave, eb)
+    sched = tiled.sched
+    L = _cabi.lib()
+    args = [_ptr(tiled.vrow_ptr), _ptr(tiled.col_tiled), _ptr(tiled.val_tiled), _ptr(X), _ptr(Y), tiled.n_rows,
+            tiled.nnz, K, tiled.num_slabs, sched.P, _ptr(sched.coord_x), _ptr(sched.coord_y), int(threads_per_wave),
+            _ptr(ws), ws.numel()]
+    if phases is None:
+        fn = L.mps_spmm_tiled_f32 if eb == 4 else L.mps_spmm_tiled_f16
+        check(fn(*args, _stream()), "mps_spmm_tiled")
+    else:
+        fn = L.mps_spmm_tiled_f32_phases if eb == 4 else L.mps_spmm_tiled_f16_phases
+        check(fn(*args, int(phases), _stream()), "mps_spmm_tiled_phases")
+    return Y
+
+
 def run_spmm_row_wise(csr, X, num_waves, out=None):
     """Row-split comparison kernel (src/row_wise.cu:172-240), fp32."""
     _need(X, torch.float32, "X")
