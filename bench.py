@@ -53,8 +53,9 @@ def main():
     ap.add_argument("--spec", default="", help="generator spec overriding the workload's graph (experiments)")
     ap.add_argument("--k", type=int, default=0, help="feature width overriding the workload's K (experiments)")
     ap.add_argument("--cost", type=int, default=0, help="merge items per partition (0 = library default)")
-    ap.add_argument("--mode", default="auto", choices=["auto", "plain", "tiled"],
-                    help="plain = CSR as given; tiled = column-slab tiled copy; auto = tiled where it pays")
+    ap.add_argument("--mode", default="auto", choices=["auto", "plain", "untiled", "tiled"],
+                    help="plain = kernels on the CSR arrays as given, no plan; auto / untiled / tiled = with a plan "
+                         "(column-slab tiling where it pays / never / always)")
     ap.add_argument("--slab-bytes", type=int, default=0, help="slab size for tiling (0 = library default)")
     ap.add_argument("--tpw", type=int, default=0, help="partitions per wavefront (0 = full wavefront)")
     ap.add_argument("--seed", type=int, default=1)
@@ -92,24 +93,21 @@ def main():
     d_Y = torch.full_like(d_X, float("nan"))
     csr.validate()
     cost = args.cost if args.cost > 0 else sp.DEFAULT_COST
-    tiled = None
+    plan = None
     if args.mode != "plain":
-        if args.mode == "tiled":
-            ns, sc = sp.tile_shape(n, nnz, K, eb, args.slab_bytes)
-            if ns <= 1:  # forced: pick 2 MiB slabs regardless of the heuristic
-                sb = args.slab_bytes or (2 << 20)
-                sc = max(64, (sb // (K * eb)) // 64 * 64)
-                ns = (n + sc - 1) // sc
-            tiled = sp.build_tiles(csr, K, cost=cost, num_slabs=ns, slab_cols=sc)
-        else:
-            tiled = sp.build_tiles(csr, K, cost=cost, slab_bytes=args.slab_bytes)
-    sched = tiled.sched if tiled is not None else sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
+        tiling = {"auto": "auto", "untiled": "off", "tiled": "force"}[args.mode]
+        plan = sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes)
+        P = plan.info.num_partitions
+    else:
+        sched = sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
+        P = sched.P
     torch.cuda.synchronize()
     PH = pkg._cabi
+    tiled = plan is not None and plan.info.num_slabs > 1
 
     def step(phases=None):
-        if tiled is not None:
-            sp.spmm_merge_path_tiled(tiled, d_X, threads_per_wave=args.tpw, out=d_Y, phases=phases)
+        if plan is not None:
+            plan.spmm(d_X, out=d_Y, phases=phases)
         else:
             sp.spmm_merge_path(csr, d_X, sched, threads_per_wave=args.tpw, out=d_Y, phases=phases)
 
@@ -136,7 +134,7 @@ def main():
         b.record()
         step(PH.MPS_PHASE_FIXUP)
         c.record()
-        if tiled is not None:
+        if tiled:
             step(PH.MPS_PHASE_REDUCE)
         d.record()
     torch.cuda.synchronize()
@@ -144,21 +142,15 @@ def main():
     fix_ms = sum(b.elapsed_time(c) for _, b, c, _ in evs) / args.steps
     red_ms = sum(c.elapsed_time(d) for _, _, c, d in evs) / args.steps
 
-    # schedule build time (not part of a step)
-    p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    p0.record()
-    for _ in range(5):
-        sp.generate_mp_sched(tiled.vrow_ptr if tiled is not None else csr.row_ptr, nnz, cost=cost)
-    p1.record()
+    # preprocessing time (once per matrix, not part of a step)
     torch.cuda.synchronize()
-    plan_ms = p0.elapsed_time(p1) / 5
-    tile_ms = 0.0
-    if tiled is not None:
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        sp.build_tiles(csr, K, cost=cost, num_slabs=tiled.num_slabs, slab_cols=tiled.slab_cols)
-        torch.cuda.synchronize()
-        tile_ms = (time.perf_counter() - t1) * 1e3
+    t1 = time.perf_counter()
+    if plan is not None:
+        sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes).close()
+    else:
+        sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t1) * 1e3
 
     flops = 2.0 * nnz * K
     b_alg = algorithmic_bytes(n, nnz, K, eb, eb)
@@ -179,16 +171,16 @@ def main():
         "dtype": dt,
         "data": "synthetic (seeded generator, values U[0,1), features U[-1,1))",
         "config": {"workload": args.workload, "spec": spec, "n_rows": int(n), "nnz": int(nnz), "K": K,
-                   "max_row_degree": int(max_deg), "cost": cost, "partitions": sched.P,
+                   "max_row_degree": int(max_deg), "cost": cost, "partitions": P,
                    "threads_per_wave": args.tpw or g.max_threads_per_wave(K, eb), "seed": args.seed,
-                   "layout": ("tiled: %d column slabs of %d" % (tiled.num_slabs, tiled.slab_cols)) if tiled is not None
-                   else "plain CSR"},
+                   "layout": "plain CSR, no plan" if plan is None else
+                   ("plan: %d column slab(s) of %d, sliced, %.0f MB" % (plan.info.num_slabs, plan.info.slab_cols,
+                                                                       plan.info.device_bytes / 1e6))},
         "gbs_algorithmic_per_step": round(b_alg / (ms_per_step * 1e6), 2),
         "hbm_fraction_per_step": round(b_alg / (ms_per_step * 1e6) / PEAK_HBM_GBS, 4),
         "kernel_ms": {"mp_spmm_kernel": round(main_ms, 5), "mp_fixup_kernel": round(fix_ms, 5),
                       "tile_reduce_kernel": round(red_ms, 5),
-                      "mp_partition_kernel (once per graph)": round(plan_ms, 5),
-                      "tile build incl. allocation (once per graph)": round(tile_ms, 3)},
+                      "preprocessing, host wall time (once per matrix)": round(plan_ms, 3)},
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "roofline": {"bound": "hbm", "kernel": "mp_spmm_kernel", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None,

@@ -13,8 +13,8 @@
  *     value; HIP runtime failures return MPS_ERR_HIP + hipError_t.  Nothing
  *     throws and nothing calls exit().
  *   - "d_" arguments are device pointers, everything else is host memory.
- *   - The caller owns every buffer, including workspaces; unless a comment
- *     says otherwise the library allocates no device memory.
+ *   - The caller owns every buffer, including workspaces; the library
+ *     allocates device memory only where a comment says so (plans).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *     Calls are asynchronous with respect to the host; the caller
  *     synchronises.
@@ -206,7 +206,7 @@ int mps_spmm_f16(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_v
  * timing: phases bit 0 = the main kernel, bit 1 = the carry-out fix-up. */
 #define MPS_PHASE_MAIN 1u
 #define MPS_PHASE_FIXUP 2u
-#define MPS_PHASE_REDUCE 4u /* tiled entry points only */
+#define MPS_PHASE_REDUCE 4u /* plans with column slabs only */
 int mps_spmm_f32_phases(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
                         const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
                         const int *d_coord_x, const int *d_coord_y, int tpw,
@@ -219,65 +219,85 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
                         void *stream);
 
 /* ------------------------------------------------------------------------ */
-/* Device side: column-slab tiling of the merge-path SpMM                    */
+/* Device side: plans (per-matrix preprocessing of the merge-path SpMM)      */
 /* ------------------------------------------------------------------------ */
 
-/* The reference has no counterpart of this section.  Its kernels gather the
- * dense rows straight from global memory (src/MergePathSpMM.cu:459-460); on
- * MI355X those gathers are served by the 4 MiB L2 of the XCD a wavefront runs
- * on, and a feature matrix larger than that is bound by L2 misses.  Tiling
- * reorders the nonzeros once per matrix -- like the schedule, outside the
- * repeat loop (:192) -- so that the running wavefronts gather from one slab
- * of X at a time:
- *   - columns are cut into num_slabs slabs of slab_cols columns;
- *   - virtual row v = s * n_rows + r holds the nonzeros of row r whose
- *     column lies in slab s; the nonzeros are stored in virtual-row order
- *     (d_col_tiled, d_val_tiled) with row pointers d_vrow_ptr;
- *   - the same merge-path partitioner and SpMM kernel run over the
- *     num_slabs * n_rows virtual rows (call mps_num_partitions and
- *     mps_partition with n_rows := num_slabs * n_rows and d_vrow_ptr), writing
- *     fp32 partial rows into the workspace;
- *   - a last kernel adds the num_slabs partial rows of every row in slab
- *     order (deterministic) and writes Y.
+/* A plan is this library's counterpart of the schedule that the reference
+ * builds once per matrix before its repeat loop (generate_mp_sched and the
+ * uploads that follow it, src/MergePathSpMM.cu:192-220): everything about the
+ * sparse operand that does not change from launch to launch.  It is optional:
+ * mps_partition + mps_spmm_f32 above work from the caller's CSR arrays alone.
+ * A plan holds device memory that the library allocates (hipMalloc) at
+ * creation and frees at destruction:
  *
- * mps_tile_shape: slab count and width for an X of n_rows x K elements
- *   (slab_bytes = 0: 2 MiB slabs).  num_slabs == 1 means tiling does not pay
- *   (X fits in L2, or rows hold too few nonzeros per slab): use mps_spmm_f32.
- * mps_tile_build: builds d_vrow_ptr[num_slabs * n_rows + 1], d_col_tiled[nnz]
- *   and d_perm[nnz] (tiled position -> original nonzero index).  d_scratch:
- *   int[num_slabs * n_rows + 2049].  Synchronises the stream; returns
- *   MPS_ERR_UNSORTED when some row's column ids are not non-decreasing.
- * mps_tile_gather_values: d_val_tiled[i] = d_val[d_perm[i]]; call again
- *   whenever the values change. */
+ *   - Column-slab tiling (optional).  The dense-row gathers of the kernel are
+ *     served by the 4 MiB L2 of the XCD a wavefront runs on; a feature matrix
+ *     larger than that is bound by L2 misses.  The nonzeros are reordered
+ *     slab-major: columns are cut into num_slabs slabs of slab_cols columns,
+ *     "virtual row" v = s * n_rows + r holds the nonzeros of row r whose
+ *     column lies in slab s, and the virtual rows are stored in order, so the
+ *     running wavefronts gather from one ~2 MiB slab of X at a time.  The
+ *     kernel then produces num_slabs fp32 partial rows per row, which a last
+ *     kernel adds in slab order (deterministic).  Needs column ids sorted
+ *     (non-decreasing) within every row; otherwise the plan is built untiled.
+ *   - The merge-path partition (mps_num_partitions, mps_partition) of the
+ *     num_slabs * n_rows virtual rows for the given cost.
+ *   - The nonzeros "sliced" by that partition: the 16-nonzero windows that the
+ *     partitions of one wavefront consume in the same round are stored side
+ *     by side, so that a wavefront stages a round with one contiguous load.
+ *   - The workspace (partial rows, carry-out records).
+ *
+ * mps_tile_shape: the slab count and width mps_plan_create chooses for an X
+ *   of n_rows x K elements (slab_bytes = 0: 2 MiB slabs); num_slabs == 1
+ *   means tiling does not pay (X fits in L2, or a row holds too few nonzeros
+ *   per slab).
+ * mps_plan_create: d_val is fp32 (elem_bytes 4) or fp16 (2); cost and tpw as
+ *   for mps_num_partitions / mps_spmm_f32.  Synchronises the stream.
+ * mps_plan_set_values: the nonzero values changed, the pattern did not.
+ * mps_plan_spmm_f32 / _f16: Y = A * X; same arithmetic (fp32 accumulation)
+ *   and tolerance as mps_spmm_f32 / mps_spmm_f16, different summation order.
+ *   Calls on one plan share its workspace: do not overlap them on different
+ *   streams.
+ * mps_plan_spmm_phases: the same with the kernels selectable, for timing
+ *   (MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE).
+ * mps_plan_copy_array: copies one of the plan's device arrays to the host
+ *   (bytes must equal its size), for inspection and tests. */
+typedef struct mps_plan mps_plan;
+
+#define MPS_PLAN_NO_TILING 1u    /* never tile                                  */
+#define MPS_PLAN_FORCE_TILING 2u /* tile with slab_bytes slabs whatever the shape */
+
+typedef struct mps_plan_info {
+    int n_rows, nnz, K, elem_bytes, cost, threads_per_wave;
+    int num_slabs, slab_cols;      /* 1, n_rows when untiled                      */
+    int num_partitions, num_waves; /* P and ceil(P / threads_per_wave)            */
+    long long total_rounds;        /* sum over wavefronts of their 16-nonzero rounds */
+    long long slice_slots;         /* nonzero slots incl. padding                 */
+    size_t device_bytes;           /* device memory the plan holds                */
+} mps_plan_info;
+
+enum {
+    MPS_PLAN_ARRAY_VROW_PTR = 0,   /* int[num_slabs * n_rows + 1]                 */
+    MPS_PLAN_ARRAY_COORD_X = 1,    /* int[P + 1]                                  */
+    MPS_PLAN_ARRAY_COORD_Y = 2,    /* int[P + 1]                                  */
+    MPS_PLAN_ARRAY_WAVE_OFF = 3,   /* int[num_waves + 1]: first round of each wave */
+    MPS_PLAN_ARRAY_SLICE_COLS = 4, /* int[slice_slots]                            */
+    MPS_PLAN_ARRAY_SLICE_SRC = 5,  /* int[slice_slots]: original nonzero index, -1 = padding */
+    MPS_PLAN_ARRAY_SLICE_VALS = 6  /* elem_bytes * slice_slots                    */
+};
+
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,
                    int *slab_cols_out);
-int mps_tile_build(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int num_slabs,
-                   int slab_cols, int *d_vrow_ptr, int *d_col_tiled, int *d_perm, int *d_scratch,
-                   void *stream);
-int mps_tile_gather_values(const void *d_val, const int *d_perm, int nnz, int elem_bytes,
-                           void *d_val_tiled, void *stream);
-/* Workspace = fp32 partial rows (num_slabs * n_rows * K) + carry-out records. */
-int mps_spmm_tiled_workspace_bytes(int n_rows, int num_slabs, int P, int K, int tpw, int elem_bytes,
-                                   size_t *bytes_out);
-/* Y = A * X from the tiled arrays.  P, d_coord_x, d_coord_y: partition of the
- * virtual rows.  Same arithmetic and tolerance as mps_spmm_f32 / mps_spmm_f16
- * (fp32 accumulation; the summation order differs). */
-int mps_spmm_tiled_f32(const int *d_vrow_ptr, const int *d_col_tiled, const float *d_val_tiled,
-                       const float *d_X, float *d_Y, int n_rows, int nnz, int K, int num_slabs, int P,
-                       const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
-                       size_t workspace_bytes, void *stream);
-int mps_spmm_tiled_f16(const int *d_vrow_ptr, const int *d_col_tiled, const uint16_t *d_val_tiled,
-                       const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K, int num_slabs,
-                       int P, const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
-                       size_t workspace_bytes, void *stream);
-int mps_spmm_tiled_f32_phases(const int *d_vrow_ptr, const int *d_col_tiled, const float *d_val_tiled,
-                              const float *d_X, float *d_Y, int n_rows, int nnz, int K, int num_slabs,
-                              int P, const int *d_coord_x, const int *d_coord_y, int tpw,
-                              void *d_workspace, size_t workspace_bytes, unsigned phases, void *stream);
-int mps_spmm_tiled_f16_phases(const int *d_vrow_ptr, const int *d_col_tiled, const uint16_t *d_val_tiled,
-                              const uint16_t *d_X, uint16_t *d_Y, int n_rows, int nnz, int K,
-                              int num_slabs, int P, const int *d_coord_x, const int *d_coord_y, int tpw,
-                              void *d_workspace, size_t workspace_bytes, unsigned phases, void *stream);
+int mps_plan_create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz,
+                    int K, int elem_bytes, int cost, int tpw, unsigned flags, size_t slab_bytes,
+                    void *stream, mps_plan **plan_out);
+void mps_plan_destroy(mps_plan *plan);
+int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info);
+int mps_plan_set_values(mps_plan *plan, const void *d_val, void *stream);
+int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t bytes);
+int mps_plan_spmm_f32(const mps_plan *plan, const float *d_X, float *d_Y, void *stream);
+int mps_plan_spmm_f16(const mps_plan *plan, const uint16_t *d_X, uint16_t *d_Y, void *stream);
+int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsigned phases, void *stream);
 
 /* ------------------------------------------------------------------------ */
 /* Device side: comparison kernels                                           */

@@ -24,6 +24,18 @@ MPS_ERR_HIP = 1000
 MPS_PHASE_MAIN = 1
 MPS_PHASE_FIXUP = 2
 MPS_PHASE_REDUCE = 4
+MPS_PLAN_NO_TILING = 1
+MPS_PLAN_FORCE_TILING = 2
+(MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
+ MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS) = range(7)
+
+
+class PlanInfo(ctypes.Structure):
+    """struct mps_plan_info"""
+    _fields_ = [(n, ctypes.c_int) for n in ("n_rows", "nnz", "K", "elem_bytes", "cost", "threads_per_wave",
+                                             "num_slabs", "slab_cols", "num_partitions", "num_waves")] + \
+               [("total_rounds", ctypes.c_longlong), ("slice_slots", ctypes.c_longlong),
+                ("device_bytes", ctypes.c_size_t)]
 
 c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp, _i, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64
@@ -57,15 +69,14 @@ PROTOTYPES = {
     "mps_spmm_f16_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
                                  ctypes.c_uint, _vp]),
     "mps_tile_shape": (_i, [_i, _i, _i, _i, _sz, c_int_p, c_int_p]),
-    "mps_tile_build": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
-    "mps_tile_gather_values": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
-    "mps_spmm_tiled_workspace_bytes": (_i, [_i, _i, _i, _i, _i, _i, ctypes.POINTER(_sz)]),
-    "mps_spmm_tiled_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),
-    "mps_spmm_tiled_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),
-    "mps_spmm_tiled_f32_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
-                                       ctypes.c_uint, _vp]),
-    "mps_spmm_tiled_f16_phases": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz,
-                                       ctypes.c_uint, _vp]),
+    "mps_plan_create": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_uint, _sz, _vp, ctypes.POINTER(_vp)]),
+    "mps_plan_destroy": (None, [_vp]),
+    "mps_plan_get_info": (_i, [_vp, _vp]),
+    "mps_plan_set_values": (_i, [_vp, _vp, _vp]),
+    "mps_plan_copy_array": (_i, [_vp, _i, _vp, _sz]),
+    "mps_plan_spmm_f32": (_i, [_vp, _vp, _vp, _vp]),
+    "mps_plan_spmm_f16": (_i, [_vp, _vp, _vp, _vp]),
+    "mps_plan_spmm_phases": (_i, [_vp, _vp, _vp, ctypes.c_uint, _vp]),
     "mps_rowwise_spmm_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "mps_rowwise_bounds": (_i, [_i, _i, _vp, _vp]),
     "mps_nzsplit_max_parts": (_i, [_i, _i, _i, c_int_p]),

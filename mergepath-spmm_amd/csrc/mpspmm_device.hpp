@@ -1,0 +1,638 @@
+// Device code shared by the two halves of the library's GPU side
+// (mpspmm_kernels.hip: the CSR entry points; mpspmm_plan.hip: plans).
+// Everything lives in an anonymous namespace: each translation unit gets its
+// own copy of the kernels it launches.
+#ifndef MPSPMM_DEVICE_HPP
+#define MPSPMM_DEVICE_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdint>
+#include <cstdlib>
+
+#include "mpspmm.h"
+#include "mpspmm_internal.h"
+
+#define MPS_HIP_TRY(expr)                                       \
+    do {                                                        \
+        hipError_t e_ = (expr);                                 \
+        if (e_ != hipSuccess) return MPS_ERR_HIP + (int)e_;     \
+    } while (0)
+
+namespace {
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = 64 * kWavesPerBlock;
+constexpr int kWindow = 16;  // nonzeros staged per lane-group per round
+constexpr int kXcds = 8;     // accelerator dies of an MI355X, each with its own L2
+
+using half_t = _Float16;
+typedef half_t half8_t __attribute__((ext_vector_type(8)));
+typedef half_t half4_t __attribute__((ext_vector_type(4)));
+// 4-byte aligned 16-byte vectors: windows start at any nonzero index
+typedef int int4u_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef float float4u_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef half_t half4u_t __attribute__((ext_vector_type(4), aligned(2)));
+
+// LDS traffic here is private to one wavefront (each wave owns its slice), and
+// a wave's LDS operations execute in order, so a compiler-level barrier is all
+// that is needed between its writes and its reads.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---------------------------------------------------------------------------
+// Per-(element type, vector width) access to the dense input.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+struct XOps;
+
+template <>
+struct XOps<float, 4> {
+    using Raw = float4;
+    static __device__ __forceinline__ void fma(float (&acc)[4], float v, const Raw &r)
+    {
+        acc[0] = __builtin_fmaf(v, r.x, acc[0]);
+        acc[1] = __builtin_fmaf(v, r.y, acc[1]);
+        acc[2] = __builtin_fmaf(v, r.z, acc[2]);
+        acc[3] = __builtin_fmaf(v, r.w, acc[3]);
+    }
+};
+
+template <>
+struct XOps<float, 1> {
+    using Raw = float;
+    static __device__ __forceinline__ void fma(float (&acc)[1], float v, const Raw &r)
+    {
+        acc[0] = __builtin_fmaf(v, r, acc[0]);
+    }
+};
+
+template <>
+struct XOps<half_t, 8> {
+    using Raw = half8_t;
+    static __device__ __forceinline__ void fma(float (&acc)[8], float v, const Raw &r)
+    {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(v, (float)r[i], acc[i]);
+    }
+};
+
+template <>
+struct XOps<half_t, 1> {
+    using Raw = half_t;
+    static __device__ __forceinline__ void fma(float (&acc)[1], float v, const Raw &r)
+    {
+        acc[0] = __builtin_fmaf(v, (float)r, acc[0]);
+    }
+};
+
+// VEC accumulators -> VEC adjacent outputs (fp32 or fp16), one vector store
+// where the width allows.
+template <int VEC>
+__device__ __forceinline__ void store_acc(float *p, const float (&acc)[VEC])
+{
+    if constexpr (VEC % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4)
+            *reinterpret_cast<float4 *>(p + i) = make_float4(acc[i], acc[i + 1], acc[i + 2], acc[i + 3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) p[i] = acc[i];
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void store_acc(half_t *p, const float (&acc)[VEC])
+{
+    if constexpr (VEC == 8) {
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (half_t)acc[i];
+        *reinterpret_cast<half8_t *>(p) = o;
+    } else if constexpr (VEC == 4) {
+        half4_t o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (half_t)acc[i];
+        *reinterpret_cast<half4_t *>(p) = o;
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) p[i] = (half_t)acc[i];
+    }
+}
+
+// Address of the VEC columns a lane owns in row `c` of X.  POW2: the row
+// pitch is a power of two and the matrix is below 4 GiB, so the byte offset
+// is one shift-or in 32 bits (the load then takes its base from SGPRs).
+template <typename T, int VEC, bool POW2>
+struct Gather {
+    using Raw = typename XOps<T, VEC>::Raw;
+    const char *xb;
+    size_t row_bytes;
+    unsigned col_byte;
+    int row_shift;
+    __device__ __forceinline__ Raw load(int c) const
+    {
+        if constexpr (POW2) {
+            unsigned off = ((unsigned)c << row_shift) | col_byte;
+            return *reinterpret_cast<const Raw *>(xb + off);
+        } else {
+            size_t off = (size_t)c * row_bytes + col_byte;
+            return *reinterpret_cast<const Raw *>(xb + off);
+        }
+    }
+};
+
+// Four consecutive nonzeros of a window, as registers.
+struct Win {
+    int4 c;
+    float4 v;
+};
+
+__device__ __forceinline__ float4 load_val4(const float *p)
+{
+    float4u_t t = __builtin_nontemporal_load(reinterpret_cast<const float4u_t *>(p));
+    return make_float4(t[0], t[1], t[2], t[3]);
+}
+__device__ __forceinline__ float4 load_val4(const half_t *p)
+{
+    half4u_t h = __builtin_nontemporal_load(reinterpret_cast<const half4u_t *>(p));
+    return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+}
+
+// Nonzeros [i0, i0 + 4) of col_idx / val (those below nnz).  The sparse
+// stream is read once: non-temporal loads keep it from displacing X in L2.
+template <typename T>
+__device__ __forceinline__ Win load_win(const int *__restrict__ col_idx, const T *__restrict__ val, int nnz, int i0)
+{
+    Win w;
+    w.c = make_int4(0, 0, 0, 0);
+    w.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i0 + 3 < nnz) {
+        int4u_t t = __builtin_nontemporal_load(reinterpret_cast<const int4u_t *>(col_idx + i0));
+        w.c = make_int4(t[0], t[1], t[2], t[3]);
+        w.v = load_val4(val + i0);
+    } else {
+        if (i0 + 0 < nnz) { w.c.x = col_idx[i0 + 0]; w.v.x = (float)val[i0 + 0]; }
+        if (i0 + 1 < nnz) { w.c.y = col_idx[i0 + 1]; w.v.y = (float)val[i0 + 1]; }
+        if (i0 + 2 < nnz) { w.c.z = col_idx[i0 + 2]; w.v.z = (float)val[i0 + 2]; }
+    }
+    return w;
+}
+
+
+// Elements [e0, e0 + 4) of a plan's sliced arrays: 16-byte aligned, padded to
+// whole round blocks, so no bounds are needed.
+__device__ __forceinline__ Win load_slice_vals(const float *p, Win w)
+{
+    typedef float f4_t __attribute__((ext_vector_type(4)));
+    f4_t t = __builtin_nontemporal_load(reinterpret_cast<const f4_t *>(p));
+    w.v = make_float4(t[0], t[1], t[2], t[3]);
+    return w;
+}
+__device__ __forceinline__ Win load_slice_vals(const half_t *p, Win w)
+{
+    half4_t h = __builtin_nontemporal_load(reinterpret_cast<const half4_t *>(p));
+    w.v = make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+    return w;
+}
+template <typename T>
+__device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T *__restrict__ vals, size_t e0)
+{
+    typedef int i4_t __attribute__((ext_vector_type(4)));
+    Win w;
+    i4_t t = __builtin_nontemporal_load(reinterpret_cast<const i4_t *>(cols + e0));
+    w.c = make_int4(t[0], t[1], t[2], t[3]);
+    return load_slice_vals(vals + e0, w);
+}
+
+// ---------------------------------------------------------------------------
+// Merge-path SpMM, main kernel.
+// ---------------------------------------------------------------------------
+//
+// SLICED = false: col_idx / val are the CSR arrays; every lane-group stages
+//   its own 16-nonzero windows (two 64-byte loads per window).
+// SLICED = true: col_idx / val are the sliced arrays of a plan: the windows
+//   of the groups of one wavefront for one round lie side by side
+//   (wave_off[w] + round) * tpw * 16 elements into the arrays, so the whole
+//   wavefront stages a round with one contiguous, fully coalesced load per
+//   array; wave_off[w + 1] - wave_off[w] is the number of rounds of wave w.
+template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED>
+__global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
+    const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
+    const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
+    const int *__restrict__ coord_y, const int *__restrict__ wave_off, int nnz, int K, int P,
+    int lanes_log2, int tpw, int num_waves, int row_shift, int *__restrict__ ws_head_row,
+    float *__restrict__ ws_head, float *__restrict__ ws_tail)
+{
+    using XO = XOps<T, VEC>;
+    using Raw = typename XO::Raw;
+    constexpr int kCombine = 64 * VEC;  // floats per wave for heads (and for tails)
+    constexpr int kSlice = (2 * kCombine > 2 * 16 * kWindow) ? 2 * kCombine : 2 * 16 * kWindow;
+    __shared__ float s_buf[kWavesPerBlock][kSlice];
+    __shared__ int s_hrow[kWavesPerBlock][16];
+
+    const int wib = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    // Workgroups are dealt round-robin to the 8 XCDs.  Give XCD k the k-th
+    // contiguous eighth of the partitions, so that the wavefronts sharing an L2
+    // work on neighbouring rows (and, in a tiled plan, on the same column slab).
+    const int blocks_per_xcd = gridDim.x / kXcds;
+    const int lblock = (blockIdx.x % kXcds) * blocks_per_xcd + blockIdx.x / kXcds;
+    const int w = lblock * kWavesPerBlock + wib;
+    if (w >= num_waves) return;
+
+    const int L = 1 << lanes_log2;
+    const int g = lane >> lanes_log2;
+    const int s = lane & (L - 1);
+    const int KT = L * VEC;  // columns covered by one pass of the wave
+    const int kcol = blockIdx.y * KT + s * VEC;
+    const bool col_ok = kcol < K;
+    // lanes beyond K gather column 0 (a valid address) and never store
+    const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
+                                  col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
+
+    int *s_col_wave = reinterpret_cast<int *>(&s_buf[wib][0]);
+    float *s_val_wave = &s_buf[wib][16 * kWindow];
+    int *s_col = s_col_wave + g * kWindow;
+    float *s_val = s_val_wave + g * kWindow;
+
+    const int p = w * tpw + g;
+    const bool part_ok = (g < tpw) && (p < P);
+    int x = 1, x_end = 1, y_begin = 0, y_end = 0;
+    if (part_ok) {
+        x = max(coord_x[p], 1);
+        x_end = coord_x[p + 1];
+        y_begin = coord_y[p];
+        y_end = coord_y[p + 1];
+    }
+    // Row x - 1 is in progress; it ends where nonzero index row_ptr[x] begins.
+    // The two row ends after it are loaded ahead, so that finishing a row does
+    // not wait on memory.
+    auto row_end_at = [&](int xx) { return (xx < x_end) ? row_ptr[xx] : INT_MAX; };
+    int row_end = row_end_at(x), row_end1 = row_end_at(x + 1), row_end2 = row_end_at(x + 2);
+
+    float acc[VEC], head[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) { acc[i] = 0.f; head[i] = 0.f; }
+    int head_row = -1;
+
+    auto emit = [&]() {
+        const int row = x - 1;
+        if (head_row < 0) {
+            head_row = row;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) head[i] = acc[i];
+        } else if (col_ok) {
+            store_acc<VEC>(Y + (size_t)row * K + kcol, acc);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+        ++x;
+        row_end = row_end1;
+        row_end1 = row_end2;
+        row_end2 = row_end_at(x + 2);
+    };
+
+    int wbase = y_begin;
+    Win pw;
+    pw.c = make_int4(0, 0, 0, 0);
+    pw.v = make_float4(0.f, 0.f, 0.f, 0.f);
+    // sliced staging: lane l moves elements [4l, 4l + 4) of the wave's round block
+    const int round_elems = tpw * kWindow;
+    const bool stager = SLICED ? (4 * lane < round_elems) : (s < 4);
+    int round = 0, round_end = 0;
+    if constexpr (SLICED) {
+        round = wave_off[w];
+        round_end = wave_off[w + 1];
+        if (stager && round < round_end) pw = load_slice<T>(col_idx, val, (size_t)round * round_elems + 4 * lane);
+    } else {
+        if (stager && wbase < y_end) pw = load_win<T>(col_idx, val, nnz, wbase + 4 * s);
+    }
+
+    while (SLICED ? (round < round_end) : (__any(wbase < y_end) != 0)) {
+        const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
+        if constexpr (SLICED) {
+            if (stager) {
+                *reinterpret_cast<int4 *>(s_col_wave + 4 * lane) = pw.c;
+                *reinterpret_cast<float4 *>(s_val_wave + 4 * lane) = pw.v;
+            }
+        } else {
+            if (stager && nvalid > 0) {
+                *reinterpret_cast<int4 *>(s_col + 4 * s) = pw.c;
+                *reinterpret_cast<float4 *>(s_val + 4 * s) = pw.v;
+            }
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int b = 0; b < kWindow; b += BATCH) {
+            int cols[BATCH];
+            float vals[BATCH];
+            Raw xr[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                cols[j] = s_col[b + j];
+                vals[j] = s_val[b + j];
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j)
+                if (b + j < nvalid) xr[j] = gx.load(cols[j]);
+            if (b == 0) {
+                // next window: in flight while this one is consumed
+                if constexpr (SLICED) {
+                    if (stager && round + 1 < round_end)
+                        pw = load_slice<T>(col_idx, val, (size_t)(round + 1) * round_elems + 4 * lane);
+                } else {
+                    const int nb = wbase + kWindow;
+                    if (stager && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                if (b + j < nvalid) {
+                    const int idx = wbase + b + j;
+                    while (idx == row_end) emit();
+                    XO::fma(acc, vals[j], xr[j]);
+                }
+            }
+        }
+        wbase += kWindow;
+        ++round;
+        wave_lds_sync();
+    }
+    while (x < x_end) emit();  // rows that end exactly where the partition ends
+
+    // ---- combine the groups of this wavefront -------------------------------
+    float *heads = &s_buf[wib][0];
+    float *tails = heads + kCombine;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        heads[g * KT + s * VEC + i] = head[i];
+        tails[g * KT + s * VEC + i] = acc[i];
+    }
+    if (s == 0) s_hrow[wib][g] = head_row;
+    wave_lds_sync();
+
+    const int ng = min(tpw, P - w * tpw);
+    for (int c = lane; c < KT; c += 64) {
+        const int kc = blockIdx.y * KT + c;
+        const bool kc_ok = kc < K;
+        float carry = 0.f;
+        bool first = true;
+        for (int gg = 0; gg < ng; ++gg) {
+            const int hr = s_hrow[wib][gg];
+            const float t = tails[gg * KT + c];
+            if (hr >= 0) {
+                const float v = heads[gg * KT + c] + carry;
+                if (first) {
+                    if (kc_ok) ws_head[(size_t)w * K + kc] = v;
+                    if (kc == 0) ws_head_row[w] = hr;
+                    first = false;
+                } else if (kc_ok) {
+                    Y[(size_t)hr * K + kc] = (TOut)v;
+                }
+                carry = t;
+            } else {
+                carry += t;
+            }
+        }
+        if (first && kc == 0) ws_head_row[w] = -1;
+        if (kc_ok) ws_tail[(size_t)w * K + kc] = carry;
+    }
+}
+
+// Carry-out fix-up: the first row that ends inside wavefront w also received
+// nonzeros from the wavefronts before it, back to (and including) the nearest
+// one that itself saw a row end.
+template <typename TOut>
+__global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ ws_head_row,
+                                                        const float *__restrict__ ws_head,
+                                                        const float *__restrict__ ws_tail,
+                                                        TOut *__restrict__ Y, int num_waves, int K)
+{
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long w64 = idx / K;
+    if (w64 >= num_waves) return;
+    const int w = (int)w64;
+    const int k = (int)(idx - w64 * K);
+    const int hr = ws_head_row[w];
+    if (hr < 0) return;
+    float sum = ws_head[(size_t)w * K + k];
+    int j = w - 1;
+    while (j >= 0) {
+        // four records at a time so that their loads overlap
+        float t[4];
+        int h[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int jj = j - u;
+            t[u] = jj >= 0 ? ws_tail[(size_t)jj * K + k] : 0.f;
+            h[u] = jj >= 0 ? ws_head_row[jj] : 0;
+        }
+        bool done = false;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (!done) {
+                sum += t[u];
+                if (h[u] >= 0) done = true;
+            }
+        }
+        if (done) break;
+        j -= 4;
+    }
+    Y[(size_t)hr * K + k] = (TOut)sum;
+}
+
+// ---------------------------------------------------------------------------
+// Exclusive prefix sum of an int array, in place (three launches).
+// ---------------------------------------------------------------------------
+constexpr int kScanThreads = 1024;
+constexpr int kScanMaxBlocks = 2048;
+
+// Inclusive scan of one value per thread across a 1024-thread block.
+__device__ __forceinline__ int block_inclusive_scan(int v, int *s_wave /*[16]*/, int &block_total)
+{
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    if (lane == 63) s_wave[wv] = v;
+    __syncthreads();
+    int wave_off = 0, total = 0;
+    for (int i = 0; i < kScanThreads / 64; ++i) {
+        int t = s_wave[i];
+        if (i < wv) wave_off += t;
+        total += t;
+    }
+    __syncthreads();
+    block_total = total;
+    return v + wave_off;
+}
+
+// PHASE 1: per-segment sums.  PHASE 3: exclusive offsets written back.
+template <int PHASE>
+__global__ __launch_bounds__(kScanThreads) void scan_segments_kernel(int *__restrict__ data, int n, int seg_len,
+                                                                     int *__restrict__ sums)
+{
+    __shared__ int s_wave[kScanThreads / 64];
+    const int seg_begin = blockIdx.x * seg_len;
+    const int seg_end = min(seg_begin + seg_len, n);
+    int running = (PHASE == 3) ? sums[blockIdx.x] : 0;
+    for (int base = seg_begin; base < seg_end; base += kScanThreads) {
+        const int i = base + threadIdx.x;
+        int v = (i < seg_end) ? data[i] : 0;
+        int total;
+        int incl = block_inclusive_scan(v, s_wave, total);
+        if (PHASE == 3 && i < seg_end) data[i] = running + incl - v;
+        running += total;
+    }
+    if (PHASE == 1 && threadIdx.x == 0) sums[blockIdx.x] = running;
+}
+
+// PHASE 2: exclusive scan of the (<= 2048) segment sums in place.
+__global__ __launch_bounds__(kScanThreads) void scan_sums_kernel(int *__restrict__ sums, int nseg)
+{
+    __shared__ int s_wave[kScanThreads / 64];
+    int running = 0;
+    for (int base = 0; base < nseg; base += kScanThreads) {
+        const int i = base + threadIdx.x;
+        int v = i < nseg ? sums[i] : 0;
+        int total;
+        int incl = block_inclusive_scan(v, s_wave, total);
+        if (i < nseg) sums[i] = running + incl - v;
+        running += total;
+    }
+}
+
+// data[0..n) -> exclusive prefix sums; sums: int[2048] scratch.
+inline int scan_exclusive_inplace(int *data, int n, int *sums, hipStream_t st)
+{
+    if (n <= 0) return MPS_OK;
+    int nseg = (n + kScanThreads - 1) / kScanThreads;
+    if (nseg > kScanMaxBlocks) nseg = kScanMaxBlocks;
+    int seg_len = (n + nseg - 1) / nseg;
+    seg_len = (seg_len + kScanThreads - 1) / kScanThreads * kScanThreads;
+    nseg = (n + seg_len - 1) / seg_len;
+    hipLaunchKernelGGL((scan_segments_kernel<1>), dim3(nseg), dim3(kScanThreads), 0, st, data, n, seg_len, sums);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kScanThreads), 0, st, sums, nseg);
+    hipLaunchKernelGGL((scan_segments_kernel<3>), dim3(nseg), dim3(kScanThreads), 0, st, data, n, seg_len, sums);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+
+// ---------------------------------------------------------------------------
+// Launch helpers shared by the entry points
+// ---------------------------------------------------------------------------
+inline bool aligned_to(const void *p, unsigned a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// log2 of the row pitch in bytes when the fast addressing applies, else -1.
+inline int pow2_row_shift(int n_rows, int K, int elem_bytes)
+{
+    uint64_t rb = (uint64_t)K * elem_bytes;
+    if (rb & (rb - 1)) return -1;
+    if ((uint64_t)(n_rows > 0 ? n_rows : 1) * rb >= (1ull << 32)) return -1;
+    int sh = 0;
+    while ((1ull << sh) < rb) ++sh;
+    return sh;
+}
+
+struct SpmmShape {
+    mps_lane_shape ls;
+    int tpw;
+    int num_waves;
+    int row_shift;  // >= 0: power-of-two pitch, 32-bit offsets
+};
+
+inline int make_spmm_shape(int n_rows, int K, int P, int tpw, int elem_bytes, SpmmShape &sh)
+{
+    if (K < 1 || P < 1 || tpw < 0) return MPS_ERR_INVALID_ARG;
+    sh.ls = mps_make_lane_shape(K, elem_bytes);
+    if (tpw == 0) tpw = sh.ls.groups;
+    if (tpw > sh.ls.groups) return MPS_ERR_TPW;
+    sh.tpw = tpw;
+    sh.num_waves = (P + tpw - 1) / tpw;
+    sh.row_shift = pow2_row_shift(n_rows, K, elem_bytes);
+    return MPS_OK;
+}
+
+inline size_t carry_bytes_for(int num_waves, int K)
+{
+    size_t rows = ((size_t)num_waves + 63) / 64 * 64;
+    return rows * sizeof(int) + 2 * (size_t)num_waves * K * sizeof(float);
+}
+
+// Gathers in flight per lane between waits: tuning knob, 8 or 16.
+inline int gather_batch()
+{
+    static int b = [] {
+        const char *e = std::getenv("MPS_GATHER_BATCH");
+        int v = e ? std::atoi(e) : 0;
+        return v == 16 ? 16 : 8;
+    }();
+    return b;
+}
+
+// wave_off == nullptr: CSR arrays; else the sliced arrays of a plan.
+template <typename T, typename TOut, int VEC>
+int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X, TOut *Y, int nnz, int K, int P,
+                const int *cx, const int *cy, const int *wave_off, const SpmmShape &sh, void *ws, unsigned phases,
+                hipStream_t st)
+{
+    const int W = sh.num_waves;
+    size_t rows = ((size_t)W + 63) / 64 * 64;
+    int *ws_head_row = static_cast<int *>(ws);
+    float *ws_head = reinterpret_cast<float *>(ws_head_row + rows);
+    float *ws_tail = ws_head + (size_t)W * K;
+    if (phases & MPS_PHASE_MAIN) {
+        const int nblocks = (W + kWavesPerBlock - 1) / kWavesPerBlock;
+        dim3 grid((nblocks + kXcds - 1) / kXcds * kXcds, sh.ls.col_tiles);
+#define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED)                                                                  \
+    hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED>), grid, dim3(kBlock), 0, st, row_ptr, \
+                       col_idx, val, X, Y, cx, cy, wave_off, nnz, K, P, sh.ls.lanes_log2, sh.tpw, W,           \
+                       sh.row_shift, ws_head_row, ws_head, ws_tail)
+        if (wave_off) {
+            if (sh.row_shift >= 0) {
+                if (gather_batch() == 16) MPS_LAUNCH_MAIN(true, 16, true); else MPS_LAUNCH_MAIN(true, 8, true);
+            } else {
+                MPS_LAUNCH_MAIN(false, 8, true);
+            }
+        } else {
+            if (sh.row_shift >= 0) {
+                if (gather_batch() == 16) MPS_LAUNCH_MAIN(true, 16, false); else MPS_LAUNCH_MAIN(true, 8, false);
+            } else {
+                MPS_LAUNCH_MAIN(false, 8, false);
+            }
+        }
+#undef MPS_LAUNCH_MAIN
+        MPS_HIP_TRY(hipGetLastError());
+    }
+    if (phases & MPS_PHASE_FIXUP) {
+        long long threads = (long long)W * K;
+        unsigned blocks = (unsigned)((threads + 255) / 256);
+        hipLaunchKernelGGL((mp_fixup_kernel<TOut>), dim3(blocks), dim3(256), 0, st, ws_head_row, ws_head, ws_tail,
+                           Y, W, K);
+        MPS_HIP_TRY(hipGetLastError());
+    }
+    return MPS_OK;
+}
+
+template <typename T, typename TOut>
+int launch_spmm_any(const int *row_ptr, const int *col_idx, const T *val, const T *X, TOut *Y, int nnz, int K,
+                    int P, const int *cx, const int *cy, const int *wave_off, const SpmmShape &sh, void *ws,
+                    unsigned phases, hipStream_t st)
+{
+    if (sh.ls.vec == 1)
+        return launch_spmm<T, TOut, 1>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, wave_off, sh, ws, phases, st);
+    return launch_spmm<T, TOut, 16 / (int)sizeof(T)>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, wave_off, sh, ws,
+                                                     phases, st);
+}
+
+}  // namespace
+
+#endif

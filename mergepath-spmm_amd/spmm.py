@@ -125,34 +125,6 @@ def spmm_merge_path(csr, X, sched, threads_per_wave=0, out=None, phases=None):
     return Y
 
 
-class TiledCsr:
-    """Column-slab tiled copy of a CSR matrix plus the merge-path schedule over
-    its virtual rows (mps_tile_build; no counterpart in the reference)."""
-
-    def __init__(self, csr, num_slabs, slab_cols, vrow_ptr, col_tiled, perm, val_tiled):
-        self.n_rows, self.nnz = csr.n_rows, csr.nnz
-        self.num_slabs, self.slab_cols = num_slabs, slab_cols
-        self.vrow_ptr, self.col_tiled, self.perm, self.val_tiled = vrow_ptr, col_tiled, perm, val_tiled
-        self.sched = None
-        self._ws = {}
-
-    def set_values(self, val):
-        """Re-gather the tiled values after the caller changed val."""
-        eb = 4 if val.dtype == torch.float32 else 2
-        check(_cabi.lib().mps_tile_gather_values(_ptr(val), _ptr(self.perm), self.nnz, eb, _ptr(self.val_tiled),
-                                                 _stream()), "mps_tile_gather_values")
-
-    def workspace(self, K, tpw, elem_bytes):
-        key = (K, tpw, elem_bytes)
-        if key not in self._ws:
-            nbytes = ctypes.c_size_t()
-            check(_cabi.lib().mps_spmm_tiled_workspace_bytes(self.n_rows, self.num_slabs, self.sched.P, K, tpw,
-                                                             elem_bytes, ctypes.byref(nbytes)),
-                  "mps_spmm_tiled_workspace_bytes")
-            self._ws[key] = torch.empty(max(int(nbytes.value), 16), dtype=torch.uint8, device=self.vrow_ptr.device)
-        return self._ws[key]
-
-
 def tile_shape(n_rows, nnz, K, elem_bytes=4, slab_bytes=0):
     ns, sc = ctypes.c_int(), ctypes.c_int()
     check(_cabi.lib().mps_tile_shape(int(n_rows), int(nnz), int(K), int(elem_bytes), int(slab_bytes),
@@ -160,55 +132,76 @@ def tile_shape(n_rows, nnz, K, elem_bytes=4, slab_bytes=0):
     return ns.value, sc.value
 
 
-def build_tiles(csr, K, cost=None, slab_bytes=0, num_slabs=None, slab_cols=None):
-    """Tile csr for feature width K and build the schedule over the virtual rows.
-    Returns None when tiling does not pay for this shape (unless slabs are forced)."""
-    eb = 4 if csr.val.dtype == torch.float32 else 2
-    if num_slabs is None:
-        num_slabs, slab_cols = tile_shape(csr.n_rows, csr.nnz, K, eb, slab_bytes)
-        if num_slabs <= 1:
-            return None
-    dev = csr.row_ptr.device
-    nv = num_slabs * csr.n_rows
-    vrow_ptr = torch.empty(nv + 1, dtype=torch.int32, device=dev)
-    col_tiled = torch.empty(max(csr.nnz, 1), dtype=torch.int32, device=dev)
-    perm = torch.empty(max(csr.nnz, 1), dtype=torch.int32, device=dev)
-    scratch = torch.empty(nv + 2049, dtype=torch.int32, device=dev)
-    check(_cabi.lib().mps_tile_build(_ptr(csr.row_ptr), _ptr(csr.col_idx), csr.n_rows, csr.nnz, num_slabs, slab_cols,
-                                     _ptr(vrow_ptr), _ptr(col_tiled), _ptr(perm), _ptr(scratch), _stream()),
-          "mps_tile_build")
-    del scratch
-    val_tiled = torch.empty(max(csr.nnz, 1), dtype=csr.val.dtype, device=dev)
-    t = TiledCsr(csr, num_slabs, slab_cols, vrow_ptr, col_tiled, perm, val_tiled)
-    t.set_values(csr.val)
-    t.sched = generate_mp_sched(vrow_ptr, csr.nnz, cost=cost)
-    return t
+class Plan:
+    """Per-matrix preprocessing (mps_plan_create): optional column-slab tiling,
+    the merge-path partition of the (virtual) rows, the sliced nonzero arrays
+    and the workspace.  The counterpart of what the reference sets up once
+    before its repeat loop (src/MergePathSpMM.cu:192-220)."""
 
+    def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0):
+        import numpy as np
+        self._np = np
+        self._h = ctypes.c_void_p()
+        self.dtype = csr.val.dtype
+        eb = 4 if self.dtype == torch.float32 else 2
+        flags = {"auto": 0, "off": _cabi.MPS_PLAN_NO_TILING, "force": _cabi.MPS_PLAN_FORCE_TILING}[tiling]
+        check(_cabi.lib().mps_plan_create(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
+                                          int(K), eb, int(DEFAULT_COST if cost is None else cost),
+                                          int(threads_per_wave), flags, int(slab_bytes), _stream(),
+                                          ctypes.byref(self._h)), "mps_plan_create")
+        self.K, self.n_rows = int(K), csr.n_rows
+        info = _cabi.PlanInfo()
+        check(_cabi.lib().mps_plan_get_info(self._h, ctypes.byref(info)), "mps_plan_get_info")
+        self.info = info
 
-def spmm_merge_path_tiled(tiled, X, threads_per_wave=0, out=None, phases=None):
-    """Y = A @ X from the tiled arrays (mps_spmm_tiled_f32 / _f16)."""
-    dtype = X.dtype
-    if dtype not in (torch.float32, torch.float16) or tiled.val_tiled.dtype != dtype:
-        raise TypeError("X and val must both be float32 or both float16")
-    _need(X, dtype, "X")
-    if X.dim() != 2 or X.shape[0] != tiled.n_rows:
-        raise ValueError("X must be [n_rows, K]")
-    K = int(X.shape[1])
-    Y = out if out is not None else torch.empty_like(X)
-    eb = 4 if dtype == torch.float32 else 2
-    ws = tiled.workspace(K, threads_per_wave, eb)
-    sched = tiled.sched
-    L = _cabi.lib()
-    args = [_ptr(tiled.vrow_ptr), _ptr(tiled.col_tiled), _ptr(tiled.val_tiled), _ptr(X), _ptr(Y), tiled.n_rows,
-            tiled.nnz, K, tiled.num_slabs, sched.P, _ptr(sched.coord_x), _ptr(sched.coord_y), int(threads_per_wave),
-            _ptr(ws), ws.numel()]
-    if phases is None:
-        fn = L.mps_spmm_tiled_f32 if eb == 4 else L.mps_spmm_tiled_f16
-        check(fn(*args, _stream()), "mps_spmm_tiled")
-    else:
-        fn = L.mps_spmm_tiled_f32_phases if eb == 4 else L.mps_spmm_tiled_f16_phases
-        check(fn(*args, int(phases), _stream()), "mps_spmm_tiled_phases")
-    return Y
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h.value and _cabi is not None:
+            _cabi.lib().mps_plan_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_values(self, val):
+        """The nonzero values changed, the pattern did not."""
+        _need(val, self.dtype, "val")
+        check(_cabi.lib().mps_plan_set_values(self._h, _ptr(val), _stream()), "mps_plan_set_values")
+
+    def array(self, which):
+        """Host copy of one of the plan's device arrays (numpy)."""
+        np, i = self._np, self.info
+        slots = int(i.slice_slots)
+        shapes = {
+            _cabi.MPS_PLAN_ARRAY_VROW_PTR: (i.num_slabs * i.n_rows + 1, np.int32),
+            _cabi.MPS_PLAN_ARRAY_COORD_X: (i.num_partitions + 1, np.int32),
+            _cabi.MPS_PLAN_ARRAY_COORD_Y: (i.num_partitions + 1, np.int32),
+            _cabi.MPS_PLAN_ARRAY_WAVE_OFF: (i.num_waves + 1, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SLICE_COLS: (slots, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SLICE_SRC: (slots, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SLICE_VALS: (slots, np.float32 if i.elem_bytes == 4 else np.float16),
+        }
+        n, dt = shapes[which]
+        out = np.empty(n, dtype=dt)
+        check(_cabi.lib().mps_plan_copy_array(self._h, int(which), out.ctypes.data, out.nbytes), "mps_plan_copy_array")
+        return out
+
+    def spmm(self, X, out=None, phases=None):
+        """Y = A @ X."""
+        _need(X, self.dtype, "X")
+        if X.dim() != 2 or X.shape[0] != self.n_rows or X.shape[1] != self.K:
+            raise ValueError("X must be [n_rows, K] with the K the plan was made for")
+        Y = out if out is not None else torch.empty_like(X)
+        _need(Y, self.dtype, "out")
+        L = _cabi.lib()
+        if phases is None:
+            fn = L.mps_plan_spmm_f32 if self.dtype == torch.float32 else L.mps_plan_spmm_f16
+            check(fn(self._h, _ptr(X), _ptr(Y), _stream()), "mps_plan_spmm")
+        else:
+            check(L.mps_plan_spmm_phases(self._h, _ptr(X), _ptr(Y), int(phases), _stream()), "mps_plan_spmm_phases")
+        return Y
 
 
 def run_spmm_row_wise(csr, X, num_waves, out=None):

@@ -1,0 +1,189 @@
+"""Plans (mps_plan_*): column-slab tiling, partition of the virtual rows and
+sliced nonzero arrays, checked against numpy restatements of their layout; the
+SpMM through a plan meets the same bar against the oracle's fp64 row loop."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import check_fp32, make_csr, random_csr, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def slab_major_reference(rp, ci, num_slabs, slab_cols):
+    """(vrow_ptr, perm): virtual row s*n + r holds row r's nonzeros with
+    s*slab_cols <= col < (s+1)*slab_cols, in their original order."""
+    n = rp.size - 1
+    rows = np.repeat(np.arange(n, dtype=np.int64), np.diff(rp))
+    slab = np.minimum(ci.astype(np.int64) // slab_cols, num_slabs - 1)
+    v = slab * n + rows
+    perm = np.argsort(v, kind="stable")
+    counts = np.bincount(v, minlength=num_slabs * n)
+    vrp = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    return vrp, perm.astype(np.int32)
+
+
+def check_plan_layout(pkg, orc, plan, rp, ci, val):
+    c, i = pkg._cabi, plan.info
+    n, nnz = rp.size - 1, ci.size
+    vrp, perm = slab_major_reference(rp, ci, i.num_slabs, i.slab_cols)
+    assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_VROW_PTR), vrp)
+    # the partition of the virtual rows is the reference split (oracle restatement)
+    assert i.num_partitions == orc.num_partitions(i.num_slabs * n, nnz, i.cost)
+    xs, ys = orc.partition_coords(vrp, nnz, i.num_partitions)
+    assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_COORD_X), xs)
+    assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_COORD_Y), ys)
+    # slices: wave w, round r, group g, element j  <-  virtual nonzero ys[p] + 16 r + j
+    G, W = i.threads_per_wave, i.num_waves
+    cnt = np.diff(ys)
+    rounds = np.zeros(W, dtype=np.int64)
+    for w in range(W):
+        seg = cnt[w * G:(w + 1) * G]
+        rounds[w] = ((seg + 15) // 16).max() if seg.size else 0
+    wave_off = np.concatenate([[0], np.cumsum(rounds)])
+    assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_WAVE_OFF), wave_off)
+    assert i.total_rounds == wave_off[-1] and i.slice_slots == wave_off[-1] * G * 16
+    src = plan.array(c.MPS_PLAN_ARRAY_SLICE_SRC)
+    cols = plan.array(c.MPS_PLAN_ARRAY_SLICE_COLS)
+    vals = plan.array(c.MPS_PLAN_ARRAY_SLICE_VALS)
+    want_src = np.full(src.size, -1, dtype=np.int64)
+    for p in range(i.num_partitions):
+        w, g = divmod(p, G)
+        k = np.arange(cnt[p])
+        slot = (wave_off[w] + k // 16) * (G * 16) + g * 16 + k % 16
+        want_src[slot] = perm[ys[p] + k]
+    assert np.array_equal(src, want_src)
+    live = want_src >= 0
+    assert live.sum() == nnz
+    assert np.array_equal(cols[live], ci[want_src[live]]) and (cols[~live] == 0).all()
+    assert np.array_equal(vals[live], val[want_src[live]]) and (vals[~live] == 0).all()
+
+
+@pytest.mark.parametrize("tiling,slab_bytes,cost,tpw", [("off", 0, 16, 0), ("force", 16384, 16, 0), ("force", 4096, 7, 3),
+                                                        ("force", 1 << 20, 64, 16), ("force", 8192, 128, 1)])
+def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw):
+    rng = np.random.default_rng(cost + slab_bytes)
+    n = 500
+    rp, ci = random_csr(rng, n, 40, hub_rows=[(3, 450), (499, 300)])
+    val = rng.random(ci.size).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    plan = pkg.spmm.Plan(csr, 16, cost=cost, threads_per_wave=tpw, tiling=tiling, slab_bytes=slab_bytes)
+    if tiling == "force":
+        assert plan.info.num_slabs == -(-n // plan.info.slab_cols) and plan.info.slab_cols % 64 == 0
+    else:
+        assert plan.info.num_slabs == 1
+    check_plan_layout(pkg, orc, plan, rp, ci, val)
+    # new values flow through set_values
+    val2 = rng.random(ci.size).astype(np.float32)
+    plan.set_values(torch.from_numpy(val2).to(dev))
+    check_plan_layout(pkg, orc, plan, rp, ci, val2)
+    plan.close()
+
+
+def test_unsorted_rows(pkg, dev):
+    n = 130  # two 64-column slabs
+    rp = np.concatenate([[0, 3, 5], np.full(n - 2, 5)]).astype(np.int32)
+    ci = np.array([100, 70, 0, 0, 129], dtype=np.int32)  # row 0 decreasing
+    csr = make_csr(pkg, dev, rp, ci, np.ones(5, dtype=np.float32))
+    with pytest.raises(pkg.MpsError) as e:
+        pkg.spmm.Plan(csr, 16, cost=4, tiling="force", slab_bytes=4096)
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSORTED
+    # a decrease exactly at a row boundary is fine, and so are repeated ids
+    ci_ok = np.array([0, 70, 70, 0, 129], dtype=np.int32)
+    csr = make_csr(pkg, dev, rp, ci_ok, np.ones(5, dtype=np.float32))
+    assert pkg.spmm.Plan(csr, 16, cost=4, tiling="force", slab_bytes=4096).info.num_slabs == 3
+
+
+def test_unsorted_rows_fall_back_to_untiled_in_auto_mode(pkg, orc, dev):
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=60000,nnz=6000000,gamma=2.1,dmax=5000", seed=4)
+    n, K = rp.size - 1, 16
+    ci = ci.copy()
+    lo, hi = rp[10], rp[11]
+    ci[lo:hi] = ci[lo:hi][::-1]  # one row descending
+    val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+    X = g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    assert pkg.spmm.tile_shape(n, ci.size, K)[0] > 1
+    plan = pkg.spmm.Plan(csr, K, cost=64)
+    assert plan.info.num_slabs == 1
+    (d_X,) = to_dev(dev, X)
+    Y = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+
+
+@pytest.mark.parametrize("K", [1, 4, 16, 20, 64, 256, 260])
+def test_plan_spmm_against_oracle(pkg, orc, dev, K):
+    rng = np.random.default_rng(100 + K)
+    n = 900
+    rp, ci = random_csr(rng, n, 60, hub_rows=[(0, 800), (450, 777), (899, 600)])
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    for tiling, slab_bytes, cost, tpw in (("off", 0, 32, 0), ("force", 320 * K * 4, 32, 0), ("force", 128 * K * 4, 128, 0),
+                                          ("force", 64 * K * 4, 7, 1), ("off", 0, 7, 0)):
+        plan = pkg.spmm.Plan(csr, K, cost=cost, threads_per_wave=tpw, tiling=tiling, slab_bytes=slab_bytes)
+        out = torch.full_like(d_X, float("nan"))
+        Y = plan.spmm(d_X, out=out)
+        torch.cuda.synchronize()
+        check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+        again = plan.spmm(d_X, out=torch.empty_like(d_X))
+        assert torch.equal(Y, again)  # deterministic
+        plan.close()
+
+
+def test_plan_edge_shapes(pkg, orc, dev):
+    rng = np.random.default_rng(6)
+    K = 16
+    for deg in (np.array([300, 0, 0, 1, 2, 0]), np.array([0, 0, 5000, 0]), np.zeros(50, dtype=np.int64), np.array([9]),
+                np.array([1, 1, 1, 1, 777]), np.array([0, 1, 0])):
+        n = max(int(deg.size), int(deg.max()) if deg.size else 1, 16)
+        deg_full = np.zeros(n, dtype=np.int64)
+        deg_full[: deg.size] = deg
+        rp = np.concatenate([[0], np.cumsum(deg_full)]).astype(np.int32)
+        ci = np.concatenate([np.sort(rng.choice(n, size=int(d), replace=False)) for d in deg_full] +
+                            [np.zeros(0, dtype=np.int64)]).astype(np.int32)
+        val = rng.random(ci.size).astype(np.float32)
+        X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+        ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+        csr = make_csr(pkg, dev, rp, ci, val)
+        (d_X,) = to_dev(dev, X)
+        for tiling, sb, cost in (("off", 0, 1), ("off", 0, 64), ("force", 64 * K * 4, 5), ("force", 1024 * K * 4, 256)):
+            plan = pkg.spmm.Plan(csr, K, cost=cost, tiling=tiling, slab_bytes=sb)
+            Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan"))).cpu().numpy()
+            check_fp32(Y, ref, scale, rel_elem=False)
+            assert (Y[deg_full == 0] == 0).all()
+            plan.close()
+
+
+def test_tile_shape_heuristic(pkg):
+    sp = pkg.spmm
+    # config 2: X = 14.9 MB, ~492 nonzeros per row -> 8 slabs of ~2 MiB
+    ns, sc = sp.tile_shape(232965, 114604189, 16, 4)
+    assert ns == 8 and sc * 16 * 4 <= (2 << 20) + 64 * 64 and ns * sc >= 232965
+    assert sp.tile_shape(4096, 32731, 16, 4)[0] == 1  # X fits in L2
+    assert sp.tile_shape(1048576, 16086273, 16, 4)[0] == 1  # too few nonzeros per row and slab
+
+
+def test_power_law_graph_auto_plan(pkg, orc, dev):
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=100000,nnz=20000000,gamma=2.1,dmax=9000", seed=2)
+    n, K = rp.size - 1, 16
+    val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+    X = g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, K, cost=128)
+    assert plan.info.num_slabs == 4
+    Y = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    # the plain path on the caller's CSR agrees to rounding
+    sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz, cost=128)
+    Y0 = pkg.spmm.spmm_merge_path(csr, d_X, sched)
+    assert (Y - Y0).abs().max().item() <= 1e-3
