@@ -1,0 +1,124 @@
+"""The four driver programs end to end on the GPU: reference command lines,
+first stdout line, error exits, and the result matrix against the oracle."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "mergepath-spmm_amd", "csrc")
+
+
+def run(prog, *args, expect=0):
+    exe = os.path.join(CSRC, prog)
+    assert os.path.exists(exe), "driver %s is not built" % prog
+    p = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=110)
+    assert p.returncode == expect, (prog, args, p.returncode, p.stdout[-2000:], p.stderr[-2000:])
+    return p.stdout
+
+
+def inputs(pkg, path, K, half=False):
+    g = pkg.graphs
+    rp, ci, _ = g.read_csr(path)
+    n = rp.size - 1
+    fill = g.fill_uniform_f16 if half else g.fill_uniform_f32
+    return rp, ci, fill(ci.size, 11, 0.0, 1.0), fill(n * K, 13, -1.0, 1.0).reshape(n, K)
+
+
+@pytest.fixture(scope="module")
+def graph_file(pkg, tmp_path_factory):
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=3000,nnz=90000,gamma=2.1,dmax=900", seed=5)
+    path = tmp_path_factory.mktemp("csr") / "g.csr"
+    g.write_csr(path, rp, ci)
+    return str(path)
+
+
+def last_json(out):
+    return json.loads(out.strip().splitlines()[-1])
+
+
+def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
+    K = 16
+    rp, ci, val, X = inputs(pkg, graph_file, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    for cost, tpw in ((32, 16), ("default", 64), (7, 1), (128, 0)):
+        dump = tmp_path / "y.bin"
+        out = run("MergePathSpMM", graph_file, K, cost, tpw, 3, "--dump", dump)
+        assert out.splitlines()[0] == "Total number of rows: %d and non-zeros: %d" % (rp.size - 1, ci.size)
+        Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
+        err = np.abs(Y - ref)
+        assert (err <= 1e-5 * scale + 1e-6).all()
+        j = last_json(out)
+        assert j["kernel"] == "merge_path" and j["repeat"] == 3 and j["nnz"] == ci.size
+        assert j["P"] == orc.num_partitions(rp.size - 1, ci.size, 128 if cost == "default" else cost)
+        assert abs(j["checksum"] - Y.astype(np.float64).sum()) <= 1e-6 * np.abs(Y).sum() + 1e-6
+
+
+def test_merge_path_driver_errors(graph_file):
+    out = run("MergePathSpMM", graph_file, 16, 32, expect=255)  # too few arguments -> usage, exit(-1)
+    assert out.startswith("Usage: ./application <input_file> <dimension> <cost> <threads_per_wave> <repeat>")
+    out = run("MergePathSpMM", graph_file, 16, 32, 17, 1, expect=255)  # more partitions than a wave holds
+    assert "Cannot process the given number of threads withing a warp." in out
+    assert "Max threads per warp can be 16" in out
+    run("MergePathSpMM", "/nonexistent/file.csr", 16, 32, 16, 1, expect=1)
+    run("MergePathSpMM", os.path.join(ROOT, "tests", "golden", "bad_cell.csr"), 16, 32, 16, 1, expect=1)
+
+
+def test_merge_path_driver_synthetic_and_wide(pkg, orc, tmp_path):
+    dump = tmp_path / "y.bin"
+    out = run("MergePathSpMM", "gen:er:n=4096,deg=8", 64, 16, 4, 2, "--dump", dump, "--seed", 1)
+    rp, ci, _ = pkg.graphs.generate("er:n=4096,deg=8", seed=1)
+    assert out.splitlines()[0] == "Total number of rows: 4096 and non-zeros: %d" % ci.size
+    val = pkg.graphs.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+    X = pkg.graphs.fill_uniform_f32(4096 * 64, 13, -1.0, 1.0).reshape(4096, 64)
+    ref = orc.spmm_f64(rp, ci, val, X)
+    Y = np.fromfile(dump, dtype=np.float32).reshape(-1, 64)
+    assert (np.abs(Y - ref) <= 1e-5 * np.abs(ref) + 1e-6).all()
+
+
+def test_fp16_driver(pkg, orc, graph_file, tmp_path):
+    K = 64
+    rp, ci, val, X = inputs(pkg, graph_file, K, half=True)
+    ref, scale = orc.spmm_f64_f16in(rp, ci, val, X, want_abs=True)
+    dump = tmp_path / "y.bin"
+    out = run("MergePathSpMM_fp16", graph_file, K, 64, 8, 2, "--dump", dump)
+    Y = np.fromfile(dump, dtype=np.float16).reshape(-1, K).astype(np.float64)
+    assert (np.abs(Y - ref) <= 2e-2 * np.abs(ref) + 2e-5 * scale + 1e-6).all()
+    assert last_json(out)["dtype"] == "fp16"
+    out = run("MergePathSpMM_fp16", graph_file, K, 64, 9, 2, expect=255)
+    assert "Max threads per warp can be 8" in out
+
+
+def test_row_wise_driver(pkg, orc, graph_file, tmp_path):
+    K = 16
+    rp, ci, val, X = inputs(pkg, graph_file, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    dump = tmp_path / "y.bin"
+    out = run("row_wise", graph_file, K, 512, 2, "--dump", dump)
+    assert out.splitlines()[0].startswith("Total number of rows: 3000 and non-zeros:")
+    Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
+    assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
+    assert run("row_wise", graph_file, K, expect=255).startswith("Usage: ./application <input_file> <dimension> <num_warps> <repeat>")
+    # --print: the text dump of the reference program, one row per line, values followed by '-'
+    small = tmp_path / "tiny.csr"
+    pkg.graphs.write_csr(small, np.array([0, 2, 3, 4]), np.array([1, 2, 0, 1]))
+    lines = run("row_wise", small, 4, 2, 1, "--print").splitlines()
+    rows = [ln for ln in lines if ln.endswith("-") and ln.count("-") >= 4]
+    assert len(rows) == 3
+
+
+def test_nz_splitting_driver(pkg, orc, graph_file, tmp_path):
+    K = 16
+    rp, ci, val, X = inputs(pkg, graph_file, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    dump = tmp_path / "y.bin"
+    out = run("nz_splitting", graph_file, K, 32, 3, "--dump", dump)
+    Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
+    assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
+    assert last_json(out)["num_parts"] == orc.calculate_part_num(32, rp)
+    assert run("nz_splitting", graph_file, expect=255).startswith("Usage: ./application <input_file> <dimension> <part_size> <repeat>")
