@@ -68,6 +68,12 @@ const char *mps_version(void);
  * cost <= 0 is rejected (the reference divides by it). */
 int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out);
 
+/* The cost this library uses when the caller names none (the reference has
+ * no default; src/MergePathSpMM.cu:121 takes it from argv): 128 merge items
+ * per partition, fewer for small matrices (64 below 2^24 items, 32 below
+ * 2^21) so that the partitions still fill the GPU. */
+int mps_default_cost(int n_rows, int nnz, int *cost_out);
+
 /* Merge items per partition, src/MergePathSpMM.cu:327-328:
  *   ceil((n_rows + 1 + nnz) / P). */
 int mps_items_per_partition(int n_rows, int nnz, int P, int *ipt_out);
@@ -236,7 +242,7 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     slab-major: columns are cut into num_slabs slabs of slab_cols columns,
  *     "virtual row" v = s * n_rows + r holds the nonzeros of row r whose
  *     column lies in slab s, and the virtual rows are stored in order, so the
- *     running wavefronts gather from one ~2 MiB slab of X at a time.  The
+ *     running wavefronts gather from one ~3 MiB slab of X at a time.  The
  *     kernel then produces num_slabs fp32 partial rows per row, which a last
  *     kernel adds in slab order (deterministic).  Needs column ids sorted
  *     (non-decreasing) within every row; otherwise the plan is built untiled.
@@ -248,7 +254,7 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *   - The workspace (partial rows, carry-out records).
  *
  * mps_tile_shape: the slab count and width mps_plan_create chooses for an X
- *   of n_rows x K elements (slab_bytes = 0: 2 MiB slabs); num_slabs == 1
+ *   of n_rows x K elements (slab_bytes = 0: 3 MiB slabs); num_slabs == 1
  *   means tiling does not pay (X fits in L2, or a row holds too few nonzeros
  *   per slab).
  * mps_plan_create: d_val is fp32 (elem_bytes 4) or fp16 (2); cost and tpw as

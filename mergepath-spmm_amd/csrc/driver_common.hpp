@@ -20,7 +20,6 @@
 
 namespace drv {
 
-constexpr int kDefaultCost = 128;       // merge items per partition when <cost> is "default" or 0
 constexpr double kPeakGBs = 8000.0;     // MI355X HBM3E
 constexpr uint64_t kSeedVal = 11, kSeedX = 13, kSeedGraph = 1;
 
@@ -201,12 +200,8 @@ double finish_output(const std::vector<T> &Y, int n_rows, int K, const Options &
     return sum;
 }
 
-inline int parse_cost(const std::string &s)
-{
-    if (s == "default") return kDefaultCost;
-    int c = std::atoi(s.c_str());
-    return c == 0 ? kDefaultCost : c;
-}
+// <cost>: a number, or "default" / 0 for the library's choice (resolved once the graph is known)
+inline int parse_cost(const std::string &s) { return s == "default" ? 0 : std::atoi(s.c_str()); }
 
 }  // namespace drv
 #endif

@@ -34,7 +34,7 @@ int mergepath_main(int argc, char **argv)
         std::exit(-1);
     }
     const int dimension = std::atoi(pos[1].c_str());
-    const int cost = parse_cost(pos[2]);
+    int cost = parse_cost(pos[2]);
     int threads_per_wave = std::atoi(pos[3].c_str());
     const int repeats = std::atoi(pos[4].c_str());
     if (dimension < 1) die("dimension must be positive");
@@ -43,6 +43,7 @@ int mergepath_main(int argc, char **argv)
     Graph gr;
     load_graph(pos[0], opt.seed, gr);
     const int N = gr.n_rows, nnz = gr.nnz, K = dimension;
+    if (cost == 0) mps_ok(mps_default_cost(N, nnz, &cost), "mps_default_cost");
 
     int max_tpw = 0;
     mps_ok(mps_max_threads_per_wave(K, (int)sizeof(T), &max_tpw), "mps_max_threads_per_wave");

@@ -20,6 +20,10 @@
         if (e_ != hipSuccess) return MPS_ERR_HIP + (int)e_;     \
     } while (0)
 
+#ifndef MPS_MAIN_KERNEL_ATTR
+#define MPS_MAIN_KERNEL_ATTR
+#endif
+
 namespace {
 
 constexpr int kWavesPerBlock = 4;
@@ -221,7 +225,7 @@ __device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T 
 //   wavefront stages a round with one contiguous, fully coalesced load per
 //   array; wave_off[w + 1] - wave_off[w] is the number of rounds of wave w.
 template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED>
-__global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
+__global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
     const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
     const int *__restrict__ coord_y, const int *__restrict__ wave_off, int nnz, int K, int P,
@@ -230,9 +234,10 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
 {
     using XO = XOps<T, VEC>;
     using Raw = typename XO::Raw;
-    constexpr int kCombine = 64 * VEC;  // floats per wave for heads (and for tails)
-    constexpr int kSlice = (2 * kCombine > 2 * 16 * kWindow) ? 2 * kCombine : 2 * 16 * kWindow;
-    __shared__ float s_buf[kWavesPerBlock][kSlice];
+    constexpr int kCombine = 64 * VEC;  // floats per wave for the head partials (and for the tails)
+    constexpr int kStage = (kCombine > 2 * 16 * kWindow) ? kCombine : 2 * 16 * kWindow;
+    __shared__ float s_stage[kWavesPerBlock][kStage];   // windows; at the end, the tail partials
+    __shared__ float s_heads[kWavesPerBlock][kCombine]; // first finished row of every group
     __shared__ int s_hrow[kWavesPerBlock][16];
 
     const int wib = threadIdx.x >> 6;
@@ -255,10 +260,11 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
     const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
                                   col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
 
-    int *s_col_wave = reinterpret_cast<int *>(&s_buf[wib][0]);
-    float *s_val_wave = &s_buf[wib][16 * kWindow];
-    int *s_col = s_col_wave + g * kWindow;
-    float *s_val = s_val_wave + g * kWindow;
+    int *s_col_wave = reinterpret_cast<int *>(&s_stage[wib][0]);
+    float *s_val_wave = &s_stage[wib][16 * kWindow];
+    const int *s_col = s_col_wave + g * kWindow;
+    const float *s_val = s_val_wave + g * kWindow;
+    float *my_head = &s_heads[wib][g * KT + s * VEC];
 
     const int p = w * tpw + g;
     const bool part_ok = (g < tpw) && (p < P);
@@ -270,14 +276,14 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
         y_end = coord_y[p + 1];
     }
     // Row x - 1 is in progress; it ends where nonzero index row_ptr[x] begins.
-    // The two row ends after it are loaded ahead, so that finishing a row does
-    // not wait on memory.
+    // The row end after it is loaded ahead, so that finishing a row does not
+    // wait on memory.
     auto row_end_at = [&](int xx) { return (xx < x_end) ? row_ptr[xx] : INT_MAX; };
-    int row_end = row_end_at(x), row_end1 = row_end_at(x + 1), row_end2 = row_end_at(x + 2);
+    int row_end = row_end_at(x), row_end1 = row_end_at(x + 1);
 
-    float acc[VEC], head[VEC];
+    float acc[VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) { acc[i] = 0.f; head[i] = 0.f; }
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
     int head_row = -1;
 
     auto emit = [&]() {
@@ -285,7 +291,7 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
         if (head_row < 0) {
             head_row = row;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) head[i] = acc[i];
+            for (int i = 0; i < VEC; ++i) my_head[i] = acc[i];
         } else if (col_ok) {
             store_acc<VEC>(Y + (size_t)row * K + kcol, acc);
         }
@@ -293,8 +299,7 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
         ++x;
         row_end = row_end1;
-        row_end1 = row_end2;
-        row_end2 = row_end_at(x + 2);
+        row_end1 = row_end_at(x + 1);
     };
 
     int wbase = y_begin;
@@ -312,6 +317,16 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
     } else {
         if (stager && wbase < y_end) pw = load_win<T>(col_idx, val, nnz, wbase + 4 * s);
     }
+    auto prefetch_next = [&]() {
+        // next window: in flight while this one is consumed
+        if constexpr (SLICED) {
+            if (stager && round + 1 < round_end)
+                pw = load_slice<T>(col_idx, val, (size_t)(round + 1) * round_elems + 4 * lane);
+        } else {
+            const int nb = wbase + kWindow;
+            if (stager && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
+        }
+    };
 
     while (SLICED ? (round < round_end) : (__any(wbase < y_end) != 0)) {
         const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
@@ -322,40 +337,41 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
             }
         } else {
             if (stager && nvalid > 0) {
-                *reinterpret_cast<int4 *>(s_col + 4 * s) = pw.c;
-                *reinterpret_cast<float4 *>(s_val + 4 * s) = pw.v;
+                *reinterpret_cast<int4 *>(s_col_wave + g * kWindow + 4 * s) = pw.c;
+                *reinterpret_cast<float4 *>(s_val_wave + g * kWindow + 4 * s) = pw.v;
             }
         }
         wave_lds_sync();
+        if (__all(nvalid == kWindow)) {
+            // every group of the wave has a full window: no bounds to test
 #pragma unroll
-        for (int b = 0; b < kWindow; b += BATCH) {
-            int cols[BATCH];
-            float vals[BATCH];
-            Raw xr[BATCH];
+            for (int b = 0; b < kWindow; b += BATCH) {
+                Raw xr[BATCH];
 #pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                cols[j] = s_col[b + j];
-                vals[j] = s_val[b + j];
-            }
+                for (int j = 0; j < BATCH; ++j) xr[j] = gx.load(s_col[b + j]);
+                if (b == 0) prefetch_next();
 #pragma unroll
-            for (int j = 0; j < BATCH; ++j)
-                if (b + j < nvalid) xr[j] = gx.load(cols[j]);
-            if (b == 0) {
-                // next window: in flight while this one is consumed
-                if constexpr (SLICED) {
-                    if (stager && round + 1 < round_end)
-                        pw = load_slice<T>(col_idx, val, (size_t)(round + 1) * round_elems + 4 * lane);
-                } else {
-                    const int nb = wbase + kWindow;
-                    if (stager && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                if (b + j < nvalid) {
+                for (int j = 0; j < BATCH; ++j) {
                     const int idx = wbase + b + j;
                     while (idx == row_end) emit();
-                    XO::fma(acc, vals[j], xr[j]);
+                    XO::fma(acc, s_val[b + j], xr[j]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < kWindow; b += BATCH) {
+                Raw xr[BATCH];
+#pragma unroll
+                for (int j = 0; j < BATCH; ++j)
+                    if (b + j < nvalid) xr[j] = gx.load(s_col[b + j]);
+                if (b == 0) prefetch_next();
+#pragma unroll
+                for (int j = 0; j < BATCH; ++j) {
+                    if (b + j < nvalid) {
+                        const int idx = wbase + b + j;
+                        while (idx == row_end) emit();
+                        XO::fma(acc, s_val[b + j], xr[j]);
+                    }
                 }
             }
         }
@@ -366,13 +382,10 @@ __global__ __launch_bounds__(kBlock) void mp_spmm_kernel(
     while (x < x_end) emit();  // rows that end exactly where the partition ends
 
     // ---- combine the groups of this wavefront -------------------------------
-    float *heads = &s_buf[wib][0];
-    float *tails = heads + kCombine;
+    const float *heads = &s_heads[wib][0];
+    float *tails = &s_stage[wib][0];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        heads[g * KT + s * VEC + i] = head[i];
-        tails[g * KT + s * VEC + i] = acc[i];
-    }
+    for (int i = 0; i < VEC; ++i) tails[g * KT + s * VEC + i] = acc[i];
     if (s == 0) s_hrow[wib][g] = head_row;
     wave_lds_sync();
 
@@ -567,13 +580,15 @@ inline size_t carry_bytes_for(int num_waves, int K)
     return rows * sizeof(int) + 2 * (size_t)num_waves * K * sizeof(float);
 }
 
-// Gathers in flight per lane between waits: tuning knob, 8 or 16.
+// Gathers in flight per lane between waits.  Fewer means fewer registers and
+// more resident wavefronts, which is what keeps the L1's request queue full;
+// 4 measured best on MI355X.  MPS_GATHER_BATCH=2|4|8 overrides it for tuning.
 inline int gather_batch()
 {
     static int b = [] {
         const char *e = std::getenv("MPS_GATHER_BATCH");
         int v = e ? std::atoi(e) : 0;
-        return v == 16 ? 16 : 8;
+        return (v == 8 || v == 2) ? v : 4;
     }();
     return b;
 }
@@ -596,17 +611,22 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
     hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED>), grid, dim3(kBlock), 0, st, row_ptr, \
                        col_idx, val, X, Y, cx, cy, wave_off, nnz, K, P, sh.ls.lanes_log2, sh.tpw, W,           \
                        sh.row_shift, ws_head_row, ws_head, ws_tail)
+        const int batch = gather_batch();
         if (wave_off) {
             if (sh.row_shift >= 0) {
-                if (gather_batch() == 16) MPS_LAUNCH_MAIN(true, 16, true); else MPS_LAUNCH_MAIN(true, 8, true);
+                if (batch == 8) MPS_LAUNCH_MAIN(true, 8, true);
+                else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, true);
+                else MPS_LAUNCH_MAIN(true, 4, true);
             } else {
-                MPS_LAUNCH_MAIN(false, 8, true);
+                MPS_LAUNCH_MAIN(false, 4, true);
             }
         } else {
             if (sh.row_shift >= 0) {
-                if (gather_batch() == 16) MPS_LAUNCH_MAIN(true, 16, false); else MPS_LAUNCH_MAIN(true, 8, false);
+                if (batch == 8) MPS_LAUNCH_MAIN(true, 8, false);
+                else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, false);
+                else MPS_LAUNCH_MAIN(true, 4, false);
             } else {
-                MPS_LAUNCH_MAIN(false, 8, false);
+                MPS_LAUNCH_MAIN(false, 4, false);
             }
         }
 #undef MPS_LAUNCH_MAIN

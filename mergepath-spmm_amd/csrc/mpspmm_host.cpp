@@ -659,6 +659,14 @@ int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out)
     return MPS_OK;
 }
 
+int mps_default_cost(int n_rows, int nnz, int *cost_out)
+{
+    if (!cost_out || n_rows < 0 || nnz < 0) return MPS_ERR_INVALID_ARG;
+    const int64_t total = (int64_t)n_rows + 1 + nnz;
+    *cost_out = total >= (1 << 24) ? 128 : total >= (1 << 21) ? 64 : 32;
+    return MPS_OK;
+}
+
 int mps_items_per_partition(int n_rows, int nnz, int P, int *ipt_out)
 {
     if (!ipt_out || n_rows < 0 || nnz < 0 || P <= 0) return MPS_ERR_INVALID_ARG;

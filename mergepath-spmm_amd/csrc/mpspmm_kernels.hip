@@ -15,14 +15,8 @@
 // wavefront through LDS, and what still crosses the wavefront boundary is
 // written to a carry-out record that a second kernel folds in.  No atomics.
 //
-// Column-slab tiling.  The dense-row gathers are served by the L2 of the XCD
-// the wavefront runs on (4 MiB each); a feature matrix larger than that
-// misses to the fabric, whose request rate then bounds the kernel.  The tiled
-// entry points reorder the nonzeros slab-major (all rows of column slab 0,
-// then slab 1, ...), so that at any moment the running wavefronts gather from
-// one ~2 MiB slab of X, and run the same merge-path kernel over the resulting
-// num_slabs * n_rows "virtual rows"; a last kernel adds the per-slab partial
-// rows in slab order.
+// Plans (mpspmm_plan.hip) run the same kernel over a column-slab tiled,
+// sliced copy of the matrix.
 #include "mpspmm_device.hpp"
 
 namespace {
@@ -483,7 +477,7 @@ int mps_rowwise_spmm_f32(const int *d_row_ptr, const int *d_col_idx, const float
     dim3 grid((num_waves + kWavesPerBlock - 1) / kWavesPerBlock, ls.col_tiles);
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define MPS_LAUNCH_ROWWISE(VEC, POW2)                                                                     \
-    hipLaunchKernelGGL((rowwise_spmm_kernel<float, VEC, POW2, 8>), grid, dim3(kBlock), 0, st, d_row_ptr,  \
+    hipLaunchKernelGGL((rowwise_spmm_kernel<float, VEC, POW2, 4>), grid, dim3(kBlock), 0, st, d_row_ptr,  \
                        d_col_idx, d_val, d_X, d_Y, n_rows, nnz, K, ls.lanes_log2, num_waves, row_shift, step)
     if (ls.vec == 4) { if (row_shift >= 0) MPS_LAUNCH_ROWWISE(4, true); else MPS_LAUNCH_ROWWISE(4, false); }
     else { if (row_shift >= 0) MPS_LAUNCH_ROWWISE(1, true); else MPS_LAUNCH_ROWWISE(1, false); }
@@ -554,7 +548,7 @@ int mps_nzsplit_spmm_f32(const int *d_col_idx, const float *d_val, const float *
     int num_waves = (num_parts + ls.groups - 1) / ls.groups;
     dim3 grid((num_waves + kWavesPerBlock - 1) / kWavesPerBlock, ls.col_tiles);
 #define MPS_LAUNCH_NZSPLIT(VEC, POW2)                                                                    \
-    hipLaunchKernelGGL((nzsplit_spmm_kernel<float, VEC, POW2, 8>), grid, dim3(kBlock), 0, st, d_col_idx, \
+    hipLaunchKernelGGL((nzsplit_spmm_kernel<float, VEC, POW2, 4>), grid, dim3(kBlock), 0, st, d_col_idx, \
                        d_val, d_X, d_Y, nnz, K, ls.lanes_log2, row_shift, d_part_ptr, d_part2node,       \
                        num_parts, num_waves)
     if (ls.vec == 4) { if (row_shift >= 0) MPS_LAUNCH_NZSPLIT(4, true); else MPS_LAUNCH_NZSPLIT(4, false); }

@@ -13,8 +13,11 @@ import torch
 from . import _cabi
 from ._cabi import check
 
-# Merge items (row ends + nonzeros) per partition when the caller gives no cost.
-DEFAULT_COST = 128
+def default_cost(n_rows, nnz):
+    """Merge items (row ends + nonzeros) per partition when the caller gives no cost."""
+    c = ctypes.c_int()
+    check(_cabi.lib().mps_default_cost(int(n_rows), int(nnz), ctypes.byref(c)), "mps_default_cost")
+    return c.value
 
 
 def _stream():
@@ -92,7 +95,7 @@ def generate_mp_sched(row_ptr, nnz, cost=None, P=None):
     _need(row_ptr, torch.int32, "row_ptr")
     n_rows = int(row_ptr.numel()) - 1
     if P is None:
-        P = num_partitions(n_rows, nnz, DEFAULT_COST if cost is None else cost)
+        P = num_partitions(n_rows, nnz, default_cost(n_rows, nnz) if cost is None else cost)
     cx = torch.empty(P + 1, dtype=torch.int32, device=row_ptr.device)
     cy = torch.empty(P + 1, dtype=torch.int32, device=row_ptr.device)
     check(_cabi.lib().mps_partition(_ptr(row_ptr), n_rows, int(nnz), int(P), _ptr(cx), _ptr(cy), _stream()),
@@ -146,7 +149,7 @@ class Plan:
         eb = 4 if self.dtype == torch.float32 else 2
         flags = {"auto": 0, "off": _cabi.MPS_PLAN_NO_TILING, "force": _cabi.MPS_PLAN_FORCE_TILING}[tiling]
         check(_cabi.lib().mps_plan_create(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
-                                          int(K), eb, int(DEFAULT_COST if cost is None else cost),
+                                          int(K), eb, int(default_cost(csr.n_rows, csr.nnz) if cost is None else cost),
                                           int(threads_per_wave), flags, int(slab_bytes), _stream(),
                                           ctypes.byref(self._h)), "mps_plan_create")
         self.K, self.n_rows = int(K), csr.n_rows

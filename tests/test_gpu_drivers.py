@@ -55,7 +55,7 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
         assert (err <= 1e-5 * scale + 1e-6).all()
         j = last_json(out)
         assert j["kernel"] == "merge_path" and j["repeat"] == 3 and j["nnz"] == ci.size
-        assert j["P"] == orc.num_partitions(rp.size - 1, ci.size, 128 if cost == "default" else cost)
+        assert j["P"] == orc.num_partitions(rp.size - 1, ci.size, 32 if cost == "default" else cost)  # small graph: 32
         assert abs(j["checksum"] - Y.astype(np.float64).sum()) <= 1e-6 * np.abs(Y).sum() + 1e-6
 
 

@@ -51,6 +51,8 @@ def test_num_partitions_matches_oracle(pkg, orc):
         pkg.graphs.num_partitions(2 ** 30, 2 ** 30 + 5, 16)
     assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
     assert pkg.graphs.items_per_partition(6, 15, 5) == 5
+    assert pkg.spmm.default_cost(232965, 114604189) == 128 and pkg.spmm.default_cost(416349, 2081148) == 64
+    assert pkg.spmm.default_cost(4096, 32731) == 32
 
 
 def test_max_threads_per_wave(pkg):
