@@ -96,17 +96,21 @@ struct XOps<half_t, 1> {
 };
 
 // VEC accumulators -> VEC adjacent outputs (fp32 or fp16), one vector store
-// where the width allows.
+// where the width allows.  Non-temporal: output rows are written once and not
+// read again by the kernel, so they should not displace X in L2.
 template <int VEC>
 __device__ __forceinline__ void store_acc(float *p, const float (&acc)[VEC])
 {
+    typedef float f4_t __attribute__((ext_vector_type(4)));
     if constexpr (VEC % 4 == 0) {
 #pragma unroll
-        for (int i = 0; i < VEC; i += 4)
-            *reinterpret_cast<float4 *>(p + i) = make_float4(acc[i], acc[i + 1], acc[i + 2], acc[i + 3]);
+        for (int i = 0; i < VEC; i += 4) {
+            f4_t v = {acc[i], acc[i + 1], acc[i + 2], acc[i + 3]};
+            __builtin_nontemporal_store(v, reinterpret_cast<f4_t *>(p + i));
+        }
     } else {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) p[i] = acc[i];
+        for (int i = 0; i < VEC; ++i) __builtin_nontemporal_store(acc[i], p + i);
     }
 }
 template <int VEC>
@@ -116,15 +120,15 @@ __device__ __forceinline__ void store_acc(half_t *p, const float (&acc)[VEC])
         half8_t o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = (half_t)acc[i];
-        *reinterpret_cast<half8_t *>(p) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<half8_t *>(p));
     } else if constexpr (VEC == 4) {
         half4_t o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = (half_t)acc[i];
-        *reinterpret_cast<half4_t *>(p) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<half4_t *>(p));
     } else {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) p[i] = (half_t)acc[i];
+        for (int i = 0; i < VEC; ++i) __builtin_nontemporal_store((half_t)acc[i], p + i);
     }
 }
 
