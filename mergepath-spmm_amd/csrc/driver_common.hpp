@@ -48,6 +48,9 @@ struct Options {
     bool print_matrix = false;  // --print: the "v-" text dump of src/row_wise.cu:162-168
     int warmup = 3;
     uint64_t seed = kSeedGraph;
+    bool use_plan = true;       // --no-plan: CSR entry points on the caller's arrays, no preprocessing
+    int tiling = 0;             // --tiling off|force (default: where it pays)
+    size_t slab_bytes = 0;      // --slab-bytes N (default: the library's 3 MiB)
 };
 
 // Strips the optional trailing flags; returns the positional arguments.
@@ -58,6 +61,12 @@ inline std::vector<std::string> split_args(int argc, char **argv, Options &opt)
         std::string a = argv[i];
         if (a == "--dump" && i + 1 < argc) opt.dump_path = argv[++i];
         else if (a == "--print") opt.print_matrix = true;
+        else if (a == "--no-plan") opt.use_plan = false;
+        else if (a == "--slab-bytes" && i + 1 < argc) opt.slab_bytes = std::strtoull(argv[++i], nullptr, 10);
+        else if (a == "--tiling" && i + 1 < argc) {
+            std::string t = argv[++i];
+            opt.tiling = t == "off" ? MPS_PLAN_NO_TILING : t == "force" ? MPS_PLAN_FORCE_TILING : 0;
+        }
         else if (a == "--warmup" && i + 1 < argc) opt.warmup = std::atoi(argv[++i]);
         else if (a == "--seed" && i + 1 < argc) opt.seed = std::strtoull(argv[++i], nullptr, 10);
         else pos.push_back(a);

@@ -15,6 +15,7 @@ template <> struct Elem<float> {
     static int spmm(const int *rp, const int *ci, const float *v, const float *X, float *Y, int n, int nnz, int K, int P,
                     const int *cx, const int *cy, int tpw, void *ws, size_t wsb)
     { return mps_spmm_f32(rp, ci, v, X, Y, n, nnz, K, P, cx, cy, tpw, ws, wsb, nullptr); }
+    static int plan_spmm(const mps_plan *pl, const float *X, float *Y) { return mps_plan_spmm_f32(pl, X, Y, nullptr); }
 };
 template <> struct Elem<uint16_t> {
     static constexpr const char *name = "fp16";
@@ -22,6 +23,7 @@ template <> struct Elem<uint16_t> {
     static int spmm(const int *rp, const int *ci, const uint16_t *v, const uint16_t *X, uint16_t *Y, int n, int nnz, int K,
                     int P, const int *cx, const int *cy, int tpw, void *ws, size_t wsb)
     { return mps_spmm_f16(rp, ci, v, X, Y, n, nnz, K, P, cx, cy, tpw, ws, wsb, nullptr); }
+    static int plan_spmm(const mps_plan *pl, const uint16_t *X, uint16_t *Y) { return mps_plan_spmm_f16(pl, X, Y, nullptr); }
 };
 
 template <typename T>
@@ -55,9 +57,8 @@ int mergepath_main(int argc, char **argv)
         std::exit(-1);
     }
 
-    int P = 0, ipt = 0;
+    int P = 0;
     mps_ok(mps_num_partitions(N, nnz, cost, &P), "mps_num_partitions");
-    mps_ok(mps_items_per_partition(N, nnz, P, &ipt), "mps_items_per_partition");
 
     std::vector<T> h_val((size_t)nnz), h_X((size_t)N * K), h_Y((size_t)N * K);
     mps_ok(Elem<T>::fill(h_val.data(), h_val.size(), kSeedVal, 0.0f, 1.0f), "fill val");
@@ -71,27 +72,49 @@ int mergepath_main(int argc, char **argv)
     d_X.upload(h_X.data());
     mps_ok(mps_csr_validate(d_rp.p, d_ci.p, N, N, nnz, nullptr), "mps_csr_validate");
 
+    // Everything that depends on the matrix alone is built once, outside the
+    // repeat loop, as generate_mp_sched and its uploads are (:192-220): with a
+    // plan (default) the tiled / sliced copy and the partition; with --no-plan
+    // the partition of the caller's arrays only.
     size_t ws_bytes = 0;
-    mps_ok(mps_spmm_workspace_bytes(P, K, threads_per_wave, (int)sizeof(T), &ws_bytes), "mps_spmm_workspace_bytes");
-    DevBuf<unsigned char> d_ws(ws_bytes);
-
-    // the schedule is built once, outside the repeat loop, as generate_mp_sched is (:192)
-    Timing plan = time_launches(1, 3, [&] { mps_ok(mps_partition(d_rp.p, N, nnz, P, d_cx.p, d_cy.p, nullptr), "mps_partition"); });
-
+    DevBuf<unsigned char> d_ws;
+    mps_plan *plan = nullptr;
+    mps_plan_info info{};
+    Timing prep;
     hip_ok(hipMemset(d_Y.p, 0xff, d_Y.n * sizeof(T)), "hipMemset");
-    Timing t = time_launches(opt.warmup, repeats, [&] {
-        mps_ok(Elem<T>::spmm(d_rp.p, d_ci.p, d_val.p, d_X.p, d_Y.p, N, nnz, K, P, d_cx.p, d_cy.p, threads_per_wave, d_ws.p,
-                             ws_bytes), "mps_spmm");
-    });
+    Timing t;
+    if (opt.use_plan) {
+        hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        prep = time_launches(0, 1, [&] {
+            mps_ok(mps_plan_create(d_rp.p, d_ci.p, d_val.p, N, nnz, K, (int)sizeof(T), cost, threads_per_wave,
+                                   (unsigned)opt.tiling, opt.slab_bytes, nullptr, &plan), "mps_plan_create");
+        });
+        mps_ok(mps_plan_get_info(plan, &info), "mps_plan_get_info");
+        P = info.num_partitions;
+        t = time_launches(opt.warmup, repeats, [&] { mps_ok(Elem<T>::plan_spmm(plan, d_X.p, d_Y.p), "mps_plan_spmm"); });
+    } else {
+        mps_ok(mps_spmm_workspace_bytes(P, K, threads_per_wave, (int)sizeof(T), &ws_bytes), "mps_spmm_workspace_bytes");
+        d_ws.alloc(ws_bytes);
+        prep = time_launches(1, 3, [&] { mps_ok(mps_partition(d_rp.p, N, nnz, P, d_cx.p, d_cy.p, nullptr), "mps_partition"); });
+        t = time_launches(opt.warmup, repeats, [&] {
+            mps_ok(Elem<T>::spmm(d_rp.p, d_ci.p, d_val.p, d_X.p, d_Y.p, N, nnz, K, P, d_cx.p, d_cy.p, threads_per_wave, d_ws.p,
+                                 ws_bytes), "mps_spmm");
+        });
+    }
     d_Y.download(h_Y.data());
     double checksum = finish_output(h_Y, N, K, opt);
 
-    std::printf("partitions: %d (cost %d, %d merge items each), threads_per_wave %d, max row degree %d\n", P, cost, ipt,
-                threads_per_wave, gr.max_degree);
-    std::printf("partitioner: avg %.2f us per build (not in the launch time below)\n", plan.avg_us);
+    std::printf("partitions: %d (cost %d), threads_per_wave %d, max row degree %d\n", P, cost, threads_per_wave,
+                gr.max_degree);
+    if (plan)
+        std::printf("plan: %d column slab(s) of %d columns, %lld sliced rounds, %.1f MB of device memory\n", info.num_slabs,
+                    info.slab_cols, info.total_rounds, info.device_bytes / 1e6);
+    std::printf("preprocessing: %.2f us, once per matrix (not in the launch time below)\n", prep.avg_us);
     char extra[256];
-    std::snprintf(extra, sizeof extra, ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan_us\": %.3f", P, cost,
-                  threads_per_wave, plan.avg_us);
+    std::snprintf(extra, sizeof extra,
+                  ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan\": %s, \"num_slabs\": %d, \"prep_us\": %.3f", P,
+                  cost, threads_per_wave, plan ? "true" : "false", plan ? info.num_slabs : 1, prep.avg_us);
+    mps_plan_destroy(plan);
     report("merge_path", Elem<T>::name, N, nnz, K, (int)sizeof(T), (int)sizeof(T), repeats, t, checksum, extra);
     return 0;
 }

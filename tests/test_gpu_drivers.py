@@ -46,16 +46,19 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
     K = 16
     rp, ci, val, X = inputs(pkg, graph_file, K)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
-    for cost, tpw in ((32, 16), ("default", 64), (7, 1), (128, 0)):
+    for cost, tpw, extra in ((32, 16, ()), ("default", 64, ()), (7, 1, ("--no-plan",)), (128, 0, ("--no-plan",)),
+                             (16, 16, ("--tiling", "force", "--slab-bytes", 65536))):
         dump = tmp_path / "y.bin"
-        out = run("MergePathSpMM", graph_file, K, cost, tpw, 3, "--dump", dump)
+        out = run("MergePathSpMM", graph_file, K, cost, tpw, 3, "--dump", dump, *extra)
         assert out.splitlines()[0] == "Total number of rows: %d and non-zeros: %d" % (rp.size - 1, ci.size)
         Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
         err = np.abs(Y - ref)
         assert (err <= 1e-5 * scale + 1e-6).all()
         j = last_json(out)
         assert j["kernel"] == "merge_path" and j["repeat"] == 3 and j["nnz"] == ci.size
-        assert j["P"] == orc.num_partitions(rp.size - 1, ci.size, 32 if cost == "default" else cost)  # small graph: 32
+        slabs = j["num_slabs"]
+        assert j["plan"] == ("--no-plan" not in extra) and (slabs > 1) == ("force" in extra)
+        assert j["P"] == orc.num_partitions(slabs * (rp.size - 1), ci.size, 32 if cost == "default" else cost)  # small graph: 32
         assert abs(j["checksum"] - Y.astype(np.float64).sum()) <= 1e-6 * np.abs(Y).sum() + 1e-6
 
 
