@@ -25,6 +25,14 @@ import __graft_entry__ as entry  # noqa: E402
 
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch of the main kernel, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
+# profiles/mp_spmm_kernel_chunglu_233k_f32_k16.md (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors the copy
+# probe gives, profiles/hbm_copy_probe_fetch_write_calibration.md).  Keyed by (workload, layout); other
+# configurations report null.
+MEASURED_TRAFFIC = {
+    ("chunglu_233k_f32_k16", "plan", 5, 128): int(544711 * 1024 * 2.0 + 80402 * 1024 * 1.0),
+}
+
 WORKLOADS = {
     # name: (generator spec, K, dtype)
     "chunglu_233k_f32_k16": ("chunglu:n=232965,nnz=114600000,gamma=2.1,dmax=20000", 16, "f32"),
@@ -183,7 +191,9 @@ def main():
                       "preprocessing, host wall time (once per matrix)": round(plan_ms, 3)},
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "roofline": {"bound": "hbm", "kernel": "mp_spmm_kernel", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, "plan" if plan is not None else "plain",
+                                                      plan.info.num_slabs if plan is not None else 1, cost)),
                      "algorithmic_bytes": int(b_alg)},
         "host_generate_s": round(gen_s, 2),
     }
