@@ -64,6 +64,8 @@ def main():
     ap.add_argument("--mode", default="auto", choices=["auto", "plain", "untiled", "tiled"],
                     help="plain = kernels on the CSR arrays as given, no plan; auto / untiled / tiled = with a plan "
                          "(column-slab tiling where it pays / never / always)")
+    ap.add_argument("--hot", default="auto", choices=["auto", "off", "force"],
+                    help="hot columns of a tiled plan (their rows of X in LDS): where they pay / never / always")
     ap.add_argument("--slab-bytes", type=int, default=0, help="slab size for tiling (0 = library default)")
     ap.add_argument("--tpw", type=int, default=0, help="partitions per wavefront (0 = full wavefront)")
     ap.add_argument("--seed", type=int, default=1)
@@ -104,7 +106,7 @@ def main():
     plan = None
     if args.mode != "plain":
         tiling = {"auto": "auto", "untiled": "off", "tiled": "force"}[args.mode]
-        plan = sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes)
+        plan = sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes, hot=args.hot)
         P = plan.info.num_partitions
     else:
         sched = sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
@@ -154,7 +156,7 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     if plan is not None:
-        sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes).close()
+        sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes, hot=args.hot).close()
     else:
         sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
     torch.cuda.synchronize()
@@ -183,7 +185,10 @@ def main():
                    "threads_per_wave": args.tpw or g.max_threads_per_wave(K, eb), "seed": args.seed,
                    "layout": "plain CSR, no plan" if plan is None else
                    ("plan: %d column slab(s) of %d, sliced, %.0f MB" % (plan.info.num_slabs, plan.info.slab_cols,
-                                                                       plan.info.device_bytes / 1e6))},
+                                                                       plan.info.device_bytes / 1e6)) +
+                   ("" if plan is None or plan.info.hot_rows == 0 else
+                    ", %d hot columns per slab in LDS (%.1f %% of the nonzeros)"
+                    % (plan.info.hot_rows, 100.0 * plan.info.hot_nnz / max(nnz, 1)))},
         "gbs_algorithmic_per_step": round(b_alg / (ms_per_step * 1e6), 2),
         "hbm_fraction_per_step": round(b_alg / (ms_per_step * 1e6) / PEAK_HBM_GBS, 4),
         "kernel_ms": {"mp_spmm_kernel": round(main_ms, 5), "mp_fixup_kernel": round(fix_ms, 5),

@@ -246,8 +246,19 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     kernel then produces num_slabs fp32 partial rows per row, which a last
  *     kernel adds in slab order (deterministic).  Needs column ids sorted
  *     (non-decreasing) within every row; otherwise the plan is built untiled.
+ *   - Hot columns (tiled plans, row pitch a power of two up to ~256 bytes).
+ *     Inside every slab the hot_rows columns with the most nonzeros (as many
+ *     rows of X as fit in the 160 KiB LDS of a CU beside the kernel's own
+ *     buffers: 1,728 at K = 16 fp32) form a "hot" segment; the workgroups
+ *     that process it copy those rows of X into LDS once and gather from
+ *     there, the remaining columns of the slab form the "cold" segment,
+ *     gathered through L2.  Segments are ordered hot first (virtual row
+ *     v = seg * n_rows + r, 2 * num_slabs segments), each is partitioned on
+ *     its own, and the plan runs two launches of the same kernel.  Used when
+ *     the hot columns hold at least 15 % of the nonzeros.
  *   - The merge-path partition (mps_num_partitions, mps_partition) of the
- *     num_slabs * n_rows virtual rows for the given cost.
+ *     virtual rows for the given cost: one split of all of them, or, with hot
+ *     columns, one split per segment (padded to whole workgroups).
  *   - The nonzeros "sliced" by that partition: the 16-nonzero windows that the
  *     partitions of one wavefront consume in the same round are stored side
  *     by side, so that a wavefront stages a round with one contiguous load.
@@ -272,6 +283,8 @@ typedef struct mps_plan mps_plan;
 
 #define MPS_PLAN_NO_TILING 1u    /* never tile                                  */
 #define MPS_PLAN_FORCE_TILING 2u /* tile with slab_bytes slabs whatever the shape */
+#define MPS_PLAN_NO_HOT 4u       /* never keep hot columns' rows of X in LDS     */
+#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros */
 
 typedef struct mps_plan_info {
     int n_rows, nnz, K, elem_bytes, cost, threads_per_wave;
@@ -280,6 +293,13 @@ typedef struct mps_plan_info {
     long long total_rounds;        /* sum over wavefronts of their 16-nonzero rounds */
     long long slice_slots;         /* nonzero slots incl. padding                 */
     size_t device_bytes;           /* device memory the plan holds                */
+    int num_segments;              /* virtual-row segments: num_slabs, or 2 * num_slabs with hot columns */
+    int hot_rows;                  /* rows of X per LDS table (0: no hot launch)  */
+    int hot_waves;                 /* wavefronts of the hot launch                */
+    long long hot_nnz;             /* nonzeros gathered from LDS                  */
+    int hot_cost;                  /* merge items per partition of the hot segments */
+    int mark_shift;                /* > 0: SLICE_COLS entries are column | row_ends << mark_shift */
+    int hot_mark_shift;            /* the same for the entries of the hot wavefronts (column = LDS slot) */
 } mps_plan_info;
 
 enum {
@@ -289,7 +309,8 @@ enum {
     MPS_PLAN_ARRAY_WAVE_OFF = 3,   /* int[num_waves + 1]: first round of each wave */
     MPS_PLAN_ARRAY_SLICE_COLS = 4, /* int[slice_slots]                            */
     MPS_PLAN_ARRAY_SLICE_SRC = 5,  /* int[slice_slots]: original nonzero index, -1 = padding */
-    MPS_PLAN_ARRAY_SLICE_VALS = 6  /* elem_bytes * slice_slots                    */
+    MPS_PLAN_ARRAY_SLICE_VALS = 6, /* elem_bytes * slice_slots                    */
+    MPS_PLAN_ARRAY_HOT_COLS = 7    /* int[num_slabs * hot_rows]: column of each LDS slot, -1 = unused */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,

@@ -26,8 +26,10 @@ MPS_PHASE_FIXUP = 2
 MPS_PHASE_REDUCE = 4
 MPS_PLAN_NO_TILING = 1
 MPS_PLAN_FORCE_TILING = 2
+MPS_PLAN_NO_HOT = 4
+MPS_PLAN_FORCE_HOT = 8
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
- MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS) = range(7)
+ MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS) = range(8)
 
 
 class PlanInfo(ctypes.Structure):
@@ -35,7 +37,9 @@ class PlanInfo(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int) for n in ("n_rows", "nnz", "K", "elem_bytes", "cost", "threads_per_wave",
                                              "num_slabs", "slab_cols", "num_partitions", "num_waves")] + \
                [("total_rounds", ctypes.c_longlong), ("slice_slots", ctypes.c_longlong),
-                ("device_bytes", ctypes.c_size_t)]
+                ("device_bytes", ctypes.c_size_t), ("num_segments", ctypes.c_int), ("hot_rows", ctypes.c_int),
+                ("hot_waves", ctypes.c_int), ("hot_nnz", ctypes.c_longlong), ("hot_cost", ctypes.c_int), ("mark_shift", ctypes.c_int),
+                ("hot_mark_shift", ctypes.c_int)]
 
 c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp, _i, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64

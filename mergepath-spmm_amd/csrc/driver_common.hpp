@@ -51,6 +51,7 @@ struct Options {
     bool use_plan = true;       // --no-plan: CSR entry points on the caller's arrays, no preprocessing
     int tiling = 0;             // --tiling off|force (default: where it pays)
     size_t slab_bytes = 0;      // --slab-bytes N (default: the library's 3 MiB)
+    int hot = 0;                // --hot off|force (default: where it pays)
 };
 
 // Strips the optional trailing flags; returns the positional arguments.
@@ -66,6 +67,10 @@ inline std::vector<std::string> split_args(int argc, char **argv, Options &opt)
         else if (a == "--tiling" && i + 1 < argc) {
             std::string t = argv[++i];
             opt.tiling = t == "off" ? MPS_PLAN_NO_TILING : t == "force" ? MPS_PLAN_FORCE_TILING : 0;
+        }
+        else if (a == "--hot" && i + 1 < argc) {
+            std::string t = argv[++i];
+            opt.hot = t == "off" ? MPS_PLAN_NO_HOT : t == "force" ? MPS_PLAN_FORCE_HOT : 0;
         }
         else if (a == "--warmup" && i + 1 < argc) opt.warmup = std::atoi(argv[++i]);
         else if (a == "--seed" && i + 1 < argc) opt.seed = std::strtoull(argv[++i], nullptr, 10);

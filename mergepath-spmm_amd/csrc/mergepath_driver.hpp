@@ -87,7 +87,7 @@ int mergepath_main(int argc, char **argv)
         hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize");
         prep = time_launches(0, 1, [&] {
             mps_ok(mps_plan_create(d_rp.p, d_ci.p, d_val.p, N, nnz, K, (int)sizeof(T), cost, threads_per_wave,
-                                   (unsigned)opt.tiling, opt.slab_bytes, nullptr, &plan), "mps_plan_create");
+                                   (unsigned)(opt.tiling | opt.hot), opt.slab_bytes, nullptr, &plan), "mps_plan_create");
         });
         mps_ok(mps_plan_get_info(plan, &info), "mps_plan_get_info");
         P = info.num_partitions;
@@ -109,11 +109,16 @@ int mergepath_main(int argc, char **argv)
     if (plan)
         std::printf("plan: %d column slab(s) of %d columns, %lld sliced rounds, %.1f MB of device memory\n", info.num_slabs,
                     info.slab_cols, info.total_rounds, info.device_bytes / 1e6);
+    if (plan && info.hot_rows > 0)
+        std::printf("hot columns: %d rows of X per slab in LDS, %lld of %d nonzeros (%.1f %%), %d of %d wavefronts\n",
+                    info.hot_rows, info.hot_nnz, nnz, nnz ? 100.0 * (double)info.hot_nnz / nnz : 0.0, info.hot_waves,
+                    info.num_waves);
     std::printf("preprocessing: %.2f us, once per matrix (not in the launch time below)\n", prep.avg_us);
     char extra[256];
     std::snprintf(extra, sizeof extra,
-                  ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan\": %s, \"num_slabs\": %d, \"prep_us\": %.3f", P,
-                  cost, threads_per_wave, plan ? "true" : "false", plan ? info.num_slabs : 1, prep.avg_us);
+                  ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan\": %s, \"num_slabs\": %d, \"hot_rows\": %d, \"prep_us\": %.3f",
+                  P, cost, threads_per_wave, plan ? "true" : "false", plan ? info.num_slabs : 1, plan ? info.hot_rows : 0,
+                  prep.avg_us);
     mps_plan_destroy(plan);
     report("merge_path", Elem<T>::name, N, nnz, K, (int)sizeof(T), (int)sizeof(T), repeats, t, checksum, extra);
     return 0;

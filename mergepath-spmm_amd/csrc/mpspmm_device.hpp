@@ -20,6 +20,9 @@
         if (e_ != hipSuccess) return MPS_ERR_HIP + (int)e_;     \
     } while (0)
 
+#ifndef MPS_HOT_RPL
+#define MPS_HOT_RPL 4
+#endif
 #ifndef MPS_MAIN_KERNEL_ATTR
 #define MPS_MAIN_KERNEL_ATTR
 #endif
@@ -30,6 +33,8 @@ constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kWindow = 16;  // nonzeros staged per lane-group per round
 constexpr int kXcds = 8;     // accelerator dies of an MI355X, each with its own L2
+constexpr int kHotRoundsPerLoad = MPS_HOT_RPL;  // rounds of the sliced arrays a hot wavefront loads at a time
+constexpr int kHotWavesPerBlock = 16;  // workgroup of the LDS-resident ("hot") launch of a plan
 
 using half_t = _Float16;
 typedef half_t half8_t __attribute__((ext_vector_type(8)));
@@ -228,21 +233,33 @@ __device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T 
 //   (wave_off[w] + round) * tpw * 16 elements into the arrays, so the whole
 //   wavefront stages a round with one contiguous, fully coalesced load per
 //   array; wave_off[w + 1] - wave_off[w] is the number of rounds of wave w.
-template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED>
-__global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
+// MARKS = true (sliced arrays only): every column entry also says how many
+//   rows end in front of its nonzero, entry = column | ends << mark_shift, so
+//   the kernel never reads row_ptr while it works through a partition: no load
+//   of its own sits between the window prefetch and the gathers.
+// HOT = true: the column part of an entry is a row slot of the table of X rows
+//   that the workgroup keeps in LDS (see below).
+template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED, bool HOT, bool MARKS, int RPL>
+__global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
     const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
     const int *__restrict__ coord_y, const int *__restrict__ wave_off, int nnz, int K, int P,
-    int lanes_log2, int tpw, int num_waves, int row_shift, int *__restrict__ ws_head_row,
-    float *__restrict__ ws_head, float *__restrict__ ws_tail)
+    int lanes_log2, int tpw, int wave_begin, int wave_end, int row_shift, int *__restrict__ ws_head_row,
+    float *__restrict__ ws_head, float *__restrict__ ws_tail, const int *__restrict__ hot_cols,
+    const int *__restrict__ seg_part_off, int hot_rows, const int *__restrict__ hot_block_wave, int hot_blocks,
+    int mark_shift)
 {
+    static_assert(!MARKS || SLICED, "row marks live in the sliced arrays");
+    static_assert(!HOT || MARKS, "the hot launch reads marked entries");
+    constexpr int WPB = HOT ? kHotWavesPerBlock : kWavesPerBlock;
     using XO = XOps<T, VEC>;
     using Raw = typename XO::Raw;
     constexpr int kCombine = 64 * VEC;  // floats per wave for the head partials (and for the tails)
     constexpr int kStage = (kCombine > 2 * 16 * kWindow) ? kCombine : 2 * 16 * kWindow;
-    __shared__ float s_stage[kWavesPerBlock][kStage];   // windows; at the end, the tail partials
-    __shared__ float s_heads[kWavesPerBlock][kCombine]; // first finished row of every group
-    __shared__ int s_hrow[kWavesPerBlock][16];
+    __shared__ float s_stage[WPB][kStage];   // windows; at the end, the tail partials
+    __shared__ float s_heads[WPB][kCombine]; // first finished row of every group
+    __shared__ int s_hrow[WPB][16];
+    extern __shared__ __align__(16) char s_hot[];  // HOT: the hot rows of X of this block's column slab
 
     const int wib = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
@@ -251,8 +268,37 @@ __global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
     // work on neighbouring rows (and, in a tiled plan, on the same column slab).
     const int blocks_per_xcd = gridDim.x / kXcds;
     const int lblock = (blockIdx.x % kXcds) * blocks_per_xcd + blockIdx.x / kXcds;
-    const int w = lblock * kWavesPerBlock + wib;
-    if (w >= num_waves) return;
+    int w = wave_begin + lblock * WPB + wib;
+    int w_stop = wave_end;
+    if constexpr (HOT) {
+        // A hot block works through the wavefront-sized pieces [hot_block_wave[b],
+        // hot_block_wave[b + 1]) of one hot segment, 16 at a time: it copies that
+        // slab's hot rows of X into LDS once; the sliced column array then holds
+        // LDS row slots instead of column ids.
+        if (lblock >= hot_blocks) return;  // whole block
+        const int w0 = hot_block_wave[lblock];
+        w_stop = hot_block_wave[lblock + 1];
+        if (w0 >= w_stop) return;  // whole block
+        w = w0 + wib;
+        const int p0 = w0 * tpw;
+        int lo = 0, hi = seg_part_off[-1] - 1;  // the number of hot segments is stored in front of the table
+        while (lo < hi) {  // largest hot segment g with seg_part_off[g] <= p0
+            int mid = (lo + hi + 1) >> 1;
+            if (seg_part_off[mid] <= p0) lo = mid; else hi = mid - 1;
+        }
+        const int *cols = hot_cols + (size_t)lo * hot_rows;
+        const int vec_per_row = (int)(((size_t)K * sizeof(T)) >> 4);
+        const int total = hot_rows * vec_per_row;
+        const float4 *xsrc = reinterpret_cast<const float4 *>(X);
+        float4 *dst = reinterpret_cast<float4 *>(s_hot);
+        for (int i = threadIdx.x; i < total; i += 64 * WPB) {
+            const int r = i / vec_per_row;
+            const int c = cols[r];
+            if (c >= 0) dst[i] = xsrc[(size_t)c * vec_per_row + (i - r * vec_per_row)];
+        }
+        __syncthreads();
+    }
+    if (w >= w_stop) return;
 
     const int L = 1 << lanes_log2;
     const int g = lane >> lanes_log2;
@@ -264,12 +310,21 @@ __global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
     const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
                                   col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
 
+    auto gather = [&](int c) -> Raw {
+        if constexpr (HOT) {
+            return *reinterpret_cast<const Raw *>(s_hot + (((unsigned)c << row_shift) | gx.col_byte));
+        } else {
+            return gx.load(c);
+        }
+    };
+
     int *s_col_wave = reinterpret_cast<int *>(&s_stage[wib][0]);
     float *s_val_wave = &s_stage[wib][16 * kWindow];
     const int *s_col = s_col_wave + g * kWindow;
     const float *s_val = s_val_wave + g * kWindow;
     float *my_head = &s_heads[wib][g * KT + s * VEC];
 
+    for (;;) {  // one pass per wavefront-sized piece: one for a cold block, many for a hot one
     const int p = w * tpw + g;
     const bool part_ok = (g < tpw) && (p < P);
     int x = 1, x_end = 1, y_begin = 0, y_end = 0;
@@ -282,8 +337,9 @@ __global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
     // Row x - 1 is in progress; it ends where nonzero index row_ptr[x] begins.
     // The row end after it is loaded ahead, so that finishing a row does not
     // wait on memory.
-    auto row_end_at = [&](int xx) { return (xx < x_end) ? row_ptr[xx] : INT_MAX; };
-    int row_end = row_end_at(x), row_end1 = row_end_at(x + 1);
+    auto row_end_at = [&](int xx) { return (!MARKS && xx < x_end) ? row_ptr[xx] : INT_MAX; };
+    [[maybe_unused]] int row_end = row_end_at(x), row_end1 = row_end_at(x + 1);
+    [[maybe_unused]] const unsigned mark_mask = (1u << mark_shift) - 1u;
 
     float acc[VEC];
 #pragma unroll
@@ -302,86 +358,131 @@ __global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
         ++x;
-        row_end = row_end1;
-        row_end1 = row_end_at(x + 1);
+        if constexpr (!MARKS) {
+            row_end = row_end1;
+            row_end1 = row_end_at(x + 1);
+        }
     };
+    // rows that end in front of nonzero idx (entry: what the column array holds for it)
+    auto finish_rows = [&](int idx, int entry) {
+        if constexpr (MARKS) {
+            for (unsigned e = (unsigned)entry >> mark_shift; e != 0; --e) emit();
+        } else {
+            while (idx == row_end) emit();
+        }
+    };
+    auto column_of = [&](int entry) { return MARKS ? (int)((unsigned)entry & mark_mask) : entry; };
 
     int wbase = y_begin;
-    Win pw;
-    pw.c = make_int4(0, 0, 0, 0);
-    pw.v = make_float4(0.f, 0.f, 0.f, 0.f);
     // sliced staging: lane l moves elements [4l, 4l + 4) of the wave's round block
     const int round_elems = tpw * kWindow;
     const bool stager = SLICED ? (4 * lane < round_elems) : (s < 4);
-    int round = 0, round_end = 0;
-    if constexpr (SLICED) {
-        round = wave_off[w];
-        round_end = wave_off[w + 1];
-        if (stager && round < round_end) pw = load_slice<T>(col_idx, val, (size_t)round * round_elems + 4 * lane);
-    } else {
-        if (stager && wbase < y_end) pw = load_win<T>(col_idx, val, nnz, wbase + 4 * s);
-    }
-    auto prefetch_next = [&]() {
-        // next window: in flight while this one is consumed
-        if constexpr (SLICED) {
-            if (stager && round + 1 < round_end)
-                pw = load_slice<T>(col_idx, val, (size_t)(round + 1) * round_elems + 4 * lane);
-        } else {
-            const int nb = wbase + kWindow;
-            if (stager && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
-        }
-    };
 
-    while (SLICED ? (round < round_end) : (__any(wbase < y_end) != 0)) {
-        const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
-        if constexpr (SLICED) {
-            if (stager) {
-                *reinterpret_cast<int4 *>(s_col_wave + 4 * lane) = pw.c;
-                *reinterpret_cast<float4 *>(s_val_wave + 4 * lane) = pw.v;
-            }
-        } else {
-            if (stager && nvalid > 0) {
-                *reinterpret_cast<int4 *>(s_col_wave + g * kWindow + 4 * s) = pw.c;
-                *reinterpret_cast<float4 *>(s_val_wave + g * kWindow + 4 * s) = pw.v;
-            }
-        }
-        wave_lds_sync();
+    // one staged window of every group: gather, finish rows, accumulate
+    auto consume = [&](int nvalid) {
         if (__all(nvalid == kWindow)) {
             // every group of the wave has a full window: no bounds to test
 #pragma unroll
             for (int b = 0; b < kWindow; b += BATCH) {
                 Raw xr[BATCH];
-#pragma unroll
-                for (int j = 0; j < BATCH; ++j) xr[j] = gx.load(s_col[b + j]);
-                if (b == 0) prefetch_next();
+                int ent[BATCH];
+                float av[BATCH];
 #pragma unroll
                 for (int j = 0; j < BATCH; ++j) {
-                    const int idx = wbase + b + j;
-                    while (idx == row_end) emit();
-                    XO::fma(acc, s_val[b + j], xr[j]);
+                    ent[j] = s_col[b + j];
+                    av[j] = s_val[b + j];
+                    xr[j] = gather(column_of(ent[j]));
+                }
+#pragma unroll
+                for (int j = 0; j < BATCH; ++j) {
+                    finish_rows(wbase + b + j, ent[j]);
+                    XO::fma(acc, av[j], xr[j]);
                 }
             }
         } else {
 #pragma unroll
             for (int b = 0; b < kWindow; b += BATCH) {
                 Raw xr[BATCH];
-#pragma unroll
-                for (int j = 0; j < BATCH; ++j)
-                    if (b + j < nvalid) xr[j] = gx.load(s_col[b + j]);
-                if (b == 0) prefetch_next();
+                int ent[BATCH];
 #pragma unroll
                 for (int j = 0; j < BATCH; ++j) {
                     if (b + j < nvalid) {
-                        const int idx = wbase + b + j;
-                        while (idx == row_end) emit();
+                        ent[j] = s_col[b + j];
+                        xr[j] = gather(column_of(ent[j]));
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < BATCH; ++j) {
+                    if (b + j < nvalid) {
+                        finish_rows(wbase + b + j, ent[j]);
                         XO::fma(acc, s_val[b + j], xr[j]);
                     }
                 }
             }
         }
-        wbase += kWindow;
-        ++round;
-        wave_lds_sync();
+    };
+
+    if constexpr (SLICED) {
+        // RPL rounds are loaded at a time, one load ahead: 2 * RPL windows of the
+        // wavefront are in flight or in registers, which is what keeps the stream
+        // coming when only a few wavefronts fit on a CU (the hot launch).
+        int round = wave_off[w];
+        const int round_end = wave_off[w + 1];
+        Win nx[RPL];
+#pragma unroll
+        for (int h = 0; h < RPL; ++h) {
+            nx[h].c = make_int4(0, 0, 0, 0);
+            nx[h].v = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        auto load_rounds = [&](int r0) {
+#pragma unroll
+            for (int h = 0; h < RPL; ++h)
+                if (stager && r0 + h < round_end)
+                    nx[h] = load_slice<T>(col_idx, val, (size_t)(r0 + h) * round_elems + 4 * lane);
+        };
+        load_rounds(round);
+        while (round < round_end) {
+            Win cu[RPL];
+#pragma unroll
+            for (int h = 0; h < RPL; ++h) cu[h] = nx[h];
+            load_rounds(round + RPL);
+#pragma nounroll
+            for (int h = 0; h < RPL && round < round_end; ++h) {
+                const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
+                if (stager) {
+                    *reinterpret_cast<int4 *>(s_col_wave + 4 * lane) = cu[0].c;
+                    *reinterpret_cast<float4 *>(s_val_wave + 4 * lane) = cu[0].v;
+                }
+                wave_lds_sync();
+                consume(nvalid);
+                wbase += kWindow;
+                ++round;
+#pragma unroll
+                for (int q = 0; q + 1 < RPL; ++q) cu[q] = cu[q + 1];
+                wave_lds_sync();
+            }
+        }
+    } else {
+        Win pw;
+        pw.c = make_int4(0, 0, 0, 0);
+        pw.v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (stager && wbase < y_end) pw = load_win<T>(col_idx, val, nnz, wbase + 4 * s);
+        while (__any(wbase < y_end) != 0) {
+            const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
+            if (stager && nvalid > 0) {
+                *reinterpret_cast<int4 *>(s_col_wave + g * kWindow + 4 * s) = pw.c;
+                *reinterpret_cast<float4 *>(s_val_wave + g * kWindow + 4 * s) = pw.v;
+            }
+            wave_lds_sync();
+            // next window: in flight while this one is consumed.  One load site for
+            // both paths of consume(): the registers of the window in flight are the
+            // same everywhere, and nothing else has to wait for it.
+            const int nb = wbase + kWindow;
+            if (stager && nb < y_end) pw = load_win<T>(col_idx, val, nnz, nb + 4 * s);
+            consume(nvalid);
+            wbase += kWindow;
+            wave_lds_sync();
+        }
     }
     while (x < x_end) emit();  // rows that end exactly where the partition ends
 
@@ -418,6 +519,14 @@ __global__ __launch_bounds__(kBlock) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
         }
         if (first && kc == 0) ws_head_row[w] = -1;
         if (kc_ok) ws_tail[(size_t)w * K + kc] = carry;
+    }
+    if constexpr (!HOT) {
+        break;
+    } else {
+        w += WPB;
+        if (w >= w_stop) break;
+        wave_lds_sync();  // the combine above has read what the next piece overwrites
+    }
     }
 }
 
@@ -597,10 +706,23 @@ inline int gather_batch()
     return b;
 }
 
-// wave_off == nullptr: CSR arrays; else the sliced arrays of a plan.
+// What a plan adds to a launch: sliced arrays, and optionally the hot launch.
+struct PlanLaunch {
+    const int *wave_off = nullptr;      // nullptr: CSR arrays
+    int hot_waves = 0;                  // waves [0, hot_waves) gather from LDS
+    int hot_rows = 0;                   // rows of X per hot table
+    const int *hot_cols = nullptr;      // [hot segments][hot_rows] column ids, -1 = unused slot
+    const int *seg_part_off = nullptr;  // first partition of every hot segment; [-1] holds their number
+    const int *hot_block_wave = nullptr;  // [hot_blocks + 1] wave range of every hot workgroup
+    int hot_blocks = 0;
+    size_t hot_lds_bytes = 0;
+    int mark_shift = 0;      // > 0: entries of the (cold) sliced column array carry row marks above this bit
+    int hot_mark_shift = 0;  // the same for the hot waves
+};
+
 template <typename T, typename TOut, int VEC>
 int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X, TOut *Y, int nnz, int K, int P,
-                const int *cx, const int *cy, const int *wave_off, const SpmmShape &sh, void *ws, unsigned phases,
+                const int *cx, const int *cy, const PlanLaunch &pl, const SpmmShape &sh, void *ws, unsigned phases,
                 hipStream_t st)
 {
     const int W = sh.num_waves;
@@ -608,29 +730,52 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
     int *ws_head_row = static_cast<int *>(ws);
     float *ws_head = reinterpret_cast<float *>(ws_head_row + rows);
     float *ws_tail = ws_head + (size_t)W * K;
+    const int *wave_off = pl.wave_off;
     if (phases & MPS_PHASE_MAIN) {
-        const int nblocks = (W + kWavesPerBlock - 1) / kWavesPerBlock;
-        dim3 grid((nblocks + kXcds - 1) / kXcds * kXcds, sh.ls.col_tiles);
-#define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED)                                                                  \
-    hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED>), grid, dim3(kBlock), 0, st, row_ptr, \
-                       col_idx, val, X, Y, cx, cy, wave_off, nnz, K, P, sh.ls.lanes_log2, sh.tpw, W,           \
-                       sh.row_shift, ws_head_row, ws_head, ws_tail)
         const int batch = gather_batch();
-        if (wave_off) {
-            if (sh.row_shift >= 0) {
-                if (batch == 8) MPS_LAUNCH_MAIN(true, 8, true);
-                else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, true);
-                else MPS_LAUNCH_MAIN(true, 4, true);
+#define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED, HOT, MARKS, WB, WE, WPB, LDS, SHIFT)                                \
+    do {                                                                                                          \
+        const int nblocks_ = (HOT) ? pl.hot_blocks : ((WE) - (WB) + (WPB)-1) / (WPB);                             \
+        dim3 grid_((nblocks_ + kXcds - 1) / kXcds * kXcds, sh.ls.col_tiles);                                      \
+        hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED, HOT, MARKS, (HOT) ? kHotRoundsPerLoad : 1>), grid_, \
+                           dim3(64 * (WPB)), LDS, st, row_ptr, col_idx, val, X, Y, cx, cy, wave_off, nnz, K, P,   \
+                           sh.ls.lanes_log2, sh.tpw, WB, WE, sh.row_shift, ws_head_row, ws_head, ws_tail,         \
+                           pl.hot_cols, pl.seg_part_off, pl.hot_rows, pl.hot_block_wave, pl.hot_blocks, SHIFT);   \
+    } while (0)
+        if (pl.hot_waves > 0) {
+            // hot launch: only built for power-of-two pitches and vector lanes (VEC > 1)
+            if constexpr (VEC > 1) {
+                if (pl.hot_mark_shift <= 0) return MPS_ERR_INVALID_ARG;
+                auto kern = mp_spmm_kernel<T, TOut, VEC, true, 4, true, true, true, kHotRoundsPerLoad>;
+                MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.hot_lds_bytes));
+                MPS_LAUNCH_MAIN(true, 4, true, true, true, 0, pl.hot_waves, kHotWavesPerBlock, pl.hot_lds_bytes,
+                                pl.hot_mark_shift);
             } else {
-                MPS_LAUNCH_MAIN(false, 4, true);
+                return MPS_ERR_UNSUPPORTED;
             }
-        } else {
-            if (sh.row_shift >= 0) {
-                if (batch == 8) MPS_LAUNCH_MAIN(true, 8, false);
-                else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, false);
-                else MPS_LAUNCH_MAIN(true, 4, false);
+        }
+        const int cold_begin = pl.hot_waves;
+        if (cold_begin < W) {
+            if (wave_off && pl.mark_shift > 0) {
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, 4, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+                else MPS_LAUNCH_MAIN(false, 4, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+            } else if (wave_off) {
+                if (sh.row_shift >= 0) {
+                    if (batch == 8) MPS_LAUNCH_MAIN(true, 8, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
+                    else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
+                    else MPS_LAUNCH_MAIN(true, 4, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
+                } else {
+                    MPS_LAUNCH_MAIN(false, 4, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
+                }
             } else {
-                MPS_LAUNCH_MAIN(false, 4, false);
+                if (sh.row_shift >= 0) {
+                    if (batch == 8) MPS_LAUNCH_MAIN(true, 8, false, false, false, 0, W, kWavesPerBlock, 0, 0);
+                    else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, false, false, false, 0, W, kWavesPerBlock, 0, 0);
+                    else MPS_LAUNCH_MAIN(true, 4, false, false, false, 0, W, kWavesPerBlock, 0, 0);
+                } else {
+                    MPS_LAUNCH_MAIN(false, 4, false, false, false, 0, W, kWavesPerBlock, 0, 0);
+                }
             }
         }
 #undef MPS_LAUNCH_MAIN
@@ -648,12 +793,12 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
 
 template <typename T, typename TOut>
 int launch_spmm_any(const int *row_ptr, const int *col_idx, const T *val, const T *X, TOut *Y, int nnz, int K,
-                    int P, const int *cx, const int *cy, const int *wave_off, const SpmmShape &sh, void *ws,
+                    int P, const int *cx, const int *cy, const PlanLaunch &pl, const SpmmShape &sh, void *ws,
                     unsigned phases, hipStream_t st)
 {
     if (sh.ls.vec == 1)
-        return launch_spmm<T, TOut, 1>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, wave_off, sh, ws, phases, st);
-    return launch_spmm<T, TOut, 16 / (int)sizeof(T)>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, wave_off, sh, ws,
+        return launch_spmm<T, TOut, 1>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, pl, sh, ws, phases, st);
+    return launch_spmm<T, TOut, 16 / (int)sizeof(T)>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, pl, sh, ws,
                                                      phases, st);
 }
 

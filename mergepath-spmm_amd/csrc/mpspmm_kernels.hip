@@ -326,7 +326,7 @@ int spmm_entry(const int *row_ptr, const int *col_idx, const T *val, const T *X,
     if (rc != MPS_OK) return rc;
     if (!ws || ws_bytes < carry_bytes_for(sh.num_waves, K)) return MPS_ERR_WORKSPACE;
     if (!aligned_to(ws, 16)) return MPS_ERR_ALIGNMENT;
-    return launch_spmm_any<T, T>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, nullptr, sh, ws, phases,
+    return launch_spmm_any<T, T>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, PlanLaunch{}, sh, ws, phases,
                                  static_cast<hipStream_t>(stream));
 }
 

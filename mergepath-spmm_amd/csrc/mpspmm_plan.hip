@@ -16,6 +16,9 @@
 //   4. the workspace of the SpMM (per-slab partial rows, carry-out records).
 #include "mpspmm_device.hpp"
 
+#include <algorithm>
+#include <vector>
+
 struct mps_plan {
     int n_rows = 0, nnz = 0, K = 0, elem_bytes = 0, cost = 0;
     int num_slabs = 1, slab_cols = 0;
@@ -32,6 +35,18 @@ struct mps_plan {
     void *workspace = nullptr;
     size_t part_bytes = 0, workspace_bytes = 0;
     size_t device_bytes = 0;
+    // hot columns (LDS-resident rows of X), tiled plans only
+    int num_segs = 1;          // virtual-row segments: num_slabs, or 2 * num_slabs with hot columns
+    int hot_rows = 0;          // rows of X per hot table (0: no hot launch)
+    int hot_waves = 0;         // wavefronts [0, hot_waves) belong to hot segments
+    long long hot_nnz = 0;     // nonzeros whose column is hot
+    int *hot_cols = nullptr;   // [num_slabs][hot_rows] column ids by slot, -1 = unused
+    int *seg_table = nullptr;  // [0] = num_slabs, [1 + g] = first partition of hot segment g (g <= num_slabs)
+    size_t hot_lds_bytes = 0;
+    int hot_cost = 0;               // merge items per partition in the hot segments
+    int mark_shift = 0, hot_mark_shift = 0;  // row marks sit above this bit of a column entry (0: none)
+    int *hot_block_wave = nullptr;  // [hot_blocks + 1] first wave of every hot workgroup
+    int hot_blocks = 0;
 };
 
 namespace {
@@ -152,11 +167,19 @@ __global__ __launch_bounds__(256) void slice_count_kernel(const int *__restrict_
     rounds[w] = r;
 }
 
-// One thread per (virtual-order) nonzero: its slot in the sliced arrays.
+// One thread per (virtual-order) nonzero: its slot in the sliced arrays.  With
+// row marks (shift > 0: mark_shift for partitions from hot_parts on,
+// hot_mark_shift before) the column entry also carries, above bit shift, the
+// number of rows that end in front of this nonzero inside its partition: its
+// virtual row minus that of the nonzero before it, or minus the row the
+// partition starts in (coord_x - 1) for the partition's first nonzero.
 __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restrict__ col_v,
                                                              const int *__restrict__ perm,
+                                                             const int *__restrict__ vrow_ptr, int n_vrows,
+                                                             const int *__restrict__ coord_x,
                                                              const int *__restrict__ coord_y, int P, int tpw,
                                                              const int *__restrict__ wave_off, int nnz,
+                                                             int hot_parts, int hot_mark_shift, int mark_shift,
                                                              int *__restrict__ slice_cols,
                                                              int *__restrict__ slice_src)
 {
@@ -173,7 +196,24 @@ __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restric
     const int k = y - coord_y[p];
     const size_t slot = ((size_t)wave_off[w] + (size_t)(k / kWindow)) * (size_t)(tpw * kWindow) + (size_t)g * kWindow +
                         (size_t)(k % kWindow);
-    slice_cols[slot] = col_v[y];
+    unsigned entry = (unsigned)col_v[y];
+    const int shift = p < hot_parts ? hot_mark_shift : mark_shift;
+    if (shift > 0) {
+        auto row_of = [&](int yy) {  // largest v with vrow_ptr[v] <= yy
+            int a = 0, b = n_vrows - 1;
+            while (a < b) {
+                int mid = (a + b + 1) >> 1;
+                if (vrow_ptr[mid] <= yy) a = mid; else b = mid - 1;
+            }
+            return a;
+        };
+        const int row = row_of(y);
+        int before;
+        if (k == 0) before = max(coord_x[p], 1) - 1;
+        else before = vrow_ptr[row] < y ? row : row_of(y - 1);
+        entry |= (unsigned)(row - before) << shift;
+    }
+    slice_cols[slot] = (int)entry;
     slice_src[slot] = perm ? perm[y] : y;
 }
 
@@ -186,6 +226,123 @@ __global__ __launch_bounds__(256) void slice_values_kernel(const T *__restrict__
     if (i >= slots) return;
     const int src = slice_src[i];
     slice_vals[i] = src >= 0 ? val[src] : (T)0;
+}
+
+
+// ---------------------------------------------------------------------------
+// Hot columns.  Inside every column slab the hot_rows columns with the most
+// nonzeros get their rows of X copied into LDS by the workgroups that process
+// them ("hot" segments, gathered from LDS); the other columns of the slab form
+// the "cold" segment, gathered through L2 as before.  Segment order: the hot
+// segments of all slabs, then the cold segments; virtual row v = seg * n_rows + r.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void col_histogram_kernel(const int *__restrict__ col_idx, int nnz,
+                                                             int *__restrict__ deg)
+{
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e < nnz) atomicAdd(deg + col_idx[e], 1);
+}
+
+// One thread per (slab, row): where the row's nonzeros of that slab start, and
+// how many of them lie in hot columns.
+__global__ __launch_bounds__(256) void hot_count_kernel(const int *__restrict__ row_ptr,
+                                                         const int *__restrict__ col_idx, int n_rows,
+                                                         int num_slabs, int slab_cols,
+                                                         const int *__restrict__ hot_slot, int *__restrict__ first,
+                                                         int *__restrict__ counts)
+{
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long nv = (long long)num_slabs * n_rows;
+    if (t == nv) counts[2 * nv] = 0;
+    if (t >= nv) return;
+    const int s = (int)(t / n_rows);
+    const int r = (int)(t - (long long)s * n_rows);
+    const int b = row_ptr[r], e = row_ptr[r + 1];
+    auto lower = [&](long long key) {
+        int lo = b, hi = e;
+        while (lo < hi) {
+            int mid = lo + ((hi - lo) >> 1);
+            if (col_idx[mid] < key) lo = mid + 1; else hi = mid;
+        }
+        return lo;
+    };
+    const int f0 = lower((long long)s * slab_cols);
+    const int f1 = (s + 1 == num_slabs) ? e : lower((long long)(s + 1) * slab_cols);
+    int hot = 0;
+    for (int i = f0; i < f1; ++i) hot += hot_slot[col_idx[i]] >= 0;
+    first[t] = f0;
+    counts[t] = hot;                  // hot segment s
+    counts[nv + t] = (f1 - f0) - hot; // cold segment num_slabs + s
+}
+
+// One thread per (slab, row): its nonzeros go, in order, to the hot or the cold
+// virtual row; hot ones carry their LDS slot instead of the column id.
+__global__ __launch_bounds__(256) void hot_scatter_kernel(const int *__restrict__ col_idx, int n_rows, int num_slabs,
+                                                           const int *__restrict__ hot_slot,
+                                                           const int *__restrict__ first,
+                                                           const int *__restrict__ vrow_ptr,
+                                                           int *__restrict__ col_out, int *__restrict__ perm)
+{
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long nv = (long long)num_slabs * n_rows;
+    if (t >= nv) return;
+    int dh = vrow_ptr[t], dc = vrow_ptr[nv + t];
+    const int len = (vrow_ptr[t + 1] - dh) + (vrow_ptr[nv + t + 1] - dc);
+    const int f0 = first[t];
+    for (int i = f0; i < f0 + len; ++i) {
+        const int c = col_idx[i];
+        const int slot = hot_slot[c];
+        if (slot >= 0) {
+            col_out[dh] = slot;
+            perm[dh++] = i;
+        } else {
+            col_out[dc] = c;
+            perm[dc++] = i;
+        }
+    }
+}
+
+// Merge-path partition of every segment on its own (a partition never spans
+// two segments, so a wavefront gathers either from LDS or from L2).  Thread i
+// computes boundary i; seg_off[g] is the first partition of segment g,
+// seg_parts[g] the number of its partitions that carry work (the rest, up to
+// seg_off[g + 1], are empty padding), seg_ipt[g] its items per partition.
+// The search is MergePathSearch (src/MergePathSpMM.cu:280-297) on the rows of
+// the segment; x is returned as a global virtual-row coordinate.
+__global__ __launch_bounds__(256) void seg_partition_kernel(const int *__restrict__ vrow_ptr, int n_rows,
+                                                             int num_segs, const int *__restrict__ seg_off,
+                                                             const int *__restrict__ seg_parts,
+                                                             const int *__restrict__ seg_ipt, int P_total,
+                                                             int *__restrict__ coord_x, int *__restrict__ coord_y)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > P_total) return;
+    int lo = 0, hi = num_segs - 1;  // largest g with seg_off[g] <= i
+    while (lo < hi) {
+        int mid = (lo + hi + 1) >> 1;
+        if (seg_off[mid] <= i) lo = mid; else hi = mid - 1;
+    }
+    const int g = lo;
+    const int li = i - seg_off[g];
+    const long long base = (long long)g * n_rows;
+    const int y0 = vrow_ptr[base];
+    const int nnz_g = vrow_ptr[base + n_rows] - y0;
+    const int num_rows = n_rows + 1;
+    const int total = num_rows + nnz_g;
+    long long d64 = (long long)seg_ipt[g] * li;
+    int diagonal = (li <= seg_parts[g] && d64 < (long long)total) ? (int)d64 : total;
+    int x_min = max(diagonal - nnz_g, 0);
+    int x_max = min(diagonal, num_rows);
+    while (x_min < x_max) {
+        int pivot = (x_min + x_max) >> 1;
+        if (vrow_ptr[base + pivot] - y0 <= diagonal - pivot - 1)
+            x_min = pivot + 1;
+        else
+            x_max = pivot;
+    }
+    const int x_l = min(x_min, num_rows);
+    coord_x[i] = (int)base + max(x_l, 1);  // row base + x_l - 1 is in progress; a segment starts with its row 0
+    coord_y[i] = y0 + (diagonal - x_min);
 }
 
 template <typename T>
@@ -208,6 +365,9 @@ void plan_free(mps_plan *pl)
     (void)hipFree(pl->slice_vals);
     (void)hipFree(pl->slice_src);
     (void)hipFree(pl->workspace);
+    (void)hipFree(pl->hot_cols);
+    (void)hipFree(pl->seg_table);
+    (void)hipFree(pl->hot_block_wave);
     delete pl;
 }
 
@@ -235,12 +395,92 @@ int plan_set_values(mps_plan *pl, const void *d_val, hipStream_t st)
     return MPS_OK;
 }
 
+// Static LDS of a hot workgroup (see mp_spmm_kernel) and the rows of X that
+// fit beside it in the 160 KiB of a CU.
+constexpr int kHotCost = 256;  // merge items per partition of a hot segment (at least the plan's cost)
+
+size_t hot_static_lds(int vec)
+{
+    const size_t comb = 64 * (size_t)vec;
+    const size_t stage = comb > 2 * 16 * kWindow ? comb : 2 * 16 * kWindow;
+    return kHotWavesPerBlock * (stage + comb) * sizeof(float) + kHotWavesPerBlock * 16 * sizeof(int);
+}
+
+int choose_hot_rows(int K, int eb, const SpmmShape &sh)
+{
+    if (sh.row_shift < 0 || sh.ls.vec == 1 || sh.ls.col_tiles != 1) return 0;
+    const size_t budget = 160 * 1024 - hot_static_lds(sh.ls.vec) - 2048;
+    size_t rows = budget / ((size_t)K * eb);
+    rows = rows / 64 * 64;
+    return rows >= 256 ? (int)rows : 0;
+}
+
+struct BuildTmp {
+    int *first = nullptr, *col_v = nullptr, *perm = nullptr, *sums = nullptr, *deg = nullptr, *hot_slot = nullptr,
+        *seg = nullptr;
+    void drop()
+    {
+        (void)hipFree(first);
+        (void)hipFree(col_v);
+        (void)hipFree(perm);
+        (void)hipFree(sums);
+        (void)hipFree(deg);
+        (void)hipFree(hot_slot);
+        (void)hipFree(seg);
+        first = col_v = perm = sums = deg = hot_slot = seg = nullptr;
+    }
+};
+
+template <typename T>
+int tmp_alloc(T **p, size_t count)
+{
+    MPS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(p), (count ? count : 1) * sizeof(T)));
+    return MPS_OK;
+}
+
+// Picks the hot columns of every slab (host side, from the column histogram):
+// the hot_rows columns with the most nonzeros, ties to the smaller column id;
+// slots are handed out in ascending column order.  Returns the number of
+// nonzeros that fall into hot columns.
+long long select_hot_columns(const std::vector<int> &deg, int n, int num_slabs, int slab_cols, int hot_rows,
+                             std::vector<int> &hot_slot, std::vector<int> &hot_cols)
+{
+    hot_slot.assign((size_t)n, -1);
+    hot_cols.assign((size_t)num_slabs * hot_rows, -1);
+    long long hot_nnz = 0;
+    std::vector<int> order;
+    for (int s = 0; s < num_slabs; ++s) {
+        const int c0 = (int)std::min<long long>((long long)s * slab_cols, n);
+        const int c1 = (int)std::min<long long>((long long)(s + 1) * slab_cols, n);
+        order.resize((size_t)(c1 - c0));
+        for (int c = c0; c < c1; ++c) order[(size_t)(c - c0)] = c;
+        const size_t take = std::min<size_t>((size_t)hot_rows, order.size());
+        auto hotter = [&](int a, int b) { return deg[a] != deg[b] ? deg[a] > deg[b] : a < b; };
+        if (take < order.size()) std::nth_element(order.begin(), order.begin() + (long)take, order.end(), hotter);
+        std::sort(order.begin(), order.begin() + (long)take);
+        int slot = 0;
+        for (size_t k = 0; k < take; ++k) {
+            const int c = order[k];
+            if (deg[c] == 0) continue;  // a column nobody references needs no slot
+            hot_slot[(size_t)c] = slot;
+            hot_cols[(size_t)s * hot_rows + slot] = c;
+            hot_nnz += deg[c];
+            ++slot;
+        }
+    }
+    return hot_nnz;
+}
+
 // Builds everything; temporaries are released before returning.
 int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const void *d_val, unsigned flags,
                size_t slab_bytes, int tpw, hipStream_t st)
 {
     const int n = pl->n_rows, nnz = pl->nnz, K = pl->K, eb = pl->elem_bytes;
     int rc;
+    // lane shape and partitions per wavefront do not depend on the partition count
+    if ((rc = make_spmm_shape(n, K, 1, tpw, eb, pl->shape)) != MPS_OK) return rc;
+    const int G = pl->shape.tpw;
+
     // 1. slabs
     pl->num_slabs = 1;
     pl->slab_cols = n > 0 ? n : 1;
@@ -259,115 +499,268 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             if (rc != MPS_OK) return rc;
         }
     }
-    int *first = nullptr, *col_v = nullptr, *perm = nullptr, *sums = nullptr;
-    mps_plan tmp;  // byte accounting of temporaries is not kept
-    auto drop_tmp = [&] {
-        (void)hipFree(first);
-        (void)hipFree(col_v);
-        (void)hipFree(perm);
-        (void)hipFree(sums);
-        first = col_v = perm = sums = nullptr;
-    };
-    rc = dev_alloc(&tmp, &sums, (size_t)kScanMaxBlocks + 1);
-    if (rc != MPS_OK) return rc;
+    BuildTmp t;
+    if ((rc = tmp_alloc(&t.sums, (size_t)kScanMaxBlocks + 1)) != MPS_OK) return rc;
+#define MPS_BUILD_TRY(expr)                       \
+    do {                                          \
+        int rc_ = (expr);                         \
+        if (rc_ != MPS_OK) {                      \
+            t.drop();                             \
+            return rc_;                           \
+        }                                         \
+    } while (0)
+#define MPS_BUILD_HIP(expr)                                     \
+    do {                                                        \
+        hipError_t e_ = (expr);                                 \
+        if (e_ != hipSuccess) {                                 \
+            t.drop();                                           \
+            return MPS_ERR_HIP + (int)e_;                       \
+        }                                                       \
+    } while (0)
 
+    // 2. hot columns of every slab (tiled plans, shapes the hot kernel supports)
+    int hot_rows = 0;
+    std::vector<int> h_hot_cols;
+    if (pl->num_slabs > 1 && !(flags & MPS_PLAN_NO_HOT)) {
+        hot_rows = choose_hot_rows(K, eb, pl->shape);
+        if (2LL * pl->num_slabs * n + 1 + nnz > INT_MAX) hot_rows = 0;
+        if (hot_rows > 0) {
+            std::vector<int> h_deg((size_t)n), h_slot;
+            MPS_BUILD_TRY(tmp_alloc(&t.deg, (size_t)n));
+            MPS_BUILD_HIP(hipMemsetAsync(t.deg, 0, (size_t)n * sizeof(int), st));
+            hipLaunchKernelGGL(col_histogram_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st,
+                               d_col_idx, nnz, t.deg);
+            MPS_BUILD_HIP(hipGetLastError());
+            MPS_BUILD_HIP(hipMemcpyAsync(h_deg.data(), t.deg, (size_t)n * sizeof(int), hipMemcpyDeviceToHost, st));
+            MPS_BUILD_HIP(hipStreamSynchronize(st));
+            pl->hot_nnz = select_hot_columns(h_deg, n, pl->num_slabs, pl->slab_cols, hot_rows, h_slot, h_hot_cols);
+            // worth a second launch and twice the partial rows only if it takes a real share of the gathers
+            if ((double)pl->hot_nnz < 0.15 * (double)nnz && !(flags & MPS_PLAN_FORCE_HOT)) {
+                hot_rows = 0;
+                pl->hot_nnz = 0;
+            } else {
+                MPS_BUILD_TRY(tmp_alloc(&t.hot_slot, (size_t)n));
+                MPS_BUILD_HIP(hipMemcpyAsync(t.hot_slot, h_slot.data(), (size_t)n * sizeof(int), hipMemcpyHostToDevice, st));
+                MPS_BUILD_HIP(hipStreamSynchronize(st));
+            }
+        }
+    }
+
+    // 3. slab-major (and hot-first) order of the nonzeros
     for (int attempt = 0; attempt < 2; ++attempt) {
-        const long long nv = (long long)pl->num_slabs * n;
+        pl->num_segs = pl->num_slabs * (hot_rows > 0 ? 2 : 1);
+        const long long nslab_rows = (long long)pl->num_slabs * n;
+        const long long nv = (long long)pl->num_segs * n;
         pl->n_vrows = (int)nv;
-        rc = dev_alloc(pl, &pl->vrow_ptr, (size_t)nv + 1);
-        if (rc != MPS_OK) { drop_tmp(); return rc; }
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->vrow_ptr, (size_t)nv + 1));
         if (pl->num_slabs == 1) {
-            MPS_HIP_TRY(hipMemcpyAsync(pl->vrow_ptr, d_row_ptr, ((size_t)n + 1) * sizeof(int),
-                                       hipMemcpyDeviceToDevice, st));
+            MPS_BUILD_HIP(hipMemcpyAsync(pl->vrow_ptr, d_row_ptr, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToDevice, st));
             break;
         }
-        // 2. slab-major order
-        if ((rc = dev_alloc(&tmp, &first, (size_t)nv)) != MPS_OK || (rc = dev_alloc(&tmp, &col_v, (size_t)nnz)) != MPS_OK ||
-            (rc = dev_alloc(&tmp, &perm, (size_t)nnz)) != MPS_OK) {
-            drop_tmp();
-            return rc;
-        }
-        int *bad = sums + kScanMaxBlocks;
+        MPS_BUILD_TRY(tmp_alloc(&t.first, (size_t)nslab_rows));
+        MPS_BUILD_TRY(tmp_alloc(&t.col_v, (size_t)nnz));
+        MPS_BUILD_TRY(tmp_alloc(&t.perm, (size_t)nnz));
+        int *bad = t.sums + kScanMaxBlocks;
         int zero = 0, h_bad = 0;
-        MPS_HIP_TRY(hipMemcpyAsync(bad, &zero, sizeof(int), hipMemcpyHostToDevice, st));
+        MPS_BUILD_HIP(hipMemcpyAsync(bad, &zero, sizeof(int), hipMemcpyHostToDevice, st));
         if (nnz > 1)
             hipLaunchKernelGGL(tile_sorted_check_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st,
                                d_row_ptr, d_col_idx, n, nnz, bad);
-        hipLaunchKernelGGL(tile_count_kernel, dim3((unsigned)((nv + 1 + 255) / 256)), dim3(256), 0, st, d_row_ptr,
-                           d_col_idx, n, pl->num_slabs, pl->slab_cols, first, pl->vrow_ptr);
-        MPS_HIP_TRY(hipGetLastError());
-        if ((rc = scan_exclusive_inplace(pl->vrow_ptr, (int)nv + 1, sums, st)) != MPS_OK) { drop_tmp(); return rc; }
-        hipLaunchKernelGGL(tile_scatter_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st, d_row_ptr,
-                           d_col_idx, n, nnz, pl->num_slabs, pl->slab_cols, first, pl->vrow_ptr, col_v, perm);
-        MPS_HIP_TRY(hipGetLastError());
-        MPS_HIP_TRY(hipMemcpyAsync(&h_bad, bad, sizeof(int), hipMemcpyDeviceToHost, st));
-        MPS_HIP_TRY(hipStreamSynchronize(st));
-        if (!h_bad) break;
-        // rows are not sorted: tiling is impossible
-        if (flags & MPS_PLAN_FORCE_TILING) { drop_tmp(); return MPS_ERR_UNSORTED; }
-        (void)hipFree(first); (void)hipFree(col_v); (void)hipFree(perm);
-        first = col_v = perm = nullptr;
-        (void)hipFree(pl->vrow_ptr);
-        pl->vrow_ptr = nullptr;
-        pl->num_slabs = 1;
-        pl->slab_cols = n;
+        MPS_BUILD_HIP(hipMemcpyAsync(&h_bad, bad, sizeof(int), hipMemcpyDeviceToHost, st));
+        MPS_BUILD_HIP(hipStreamSynchronize(st));
+        if (h_bad) {
+            // rows are not sorted: tiling is impossible
+            if (flags & MPS_PLAN_FORCE_TILING) {
+                t.drop();
+                return MPS_ERR_UNSORTED;
+            }
+            (void)hipFree(t.first); (void)hipFree(t.col_v); (void)hipFree(t.perm);
+            t.first = t.col_v = t.perm = nullptr;
+            (void)hipFree(pl->vrow_ptr);
+            pl->vrow_ptr = nullptr;
+            pl->num_slabs = 1;
+            pl->slab_cols = n;
+            hot_rows = 0;
+            pl->hot_nnz = 0;
+            continue;
+        }
+        const unsigned row_blocks = (unsigned)((nslab_rows + 1 + 255) / 256);
+        if (hot_rows > 0) {
+            hipLaunchKernelGGL(hot_count_kernel, dim3(row_blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n, pl->num_slabs,
+                               pl->slab_cols, t.hot_slot, t.first, pl->vrow_ptr);
+            MPS_BUILD_HIP(hipGetLastError());
+            MPS_BUILD_TRY(scan_exclusive_inplace(pl->vrow_ptr, (int)nv + 1, t.sums, st));
+            hipLaunchKernelGGL(hot_scatter_kernel, dim3(row_blocks), dim3(256), 0, st, d_col_idx, n, pl->num_slabs,
+                               t.hot_slot, t.first, pl->vrow_ptr, t.col_v, t.perm);
+        } else {
+            hipLaunchKernelGGL(tile_count_kernel, dim3(row_blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n, pl->num_slabs,
+                               pl->slab_cols, t.first, pl->vrow_ptr);
+            MPS_BUILD_HIP(hipGetLastError());
+            MPS_BUILD_TRY(scan_exclusive_inplace(pl->vrow_ptr, (int)nv + 1, t.sums, st));
+            hipLaunchKernelGGL(tile_scatter_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st,
+                               d_row_ptr, d_col_idx, n, nnz, pl->num_slabs, pl->slab_cols, t.first, pl->vrow_ptr, t.col_v,
+                               t.perm);
+        }
+        MPS_BUILD_HIP(hipGetLastError());
+        break;
     }
-    const int *cols_v = pl->num_slabs == 1 ? d_col_idx : col_v;
+    const int *cols_v = pl->num_slabs == 1 ? d_col_idx : t.col_v;
+    pl->hot_rows = hot_rows;
 
-    // 3. merge-path partition of the virtual rows
-    if ((rc = mps_num_partitions(pl->n_vrows, nnz, pl->cost, &pl->P)) != MPS_OK) { drop_tmp(); return rc; }
-    if ((rc = make_spmm_shape(n, K, pl->P, tpw, eb, pl->shape)) != MPS_OK) { drop_tmp(); return rc; }
-    if ((rc = dev_alloc(pl, &pl->coord_x, (size_t)pl->P + 1)) != MPS_OK ||
-        (rc = dev_alloc(pl, &pl->coord_y, (size_t)pl->P + 1)) != MPS_OK) { drop_tmp(); return rc; }
-    if ((rc = mps_partition(pl->vrow_ptr, pl->n_vrows, nnz, pl->P, pl->coord_x, pl->coord_y, st)) != MPS_OK) {
-        drop_tmp();
-        return rc;
+    // 4. merge-path partition of the virtual rows
+    int max_cold_ipt = 0, max_hot_ipt = 0;
+    if (hot_rows == 0) {
+        // one split of all virtual rows: the reference's (src/MergePathSpMM.cu:138-139, :327-334)
+        MPS_BUILD_TRY(mps_num_partitions(pl->n_vrows, nnz, pl->cost, &pl->P));
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->coord_x, (size_t)pl->P + 1));
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->coord_y, (size_t)pl->P + 1));
+        MPS_BUILD_TRY(mps_partition(pl->vrow_ptr, pl->n_vrows, nnz, pl->P, pl->coord_x, pl->coord_y, st));
+        pl->hot_waves = 0;
+        MPS_BUILD_TRY(mps_items_per_partition(pl->n_vrows, nnz, pl->P, &max_cold_ipt));
+    } else {
+        // every segment is split on its own and padded to whole wavefronts
+        const int S2 = pl->num_segs, S = pl->num_slabs;
+        {
+            const char *e = std::getenv("MPS_HOT_COST");
+            const int v = e ? std::atoi(e) : 0;
+            pl->hot_cost = v > 0 ? v : (pl->cost > kHotCost ? pl->cost : kHotCost);
+        }
+        std::vector<int> seg_y((size_t)S2 + 1);
+        for (int g = 0; g <= S2; ++g)
+            MPS_BUILD_HIP(hipMemcpyAsync(&seg_y[(size_t)g], pl->vrow_ptr + (size_t)g * n, sizeof(int), hipMemcpyDeviceToHost, st));
+        MPS_BUILD_HIP(hipStreamSynchronize(st));
+        std::vector<int> h_seg((size_t)3 * S2 + 1);  // seg_off[S2 + 1], seg_parts[S2], seg_ipt[S2]
+        int *seg_off = h_seg.data(), *seg_parts = seg_off + S2 + 1, *seg_ipt = seg_parts + S2;
+        long long off = 0;
+        for (int g = 0; g < S2; ++g) {
+            const long long total = (long long)n + 1 + (seg_y[(size_t)g + 1] - seg_y[(size_t)g]);
+            // hot segments take long partitions: nothing to gain from small ones where
+            // every gather costs the same, and a long one hides the start-up loads
+            long long parts = (total - 1) / (g < S ? pl->hot_cost : pl->cost);
+            if (parts < 1) parts = 1;
+            const long long mult = G;  // whole wavefronts
+            seg_off[g] = (int)off;
+            seg_parts[g] = (int)parts;
+            seg_ipt[g] = (int)((total + parts - 1) / parts);
+            int &worst = g < S ? max_hot_ipt : max_cold_ipt;
+            if (seg_ipt[g] > worst) worst = seg_ipt[g];
+            off += (parts + mult - 1) / mult * mult;
+            if (off > INT_MAX / 2) {
+                t.drop();
+                return MPS_ERR_UNSUPPORTED;
+            }
+        }
+        seg_off[S2] = (int)off;
+        pl->P = (int)off;
+        pl->hot_waves = seg_off[S] / G;
+        MPS_BUILD_TRY(tmp_alloc(&t.seg, h_seg.size()));
+        MPS_BUILD_HIP(hipMemcpyAsync(t.seg, h_seg.data(), h_seg.size() * sizeof(int), hipMemcpyHostToDevice, st));
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->coord_x, (size_t)pl->P + 1));
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->coord_y, (size_t)pl->P + 1));
+        hipLaunchKernelGGL(seg_partition_kernel, dim3((unsigned)(((long long)pl->P + 1 + 255) / 256)), dim3(256), 0, st,
+                           pl->vrow_ptr, n, S2, t.seg, t.seg + S2 + 1, t.seg + 2 * S2 + 1, pl->P, pl->coord_x, pl->coord_y);
+        MPS_BUILD_HIP(hipGetLastError());
+        // what the hot kernel needs: slot -> column lists, and where the hot segments start
+        std::vector<int> h_table((size_t)S + 2);
+        h_table[0] = S;
+        for (int g = 0; g <= S; ++g) h_table[(size_t)g + 1] = seg_off[g];
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->seg_table, h_table.size()));
+        MPS_BUILD_HIP(hipMemcpyAsync(pl->seg_table, h_table.data(), h_table.size() * sizeof(int), hipMemcpyHostToDevice, st));
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->hot_cols, h_hot_cols.size()));
+        MPS_BUILD_HIP(hipMemcpyAsync(pl->hot_cols, h_hot_cols.data(), h_hot_cols.size() * sizeof(int), hipMemcpyHostToDevice, st));
+        MPS_BUILD_HIP(hipStreamSynchronize(st));
+        pl->hot_lds_bytes = (size_t)hot_rows * K * eb;
+        // Hot workgroups: one LDS table per CU at a time, so a few long-lived
+        // workgroups per CU, each with a contiguous share of one segment's waves.
+        int dev = 0, cus = 256;
+        MPS_BUILD_HIP(hipGetDevice(&dev));
+        MPS_BUILD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        const char *e = std::getenv("MPS_HOT_BLOCKS_PER_CU");
+        int per_cu = e ? std::atoi(e) : 1;
+        if (per_cu < 1 || per_cu > 64) per_cu = 1;
+        const long long target = (long long)cus * per_cu;
+        std::vector<int> h_blocks;
+        for (int g = 0; g < S; ++g) {
+            const int w0 = seg_off[g] / G, w1 = seg_off[g + 1] / G;
+            const long long wg = w1 - w0;
+            long long blocks = (target * wg + pl->hot_waves / 2) / (pl->hot_waves > 0 ? pl->hot_waves : 1);
+            const long long most = (wg + kHotWavesPerBlock - 1) / kHotWavesPerBlock;
+            if (blocks > most) blocks = most;
+            if (blocks < 1) blocks = 1;
+            // equal shares, whatever the remainder: the 16 wavefronts of a workgroup
+            // take the pieces of its share in turn
+            for (long long b = 0; b < blocks; ++b) h_blocks.push_back((int)(w0 + wg * b / blocks));
+        }
+        h_blocks.push_back(pl->hot_waves);
+        pl->hot_blocks = (int)h_blocks.size() - 1;
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->hot_block_wave, h_blocks.size()));
+        MPS_BUILD_HIP(hipMemcpyAsync(pl->hot_block_wave, h_blocks.data(), h_blocks.size() * sizeof(int), hipMemcpyHostToDevice, st));
+        MPS_BUILD_HIP(hipStreamSynchronize(st));
+    }
+    pl->shape.num_waves = (pl->P + G - 1) / G;
+    // Row marks: a partition holds at most items-per-partition row ends, so that
+    // many values must fit above the column (or LDS slot) bits of an entry.
+    auto bits_for = [](long long v) { int b = 1; while ((v >> b) != 0) ++b; return b; };  // values 0..v
+    {
+        const char *e = std::getenv("MPS_ROW_MARKS");
+        const bool want = !(e && std::atoi(e) == 0);
+        const int col_bits = bits_for(n > 1 ? n - 1 : 1);
+        pl->mark_shift = (want && nnz > 0 && col_bits + bits_for(max_cold_ipt) <= 32) ? col_bits : 0;
+        if (hot_rows > 0) {
+            const int slot_bits = bits_for(hot_rows - 1);
+            if (slot_bits + bits_for(max_hot_ipt) > 32) {
+                t.drop();
+                return MPS_ERR_UNSUPPORTED;
+            }
+            pl->hot_mark_shift = slot_bits;
+        }
     }
 
-    // 4. slices
-    const int W = pl->shape.num_waves, G = pl->shape.tpw;
-    if ((rc = dev_alloc(pl, &pl->wave_off, (size_t)W + 1)) != MPS_OK) { drop_tmp(); return rc; }
+    // 5. slices
+    const int W = pl->shape.num_waves;
+    MPS_BUILD_TRY(dev_alloc(pl, &pl->wave_off, (size_t)W + 1));
     hipLaunchKernelGGL(slice_count_kernel, dim3((unsigned)((W + 1 + 255) / 256)), dim3(256), 0, st, pl->coord_y, pl->P, G, W,
                        pl->wave_off);
-    MPS_HIP_TRY(hipGetLastError());
-    if ((rc = scan_exclusive_inplace(pl->wave_off, W + 1, sums, st)) != MPS_OK) { drop_tmp(); return rc; }
+    MPS_BUILD_HIP(hipGetLastError());
+    MPS_BUILD_TRY(scan_exclusive_inplace(pl->wave_off, W + 1, t.sums, st));
     int total_rounds = 0;
-    MPS_HIP_TRY(hipMemcpyAsync(&total_rounds, pl->wave_off + W, sizeof(int), hipMemcpyDeviceToHost, st));
-    MPS_HIP_TRY(hipStreamSynchronize(st));
+    MPS_BUILD_HIP(hipMemcpyAsync(&total_rounds, pl->wave_off + W, sizeof(int), hipMemcpyDeviceToHost, st));
+    MPS_BUILD_HIP(hipStreamSynchronize(st));
     pl->total_rounds = total_rounds;
     const size_t slots = (size_t)total_rounds * (size_t)(G * kWindow);
-    if ((rc = dev_alloc(pl, &pl->slice_cols, slots)) != MPS_OK || (rc = dev_alloc(pl, &pl->slice_src, slots)) != MPS_OK) {
-        drop_tmp();
-        return rc;
-    }
+    MPS_BUILD_TRY(dev_alloc(pl, &pl->slice_cols, slots));
+    MPS_BUILD_TRY(dev_alloc(pl, &pl->slice_src, slots));
     {
         unsigned char *sv = nullptr;
-        if ((rc = dev_alloc(pl, &sv, (slots ? slots : 1) * (size_t)eb)) != MPS_OK) { drop_tmp(); return rc; }
+        MPS_BUILD_TRY(dev_alloc(pl, &sv, (slots ? slots : 1) * (size_t)eb));
         pl->slice_vals = sv;
     }
     if (slots) {
-        MPS_HIP_TRY(hipMemsetAsync(pl->slice_cols, 0, slots * sizeof(int), st));
-        MPS_HIP_TRY(hipMemsetAsync(pl->slice_src, 0xff, slots * sizeof(int), st));
+        MPS_BUILD_HIP(hipMemsetAsync(pl->slice_cols, 0, slots * sizeof(int), st));
+        MPS_BUILD_HIP(hipMemsetAsync(pl->slice_src, 0xff, slots * sizeof(int), st));
     }
     if (nnz > 0) {
         hipLaunchKernelGGL(slice_scatter_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st, cols_v,
-                           pl->num_slabs == 1 ? nullptr : perm, pl->coord_y, pl->P, G, pl->wave_off, nnz, pl->slice_cols,
-                           pl->slice_src);
-        MPS_HIP_TRY(hipGetLastError());
+                           pl->num_slabs == 1 ? nullptr : t.perm, pl->vrow_ptr, pl->n_vrows, pl->coord_x, pl->coord_y,
+                           pl->P, G, pl->wave_off, nnz, pl->hot_waves * G, pl->hot_mark_shift, pl->mark_shift,
+                           pl->slice_cols, pl->slice_src);
+        MPS_BUILD_HIP(hipGetLastError());
     }
-    if ((rc = plan_set_values(pl, d_val, st)) != MPS_OK) { drop_tmp(); return rc; }
+    MPS_BUILD_TRY(plan_set_values(pl, d_val, st));
 
-    // 5. workspace
-    pl->part_bytes = part_bytes_for(n, pl->num_slabs, K);
+    // 6. workspace
+    pl->part_bytes = part_bytes_for(n, pl->num_segs, K);
     pl->workspace_bytes = pl->part_bytes + carry_bytes_for(W, K);
     {
         unsigned char *ws = nullptr;
-        if ((rc = dev_alloc(pl, &ws, pl->workspace_bytes)) != MPS_OK) { drop_tmp(); return rc; }
+        MPS_BUILD_TRY(dev_alloc(pl, &ws, pl->workspace_bytes));
         pl->workspace = ws;
     }
-    MPS_HIP_TRY(hipStreamSynchronize(st));
-    drop_tmp();
+    MPS_BUILD_HIP(hipStreamSynchronize(st));
+    t.drop();
     return MPS_OK;
+#undef MPS_BUILD_TRY
+#undef MPS_BUILD_HIP
 }
 
 template <typename T>
@@ -379,21 +772,32 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     if (!aligned_to(X, 16) || !aligned_to(Y, 16)) return MPS_ERR_ALIGNMENT;
     const T *vals = static_cast<const T *>(pl->slice_vals);
     void *carry = static_cast<char *>(pl->workspace) + pl->part_bytes;
-    if (pl->num_slabs == 1)
+    PlanLaunch how;
+    how.wave_off = pl->wave_off;
+    how.hot_waves = pl->hot_waves;
+    how.hot_rows = pl->hot_rows;
+    how.hot_cols = pl->hot_cols;
+    how.seg_part_off = pl->seg_table ? pl->seg_table + 1 : nullptr;
+    how.hot_lds_bytes = pl->hot_lds_bytes;
+    how.hot_block_wave = pl->hot_block_wave;
+    how.hot_blocks = pl->hot_blocks;
+    how.mark_shift = pl->mark_shift;
+    how.hot_mark_shift = pl->hot_mark_shift;
+    if (pl->num_segs == 1)
         return launch_spmm_any<T, T>(pl->vrow_ptr, pl->slice_cols, vals, X, Y, pl->nnz, pl->K, pl->P, pl->coord_x,
-                                     pl->coord_y, pl->wave_off, pl->shape, carry, phases, st);
+                                     pl->coord_y, how, pl->shape, carry, phases, st);
     float *part = static_cast<float *>(pl->workspace);
     int rc = launch_spmm_any<T, float>(pl->vrow_ptr, pl->slice_cols, vals, X, part, pl->nnz, pl->K, pl->P, pl->coord_x,
-                                       pl->coord_y, pl->wave_off, pl->shape, carry, phases, st);
+                                       pl->coord_y, how, pl->shape, carry, phases, st);
     if (rc != MPS_OK) return rc;
     if (phases & MPS_PHASE_REDUCE) {
         const size_t per_slab = (size_t)pl->n_rows * pl->K;
         if (pl->K % 4 == 0)
             hipLaunchKernelGGL((tile_reduce_kernel<T, 4>), dim3((unsigned)((per_slab / 4 + 255) / 256)), dim3(256), 0, st,
-                               part, Y, pl->n_rows, pl->K, pl->num_slabs);
+                               part, Y, pl->n_rows, pl->K, pl->num_segs);
         else
             hipLaunchKernelGGL((tile_reduce_kernel<T, 1>), dim3((unsigned)((per_slab + 255) / 256)), dim3(256), 0, st, part,
-                               Y, pl->n_rows, pl->K, pl->num_slabs);
+                               Y, pl->n_rows, pl->K, pl->num_segs);
         MPS_HIP_TRY(hipGetLastError());
     }
     return MPS_OK;
@@ -475,6 +879,13 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->total_rounds = plan->total_rounds;
     info->slice_slots = plan->total_rounds * (long long)(plan->shape.tpw * kWindow);
     info->device_bytes = plan->device_bytes;
+    info->num_segments = plan->num_segs;
+    info->hot_rows = plan->hot_rows;
+    info->hot_waves = plan->hot_waves;
+    info->hot_nnz = plan->hot_nnz;
+    info->hot_cost = plan->hot_cost;
+    info->mark_shift = plan->mark_shift;
+    info->hot_mark_shift = plan->hot_mark_shift;
     return MPS_OK;
 }
 
@@ -498,6 +909,10 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
     case MPS_PLAN_ARRAY_SLICE_COLS: src = plan->slice_cols; have = slots * sizeof(int); break;
     case MPS_PLAN_ARRAY_SLICE_SRC: src = plan->slice_src; have = slots * sizeof(int); break;
     case MPS_PLAN_ARRAY_SLICE_VALS: src = plan->slice_vals; have = slots * (size_t)plan->elem_bytes; break;
+    case MPS_PLAN_ARRAY_HOT_COLS:
+        src = plan->hot_cols;
+        have = (size_t)(plan->hot_rows > 0 ? plan->num_slabs : 0) * (size_t)plan->hot_rows * sizeof(int);
+        break;
     default: return MPS_ERR_INVALID_ARG;
     }
     if (bytes != have) return MPS_ERR_INVALID_ARG;

@@ -141,13 +141,14 @@ class Plan:
     and the workspace.  The counterpart of what the reference sets up once
     before its repeat loop (src/MergePathSpMM.cu:192-220)."""
 
-    def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0):
+    def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto"):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
         self.dtype = csr.val.dtype
         eb = 4 if self.dtype == torch.float32 else 2
         flags = {"auto": 0, "off": _cabi.MPS_PLAN_NO_TILING, "force": _cabi.MPS_PLAN_FORCE_TILING}[tiling]
+        flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_HOT, "force": _cabi.MPS_PLAN_FORCE_HOT}[hot]
         check(_cabi.lib().mps_plan_create(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
                                           int(K), eb, int(default_cost(csr.n_rows, csr.nnz) if cost is None else cost),
                                           int(threads_per_wave), flags, int(slab_bytes), _stream(),
@@ -178,13 +179,14 @@ class Plan:
         np, i = self._np, self.info
         slots = int(i.slice_slots)
         shapes = {
-            _cabi.MPS_PLAN_ARRAY_VROW_PTR: (i.num_slabs * i.n_rows + 1, np.int32),
+            _cabi.MPS_PLAN_ARRAY_VROW_PTR: (i.num_segments * i.n_rows + 1, np.int32),
             _cabi.MPS_PLAN_ARRAY_COORD_X: (i.num_partitions + 1, np.int32),
             _cabi.MPS_PLAN_ARRAY_COORD_Y: (i.num_partitions + 1, np.int32),
             _cabi.MPS_PLAN_ARRAY_WAVE_OFF: (i.num_waves + 1, np.int32),
             _cabi.MPS_PLAN_ARRAY_SLICE_COLS: (slots, np.int32),
             _cabi.MPS_PLAN_ARRAY_SLICE_SRC: (slots, np.int32),
             _cabi.MPS_PLAN_ARRAY_SLICE_VALS: (slots, np.float32 if i.elem_bytes == 4 else np.float16),
+            _cabi.MPS_PLAN_ARRAY_HOT_COLS: (i.num_slabs * i.hot_rows, np.int32),
         }
         n, dt = shapes[which]
         out = np.empty(n, dtype=dt)

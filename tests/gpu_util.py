@@ -40,3 +40,16 @@ def check_fp32(Y, ref, scale, rel_elem=True):
     if rel_elem:
         assert (err <= 1e-5 * np.abs(ref) + 1e-6).all()
     return float(err.max())
+
+
+def check_fp16(Y, ref, scale):
+    """fp16 bar: 2e-2 relative.  The device accumulates in fp32 and rounds once
+    to half, so the error is half an ulp of the result (2^-11 relative) plus the
+    fp32 accumulation error, far inside the bar; rows whose terms cancel are
+    again measured against sum_j |a_ij x_jk|."""
+    Y = Y.astype(np.float64)
+    err = np.abs(Y - ref)
+    assert np.isfinite(Y).all()
+    assert (err <= 2e-2 * np.abs(ref) + 2e-2 * 1e-3 * scale + 1e-6).all()
+    # what the arithmetic actually delivers: one half rounding of the result
+    assert (err <= 2.0 ** -10 * np.abs(ref) + 1e-5 * scale + 1e-7).all()

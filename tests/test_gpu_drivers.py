@@ -47,6 +47,7 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
     rp, ci, val, X = inputs(pkg, graph_file, K)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     for cost, tpw, extra in ((32, 16, ()), ("default", 64, ()), (7, 1, ("--no-plan",)), (128, 0, ("--no-plan",)),
+                             (16, 16, ("--tiling", "force", "--slab-bytes", 65536, "--hot", "off")),
                              (16, 16, ("--tiling", "force", "--slab-bytes", 65536))):
         dump = tmp_path / "y.bin"
         out = run("MergePathSpMM", graph_file, K, cost, tpw, 3, "--dump", dump, *extra)
@@ -58,7 +59,10 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
         assert j["kernel"] == "merge_path" and j["repeat"] == 3 and j["nnz"] == ci.size
         slabs = j["num_slabs"]
         assert j["plan"] == ("--no-plan" not in extra) and (slabs > 1) == ("force" in extra)
-        assert j["P"] == orc.num_partitions(slabs * (rp.size - 1), ci.size, 32 if cost == "default" else cost)  # small graph: 32
+        hot = "force" in extra and "off" not in extra  # forced slabs are narrower than the LDS table: all columns hot
+        assert (j["hot_rows"] > 0) == hot and ("hot columns: " in out) == hot
+        if not hot:  # with hot columns every segment is split on its own
+            assert j["P"] == orc.num_partitions(slabs * (rp.size - 1), ci.size, 32 if cost == "default" else cost)  # small graph: 32
         assert abs(j["checksum"] - Y.astype(np.float64).sum()) <= 1e-6 * np.abs(Y).sum() + 1e-6
 
 

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import check_fp32, make_csr, random_csr, to_dev
+from gpu_util import check_fp16, check_fp32, make_csr, random_csr, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -23,14 +23,83 @@ def slab_major_reference(rp, ci, num_slabs, slab_cols):
     return vrp, perm.astype(np.int32)
 
 
+def hot_reference(rp, ci, num_slabs, slab_cols, hot_rows):
+    """(hot_slot[n], hot_cols[num_slabs * hot_rows]): per slab the hot_rows
+    columns with the most nonzeros (ties to the smaller id, unreferenced
+    columns never), slots in ascending column order."""
+    n = rp.size - 1
+    deg = np.bincount(ci, minlength=n)
+    hot_slot = np.full(n, -1, dtype=np.int64)
+    hot_cols = np.full(num_slabs * hot_rows, -1, dtype=np.int32)
+    for s in range(num_slabs):
+        c0, c1 = min(s * slab_cols, n), min((s + 1) * slab_cols, n)
+        cols = np.arange(c0, c1)
+        order = cols[np.lexsort((cols, -deg[c0:c1]))][:hot_rows]
+        order = np.sort(order[deg[order] > 0])
+        hot_slot[order] = np.arange(order.size)
+        hot_cols[s * hot_rows:s * hot_rows + order.size] = order
+    return hot_slot, hot_cols
+
+
+def segment_major_reference(rp, ci, num_slabs, slab_cols, hot_slot):
+    """Like slab_major_reference with 2 * num_slabs segments: segment s holds
+    the nonzeros of slab s in hot columns, segment num_slabs + s the others."""
+    n = rp.size - 1
+    rows = np.repeat(np.arange(n, dtype=np.int64), np.diff(rp))
+    slab = np.minimum(ci.astype(np.int64) // slab_cols, num_slabs - 1)
+    seg = np.where(hot_slot[ci] >= 0, slab, num_slabs + slab)
+    v = seg * n + rows
+    perm = np.argsort(v, kind="stable")
+    counts = np.bincount(v, minlength=2 * num_slabs * n)
+    vrp = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    return vrp, perm.astype(np.int32)
+
+
+def segmented_partition_reference(orc, vrp, n, num_slabs, cost, hot_cost, G):
+    """Every segment split on its own with the reference search and padded
+    with empty partitions to whole wavefronts.  Returns (xs, ys, hot_partitions)."""
+    xs, ys = [], []
+    hot_parts = 0
+    for g in range(2 * num_slabs):
+        seg_rp = vrp[g * n:(g + 1) * n + 1].astype(np.int64)
+        y0 = int(seg_rp[0])
+        nnz_g = int(seg_rp[-1]) - y0
+        total = n + 1 + nnz_g
+        parts = max(1, (total - 1) // (hot_cost if g < num_slabs else cost))
+        lx, ly = orc.partition_coords((seg_rp - y0).astype(np.int32), nnz_g, parts)
+        padded = -(-parts // G) * G
+        lx = np.concatenate([lx[:parts], np.full(padded - parts, n + 1)])
+        ly = np.concatenate([ly[:parts], np.full(padded - parts, nnz_g)])
+        xs.append(g * n + np.maximum(lx, 1))
+        ys.append(y0 + ly)
+        if g < num_slabs:
+            hot_parts += padded
+    xs.append([2 * num_slabs * n + 1])
+    ys.append([int(vrp[-1])])
+    return np.concatenate(xs).astype(np.int32), np.concatenate(ys).astype(np.int32), hot_parts
+
+
 def check_plan_layout(pkg, orc, plan, rp, ci, val):
     c, i = pkg._cabi, plan.info
     n, nnz = rp.size - 1, ci.size
-    vrp, perm = slab_major_reference(rp, ci, i.num_slabs, i.slab_cols)
-    assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_VROW_PTR), vrp)
-    # the partition of the virtual rows is the reference split (oracle restatement)
-    assert i.num_partitions == orc.num_partitions(i.num_slabs * n, nnz, i.cost)
-    xs, ys = orc.partition_coords(vrp, nnz, i.num_partitions)
+    if i.hot_rows > 0:
+        assert i.num_segments == 2 * i.num_slabs and i.hot_cost == max(i.cost, 256)
+        hot_slot, hot_cols = hot_reference(rp, ci, i.num_slabs, i.slab_cols, i.hot_rows)
+        assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_HOT_COLS), hot_cols)
+        assert i.hot_nnz == int((hot_slot[ci] >= 0).sum())
+        vrp, perm = segment_major_reference(rp, ci, i.num_slabs, i.slab_cols, hot_slot)
+        assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_VROW_PTR), vrp)
+        xs, ys, hot_parts = segmented_partition_reference(orc, vrp, n, i.num_slabs, i.cost, i.hot_cost, i.threads_per_wave)
+        assert i.num_partitions == xs.size - 1 and i.hot_waves * i.threads_per_wave == hot_parts
+        want_cols = np.where(hot_slot[ci] >= 0, hot_slot[ci], ci)  # hot nonzeros carry their LDS slot
+    else:
+        assert i.num_segments == i.num_slabs and i.hot_waves == 0 and i.hot_nnz == 0
+        vrp, perm = slab_major_reference(rp, ci, i.num_slabs, i.slab_cols)
+        assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_VROW_PTR), vrp)
+        # the partition of the virtual rows is the reference split (oracle restatement)
+        assert i.num_partitions == orc.num_partitions(i.num_slabs * n, nnz, i.cost)
+        xs, ys = orc.partition_coords(vrp, nnz, i.num_partitions)
+        want_cols = ci
     assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_COORD_X), xs)
     assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_COORD_Y), ys)
     # slices: wave w, round r, group g, element j  <-  virtual nonzero ys[p] + 16 r + j
@@ -55,29 +124,85 @@ def check_plan_layout(pkg, orc, plan, rp, ci, val):
     assert np.array_equal(src, want_src)
     live = want_src >= 0
     assert live.sum() == nnz
-    assert np.array_equal(cols[live], ci[want_src[live]]) and (cols[~live] == 0).all()
+    # column entries: column (or LDS slot) below the mark shift, above it the number of rows that end in front
+    # of the nonzero inside its partition
+    row_of = np.searchsorted(vrp, np.arange(nnz), side="right") - 1
+    ends = np.diff(row_of, prepend=0)
+    first = ys[:-1][cnt > 0]
+    ends[first] = row_of[first] - (np.maximum(xs[:-1][cnt > 0], 1) - 1)
+    slot_part = np.repeat(np.arange(W), (wave_off[1:] - wave_off[:-1]) * G * 16)  # wave of every slot
+    shift = np.where(slot_part < i.hot_waves, i.hot_mark_shift, i.mark_shift)
+    assert (i.hot_mark_shift > 0) == (i.hot_rows > 0)
+    cols_u = cols.astype(np.int64) & 0xFFFFFFFF
+    got_col = np.where(shift > 0, cols_u & ((1 << shift) - 1), cols_u)
+    got_ends = np.where(shift > 0, cols_u >> shift, 0)
+    inv = np.empty(nnz, dtype=np.int64)
+    inv[perm] = np.arange(nnz)  # original nonzero -> virtual position
+    vpos = inv[want_src[live]]
+    assert np.array_equal(got_col[live], want_cols[want_src[live]]) and (cols[~live] == 0).all()
+    assert np.array_equal(got_ends[live], np.where(shift[live] > 0, ends[vpos], 0))
     assert np.array_equal(vals[live], val[want_src[live]]) and (vals[~live] == 0).all()
 
 
-@pytest.mark.parametrize("tiling,slab_bytes,cost,tpw", [("off", 0, 16, 0), ("force", 16384, 16, 0), ("force", 4096, 7, 3),
-                                                        ("force", 1 << 20, 64, 16), ("force", 8192, 128, 1)])
-def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw):
+@pytest.mark.parametrize("tiling,slab_bytes,cost,tpw,hot",
+                         [("off", 0, 16, 0, "auto"), ("force", 16384, 16, 0, "off"), ("force", 4096, 7, 3, "off"),
+                          ("force", 1 << 20, 64, 16, "off"), ("force", 8192, 128, 1, "off"),
+                          ("force", 16384, 16, 0, "auto"), ("force", 4096, 7, 3, "force"), ("force", 8192, 128, 1, "auto")])
+def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw, hot):
     rng = np.random.default_rng(cost + slab_bytes)
     n = 500
     rp, ci = random_csr(rng, n, 40, hub_rows=[(3, 450), (499, 300)])
     val = rng.random(ci.size).astype(np.float32)
     csr = make_csr(pkg, dev, rp, ci, val)
-    plan = pkg.spmm.Plan(csr, 16, cost=cost, threads_per_wave=tpw, tiling=tiling, slab_bytes=slab_bytes)
+    plan = pkg.spmm.Plan(csr, 16, cost=cost, threads_per_wave=tpw, tiling=tiling, slab_bytes=slab_bytes, hot=hot)
     if tiling == "force":
         assert plan.info.num_slabs == -(-n // plan.info.slab_cols) and plan.info.slab_cols % 64 == 0
+        # slabs narrower than the LDS table: every referenced column is hot
+        assert plan.info.hot_rows == (0 if hot == "off" else 1728)
     else:
-        assert plan.info.num_slabs == 1
+        assert plan.info.num_slabs == 1 and plan.info.hot_rows == 0
     check_plan_layout(pkg, orc, plan, rp, ci, val)
     # new values flow through set_values
     val2 = rng.random(ci.size).astype(np.float32)
     plan.set_values(torch.from_numpy(val2).to(dev))
     check_plan_layout(pkg, orc, plan, rp, ci, val2)
     plan.close()
+
+
+@pytest.mark.parametrize("K,dtype,hot_rows", [(16, np.float32, 1728), (32, np.float32, 832), (64, np.float16, 704)])
+def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
+    """Slabs wider than the LDS table: part of every slab is hot, part cold."""
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=9000,nnz=400000,gamma=2.1,dmax=3000", seed=21)
+    n = rp.size - 1
+    val = g.fill_uniform_f32(ci.size, 5, 0.0, 1.0).astype(dtype)
+    X = g.fill_uniform_f32(n * K, 6, -1.0, 1.0).reshape(n, K).astype(dtype)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    slab_cols = 4096
+    plan = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize)
+    i = plan.info
+    assert (i.num_slabs, i.slab_cols, i.hot_rows, i.num_segments) == (3, slab_cols, hot_rows, 6)
+    assert 0 < i.hot_nnz < ci.size
+    check_plan_layout(pkg, orc, plan, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    Y = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val.astype(np.float32), X.astype(np.float32), want_abs=True)
+    if dtype == np.float32:
+        check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    else:
+        check_fp16(Y.cpu().numpy(), ref, scale)
+    # the same plan without hot columns gives the same rows up to summation order
+    cold = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize, hot="off")
+    assert cold.info.hot_rows == 0 and cold.info.num_segments == 3
+    Yc = cold.spmm(d_X)
+    torch.cuda.synchronize()
+    if dtype == np.float32:
+        check_fp32(Yc.cpu().numpy(), ref, scale, rel_elem=False)
+    # twice in a row: bit-identical
+    Y2 = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    assert torch.equal(Y, Y2)
 
 
 def test_unsorted_rows(pkg, dev):
