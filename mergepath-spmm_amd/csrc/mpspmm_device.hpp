@@ -572,6 +572,122 @@ __global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ w
     Y[(size_t)hr * K + k] = (TOut)sum;
 }
 
+// The same fix-up for K a multiple of 4 up to 256, with K / 4 lanes per record
+// (16-byte loads) and as many records side by side as fit in a wavefront.  A
+// lane walks back over at most kFixupShort records on its own; a row that
+// reaches further (a hub row under a small cost spans hundreds of wavefronts)
+// is finished by the whole wavefront: it finds the end of the chain 64 records
+// per step and adds the tails with all lanes.
+constexpr int kFixupShort = 6;
+
+template <typename TOut>
+__global__ __launch_bounds__(256) void mp_fixup_wide_kernel(const int *__restrict__ ws_head_row,
+                                                             const float *__restrict__ ws_head,
+                                                             const float *__restrict__ ws_tail,
+                                                             TOut *__restrict__ Y, int num_waves, int K)
+{
+    const int lane = threadIdx.x & 63;
+    const int lpr = K >> 2;      // lanes per record
+    const int slots = 64 / lpr;  // records side by side
+    const int slot = lane / lpr, q = lane - slot * lpr;
+    const long long first_rec = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * slots;
+    if (first_rec >= num_waves) return;  // whole wavefront
+    const int w = (int)first_rec + slot;
+    const bool valid = slot < slots && w < num_waves;
+    const float4 *tail4 = reinterpret_cast<const float4 *>(ws_tail);
+    auto add = [](float4 &a, const float4 &b) {
+        a.x += b.x;
+        a.y += b.y;
+        a.z += b.z;
+        a.w += b.w;
+    };
+    // what a row that ends one record back needs, requested at once
+    int hr = -1, hprev = 0;
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f), t1 = sum;
+    if (valid) {
+        hr = ws_head_row[w];
+        sum = reinterpret_cast<const float4 *>(ws_head)[(size_t)w * lpr + q];
+        if (w > 0) {
+            hprev = ws_head_row[w - 1];
+            t1 = tail4[(size_t)(w - 1) * lpr + q];
+        }
+    }
+    const bool mine = valid && hr >= 0;
+    // chain: records w - 1, w - 2, ... back to and including the nearest one with a row end
+    int j = w - 1;
+    bool open = mine && j >= 0;
+    if (open) {
+        add(sum, t1);
+        open = hprev < 0;
+        --j;
+    }
+    for (int step = 1; step < kFixupShort; ++step) {
+        if (open && j >= 0) {
+            const float4 t = tail4[(size_t)j * lpr + q];
+            const int hj = ws_head_row[j];
+            add(sum, t);
+            open = hj < 0;
+            --j;
+        } else {
+            open = false;
+        }
+    }
+    // long chains, one after the other, by the whole wavefront
+    unsigned long long todo = __ballot(open && j >= 0 && q == 0);
+    while (todo != 0) {
+        const int src_lane = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const int jstart = __shfl(j, src_lane, 64);  // next record of that chain
+        int len = 0;
+        for (int base = jstart; base >= 0; base -= 64) {
+            const int jj = base - lane;
+            const bool stop = jj < 0 || ws_head_row[jj] >= 0;
+            const unsigned long long m = __ballot(stop);
+            if (m != 0) {
+                const int first = __ffsll((long long)m) - 1;
+                len += first + ((base - first) >= 0 ? 1 : 0);
+                break;
+            }
+            len += 64;
+        }
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (slot < slots) {
+            int i = slot;
+            for (; i + 3 * slots < len; i += 4 * slots) {
+                float4 t[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) t[u] = tail4[(size_t)(jstart - (i + u * slots)) * lpr + q];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) add(acc, t[u]);
+            }
+            for (; i < len; i += slots) add(acc, tail4[(size_t)(jstart - i) * lpr + q]);
+        }
+        float4 total = acc;  // slots added in a fixed order: the result does not depend on timing
+        for (int sl = 1; sl < slots; ++sl) {
+            const int from = q + sl * lpr;
+            float4 v;
+            v.x = __shfl(acc.x, from, 64);
+            v.y = __shfl(acc.y, from, 64);
+            v.z = __shfl(acc.z, from, 64);
+            v.w = __shfl(acc.w, from, 64);
+            add(total, v);
+        }
+        float4 v;  // from the lanes of slot 0 to the lanes that own the row
+        v.x = __shfl(total.x, q, 64);
+        v.y = __shfl(total.y, q, 64);
+        v.z = __shfl(total.z, q, 64);
+        v.w = __shfl(total.w, q, 64);
+        if (slot * lpr == src_lane && slot < slots) add(sum, v);
+    }
+    if (mine) {
+        TOut *out = Y + (size_t)hr * K + 4 * q;
+        out[0] = (TOut)sum.x;
+        out[1] = (TOut)sum.y;
+        out[2] = (TOut)sum.z;
+        out[3] = (TOut)sum.w;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Exclusive prefix sum of an int array, in place (three launches).
 // ---------------------------------------------------------------------------
@@ -782,10 +898,17 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
         MPS_HIP_TRY(hipGetLastError());
     }
     if (phases & MPS_PHASE_FIXUP) {
-        long long threads = (long long)W * K;
-        unsigned blocks = (unsigned)((threads + 255) / 256);
-        hipLaunchKernelGGL((mp_fixup_kernel<TOut>), dim3(blocks), dim3(256), 0, st, ws_head_row, ws_head, ws_tail,
-                           Y, W, K);
+        if (K % 4 == 0 && K <= 256) {
+            const int per_wave = 64 / (K / 4);  // records per wavefront
+            const long long fix_waves = ((long long)W + per_wave - 1) / per_wave;
+            hipLaunchKernelGGL((mp_fixup_wide_kernel<TOut>), dim3((unsigned)((fix_waves + 3) / 4)), dim3(256), 0, st,
+                               ws_head_row, ws_head, ws_tail, Y, W, K);
+        } else {
+            long long threads = (long long)W * K;
+            unsigned blocks = (unsigned)((threads + 255) / 256);
+            hipLaunchKernelGGL((mp_fixup_kernel<TOut>), dim3(blocks), dim3(256), 0, st, ws_head_row, ws_head, ws_tail,
+                               Y, W, K);
+        }
         MPS_HIP_TRY(hipGetLastError());
     }
     return MPS_OK;
