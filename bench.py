@@ -102,7 +102,7 @@ def main():
     d_X = torch.from_numpy(X).to(dev)
     d_Y = torch.full_like(d_X, float("nan"))
     csr.validate()
-    cost = args.cost if args.cost > 0 else sp.default_cost(n, nnz)
+    cost = args.cost if args.cost > 0 else sp.default_cost(n, nnz, K, eb)
     plan = None
     if args.mode != "plain":
         tiling = {"auto": "auto", "untiled": "off", "tiled": "force"}[args.mode]

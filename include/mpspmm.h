@@ -69,10 +69,12 @@ const char *mps_version(void);
 int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out);
 
 /* The cost this library uses when the caller names none (the reference has
- * no default; src/MergePathSpMM.cu:121 takes it from argv): 128 merge items
- * per partition, fewer for small matrices (64 below 2^24 items, 32 below
- * 2^21) so that the partitions still fill the GPU. */
-int mps_default_cost(int n_rows, int nnz, int *cost_out);
+ * no default; src/MergePathSpMM.cu:121 takes it from argv).  Measured on
+ * MI355X: 32 merge items per partition, 64 from 2^25 items and 128 from 2^27
+ * items on; and never fewer than about 512 items per wavefront, i.e. at least
+ * min(128, 512 / partitions per wavefront) for the given K and element size
+ * (32 at K = 16 fp32, 128 from K = 64 fp32 on). */
+int mps_default_cost(int n_rows, int nnz, int K, int elem_bytes, int *cost_out);
 
 /* Merge items per partition, src/MergePathSpMM.cu:327-328:
  *   ceil((n_rows + 1 + nnz) / P). */
@@ -255,6 +257,7 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     gathered through L2.  Segments are ordered hot first (virtual row
  *     v = seg * n_rows + r, 2 * num_slabs segments), each is partitioned on
  *     its own, and the plan runs two launches of the same kernel.  Used when
+ *     a row of X has at most 64 bytes (wider rows are cheaper through L2) and
  *     the hot columns hold at least 15 % of the nonzeros.
  *   - The merge-path partition (mps_num_partitions, mps_partition) of the
  *     virtual rows for the given cost: one split of all of them, or, with hot
@@ -284,7 +287,7 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_NO_TILING 1u    /* never tile                                  */
 #define MPS_PLAN_FORCE_TILING 2u /* tile with slab_bytes slabs whatever the shape */
 #define MPS_PLAN_NO_HOT 4u       /* never keep hot columns' rows of X in LDS     */
-#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros */
+#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes */
 
 typedef struct mps_plan_info {
     int n_rows, nnz, K, elem_bytes, cost, threads_per_wave;

@@ -49,7 +49,7 @@ PROTOTYPES = {
     "mps_status_string": (ctypes.c_char_p, [_i]),
     "mps_version": (ctypes.c_char_p, []),
     "mps_num_partitions": (_i, [_i, _i, _i, c_int_p]),
-    "mps_default_cost": (_i, [_i, _i, c_int_p]),
+    "mps_default_cost": (_i, [_i, _i, _i, _i, c_int_p]),
     "mps_items_per_partition": (_i, [_i, _i, _i, c_int_p]),
     "mps_max_threads_per_wave": (_i, [_i, _i, c_int_p]),
     "mps_csr_read_header": (_i, [ctypes.c_char_p, c_int_p, c_int_p]),

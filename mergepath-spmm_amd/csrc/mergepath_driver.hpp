@@ -45,7 +45,7 @@ int mergepath_main(int argc, char **argv)
     Graph gr;
     load_graph(pos[0], opt.seed, gr);
     const int N = gr.n_rows, nnz = gr.nnz, K = dimension;
-    if (cost == 0) mps_ok(mps_default_cost(N, nnz, &cost), "mps_default_cost");
+    if (cost == 0) mps_ok(mps_default_cost(N, nnz, K, (int)sizeof(T), &cost), "mps_default_cost");
 
     int max_tpw = 0;
     mps_ok(mps_max_threads_per_wave(K, (int)sizeof(T), &max_tpw), "mps_max_threads_per_wave");

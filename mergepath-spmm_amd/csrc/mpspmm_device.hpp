@@ -20,8 +20,11 @@
         if (e_ != hipSuccess) return MPS_ERR_HIP + (int)e_;     \
     } while (0)
 
+#ifndef MPS_HOT_WPB
+#define MPS_HOT_WPB 16
+#endif
 #ifndef MPS_HOT_RPL
-#define MPS_HOT_RPL 4
+#define MPS_HOT_RPL 1
 #endif
 #ifndef MPS_MAIN_KERNEL_ATTR
 #define MPS_MAIN_KERNEL_ATTR
@@ -34,7 +37,7 @@ constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kWindow = 16;  // nonzeros staged per lane-group per round
 constexpr int kXcds = 8;     // accelerator dies of an MI355X, each with its own L2
 constexpr int kHotRoundsPerLoad = MPS_HOT_RPL;  // rounds of the sliced arrays a hot wavefront loads at a time
-constexpr int kHotWavesPerBlock = 16;  // workgroup of the LDS-resident ("hot") launch of a plan
+constexpr int kHotWavesPerBlock = MPS_HOT_WPB;  // workgroup of the LDS-resident ("hot") launch of a plan
 
 using half_t = _Float16;
 typedef half_t half8_t __attribute__((ext_vector_type(8)));
@@ -423,9 +426,10 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) MP
     };
 
     if constexpr (SLICED) {
-        // RPL rounds are loaded at a time, one load ahead: 2 * RPL windows of the
-        // wavefront are in flight or in registers, which is what keeps the stream
-        // coming when only a few wavefronts fit on a CU (the hot launch).
+        // RPL rounds are loaded at a time, one load ahead: up to 2 * RPL windows of
+        // the wavefront are in flight or in registers.  Measured on MI355X, RPL = 1,
+        // 2 and 4 run the hot launch (16 wavefronts per CU) at the same speed, so
+        // both launches use 1.
         int round = wave_off[w];
         const int round_end = wave_off[w + 1];
         Win nx[RPL];

@@ -659,11 +659,15 @@ int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out)
     return MPS_OK;
 }
 
-int mps_default_cost(int n_rows, int nnz, int *cost_out)
+int mps_default_cost(int n_rows, int nnz, int K, int elem_bytes, int *cost_out)
 {
-    if (!cost_out || n_rows < 0 || nnz < 0) return MPS_ERR_INVALID_ARG;
+    if (!cost_out || n_rows < 0 || nnz < 0 || K <= 0 || (elem_bytes != 2 && elem_bytes != 4)) return MPS_ERR_INVALID_ARG;
     const int64_t total = (int64_t)n_rows + 1 + nnz;
-    *cost_out = total >= (1 << 24) ? 128 : total >= (1 << 21) ? 64 : 32;
+    const int by_size = total >= (1 << 27) ? 128 : total >= (1 << 25) ? 64 : 32;
+    // a wavefront should have some 512 merge items whatever number of partitions it holds
+    const int groups = mps_make_lane_shape(K, elem_bytes).groups;
+    const int by_width = 512 / groups < 128 ? 512 / groups : 128;
+    *cost_out = by_size > by_width ? by_size : by_width;
     return MPS_OK;
 }
 

@@ -406,9 +406,14 @@ size_t hot_static_lds(int vec)
     return kHotWavesPerBlock * (stage + comb) * sizeof(float) + kHotWavesPerBlock * 16 * sizeof(int);
 }
 
-int choose_hot_rows(int K, int eb, const SpmmShape &sh)
+int choose_hot_rows(int K, int eb, const SpmmShape &sh, bool force)
 {
     if (sh.row_shift < 0 || sh.ls.vec == 1 || sh.ls.col_tiles != 1) return 0;
+    // Measured on MI355X (Chung-Lu 233k): with 64-byte rows of X the hot launch wins
+    // (0.58 against 0.66 ms at K = 16 fp32); with 128-byte rows and more the L2 path
+    // moves twice the bytes per request at no extra cost while the LDS table holds
+    // half the rows, and the hot launch loses (1.16 against 0.99 ms at K = 32).
+    if (!force && (size_t)K * eb > 64) return 0;
     const size_t budget = 160 * 1024 - hot_static_lds(sh.ls.vec) - 2048;
     size_t rows = budget / ((size_t)K * eb);
     rows = rows / 64 * 64;
@@ -522,7 +527,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
     int hot_rows = 0;
     std::vector<int> h_hot_cols;
     if (pl->num_slabs > 1 && !(flags & MPS_PLAN_NO_HOT)) {
-        hot_rows = choose_hot_rows(K, eb, pl->shape);
+        hot_rows = choose_hot_rows(K, eb, pl->shape, (flags & MPS_PLAN_FORCE_HOT) != 0);
         if (2LL * pl->num_slabs * n + 1 + nnz > INT_MAX) hot_rows = 0;
         if (hot_rows > 0) {
             std::vector<int> h_deg((size_t)n), h_slot;

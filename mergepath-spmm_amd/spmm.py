@@ -13,10 +13,10 @@ import torch
 from . import _cabi
 from ._cabi import check
 
-def default_cost(n_rows, nnz):
+def default_cost(n_rows, nnz, K=16, elem_bytes=4):
     """Merge items (row ends + nonzeros) per partition when the caller gives no cost."""
     c = ctypes.c_int()
-    check(_cabi.lib().mps_default_cost(int(n_rows), int(nnz), ctypes.byref(c)), "mps_default_cost")
+    check(_cabi.lib().mps_default_cost(int(n_rows), int(nnz), int(K), int(elem_bytes), ctypes.byref(c)), "mps_default_cost")
     return c.value
 
 
@@ -150,7 +150,7 @@ class Plan:
         flags = {"auto": 0, "off": _cabi.MPS_PLAN_NO_TILING, "force": _cabi.MPS_PLAN_FORCE_TILING}[tiling]
         flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_HOT, "force": _cabi.MPS_PLAN_FORCE_HOT}[hot]
         check(_cabi.lib().mps_plan_create(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
-                                          int(K), eb, int(default_cost(csr.n_rows, csr.nnz) if cost is None else cost),
+                                          int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
                                           int(threads_per_wave), flags, int(slab_bytes), _stream(),
                                           ctypes.byref(self._h)), "mps_plan_create")
         self.K, self.n_rows = int(K), csr.n_rows

@@ -169,7 +169,8 @@ def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw,
     plan.close()
 
 
-@pytest.mark.parametrize("K,dtype,hot_rows", [(16, np.float32, 1728), (32, np.float32, 832), (64, np.float16, 704)])
+@pytest.mark.parametrize("K,dtype,hot_rows", [(16, np.float32, 1728), (32, np.float16, 1472), (32, np.float32, 832),
+                                              (64, np.float16, 704)])
 def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
     """Slabs wider than the LDS table: part of every slab is hot, part cold."""
     g = pkg.graphs
@@ -179,7 +180,13 @@ def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
     X = g.fill_uniform_f32(n * K, 6, -1.0, 1.0).reshape(n, K).astype(dtype)
     csr = make_csr(pkg, dev, rp, ci, val)
     slab_cols = 4096
-    plan = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize)
+    wide = K * val.itemsize > 64  # rows of X wider than 64 bytes: hot columns only on request
+    if wide:
+        auto = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize)
+        assert auto.info.hot_rows == 0
+        auto.close()
+    plan = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize,
+                         hot="force" if wide else "auto")
     i = plan.info
     assert (i.num_slabs, i.slab_cols, i.hot_rows, i.num_segments) == (3, slab_cols, hot_rows, 6)
     assert 0 < i.hot_nnz < ci.size

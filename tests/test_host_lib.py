@@ -51,8 +51,11 @@ def test_num_partitions_matches_oracle(pkg, orc):
         pkg.graphs.num_partitions(2 ** 30, 2 ** 30 + 5, 16)
     assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
     assert pkg.graphs.items_per_partition(6, 15, 5) == 5
-    assert pkg.spmm.default_cost(232965, 114604189) == 128 and pkg.spmm.default_cost(416349, 2081148) == 64
-    assert pkg.spmm.default_cost(4096, 32731) == 32
+    dc = pkg.spmm.default_cost
+    assert dc(232965, 114604189) == 64 and dc(416349, 2081148) == 32 and dc(4096, 32731) == 32
+    assert dc(1 << 22, 140000000) == 128 and dc(1 << 20, 16086273) == 32
+    # wide rows: fewer partitions per wavefront, so more items each
+    assert dc(1 << 20, 16086273, 64, 4) == 128 and dc(1 << 20, 16086273, 64, 2) == 64 and dc(4096, 32731, 256, 4) == 128
 
 
 def test_max_threads_per_wave(pkg):
