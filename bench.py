@@ -28,9 +28,10 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the main kernel, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
 # profiles/mp_spmm_kernel_chunglu_233k_f32_k16.md (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors the copy
 # probe gives, profiles/hbm_copy_probe_fetch_write_calibration.md).  Keyed by (workload, layout); other
-# configurations report null.
+# configurations report null.  Key: (workload, layout, column slabs, cost, hot columns per slab).
 MEASURED_TRAFFIC = {
-    ("chunglu_233k_f32_k16", "plan", 5, 128): int(544711 * 1024 * 2.0 + 80402 * 1024 * 1.0),
+    # cold + hot launch of the main kernel: FETCH_SIZE 380,635 + 181,210 KiB raw, WRITE_SIZE 82,080 + 82,181 KiB
+    ("chunglu_233k_f32_k16", "plan", 5, 64, 1728): int((380635 + 181210) * 1024 * 2.0 + (82080 + 82181) * 1024 * 1.0),
 }
 
 WORKLOADS = {
@@ -162,6 +163,7 @@ def main():
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t1) * 1e3
 
+    hot_on = plan is not None and plan.info.hot_rows > 0
     flops = 2.0 * nnz * K
     b_alg = algorithmic_bytes(n, nnz, K, eb, eb)
     gflops = flops / (ms_per_step * 1e6)
@@ -195,10 +197,11 @@ def main():
                       "tile_reduce_kernel": round(red_ms, 5),
                       "preprocessing, host wall time (once per matrix)": round(plan_ms, 3)},
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
-        "roofline": {"bound": "hbm", "kernel": "mp_spmm_kernel", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
+        "roofline": {"bound": "hbm", "kernel": "mp_spmm_kernel" + (" (hot + cold launch)" if hot_on else ""), "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4),
                      "traffic": MEASURED_TRAFFIC.get((args.workload, "plan" if plan is not None else "plain",
-                                                      plan.info.num_slabs if plan is not None else 1, cost)),
+                                                      plan.info.num_slabs if plan is not None else 1, cost,
+                                                      plan.info.hot_rows if plan is not None else 0)),
                      "algorithmic_bytes": int(b_alg)},
         "host_generate_s": round(gen_s, 2),
     }

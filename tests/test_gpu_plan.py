@@ -212,6 +212,33 @@ def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
     assert torch.equal(Y, Y2)
 
 
+def test_plan_without_row_marks(pkg, orc, dev, monkeypatch):
+    """MPS_ROW_MARKS=0 at plan creation: plain column ids in the sliced array, and
+    the kernel follows row_ptr as it does on the caller's CSR arrays (the path a
+    matrix takes whose column ids and row-end counts do not fit 32 bits together)."""
+    monkeypatch.setenv("MPS_ROW_MARKS", "0")
+    rng = np.random.default_rng(77)
+    n, K = 700, 16
+    rp, ci = random_csr(rng, n, 30, hub_rows=[(0, 650), (350, 400)])
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    for tiling, slab_bytes in (("off", 0), ("force", 16384)):
+        plan = pkg.spmm.Plan(csr, K, cost=12, tiling=tiling, slab_bytes=slab_bytes, hot="off")
+        assert plan.info.mark_shift == 0 and plan.info.hot_rows == 0
+        check_plan_layout(pkg, orc, plan, rp, ci, val)
+        Y = plan.spmm(d_X)
+        torch.cuda.synchronize()
+        check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+        plan.close()
+    monkeypatch.delenv("MPS_ROW_MARKS")
+    plan = pkg.spmm.Plan(csr, K, cost=12, tiling="off")
+    assert plan.info.mark_shift == 10  # 700 columns: 10 bits
+    plan.close()
+
+
 def test_unsorted_rows(pkg, dev):
     n = 130  # two 64-column slabs
     rp = np.concatenate([[0, 3, 5], np.full(n - 2, 5)]).astype(np.int32)
