@@ -144,6 +144,25 @@ int mps_fill_uniform_f16(uint16_t *out, size_t n, uint64_t seed, float lo, float
 /* Device side: validation                                                   */
 /* ------------------------------------------------------------------------ */
 
+/* Edge weights from degrees, on the device: the reference's implicit weight
+ * written out as a value array, so that the SpMM entry points reproduce its
+ * arithmetic on request.  Replaces the degree vector and the per-nonzero
+ * product in the kernels, src/MergePathSpMM.cu:178,183-185 (degrees[i] =
+ * row_ptr[i+1] - row_ptr[i]) and :450,459 (w = __fmaf_rn(float(deg_row),
+ * float(deg_col), 0)); fp16: src/MergePathSpMM_fp16.cu:451,460 (both degrees
+ * converted to half, multiplied in half: infinity beyond 65504).  The
+ * reference's tail partials use a source weight of 1 (:468): a defect, not
+ * reproduced.
+ *   MPS_WEIGHT_DEGREE_PRODUCT  val[e] = deg(row of e) * deg(col_idx[e])
+ *   MPS_WEIGHT_GCN             val[e] = 1 / sqrt(deg(row) * deg(col)), 0 where a degree is 0
+ * The matrix must be square (column ids index row_ptr, as in the reference). */
+#define MPS_WEIGHT_DEGREE_PRODUCT 0
+#define MPS_WEIGHT_GCN 1
+int mps_degree_values_f32(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int mode, float *d_val,
+                          void *stream);
+int mps_degree_values_f16(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int mode, void *d_val,
+                          void *stream);
+
 /* Checks on the device that row_ptr starts at 0, is non-decreasing, ends at
  * nnz, and that every column id lies in [0, n_cols).  Synchronises the
  * stream and allocates a 4-byte device flag for the duration of the call.

@@ -24,6 +24,8 @@ MPS_ERR_HIP = 1000
 MPS_PHASE_MAIN = 1
 MPS_PHASE_FIXUP = 2
 MPS_PHASE_REDUCE = 4
+MPS_WEIGHT_DEGREE_PRODUCT = 0
+MPS_WEIGHT_GCN = 1
 MPS_PLAN_NO_TILING = 1
 MPS_PLAN_FORCE_TILING = 2
 MPS_PLAN_NO_HOT = 4
@@ -63,6 +65,8 @@ PROTOTYPES = {
     "mps_graph_free": (None, [_vp]),
     "mps_fill_uniform_f32": (_i, [_vp, _sz, _u64, ctypes.c_float, ctypes.c_float]),
     "mps_fill_uniform_f16": (_i, [_vp, _sz, _u64, ctypes.c_float, ctypes.c_float]),
+    "mps_degree_values_f32": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "mps_degree_values_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "mps_csr_validate": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "mps_partition": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
     "mps_schedule_legacy": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -52,6 +52,8 @@ struct Options {
     int tiling = 0;             // --tiling off|force (default: where it pays)
     size_t slab_bytes = 0;      // --slab-bytes N (default: the library's 3 MiB)
     int hot = 0;                // --hot off|force (default: where it pays)
+    int weights = -1;           // --weights explicit|degree|gcn: seeded values (default), or from degrees on the device
+    bool ones = false;          // --features ones: all features 1.0, as the reference sets them (src/MergePathSpMM.cu:180-182)
 };
 
 // Strips the optional trailing flags; returns the positional arguments.
@@ -72,6 +74,11 @@ inline std::vector<std::string> split_args(int argc, char **argv, Options &opt)
             std::string t = argv[++i];
             opt.hot = t == "off" ? MPS_PLAN_NO_HOT : t == "force" ? MPS_PLAN_FORCE_HOT : 0;
         }
+        else if (a == "--weights" && i + 1 < argc) {
+            std::string t = argv[++i];
+            opt.weights = t == "degree" ? MPS_WEIGHT_DEGREE_PRODUCT : t == "gcn" ? MPS_WEIGHT_GCN : -1;
+        }
+        else if (a == "--features" && i + 1 < argc) opt.ones = std::string(argv[++i]) == "ones";
         else if (a == "--warmup" && i + 1 < argc) opt.warmup = std::atoi(argv[++i]);
         else if (a == "--seed" && i + 1 < argc) opt.seed = std::strtoull(argv[++i], nullptr, 10);
         else pos.push_back(a);

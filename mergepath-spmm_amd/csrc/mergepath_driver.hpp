@@ -16,6 +16,9 @@ template <> struct Elem<float> {
                     const int *cx, const int *cy, int tpw, void *ws, size_t wsb)
     { return mps_spmm_f32(rp, ci, v, X, Y, n, nnz, K, P, cx, cy, tpw, ws, wsb, nullptr); }
     static int plan_spmm(const mps_plan *pl, const float *X, float *Y) { return mps_plan_spmm_f32(pl, X, Y, nullptr); }
+    static int degree_values(const int *rp, const int *ci, int n, int nnz, int mode, float *v)
+    { return mps_degree_values_f32(rp, ci, n, nnz, mode, v, nullptr); }
+    static float one() { return 1.0f; }
 };
 template <> struct Elem<uint16_t> {
     static constexpr const char *name = "fp16";
@@ -24,6 +27,9 @@ template <> struct Elem<uint16_t> {
                     int P, const int *cx, const int *cy, int tpw, void *ws, size_t wsb)
     { return mps_spmm_f16(rp, ci, v, X, Y, n, nnz, K, P, cx, cy, tpw, ws, wsb, nullptr); }
     static int plan_spmm(const mps_plan *pl, const uint16_t *X, uint16_t *Y) { return mps_plan_spmm_f16(pl, X, Y, nullptr); }
+    static int degree_values(const int *rp, const int *ci, int n, int nnz, int mode, uint16_t *v)
+    { return mps_degree_values_f16(rp, ci, n, nnz, mode, v, nullptr); }
+    static uint16_t one() { return 0x3c00; }  // 1.0 in IEEE half
 };
 
 template <typename T>
@@ -63,6 +69,7 @@ int mergepath_main(int argc, char **argv)
     std::vector<T> h_val((size_t)nnz), h_X((size_t)N * K), h_Y((size_t)N * K);
     mps_ok(Elem<T>::fill(h_val.data(), h_val.size(), kSeedVal, 0.0f, 1.0f), "fill val");
     mps_ok(Elem<T>::fill(h_X.data(), h_X.size(), kSeedX, -1.0f, 1.0f), "fill X");
+    if (opt.ones) std::fill(h_X.begin(), h_X.end(), Elem<T>::one());
 
     DevBuf<int> d_rp((size_t)N + 1), d_ci((size_t)nnz), d_cx((size_t)P + 1), d_cy((size_t)P + 1);
     DevBuf<T> d_val((size_t)nnz), d_X((size_t)N * K), d_Y((size_t)N * K);
@@ -71,6 +78,8 @@ int mergepath_main(int argc, char **argv)
     d_val.upload(h_val.data());
     d_X.upload(h_X.data());
     mps_ok(mps_csr_validate(d_rp.p, d_ci.p, N, N, nnz, nullptr), "mps_csr_validate");
+    // the reference's implicit weight deg(row) * deg(col) (:450,459), written out once
+    if (opt.weights >= 0) mps_ok(Elem<T>::degree_values(d_rp.p, d_ci.p, N, nnz, opt.weights, d_val.p), "mps_degree_values");
 
     // Everything that depends on the matrix alone is built once, outside the
     // repeat loop, as generate_mp_sched and its uploads are (:192-220): with a

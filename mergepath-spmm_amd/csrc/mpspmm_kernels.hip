@@ -300,6 +300,52 @@ __global__ __launch_bounds__(256) void csr_validate_kernel(const int *__restrict
     if (err) atomicOr(bad, 1);
 }
 
+// ---------------------------------------------------------------------------
+// Edge weights from degrees: the reference's implicit weight, written out.
+// degrees[i] = row_ptr[i + 1] - row_ptr[i] (src/MergePathSpMM.cu:183-185);
+// weight of nonzero (r, c) = float(deg r) * float(deg c), one rounded product
+// (__fmaf_rn(a, b, 0), :450,459); the fp16 program multiplies the two degrees
+// converted to half, in half (src/MergePathSpMM_fp16.cu:451,460), which
+// overflows to infinity beyond 65504.  MPS_WEIGHT_GCN is the normalisation
+// GCN layers use, 1 / sqrt(deg r * deg c), 0 where a degree is 0.
+// One thread per nonzero; its row is found by bisection of row_ptr.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void degree_values_kernel(const int *__restrict__ row_ptr,
+                                                             const int *__restrict__ col_idx, int n_rows, int nnz,
+                                                             int mode, T *__restrict__ val)
+{
+    const long long e64 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e64 >= nnz) return;
+    const int e = (int)e64;
+    int lo = 0, hi = n_rows - 1;  // largest r with row_ptr[r] <= e
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (row_ptr[mid] <= e) lo = mid; else hi = mid - 1;
+    }
+    const int c = col_idx[e];
+    const int dr = row_ptr[lo + 1] - row_ptr[lo];
+    const int dc = row_ptr[c + 1] - row_ptr[c];
+    if (mode == MPS_WEIGHT_GCN) {
+        const float p = (float)dr * (float)dc;
+        val[e] = (T)(p > 0.f ? 1.0f / sqrtf(p) : 0.f);
+    } else {
+        val[e] = (T)dr * (T)dc;  // T = float: rounded fp32 product; T = half: both factors and the product in half
+    }
+}
+
+template <typename T>
+int degree_values_entry(const int *row_ptr, const int *col_idx, int n_rows, int nnz, int mode, T *val, void *stream)
+{
+    if (!row_ptr || n_rows < 0 || nnz < 0 || (nnz > 0 && (!col_idx || !val))) return MPS_ERR_INVALID_ARG;
+    if (mode != MPS_WEIGHT_DEGREE_PRODUCT && mode != MPS_WEIGHT_GCN) return MPS_ERR_INVALID_ARG;
+    if (nnz == 0) return MPS_OK;
+    hipLaunchKernelGGL((degree_values_kernel<T>), dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), row_ptr, col_idx, n_rows, nnz, mode, val);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
 template <typename T>
 int check_spmm_args(const int *row_ptr, const int *col_idx, const T *val, const T *X, const void *Y, int n_rows,
                     long long n_vrows, int nnz, int K, int P, const int *cx, const int *cy)
@@ -362,6 +408,18 @@ int mps_csr_validate(const int *d_row_ptr, const int *d_col_idx, int n_rows, int
     if (e != hipSuccess) return MPS_ERR_HIP + (int)e;
     if (e2 != hipSuccess) return MPS_ERR_HIP + (int)e2;
     return bad ? MPS_ERR_INVALID_CSR : MPS_OK;
+}
+
+int mps_degree_values_f32(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int mode, float *d_val,
+                          void *stream)
+{
+    return degree_values_entry<float>(d_row_ptr, d_col_idx, n_rows, nnz, mode, d_val, stream);
+}
+
+int mps_degree_values_f16(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int mode, void *d_val,
+                          void *stream)
+{
+    return degree_values_entry<half_t>(d_row_ptr, d_col_idx, n_rows, nnz, mode, static_cast<half_t *>(d_val), stream);
 }
 
 int mps_partition(const int *d_row_ptr, int n_rows, int nnz, int P, int *d_coord_x, int *d_coord_y,

@@ -57,6 +57,19 @@ class CsrDevice:
                                            self.nnz, _stream()), "mps_csr_validate")
 
 
+def degree_values(row_ptr, col_idx, mode="product", dtype=torch.float32):
+    """Edge weights from degrees on the device (mps_degree_values_*): the
+    reference's implicit weight deg(row) * deg(col)
+    (src/MergePathSpMM.cu:183-185,450,459) as an explicit value array, or the
+    GCN normalisation 1 / sqrt(deg(row) * deg(col)) with mode="gcn"."""
+    m = {"product": _cabi.MPS_WEIGHT_DEGREE_PRODUCT, "gcn": _cabi.MPS_WEIGHT_GCN}[mode]
+    n_rows, nnz = row_ptr.numel() - 1, col_idx.numel()
+    val = torch.empty(nnz, dtype=dtype, device=row_ptr.device)
+    fn = _cabi.lib().mps_degree_values_f32 if dtype == torch.float32 else _cabi.lib().mps_degree_values_f16
+    check(fn(_ptr(row_ptr), _ptr(col_idx), n_rows, nnz, m, _ptr(val), _stream()), "mps_degree_values")
+    return val
+
+
 class MergePathSchedule:
     """Partition count and boundary coordinates (generate_mp_sched, :300-385)."""
 

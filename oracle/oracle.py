@@ -173,3 +173,23 @@ def build_part(part_size, row_ptr):
     pn = np.empty(max(n, 1), dtype=np.int32)
     lib().orc_build_part(int(part_size), _ip(rp), int(rp.size - 1), _ip(pp), _ip(pn))
     return pp, pn[:n]
+
+
+def degree_values(row_ptr, col_idx, mode="product", dtype=np.float32):
+    """The reference's implicit edge weight as an array.  degrees[i] =
+    row_ptr[i+1] - row_ptr[i] (src/MergePathSpMM.cu:183-185); weight of
+    nonzero (r, c) = float(deg r) * float(deg c), one rounded fp32 product
+    (:450,459).  dtype=np.float16: both degrees converted to half and
+    multiplied in half (src/MergePathSpMM_fp16.cu:451,460; infinity beyond
+    65504).  mode="gcn": 1 / sqrt(deg r * deg c) in fp32, 0 where a degree
+    is 0 (no reference counterpart)."""
+    rp, ci = _i32(row_ptr), _i32(col_idx)
+    deg = np.diff(rp)
+    rows = np.repeat(np.arange(rp.size - 1), deg)
+    with np.errstate(over="ignore", divide="ignore", invalid="ignore"):
+        if mode == "gcn":
+            p = deg[rows].astype(np.float32) * deg[ci].astype(np.float32)
+            w = np.where(p > 0, np.float32(1.0) / np.sqrt(p, dtype=np.float32), np.float32(0.0)).astype(np.float32)
+            return w.astype(dtype)
+        t = np.dtype(dtype).type
+        return (deg[rows].astype(t) * deg[ci].astype(t)).astype(dtype)

@@ -66,6 +66,35 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
         assert abs(j["checksum"] - Y.astype(np.float64).sum()) <= 1e-6 * np.abs(Y).sum() + 1e-6
 
 
+def test_merge_path_driver_reference_setting(pkg, orc, graph_file, tmp_path):
+    """--weights degree --features ones: what the reference computes (weights
+    deg(row) * deg(col), features 1.0, src/MergePathSpMM.cu:180-185,450,459),
+    without its unit-weight tail defect: every column is the row sum of the weights."""
+    K = 16
+    rp, ci, _, _ = inputs(pkg, graph_file, K)
+    val = orc.degree_values(rp, ci)
+    rows = np.repeat(np.arange(rp.size - 1), np.diff(rp))
+    sums = np.bincount(rows, weights=val.astype(np.float64), minlength=rp.size - 1)
+    dump = tmp_path / "y.bin"
+    for prog, dt, tol in (("MergePathSpMM", np.float32, 1e-5), ("MergePathSpMM_fp16", np.float16, 2e-2)):
+        run(prog, graph_file, K, 32, 0, 2, "--dump", dump, "--weights", "degree", "--features", "ones")
+        Y = np.fromfile(dump, dtype=dt).reshape(-1, K).astype(np.float64)
+        if dt == np.float16:  # half weights overflow beyond 65504, as in the reference's fp16 program
+            valh = orc.degree_values(rp, ci, dtype=np.float16).astype(np.float64)
+            want = np.bincount(rows, weights=valh, minlength=rp.size - 1)
+            fin = np.isfinite(want) & (want < 65504)
+            assert fin.any() and np.allclose(Y[fin, 0], want[fin], rtol=tol, atol=1e-3)
+        else:
+            assert np.allclose(Y[:, 0], sums, rtol=tol, atol=1e-6)
+        ok = np.isfinite(Y[:, 0])
+        assert (Y[ok] == Y[ok][:, :1]).all()
+    run("MergePathSpMM", graph_file, K, 32, 16, 2, "--dump", dump, "--weights", "gcn")
+    Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
+    X = pkg.graphs.fill_uniform_f32((rp.size - 1) * K, 13, -1.0, 1.0).reshape(-1, K)
+    ref, scale = orc.spmm_f64(rp, ci, orc.degree_values(rp, ci, mode="gcn"), X, want_abs=True)
+    assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
+
+
 def test_merge_path_driver_errors(graph_file):
     out = run("MergePathSpMM", graph_file, 16, 32, expect=255)  # too few arguments -> usage, exit(-1)
     assert out.startswith("Usage: ./application <input_file> <dimension> <cost> <threads_per_wave> <repeat>")

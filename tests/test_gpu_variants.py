@@ -124,3 +124,52 @@ def test_large_scan_of_groups(pkg, orc, dev):
     pp, pn = orc.build_part(2, rp)
     assert np.array_equal(parts.part_ptr.cpu().numpy(), pp)
     assert np.array_equal(parts.part2node.cpu().numpy(), pn)
+
+
+@pytest.mark.parametrize("mode", ["product", "gcn"])
+def test_degree_values(pkg, orc, dev, mode):
+    """mps_degree_values_*: the reference's implicit weight deg(row) * deg(col)
+    (src/MergePathSpMM.cu:183-185,450,459) as an array; bit-exact for the
+    product (fp32 and half), one ulp for 1/sqrt."""
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=6000,nnz=300000,gamma=2.1,dmax=5000", seed=9)
+    # plus two hub rows that point at each other: 4097 * 4099 needs 25 bits, one fp32 rounding
+    n = rp.size - 1
+    hub = [np.r_[n + 1, np.arange(0, 4096)], np.r_[n, np.arange(0, 4098)]]
+    ci = np.concatenate([ci] + hub).astype(np.int32)
+    rp = np.concatenate([rp, [rp[-1] + 4097, rp[-1] + 4097 + 4099]]).astype(np.int32)
+    d_rp, d_ci = to_dev(dev, rp, ci)
+    for dtype, tdt in ((np.float32, torch.float32), (np.float16, torch.float16)):
+        got = pkg.spmm.degree_values(d_rp, d_ci, mode=mode, dtype=tdt).cpu().numpy()
+        want = orc.degree_values(rp, ci, mode=mode, dtype=dtype)
+        if mode == "product":
+            assert np.array_equal(got, want)  # inf == inf where half overflows
+            if dtype == np.float16:
+                assert np.isinf(want).any()
+            else:
+                assert (want > 2 ** 24).any()
+        else:
+            assert np.isfinite(got).all()
+            ulp = np.spacing(np.abs(want).astype(dtype))
+            assert (np.abs(got.astype(np.float64) - want.astype(np.float64)) <= ulp).all()
+
+
+def test_spmm_with_degree_weights_and_unit_features(pkg, orc, dev):
+    """The reference's setting (weights from degrees, all features 1.0): every
+    output column is the row sum of the weights."""
+    g = pkg.graphs
+    rp, ci, _ = g.generate("rmat:scale=12,ef=8,a=0.57,b=0.19,c=0.19", seed=3)
+    n, K = rp.size - 1, 16
+    d_rp, d_ci = to_dev(dev, rp, ci)
+    d_val = pkg.spmm.degree_values(d_rp, d_ci)
+    val = orc.degree_values(rp, ci)
+    X = np.ones((n, K), dtype=np.float32)
+    csr = pkg.spmm.CsrDevice(d_rp, d_ci, d_val)
+    plan = pkg.spmm.Plan(csr, K)
+    (d_X,) = to_dev(dev, X)
+    Y = plan.spmm(d_X).cpu().numpy()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y, ref, scale, rel_elem=False)
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    sums = np.bincount(rows, weights=val.astype(np.float64), minlength=n)
+    assert np.allclose(Y[:, 0], sums, rtol=1e-5, atol=1e-6) and (Y == Y[:, :1]).all()

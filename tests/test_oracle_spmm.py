@@ -85,3 +85,34 @@ def test_half_inputs(orc):
     # bit patterns: subnormal, one, max, -2
     for bits, want in ((0x0001, 2.0 ** -24), (0x3c00, 1.0), (0x7bff, 65504.0), (0xc000, -2.0), (0x0000, 0.0)):
         assert orc.lib().orc_half_to_double(bits) == want
+
+
+def test_degree_values_hand_example(orc):
+    # degrees 2, 1, 0, 3; weight of (r, c) = deg r * deg c (src/MergePathSpMM.cu:183-185,450,459)
+    rp = np.array([0, 2, 3, 3, 6], dtype=np.int32)
+    ci = np.array([1, 3, 0, 0, 1, 3], dtype=np.int32)
+    assert orc.degree_values(rp, ci).tolist() == [2.0, 6.0, 2.0, 6.0, 3.0, 9.0]
+    assert orc.degree_values(rp, ci, dtype=np.float16).tolist() == [2.0, 6.0, 2.0, 6.0, 3.0, 9.0]
+    g = orc.degree_values(rp, ci, mode="gcn")
+    want = [2 ** -0.5, 6 ** -0.5, 2 ** -0.5, 6 ** -0.5, 3 ** -0.5, 1 / 3]
+    assert np.allclose(g, want, rtol=2e-7, atol=0) and g.dtype == np.float32
+
+
+def test_degree_values_rounding_and_half_overflow(orc):
+    # two hub rows that point at each other: 4097 * 4099 = 16,793,603 needs 25 bits -> one fp32 rounding
+    n = 4100
+    deg = np.zeros(n, dtype=np.int64)
+    deg[0], deg[1] = 4097, 4099
+    rp = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    ci = np.concatenate([np.r_[1, np.arange(2, 4098)], np.r_[0, np.arange(2, 4100)]]).astype(np.int32)
+    w = orc.degree_values(rp, ci)
+    assert w[0] == np.float32(16793603) and float(w[0]) in (16793602.0, 16793604.0)
+    assert w[4097] == w[0] and w[1] == 0.0  # column 2 has degree 0
+    h = orc.degree_values(rp, ci, dtype=np.float16)
+    assert np.isinf(h[0]) and h[1] == 0.0  # half(4097) * half(4099) = 4096 * 4100 > 65504
+    rp2 = np.array([0, 200, 400] + [400] * 198, dtype=np.int32)  # degrees 200, 200, then empty rows
+    ci2 = np.concatenate([np.arange(200), np.arange(200)]).astype(np.int32)
+    h2 = orc.degree_values(rp2, ci2, dtype=np.float16)
+    assert h2[0] == 40000.0 and h2[1] == 40000.0 and h2[2] == 0.0  # 200 * 200 fits half
+    g = orc.degree_values(rp2, ci2, mode="gcn")
+    assert g[0] == np.float32(1.0) / np.float32(200.0) and g[2] == 0.0
