@@ -348,6 +348,26 @@ int mps_plan_spmm_f32(const mps_plan *plan, const float *d_X, float *d_Y, void *
 int mps_plan_spmm_f16(const mps_plan *plan, const uint16_t *d_X, uint16_t *d_Y, void *stream);
 int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsigned phases, void *stream);
 
+/* Parameter sweep for one matrix and K — what the reference leaves to the
+ * user's hand (cost and partitions per warp are command-line arguments,
+ * src/MergePathSpMM.cu:121-122, and its README reports the best of a sweep).
+ * Builds a plan for each candidate (costs 16 .. 256 with a full wavefront, the
+ * default cost with half the partitions per wavefront, without hot columns,
+ * without tiling), runs `repeats` timed products Y = A * X after two warm-ups
+ * (HIP events on the stream) and reports the fastest.  d_Y is overwritten.
+ * tried_out (optional) receives every candidate with its time;
+ * *n_tried_io is its capacity on entry and the number of candidates on
+ * return.  Allocates and frees one plan at a time; synchronises the stream. */
+typedef struct mps_tune_result {
+    int cost;             /* merge items per partition                       */
+    int threads_per_wave; /* partitions per wavefront                        */
+    unsigned flags;       /* MPS_PLAN_* flags of the candidate                */
+    float ms;             /* average time of one product, all kernels         */
+} mps_tune_result;
+int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz, int K,
+                      int elem_bytes, const void *d_X, void *d_Y, int repeats, void *stream,
+                      mps_tune_result *best_out, mps_tune_result *tried_out, int *n_tried_io);
+
 /* ------------------------------------------------------------------------ */
 /* Device side: comparison kernels                                           */
 /* ------------------------------------------------------------------------ */

@@ -43,6 +43,11 @@ class PlanInfo(ctypes.Structure):
                 ("hot_waves", ctypes.c_int), ("hot_nnz", ctypes.c_longlong), ("hot_cost", ctypes.c_int), ("mark_shift", ctypes.c_int),
                 ("hot_mark_shift", ctypes.c_int)]
 
+class TuneResult(ctypes.Structure):
+    """struct mps_tune_result"""
+    _fields_ = [("cost", ctypes.c_int), ("threads_per_wave", ctypes.c_int), ("flags", ctypes.c_uint),
+                ("ms", ctypes.c_float)]
+
 c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp, _i, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64
 
@@ -65,6 +70,8 @@ PROTOTYPES = {
     "mps_graph_free": (None, [_vp]),
     "mps_fill_uniform_f32": (_i, [_vp, _sz, _u64, ctypes.c_float, ctypes.c_float]),
     "mps_fill_uniform_f16": (_i, [_vp, _sz, _u64, ctypes.c_float, ctypes.c_float]),
+    "mps_plan_autotune": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, ctypes.POINTER(TuneResult),
+                               ctypes.POINTER(TuneResult), c_int_p]),
     "mps_degree_values_f32": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "mps_degree_values_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "mps_csr_validate": (_i, [_vp, _vp, _i, _i, _i, _vp]),

@@ -42,7 +42,8 @@ int mergepath_main(int argc, char **argv)
         std::exit(-1);
     }
     const int dimension = std::atoi(pos[1].c_str());
-    int cost = parse_cost(pos[2]);
+    const bool tune = pos[2] == "auto";  // sweep cost / partitions per wavefront on this matrix first
+    int cost = tune ? 0 : parse_cost(pos[2]);
     int threads_per_wave = std::atoi(pos[3].c_str());
     const int repeats = std::atoi(pos[4].c_str());
     if (dimension < 1) die("dimension must be positive");
@@ -80,6 +81,22 @@ int mergepath_main(int argc, char **argv)
     mps_ok(mps_csr_validate(d_rp.p, d_ci.p, N, N, nnz, nullptr), "mps_csr_validate");
     // the reference's implicit weight deg(row) * deg(col) (:450,459), written out once
     if (opt.weights >= 0) mps_ok(Elem<T>::degree_values(d_rp.p, d_ci.p, N, nnz, opt.weights, d_val.p), "mps_degree_values");
+
+    if (tune) {
+        mps_tune_result best{}, tried[32];
+        int n_tried = 32;
+        mps_ok(mps_plan_autotune(d_rp.p, d_ci.p, d_val.p, N, nnz, K, (int)sizeof(T), d_X.p, d_Y.p, 5, nullptr, &best, tried,
+                                 &n_tried), "mps_plan_autotune");
+        for (int i = 0; i < n_tried && i < 32; ++i)
+            std::printf("tune: cost %4d, threads_per_wave %2d, flags %u: %9.2f us\n", tried[i].cost,
+                        tried[i].threads_per_wave, tried[i].flags, tried[i].ms * 1e3);
+        cost = best.cost;
+        threads_per_wave = best.threads_per_wave;
+        opt.tiling = (int)(best.flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING));
+        opt.hot = (int)(best.flags & (MPS_PLAN_NO_HOT | MPS_PLAN_FORCE_HOT));
+        opt.use_plan = true;
+        mps_ok(mps_num_partitions(N, nnz, cost, &P), "mps_num_partitions");
+    }
 
     // Everything that depends on the matrix alone is built once, outside the
     // repeat loop, as generate_mp_sched and its uploads are (:192-220): with a

@@ -948,4 +948,65 @@ int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsig
                              static_cast<hipStream_t>(stream));
 }
 
+int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz, int K,
+                      int elem_bytes, const void *d_X, void *d_Y, int repeats, void *stream, mps_tune_result *best_out,
+                      mps_tune_result *tried_out, int *n_tried_io)
+{
+    if (!best_out || !d_row_ptr || n_rows < 0 || nnz < 0 || K < 1) return MPS_ERR_INVALID_ARG;
+    if (tried_out && !n_tried_io) return MPS_ERR_INVALID_ARG;
+    if (n_rows > 0 && (!d_X || !d_Y)) return MPS_ERR_INVALID_ARG;
+    if (repeats < 1) repeats = 5;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int max_tpw = 0, dflt = 0;
+    int rc = mps_max_threads_per_wave(K, elem_bytes, &max_tpw);
+    if (rc != MPS_OK) return rc;
+    if ((rc = mps_default_cost(n_rows, nnz, K, elem_bytes, &dflt)) != MPS_OK) return rc;
+    // what the reference's authors swept by hand: cost and partitions per wave
+    // (src/MergePathSpMM.cu:121-122), plus this library's own switch
+    std::vector<mps_tune_result> cand;
+    const int costs[] = {16, 24, 32, 48, 64, 96, 128, 256};
+    for (int c : costs) cand.push_back({c, max_tpw, 0u, 0.f});
+    if (max_tpw >= 2) cand.push_back({dflt, max_tpw / 2, 0u, 0.f});
+    cand.push_back({dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f});
+    cand.push_back({dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f});
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    MPS_HIP_TRY(hipEventCreate(&e0));
+    hipError_t he = hipEventCreate(&e1);
+    if (he != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return MPS_ERR_HIP + (int)he;
+    }
+    mps_tune_result best{0, 0, 0u, 0.f};
+    int tried = 0;
+    const int cap = (tried_out && n_tried_io) ? *n_tried_io : 0;
+    rc = MPS_OK;
+    for (mps_tune_result &c : cand) {
+        mps_plan *pl = nullptr;
+        rc = mps_plan_create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, c.cost, c.threads_per_wave, c.flags, 0,
+                             stream, &pl);
+        if (rc != MPS_OK) break;
+        const unsigned all = MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE;
+        for (int i = 0; i < 2 && rc == MPS_OK; ++i) rc = mps_plan_spmm_phases(pl, d_X, d_Y, all, stream);
+        if (rc == MPS_OK) he = hipEventRecord(e0, st);
+        for (int i = 0; i < repeats && rc == MPS_OK; ++i) rc = mps_plan_spmm_phases(pl, d_X, d_Y, all, stream);
+        if (rc == MPS_OK && he == hipSuccess) he = hipEventRecord(e1, st);
+        if (rc == MPS_OK && he == hipSuccess) he = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (rc == MPS_OK && he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+        mps_plan_destroy(pl);
+        if (rc == MPS_OK && he != hipSuccess) rc = MPS_ERR_HIP + (int)he;
+        if (rc != MPS_OK) break;
+        c.ms = ms / (float)repeats;
+        if (best.cost == 0 || c.ms < best.ms) best = c;
+        if (tried < cap) tried_out[tried] = c;
+        ++tried;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != MPS_OK) return rc;
+    if (n_tried_io) *n_tried_io = tried;
+    *best_out = best;
+    return MPS_OK;
+}
+
 }  // extern "C"

@@ -95,6 +95,19 @@ def test_merge_path_driver_reference_setting(pkg, orc, graph_file, tmp_path):
     assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
 
 
+def test_merge_path_driver_auto_cost(pkg, orc, graph_file, tmp_path):
+    K = 16
+    rp, ci, val, X = inputs(pkg, graph_file, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    dump = tmp_path / "y.bin"
+    out = run("MergePathSpMM", graph_file, K, "auto", 0, 2, "--dump", dump)
+    assert out.count("tune: cost") == 11
+    j = last_json(out)
+    assert j["plan"] and j["cost"] in (16, 24, 32, 48, 64, 96, 128, 256)
+    Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
+    assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
+
+
 def test_merge_path_driver_errors(graph_file):
     out = run("MergePathSpMM", graph_file, 16, 32, expect=255)  # too few arguments -> usage, exit(-1)
     assert out.startswith("Usage: ./application <input_file> <dimension> <cost> <threads_per_wave> <repeat>")

@@ -347,3 +347,27 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
     sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz, cost=128)
     Y0 = pkg.spmm.spmm_merge_path(csr, d_X, sched)
     assert (Y - Y0).abs().max().item() <= 1e-3
+
+
+def test_autotune_picks_a_measured_candidate(pkg, orc, dev):
+    """mps_plan_autotune: every candidate is timed, the reported best is the
+    fastest of them, and a plan built from it gives the right product."""
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", seed=8)
+    n, K = rp.size - 1, 16
+    val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+    X = g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    best, tried = pkg.spmm.autotune(csr, d_X, repeats=3)
+    assert len(tried) == 11 and all(t["ms"] > 0 for t in tried)
+    assert {t["cost"] for t in tried} >= {16, 32, 64, 128, 256}
+    assert best["ms"] == min(t["ms"] for t in tried) and best in tried
+    c = pkg._cabi
+    tiling = "off" if best["flags"] & c.MPS_PLAN_NO_TILING else "auto"
+    hot = "off" if best["flags"] & c.MPS_PLAN_NO_HOT else "auto"
+    plan = pkg.spmm.Plan(csr, K, cost=best["cost"], threads_per_wave=best["threads_per_wave"], tiling=tiling, hot=hot)
+    Y = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
