@@ -128,6 +128,12 @@ int mps_csr_write(const char *path, int n_rows, const int *row_ptr, const int *c
 typedef struct mps_graph mps_graph;
 int mps_graph_generate(const char *spec, uint64_t seed, mps_graph **graph_out);
 int mps_graph_from_csr_file(const char *path, mps_graph **graph_out);
+/* Edge list -> graph, what the reference's converter does with scipy
+ * (scripts/npz_to_csr.py:14-20: coo_matrix((1, (src_li, dst_li))).tocsr(),
+ * which sorts the column ids of every row and merges repeated edges).  The
+ * matrix is square: n_rows = 1 + the largest id on either side (the kernels
+ * index X and the degrees by column id, src/MergePathSpMM.cu:459-460). */
+int mps_graph_from_edges(const int64_t *src, const int64_t *dst, int64_t n_edges, mps_graph **graph_out);
 int mps_graph_dims(const mps_graph *g, int *n_rows_out, int *nnz_out, int *max_degree_out);
 const int *mps_graph_row_ptr(const mps_graph *g); /* host, n_rows + 1 */
 const int *mps_graph_col_idx(const mps_graph *g); /* host, nnz        */

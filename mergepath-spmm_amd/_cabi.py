@@ -63,6 +63,7 @@ PROTOTYPES = {
     "mps_csr_read": (_i, [ctypes.c_char_p, _i, _i, _vp, _vp]),
     "mps_csr_write": (_i, [ctypes.c_char_p, _i, _vp, _vp]),
     "mps_graph_generate": (_i, [ctypes.c_char_p, _u64, ctypes.POINTER(_vp)]),
+    "mps_graph_from_edges": (_i, [_vp, _vp, ctypes.c_int64, ctypes.POINTER(_vp)]),
     "mps_graph_from_csr_file": (_i, [ctypes.c_char_p, ctypes.POINTER(_vp)]),
     "mps_graph_dims": (_i, [_vp, c_int_p, c_int_p, c_int_p]),
     "mps_graph_row_ptr": (_vp, [_vp]),

@@ -569,26 +569,92 @@ int64_t parse_line(const char *&p, const char *end, int *out, int64_t cap, int *
     return count;
 }
 
+// One line of the file, [b, e) without the newline, cut at commas into pieces
+// that are parsed side by side: a counting pass gives every piece its place in
+// the output, a second pass stores the cells.  Returns the number of cells, or
+// -1 on a malformed cell; at most cap values are stored.
+int64_t parse_line_parallel(const char *b, const char *e, int *out, int64_t cap)
+{
+    const int64_t bytes = e - b;
+    const int64_t piece = 1 << 20;
+    if (bytes <= 2 * piece || host_threads() <= 1) {
+        const char *p = b;
+        return parse_line(p, e, out, cap, nullptr);
+    }
+    const int64_t pieces = (bytes + piece - 1) / piece;
+    std::vector<const char *> cut((size_t)pieces + 1);
+    cut[0] = b;
+    cut[(size_t)pieces] = e;
+    for (int64_t i = 1; i < pieces; ++i) {  // a piece starts right behind a comma
+        const char *p = b + i * piece;
+        while (p < e && p[-1] != ',') ++p;
+        cut[(size_t)i] = p;
+    }
+    std::vector<int64_t> cells((size_t)pieces + 1, 0);
+    std::atomic<bool> bad(false);
+    parallel_for(pieces, 1, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) {
+            const char *p = cut[(size_t)i];
+            int64_t c = parse_line(p, cut[(size_t)i + 1], nullptr, 0, nullptr);
+            if (c < 0) bad = true;
+            cells[(size_t)i + 1] = c < 0 ? 0 : c;
+        }
+    });
+    if (bad) return -1;
+    for (int64_t i = 0; i < pieces; ++i) cells[(size_t)i + 1] += cells[(size_t)i];
+    if (out) {
+        parallel_for(pieces, 1, [&](int64_t lo, int64_t hi) {
+            for (int64_t i = lo; i < hi; ++i) {
+                const int64_t at = cells[(size_t)i];
+                if (at >= cap) continue;
+                const char *p = cut[(size_t)i];
+                parse_line(p, cut[(size_t)i + 1], out + at, cap - at, nullptr);
+            }
+        });
+    }
+    return cells[(size_t)pieces];
+}
+
 int parse_csr(const std::vector<char> &buf, int n_rows, int nnz, int *row_ptr, int *col_idx)
 {
-    const char *p = buf.data(), *end = buf.data() + buf.size();
-    int64_t c1 = parse_line(p, end, row_ptr, (int64_t)n_rows + 1, nullptr);
+    const char *b = buf.data(), *end = buf.data() + buf.size();
+    const char *nl = static_cast<const char *>(std::memchr(b, '\n', buf.size()));
+    const char *e1 = nl ? nl : end;
+    int64_t c1 = parse_line_parallel(b, e1, row_ptr, (int64_t)n_rows + 1);
     if (c1 != (int64_t)n_rows + 1) return MPS_ERR_FORMAT;
-    int64_t c2 = parse_line(p, end, col_idx, nnz, nullptr);
+    const char *b2 = nl ? nl + 1 : end;
+    const char *nl2 = b2 < end ? static_cast<const char *>(std::memchr(b2, '\n', (size_t)(end - b2))) : nullptr;
+    int64_t c2 = parse_line_parallel(b2, nl2 ? nl2 : end, col_idx, nnz);
     if (c2 != nnz) return MPS_ERR_FORMAT;
     if (row_ptr[0] != 0 || row_ptr[n_rows] != nnz) return MPS_ERR_FORMAT;
-    for (int i = 0; i < n_rows; ++i)
-        if (row_ptr[i + 1] < row_ptr[i]) return MPS_ERR_FORMAT;
-    for (int e = 0; e < nnz; ++e)
-        if (col_idx[e] < 0 || col_idx[e] >= n_rows) return MPS_ERR_FORMAT;
-    return MPS_OK;
+    std::atomic<bool> bad(false);
+    parallel_for(n_rows, 1 << 16, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i)
+            if (row_ptr[i + 1] < row_ptr[i]) bad = true;
+    });
+    parallel_for(nnz, 1 << 18, [&](int64_t lo, int64_t hi) {
+        for (int64_t k = lo; k < hi; ++k)
+            if (col_idx[k] < 0 || col_idx[k] >= n_rows) bad = true;
+    });
+    return bad ? MPS_ERR_FORMAT : MPS_OK;
 }
 
 int header_from_buf(const std::vector<char> &buf, int *n_rows, int *nnz)
 {
-    const char *p = buf.data(), *end = buf.data() + buf.size();
+    const char *b = buf.data(), *end = buf.data() + buf.size();
+    const char *nl = static_cast<const char *>(std::memchr(b, '\n', buf.size()));
+    const char *e1 = nl ? nl : end;
+    int64_t cells = parse_line_parallel(b, e1, nullptr, 0);
+    // the last cell of the line is nnz (src/MergePathSpMM.cu:131-137)
     int last = 0;
-    int64_t cells = parse_line(p, end, nullptr, 0, &last);
+    {
+        const char *q = e1;
+        while (q > b && (q[-1] == ',' || q[-1] == ' ' || q[-1] == '\t' || q[-1] == '\r')) --q;
+        const char *t = q;
+        while (t > b && t[-1] != ',') --t;
+        const char *p = t;
+        if (cells >= 1 && parse_line(p, q, nullptr, 0, &last) != 1) return MPS_ERR_FORMAT;
+    }
     if (cells < 1 || cells > 0x7fffffffLL || last < 0) return MPS_ERR_FORMAT;
     if ((int64_t)cells + last > 0x7fffffffLL) return MPS_ERR_UNSUPPORTED;
     *n_rows = (int)cells - 1;
@@ -758,6 +824,56 @@ int mps_graph_generate(const char *spec, uint64_t seed, mps_graph **graph_out)
     if (rc != MPS_OK) {
         delete g;
         return rc;
+    }
+    finish_graph(g);
+    *graph_out = g;
+    return MPS_OK;
+}
+
+int mps_graph_from_edges(const int64_t *src, const int64_t *dst, int64_t n_edges, mps_graph **graph_out)
+{
+    if (!graph_out || n_edges < 0 || (n_edges > 0 && (!src || !dst))) return MPS_ERR_INVALID_ARG;
+    *graph_out = nullptr;
+    int64_t top = -1;
+    for (int64_t e = 0; e < n_edges; ++e) {
+        if (src[e] < 0 || dst[e] < 0) return MPS_ERR_FORMAT;
+        top = std::max(top, std::max(src[e], dst[e]));
+    }
+    const int64_t n64 = top + 1;
+    if (n64 + 1 + n_edges > 0x7fffffffLL) return MPS_ERR_UNSUPPORTED;
+    const int n = (int)n64;
+    mps_graph *g = new (std::nothrow) mps_graph;
+    if (!g) return MPS_ERR_INVALID_ARG;
+    try {
+        // counting sort by row, then every row sorted and stripped of repeats
+        std::vector<int64_t> start((size_t)n + 1, 0);
+        for (int64_t e = 0; e < n_edges; ++e) ++start[(size_t)src[e] + 1];
+        for (int i = 0; i < n; ++i) start[(size_t)i + 1] += start[(size_t)i];
+        std::vector<int> cols((size_t)n_edges);
+        {
+            std::vector<int64_t> at(start.begin(), start.end() - 1);
+            for (int64_t e = 0; e < n_edges; ++e) cols[(size_t)at[(size_t)src[e]]++] = (int)dst[e];
+        }
+        std::vector<int> kept((size_t)n, 0);
+        parallel_for(n, 1 << 12, [&](int64_t lo, int64_t hi) {
+            for (int64_t r = lo; r < hi; ++r) {
+                int *b = cols.data() + start[(size_t)r], *e = cols.data() + start[(size_t)r + 1];
+                std::sort(b, e);
+                kept[(size_t)r] = (int)(std::unique(b, e) - b);
+            }
+        });
+        g->row_ptr.resize((size_t)n + 1);
+        g->row_ptr[0] = 0;
+        for (int r = 0; r < n; ++r) g->row_ptr[(size_t)r + 1] = g->row_ptr[(size_t)r] + kept[(size_t)r];
+        g->col_idx.resize((size_t)g->row_ptr[(size_t)n]);
+        parallel_for(n, 1 << 12, [&](int64_t lo, int64_t hi) {
+            for (int64_t r = lo; r < hi; ++r)
+                std::copy(cols.data() + start[(size_t)r], cols.data() + start[(size_t)r] + kept[(size_t)r],
+                          g->col_idx.data() + g->row_ptr[(size_t)r]);
+        });
+    } catch (const std::bad_alloc &) {
+        delete g;
+        return MPS_ERR_UNSUPPORTED;
     }
     finish_graph(g);
     *graph_out = g;

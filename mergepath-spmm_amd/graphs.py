@@ -40,6 +40,19 @@ def generate(spec, seed=1):
     return _take(h)
 
 
+def from_edges(src, dst):
+    """Edge list -> (row_ptr, col_idx, max_degree): rows sorted, repeated edges
+    merged, square (what scripts/npz_to_csr.py:14-20 gets from scipy)."""
+    s = np.ascontiguousarray(src, dtype=np.int64)
+    d = np.ascontiguousarray(dst, dtype=np.int64)
+    if s.size != d.size:
+        raise ValueError("src and dst differ in length")
+    h = ctypes.c_void_p()
+    check(_cabi.lib().mps_graph_from_edges(s.ctypes.data, d.ctypes.data, ctypes.c_int64(s.size), ctypes.byref(h)),
+          "mps_graph_from_edges")
+    return _take(h)
+
+
 def read_csr(path):
     """Two-line .csr text -> (row_ptr, col_idx, max_degree)."""
     h = ctypes.c_void_p()

@@ -197,3 +197,90 @@ def test_device_entry_points_reject_bad_arguments_without_a_gpu(pkg):
     mp = ctypes.c_int()
     assert L.mps_nzsplit_max_parts(10, 100, 8, ctypes.byref(mp)) == 0 and mp.value == 22
     assert L.mps_nzsplit_max_parts(10, 100, 0, ctypes.byref(mp)) == c.MPS_ERR_INVALID_ARG
+
+
+def test_large_csr_file_is_parsed_in_pieces(pkg, tmp_path):
+    """Files beyond a few MB are cut at commas and parsed by several threads:
+    same arrays as written, whatever the thread count, and a damaged cell deep
+    inside is still an error."""
+    g = pkg.graphs
+    rp, ci, _ = g.generate("rmat:scale=16,ef=16,a=0.57,b=0.19,c=0.19", seed=2)
+    path = tmp_path / "big.csr"
+    g.write_csr(path, rp, ci)
+    assert os.path.getsize(path) > 4 << 20
+    assert g.read_csr_header(path) == (rp.size - 1, ci.size)
+    rp2, ci2, _ = g.read_csr(path)
+    assert np.array_equal(rp, rp2) and np.array_equal(ci, ci2)
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "import __graft_entry__ as e, hashlib\n"
+            "rp, ci, _ = e.load_package().graphs.read_csr(%r)\n"
+            "print(hashlib.sha256(rp.tobytes() + ci.tobytes()).hexdigest())\n" % (ROOT, str(path)))
+    import hashlib
+    want = hashlib.sha256(rp.tobytes() + ci.tobytes()).hexdigest()
+    for threads in ("1", "3", "7"):
+        env = dict(os.environ, MPS_HOST_THREADS=threads)
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True)
+        assert out.stdout.strip() == want
+    text = bytearray(path.read_bytes())
+    pos = len(text) - (3 << 20)
+    while text[pos] != ord(","):
+        pos += 1
+    text[pos + 1] = ord("x")  # a cell of the second line, deep inside a later piece
+    bad = tmp_path / "bad.csr"
+    bad.write_bytes(bytes(text))
+    with pytest.raises(pkg.MpsError) as e:
+        g.read_csr(bad)
+    assert e.value.status == pkg._cabi.MPS_ERR_FORMAT
+    # no trailing comma and no newline at the end (scripts/npz_to_csr.py:27-28 writes one, fetch_dataset.py too)
+    short = tmp_path / "short.csr"
+    short.write_bytes(path.read_bytes().rstrip(b","))
+    rp3, ci3, _ = g.read_csr(short)
+    assert np.array_equal(rp, rp3) and np.array_equal(ci, ci3)
+
+
+def reference_conversion(src, dst):
+    """What scripts/npz_to_csr.py:17-19 computes: coo_matrix((1, (src, dst))).tocsr(),
+    made square (the kernels index rows by column id)."""
+    from scipy.sparse import coo_matrix
+    n = int(max(src.max(), dst.max())) + 1 if src.size else 0
+    m = coo_matrix((np.ones(src.size), (src, dst)), shape=(n, n)).tocsr()
+    m.sum_duplicates()
+    m.sort_indices()
+    return m.indptr.astype(np.int32), m.indices.astype(np.int32)
+
+
+def test_graph_from_edges_matches_scipy(pkg):
+    rng = np.random.default_rng(4)
+    src = rng.integers(0, 3000, 60000)
+    dst = rng.integers(0, 2500, 60000)
+    src[:500], dst[:500] = src[500:1000], dst[500:1000]  # repeated edges
+    rp, ci, maxdeg = pkg.graphs.from_edges(src, dst)
+    want_rp, want_ci = reference_conversion(src, dst)
+    assert np.array_equal(rp, want_rp) and np.array_equal(ci, want_ci) and maxdeg == np.diff(want_rp).max()
+    rp, ci, _ = pkg.graphs.from_edges(np.array([], dtype=np.int64), np.array([], dtype=np.int64))
+    assert rp.tolist() == [0] and ci.size == 0
+    with pytest.raises(pkg.MpsError):
+        pkg.graphs.from_edges(np.array([1, -2]), np.array([0, 0]))
+
+
+@pytest.mark.parametrize("compressed,dtype", [(False, np.int64), (True, np.int64), (False, np.int32)])
+def test_npz_to_csr_tool(pkg, tmp_path, compressed, dtype):
+    """The native converter against the reference script's recipe
+    (scripts/npz_to_csr.py: src_li / dst_li -> coo -> csr -> two comma lines)."""
+    exe = os.path.join(ROOT, "mergepath-spmm_amd", "csrc", "npz_to_csr")
+    assert os.path.exists(exe), "npz_to_csr is not built"
+    rng = np.random.default_rng(7)
+    src = rng.integers(0, 5000, 200000).astype(dtype)
+    dst = rng.integers(0, 5000, 200000).astype(dtype)
+    npz = tmp_path / "g.npz"
+    (np.savez_compressed if compressed else np.savez)(npz, src_li=src, dst_li=dst, num_nodes=np.int64(5000))
+    out = tmp_path / "g.csr"
+    p = subprocess.run([exe, "--graph", str(npz), "--output", str(out)], capture_output=True, text=True, timeout=60)
+    assert p.returncode == 0, p.stderr
+    want_rp, want_ci = reference_conversion(src, dst)
+    want = ",".join(map(str, want_rp)) + ",\n" + ",".join(map(str, want_ci)) + ","
+    assert out.read_text() == want  # byte for byte what the script's write loop produces
+    rp, ci, _ = pkg.graphs.read_csr(out)
+    assert np.array_equal(rp, want_rp) and np.array_equal(ci, want_ci)
+    p = subprocess.run([exe, "--graph", str(out), "--output", str(tmp_path / "x.csr")], capture_output=True, text=True)
+    assert p.returncode == 1 and "npz_to_csr:" in p.stderr
