@@ -171,3 +171,28 @@ def test_nz_splitting_driver(pkg, orc, graph_file, tmp_path):
     assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
     assert last_json(out)["num_parts"] == orc.calculate_part_num(32, rp)
     assert run("nz_splitting", graph_file, expect=255).startswith("Usage: ./application <input_file> <dimension> <part_size> <repeat>")
+
+
+@pytest.mark.parametrize("prog,alg", [("rocsparse_spmm_row", "default"), ("rocsparse_spmm_row", "row_split"),
+                                      ("rocsparse_spmm_row", "merge_path"), ("rocsparse_spmm_row", "nnz_split"),
+                                      ("rocsparse_spmm_col", "default")])
+def test_rocsparse_comparison_drivers(pkg, orc, graph_file, tmp_path, prog, alg):
+    """Counterparts of src/cusparse_spmm_{row,col}.cu on rocSPARSE: same inputs as
+    the merge-path driver, and an independent library agrees with the oracle (and
+    so with MergePathSpMM) on the result."""
+    K = 16
+    rp, ci, val, X = inputs(pkg, graph_file, K)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    dump = tmp_path / "y.bin"
+    out = run(prog, graph_file, K, 3, "--alg", alg, "--dump", dump)
+    assert out.splitlines()[0] == "Total number of rows: %d and non-zeros: %d" % (rp.size - 1, ci.size)
+    Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)
+    assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
+    j = last_json(out)
+    assert j["kernel"] == prog and j["alg"] == alg and j["order"] == ("col" if prog.endswith("col") else "row")
+    ours = tmp_path / "ours.bin"
+    run("MergePathSpMM", graph_file, K, "default", 0, 1, "--dump", ours)
+    Z = np.fromfile(ours, dtype=np.float32).reshape(-1, K)
+    assert (np.abs(Y - Z) <= 2e-5 * scale + 2e-6).all()
+    out = run(prog, graph_file, K, expect=255)  # too few arguments: usage, exit(-1), as the reference's programs
+    assert out.startswith("Usage: ./application <input_file> <DIM> <repeat>")
