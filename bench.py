@@ -70,6 +70,8 @@ def main():
     ap.add_argument("--slab-bytes", type=int, default=0, help="slab size for tiling (0 = library default)")
     ap.add_argument("--tpw", type=int, default=0, help="partitions per wavefront (0 = full wavefront)")
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--graph", action="store_true",
+                    help="capture one step in a HIP graph and time replays (what a launch-bound caller would do)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the result check")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -124,13 +126,28 @@ def main():
 
     for _ in range(args.warmup):
         step()
+    timed_step = step
+    if args.graph:
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        hip_graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(hip_graph):
+            step()
+        timed_step = hip_graph.replay
+        for _ in range(args.warmup):
+            timed_step()
     # ---- timed region: exactly `steps` steps, inputs already in HBM ----------
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     w0 = time.perf_counter()
     e0.record()
     for _ in range(args.steps):
-        step()
+        timed_step()
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - w0) * 1e3
@@ -182,6 +199,7 @@ def main():
         "vs_baseline": None,
         "dtype": dt,
         "data": "synthetic (seeded generator, values U[0,1), features U[-1,1))",
+        "launch": "one HIP graph replay per step" if args.graph else "kernel launches per step",
         "config": {"workload": args.workload, "spec": spec, "n_rows": int(n), "nnz": int(nnz), "K": K,
                    "max_row_degree": int(max_deg), "cost": cost, "partitions": P,
                    "threads_per_wave": args.tpw or g.max_threads_per_wave(K, eb), "seed": args.seed,

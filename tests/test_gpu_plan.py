@@ -371,3 +371,47 @@ def test_autotune_picks_a_measured_candidate(pkg, orc, dev):
     torch.cuda.synchronize()
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+
+
+def test_plan_spmm_in_a_hip_graph(pkg, orc, dev):
+    """mps_plan_spmm_* launches kernels only (no allocation, no memset, no
+    synchronisation), so a caller can capture it: every replay, with other work
+    and synchronisations between replays, gives the eager result bit for bit."""
+    g = pkg.graphs
+    K = 16
+    for spec, kwargs in (("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", dict(tiling="force", slab_bytes=4096 * K * 4)),
+                         ("er:n=4096,deg=8", dict())):
+        rp, ci, _ = g.generate(spec, seed=8)
+        n = rp.size - 1
+        val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
+        csr = make_csr(pkg, dev, rp, ci, val)
+        plan = pkg.spmm.Plan(csr, K, **kwargs)
+        X = torch.from_numpy(g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)).to(dev)
+        Y = torch.full_like(X, float("nan"))
+        eager = plan.spmm(X).clone()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            plan.spmm(X, out=Y)  # warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            plan.spmm(X, out=Y)
+        for it in range(4):
+            Y.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(Y, eager), "replay %d" % it
+            X2 = X * (it + 2.0)  # eager work and a changed input between replays
+            want2 = plan.spmm(X2).clone()
+            torch.cuda.synchronize()
+            X.copy_(X2)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(Y, want2), "replay with new input %d" % it
+            eager = want2
+        ref, scale = orc.spmm_f64(rp, ci, val, X.cpu().numpy(), want_abs=True)
+        check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+        plan.close()
