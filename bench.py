@@ -61,6 +61,7 @@ def main():
     ap.add_argument("--workload", default="chunglu_233k_f32_k16", choices=sorted(WORKLOADS))
     ap.add_argument("--spec", default="", help="generator spec overriding the workload's graph (experiments)")
     ap.add_argument("--k", type=int, default=0, help="feature width overriding the workload's K (experiments)")
+    ap.add_argument("--dtype", default="", choices=["", "f32", "f16"], help="element type overriding the workload's (experiments)")
     ap.add_argument("--cost", type=int, default=0, help="merge items per partition (0 = library default)")
     ap.add_argument("--mode", default="auto", choices=["auto", "plain", "untiled", "tiled"],
                     help="plain = kernels on the CSR arrays as given, no plan; auto / untiled / tiled = with a plan "
@@ -90,6 +91,8 @@ def main():
         spec, args.workload = args.spec, "custom"
     if args.k:
         K, args.workload = args.k, "custom"
+    if args.dtype:
+        dt, args.workload = args.dtype, "custom"
     f16 = dt == "f16"
     eb = 2 if f16 else 4
 

@@ -281,9 +281,10 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     there, the remaining columns of the slab form the "cold" segment,
  *     gathered through L2.  Segments are ordered hot first (virtual row
  *     v = seg * n_rows + r, 2 * num_slabs segments), each is partitioned on
- *     its own, and the plan runs two launches of the same kernel.  Used when
- *     a row of X has at most 64 bytes (wider rows are cheaper through L2) and
- *     the hot columns hold at least 15 % of the nonzeros.
+ *     its own, and the plan runs two launches of the same kernel.  Used for
+ *     fp32 when a row of X has at most 64 bytes (K = 16; wider rows are
+ *     cheaper through L2, fp16 gains nothing) and the hot columns hold at
+ *     least 15 % of the nonzeros; MPS_PLAN_FORCE_HOT lifts these limits.
  *   - The merge-path partition (mps_num_partitions, mps_partition) of the
  *     virtual rows for the given cost: one split of all of them, or, with hot
  *     columns, one split per segment (padded to whole workgroups).
@@ -312,7 +313,7 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_NO_TILING 1u    /* never tile                                  */
 #define MPS_PLAN_FORCE_TILING 2u /* tile with slab_bytes slabs whatever the shape */
 #define MPS_PLAN_NO_HOT 4u       /* never keep hot columns' rows of X in LDS     */
-#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes */
+#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros, rows of X are wider than 64 bytes or fp16 */
 
 typedef struct mps_plan_info {
     int n_rows, nnz, K, elem_bytes, cost, threads_per_wave;

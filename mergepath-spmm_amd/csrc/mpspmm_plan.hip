@@ -413,7 +413,10 @@ int choose_hot_rows(int K, int eb, const SpmmShape &sh, bool force)
     // (0.58 against 0.66 ms at K = 16 fp32); with 128-byte rows and more the L2 path
     // moves twice the bytes per request at no extra cost while the LDS table holds
     // half the rows, and the hot launch loses (1.16 against 0.99 ms at K = 32).
-    if (!force && (size_t)K * eb > 64) return 0;
+    // fp16 rows of 64 bytes (K = 32): 8 conversions and 8 multiply-adds per lane and nonzero make the
+    // hot launch ALU-bound; it runs as fast as the L2 path and costs a second set of partial rows
+    // (0.672 ms either way), so it is not used.
+    if (!force && ((size_t)K * eb > 64 || eb != 4)) return 0;
     const size_t budget = 160 * 1024 - hot_static_lds(sh.ls.vec) - 2048;
     size_t rows = budget / ((size_t)K * eb);
     rows = rows / 64 * 64;
