@@ -72,8 +72,9 @@ int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out);
  * no default; src/MergePathSpMM.cu:121 takes it from argv).  Measured on
  * MI355X: 32 merge items per partition, 64 from 2^25 items and 128 from 2^27
  * items on; and never fewer than about 512 items per wavefront, i.e. at least
- * min(128, 512 / partitions per wavefront) for the given K and element size
- * (32 at K = 16 fp32, 128 from K = 64 fp32 on). */
+ * 512 / partitions per wavefront for the given K and element size (32 at
+ * K = 16 fp32, 128 at K = 64, 512 at K = 256: the carry-out records of a
+ * wavefront are 8 K bytes, so wide rows want few of them). */
 int mps_default_cost(int n_rows, int nnz, int K, int elem_bytes, int *cost_out);
 
 /* Merge items per partition, src/MergePathSpMM.cu:327-328:

@@ -732,7 +732,7 @@ int mps_default_cost(int n_rows, int nnz, int K, int elem_bytes, int *cost_out)
     const int by_size = total >= (1 << 27) ? 128 : total >= (1 << 25) ? 64 : 32;
     // a wavefront should have some 512 merge items whatever number of partitions it holds
     const int groups = mps_make_lane_shape(K, elem_bytes).groups;
-    const int by_width = 512 / groups < 128 ? 512 / groups : 128;
+    const int by_width = 512 / groups;  // 32 (16 groups) .. 512 (one group)
     *cost_out = by_size > by_width ? by_size : by_width;
     return MPS_OK;
 }

@@ -55,7 +55,8 @@ def test_num_partitions_matches_oracle(pkg, orc):
     assert dc(232965, 114604189) == 64 and dc(416349, 2081148) == 32 and dc(4096, 32731) == 32
     assert dc(1 << 22, 140000000) == 128 and dc(1 << 20, 16086273) == 32
     # wide rows: fewer partitions per wavefront, so more items each
-    assert dc(1 << 20, 16086273, 64, 4) == 128 and dc(1 << 20, 16086273, 64, 2) == 64 and dc(4096, 32731, 256, 4) == 128
+    assert dc(1 << 20, 16086273, 64, 4) == 128 and dc(1 << 20, 16086273, 64, 2) == 64 and dc(4096, 32731, 256, 4) == 512
+    assert dc(1 << 20, 16086273, 128, 4) == 256
 
 
 def test_max_threads_per_wave(pkg):
