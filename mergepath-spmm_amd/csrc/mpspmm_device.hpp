@@ -104,9 +104,11 @@ struct XOps<half_t, 1> {
 };
 
 // VEC accumulators -> VEC adjacent outputs (fp32 or fp16), one vector store
-// where the width allows.  Non-temporal: output rows are written once and not
-// read again by the kernel, so they should not displace X in L2.
-template <int VEC>
+// where the width allows.  Non-temporal (NT): output rows are written once and
+// not read again by the kernel, so they should not displace X in L2.  The hot
+// launch of a plan has no X in L2 to protect and waits less on plain stores
+// (a load that follows a store in program order also waits for the store).
+template <int VEC, bool NT = true>
 __device__ __forceinline__ void store_acc(float *p, const float (&acc)[VEC])
 {
     typedef float f4_t __attribute__((ext_vector_type(4)));
@@ -114,14 +116,15 @@ __device__ __forceinline__ void store_acc(float *p, const float (&acc)[VEC])
 #pragma unroll
         for (int i = 0; i < VEC; i += 4) {
             f4_t v = {acc[i], acc[i + 1], acc[i + 2], acc[i + 3]};
-            __builtin_nontemporal_store(v, reinterpret_cast<f4_t *>(p + i));
+            if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<f4_t *>(p + i));
+            else *reinterpret_cast<f4_t *>(p + i) = v;
         }
     } else {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) __builtin_nontemporal_store(acc[i], p + i);
     }
 }
-template <int VEC>
+template <int VEC, bool NT = true>
 __device__ __forceinline__ void store_acc(half_t *p, const float (&acc)[VEC])
 {
     if constexpr (VEC == 8) {
@@ -356,7 +359,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) MP
 #pragma unroll
             for (int i = 0; i < VEC; ++i) my_head[i] = acc[i];
         } else if (col_ok) {
-            store_acc<VEC>(Y + (size_t)row * K + kcol, acc);
+            store_acc<VEC, !HOT>(Y + (size_t)row * K + kcol, acc);
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
