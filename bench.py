@@ -30,8 +30,8 @@ PEAK_HBM_GBS = 8000.0
 # probe gives, profiles/hbm_copy_probe_fetch_write_calibration.md).  Keyed by (workload, layout); other
 # configurations report null.  Key: (workload, layout, column slabs, cost, hot columns per slab).
 MEASURED_TRAFFIC = {
-    # cold + hot launch of the main kernel: FETCH_SIZE 380,635 + 181,210 KiB raw, WRITE_SIZE 82,080 + 82,181 KiB
-    ("chunglu_233k_f32_k16", "plan", 5, 64, 1728): int((380635 + 181210) * 1024 * 2.0 + (82080 + 82181) * 1024 * 1.0),
+    # cold + hot launch of the main kernel: FETCH_SIZE 380,316 + 181,283 KiB raw, WRITE_SIZE 82,068 + 77,505 KiB
+    ("chunglu_233k_f32_k16", "plan", 5, 64, 1728): int((380316 + 181283) * 1024 * 2.0 + (82068 + 77505) * 1024 * 1.0),
 }
 
 WORKLOADS = {
