@@ -7,7 +7,7 @@ loop, as the reference builds it once on the host
 (src/MergePathSpMM.cu:192, repeat loop :231-243).
 
 Prints ONE JSON line:  metric/value = GFLOP/s (2*nnz*K/t) of the default
-workload (BASELINE config 2: Chung-Lu power-law graph, fp32, K=16), plus
+workload (benchmark configuration 2: Chung-Lu power-law graph, fp32, K=16), plus
   roofline      algorithmic bytes / average duration of the main kernel,
                 against the 8 TB/s HBM peak
   cpu_baseline  the oracle's multithreaded fp32 CSR SpMM on the host cores

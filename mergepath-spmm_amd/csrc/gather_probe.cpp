@@ -6,8 +6,8 @@
 // or far beyond it, alone or beside the sparse stream (8 bytes per nonzero,
 // one coalesced non-temporal 1 KiB load per wavefront and 8 rows), and the
 // same rows served from an LDS table by 1024-thread workgroups.  Every line
-// ends with the time the rate would need for 114.6 M nonzeros (BASELINE
-// config 2), to set beside the measured kernel times.
+// ends with the time the rate would need for 114.6 M nonzeros (the benchmark's
+// 232,965-row power-law graph), to set beside the measured kernel times.
 #include <hip/hip_runtime.h>
 
 #include <cstdio>

@@ -1,4 +1,4 @@
-"""BASELINE workloads at full size on the GPU: against the oracle's fp64 row
+"""The five benchmark workloads at full size on the GPU: against the oracle's fp64 row
 loop (OpenMP, seconds on the host) and through size-independent properties
 (all-ones features give row sums; linearity; plan and CSR entry points agree)."""
 import numpy as np

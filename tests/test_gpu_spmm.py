@@ -23,7 +23,7 @@ def run_f32(pkg, dev, rp, ci, val, X, cost=None, P=None, tpw=0, poison=True):
 
 
 def test_er_plumbing_config(pkg, orc, dev):
-    # BASELINE config 1: ER N=4096 deg 8, val U[0,1), X 4096x16 U[-1,1)
+    # benchmark configuration 1: ER N=4096 deg 8, val U[0,1), X 4096x16 U[-1,1)
     g = pkg.graphs
     rp, ci, _ = g.generate(g.CONFIG_SPECS["er_4096"], seed=1)
     n, K = rp.size - 1, 16

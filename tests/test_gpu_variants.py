@@ -35,7 +35,7 @@ def test_fp16_against_oracle(pkg, orc, dev, K):
 
 
 def test_fp16_rmat_reduced(pkg, orc, dev):
-    # BASELINE config 5 at reduced scale: R-MAT, half values / features, K = 64
+    # benchmark configuration 5 at reduced scale: R-MAT, half values / features, K = 64
     g = pkg.graphs
     rp, ci, _ = g.generate("rmat:scale=17,ef=16,a=0.57,b=0.19,c=0.19", seed=1)
     n, K = rp.size - 1, 64
