@@ -11,8 +11,11 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <exception>
 #include <map>
+#include <mutex>
 #include <string>
+#include <system_error>
 #include <thread>
 #include <vector>
 
@@ -49,19 +52,34 @@ void parallel_for(int64_t n, int64_t grain, F &&fn)
         return;
     }
     std::atomic<int64_t> next(0);
+    // an exception in a chunk (out of memory, in practice) stops the hand-out of
+    // further chunks and is thrown again on the calling thread after the join
+    std::exception_ptr failure;
+    std::mutex failure_lock;
     auto worker = [&] {
-        for (;;) {
-            int64_t c = next.fetch_add(1, std::memory_order_relaxed);
-            if (c >= chunks) break;
-            int64_t lo = c * grain, hi = std::min(n, lo + grain);
-            fn(lo, hi);
+        try {
+            for (;;) {
+                int64_t c = next.fetch_add(1, std::memory_order_relaxed);
+                if (c >= chunks) break;
+                int64_t lo = c * grain, hi = std::min(n, lo + grain);
+                fn(lo, hi);
+            }
+        } catch (...) {
+            next.store(chunks, std::memory_order_relaxed);
+            std::lock_guard<std::mutex> hold(failure_lock);
+            if (!failure) failure = std::current_exception();
         }
     };
     std::vector<std::thread> th;
     th.reserve(nt - 1);
-    for (int t = 1; t < nt; ++t) th.emplace_back(worker);
+    try {
+        for (int t = 1; t < nt; ++t) th.emplace_back(worker);
+    } catch (const std::system_error &) {
+        // fewer threads than asked for: the ones that started and this one share the chunks
+    }
     worker();
     for (auto &t : th) t.join();
+    if (failure) std::rethrow_exception(failure);
 }
 
 // ---------------------------------------------------------------------------
@@ -756,17 +774,25 @@ int mps_max_threads_per_wave(int K, int elem_bytes, int *tpw_out)
 int mps_csr_read_header(const char *path, int *n_rows_out, int *nnz_out)
 {
     if (!path || !n_rows_out || !nnz_out) return MPS_ERR_INVALID_ARG;
-    std::vector<char> buf;
-    if (!read_whole_file(path, buf)) return MPS_ERR_IO;
-    return header_from_buf(buf, n_rows_out, nnz_out);
+    try {
+        std::vector<char> buf;
+        if (!read_whole_file(path, buf)) return MPS_ERR_IO;
+        return header_from_buf(buf, n_rows_out, nnz_out);
+    } catch (const std::bad_alloc &) {
+        return MPS_ERR_UNSUPPORTED;
+    }
 }
 
 int mps_csr_read(const char *path, int n_rows, int nnz, int *row_ptr, int *col_idx)
 {
     if (!path || !row_ptr || (!col_idx && nnz > 0) || n_rows < 0 || nnz < 0) return MPS_ERR_INVALID_ARG;
-    std::vector<char> buf;
-    if (!read_whole_file(path, buf)) return MPS_ERR_IO;
-    return parse_csr(buf, n_rows, nnz, row_ptr, col_idx);
+    try {
+        std::vector<char> buf;
+        if (!read_whole_file(path, buf)) return MPS_ERR_IO;
+        return parse_csr(buf, n_rows, nnz, row_ptr, col_idx);
+    } catch (const std::bad_alloc &) {
+        return MPS_ERR_UNSUPPORTED;
+    }
 }
 
 int mps_csr_write(const char *path, int n_rows, const int *row_ptr, const int *col_idx)
@@ -810,7 +836,7 @@ int mps_graph_generate(const char *spec, uint64_t seed, mps_graph **graph_out)
     Spec sp;
     if (!parse_spec(spec, sp)) return MPS_ERR_FORMAT;
     mps_graph *g = new (std::nothrow) mps_graph;
-    if (!g) return MPS_ERR_INVALID_ARG;
+    if (!g) return MPS_ERR_UNSUPPORTED;
     int rc;
     try {
         if (sp.name == "er") rc = gen_er(sp, seed, g);
@@ -843,7 +869,7 @@ int mps_graph_from_edges(const int64_t *src, const int64_t *dst, int64_t n_edges
     if (n64 + 1 + n_edges > 0x7fffffffLL) return MPS_ERR_UNSUPPORTED;
     const int n = (int)n64;
     mps_graph *g = new (std::nothrow) mps_graph;
-    if (!g) return MPS_ERR_INVALID_ARG;
+    if (!g) return MPS_ERR_UNSUPPORTED;
     try {
         // counting sort by row, then every row sorted and stripped of repeats
         std::vector<int64_t> start((size_t)n + 1, 0);
@@ -884,24 +910,24 @@ int mps_graph_from_csr_file(const char *path, mps_graph **graph_out)
 {
     if (!path || !graph_out) return MPS_ERR_INVALID_ARG;
     *graph_out = nullptr;
-    std::vector<char> buf;
-    if (!read_whole_file(path, buf)) return MPS_ERR_IO;
-    int n = 0, nnz = 0;
-    int rc = header_from_buf(buf, &n, &nnz);
-    if (rc != MPS_OK) return rc;
-    mps_graph *g = new (std::nothrow) mps_graph;
-    if (!g) return MPS_ERR_INVALID_ARG;
+    mps_graph *g = nullptr;
     try {
+        std::vector<char> buf;
+        if (!read_whole_file(path, buf)) return MPS_ERR_IO;
+        int n = 0, nnz = 0;
+        int rc = header_from_buf(buf, &n, &nnz);
+        if (rc != MPS_OK) return rc;
+        g = new mps_graph;
         g->row_ptr.resize((size_t)n + 1);
         g->col_idx.resize((size_t)nnz);
+        rc = parse_csr(buf, n, nnz, g->row_ptr.data(), g->col_idx.data());
+        if (rc != MPS_OK) {
+            delete g;
+            return rc;
+        }
     } catch (const std::bad_alloc &) {
         delete g;
         return MPS_ERR_UNSUPPORTED;
-    }
-    rc = parse_csr(buf, n, nnz, g->row_ptr.data(), g->col_idx.data());
-    if (rc != MPS_OK) {
-        delete g;
-        return rc;
     }
     finish_graph(g);
     *graph_out = g;

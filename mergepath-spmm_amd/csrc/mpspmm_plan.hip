@@ -17,6 +17,7 @@
 #include "mpspmm_device.hpp"
 
 #include <algorithm>
+#include <new>
 #include <vector>
 
 struct mps_plan {
@@ -437,6 +438,7 @@ struct BuildTmp {
         (void)hipFree(seg);
         first = col_v = perm = sums = deg = hot_slot = seg = nullptr;
     }
+    ~BuildTmp() { drop(); }
 };
 
 template <typename T>
@@ -854,13 +856,18 @@ int mps_plan_create(const int *d_row_ptr, const int *d_col_idx, const void *d_va
     if (nnz > 0 && (!d_col_idx || !d_val)) return MPS_ERR_INVALID_ARG;
     if ((long long)n_rows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
     mps_plan *pl = new (std::nothrow) mps_plan;
-    if (!pl) return MPS_ERR_INVALID_ARG;
+    if (!pl) return MPS_ERR_UNSUPPORTED;
     pl->n_rows = n_rows;
     pl->nnz = nnz;
     pl->K = K;
     pl->elem_bytes = elem_bytes;
     pl->cost = cost;
-    int rc = plan_build(pl, d_row_ptr, d_col_idx, d_val, flags, slab_bytes, tpw, static_cast<hipStream_t>(stream));
+    int rc;
+    try {
+        rc = plan_build(pl, d_row_ptr, d_col_idx, d_val, flags, slab_bytes, tpw, static_cast<hipStream_t>(stream));
+    } catch (const std::bad_alloc &) {  // host-side tables of the build
+        rc = MPS_ERR_UNSUPPORTED;
+    }
     if (rc != MPS_OK) {
         plan_free(pl);
         return rc;
@@ -966,12 +973,13 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     if ((rc = mps_default_cost(n_rows, nnz, K, elem_bytes, &dflt)) != MPS_OK) return rc;
     // what the reference's authors swept by hand: cost and partitions per wave
     // (src/MergePathSpMM.cu:121-122), plus this library's own switch
-    std::vector<mps_tune_result> cand;
+    mps_tune_result cand[16];
+    int n_cand = 0;
     const int costs[] = {16, 24, 32, 48, 64, 96, 128, 256};
-    for (int c : costs) cand.push_back({c, max_tpw, 0u, 0.f});
-    if (max_tpw >= 2) cand.push_back({dflt, max_tpw / 2, 0u, 0.f});
-    cand.push_back({dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f});
-    cand.push_back({dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f});
+    for (int c : costs) cand[n_cand++] = {c, max_tpw, 0u, 0.f};
+    if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, 0u, 0.f};
+    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f};
+    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f};
     hipEvent_t e0 = nullptr, e1 = nullptr;
     MPS_HIP_TRY(hipEventCreate(&e0));
     hipError_t he = hipEventCreate(&e1);
@@ -983,7 +991,8 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     int tried = 0;
     const int cap = (tried_out && n_tried_io) ? *n_tried_io : 0;
     rc = MPS_OK;
-    for (mps_tune_result &c : cand) {
+    for (int ci = 0; ci < n_cand; ++ci) {
+        mps_tune_result &c = cand[ci];
         mps_plan *pl = nullptr;
         rc = mps_plan_create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, c.cost, c.threads_per_wave, c.flags, 0,
                              stream, &pl);
