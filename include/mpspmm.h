@@ -284,8 +284,10 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     v = seg * n_rows + r, 2 * num_slabs segments), each is partitioned on
  *     its own, and the plan runs two launches of the same kernel.  Used for
  *     fp32 when a row of X has at most 64 bytes (K = 16; wider rows are
- *     cheaper through L2, fp16 gains nothing) and the hot columns hold at
- *     least 15 % of the nonzeros; MPS_PLAN_FORCE_HOT lifts these limits.
+ *     cheaper through L2, fp16 gains nothing) and the gathers taken off the
+ *     L2 path outweigh the second set of partial rows (on the 232,965-row
+ *     power-law graph: from about 15 % of the nonzeros in hot columns);
+ *     MPS_PLAN_FORCE_HOT lifts these limits.
  *   - The merge-path partition (mps_num_partitions, mps_partition) of the
  *     virtual rows for the given cost: one split of all of them, or, with hot
  *     columns, one split per segment (padded to whole workgroups).
@@ -295,9 +297,11 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *   - The workspace (partial rows, carry-out records).
  *
  * mps_tile_shape: the slab count and width mps_plan_create chooses for an X
- *   of n_rows x K elements (slab_bytes = 0: 3 MiB slabs); num_slabs == 1
- *   means tiling does not pay (X fits in L2, or a row holds too few nonzeros
- *   per slab).
+ *   of n_rows x K elements (slab_bytes = 0: slabs of 3 or 6 MiB, whichever
+ *   the library's cost model prefers: gathers get cheaper with smaller slabs,
+ *   every slab adds one fp32 partial row per row); num_slabs == 1 means
+ *   tiling does not pay (X fits in L2, or a row holds too few nonzeros per
+ *   slab).
  * mps_plan_create: d_val is fp32 (elem_bytes 4) or fp16 (2); cost and tpw as
  *   for mps_num_partitions / mps_spmm_f32.  Synchronises the stream.
  * mps_plan_set_values: the nonzero values changed, the pattern did not.
@@ -361,7 +365,8 @@ int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsig
  * src/MergePathSpMM.cu:121-122, and its README reports the best of a sweep).
  * Builds a plan for each candidate (costs 16 .. 256 with a full wavefront, the
  * default cost with half the partitions per wavefront, without hot columns,
- * without tiling), runs `repeats` timed products Y = A * X after two warm-ups
+ * without tiling, with slabs of 3, 6, 12 and 24 MiB where X holds more than
+ * two of them), runs `repeats` timed products Y = A * X after two warm-ups
  * (HIP events on the stream) and reports the fastest.  d_Y is overwritten.
  * tried_out (optional) receives every candidate with its time;
  * *n_tried_io is its capacity on entry and the number of candidates on
@@ -371,6 +376,7 @@ typedef struct mps_tune_result {
     int threads_per_wave; /* partitions per wavefront                        */
     unsigned flags;       /* MPS_PLAN_* flags of the candidate                */
     float ms;             /* average time of one product, all kernels         */
+    unsigned long long slab_bytes; /* slab size of the candidate (0: the library's choice) */
 } mps_tune_result;
 int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz, int K,
                       int elem_bytes, const void *d_X, void *d_Y, int repeats, void *stream,

@@ -46,7 +46,7 @@ class PlanInfo(ctypes.Structure):
 class TuneResult(ctypes.Structure):
     """struct mps_tune_result"""
     _fields_ = [("cost", ctypes.c_int), ("threads_per_wave", ctypes.c_int), ("flags", ctypes.c_uint),
-                ("ms", ctypes.c_float)]
+                ("ms", ctypes.c_float), ("slab_bytes", ctypes.c_ulonglong)]
 
 c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp, _i, _sz, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64

@@ -88,12 +88,13 @@ int mergepath_main(int argc, char **argv)
         mps_ok(mps_plan_autotune(d_rp.p, d_ci.p, d_val.p, N, nnz, K, (int)sizeof(T), d_X.p, d_Y.p, 5, nullptr, &best, tried,
                                  &n_tried), "mps_plan_autotune");
         for (int i = 0; i < n_tried && i < 32; ++i)
-            std::printf("tune: cost %4d, threads_per_wave %2d, flags %u: %9.2f us\n", tried[i].cost,
-                        tried[i].threads_per_wave, tried[i].flags, tried[i].ms * 1e3);
+            std::printf("tune: cost %4d, threads_per_wave %2d, flags %2u, slab bytes %9llu: %9.2f us\n", tried[i].cost,
+                        tried[i].threads_per_wave, tried[i].flags, tried[i].slab_bytes, tried[i].ms * 1e3);
         cost = best.cost;
         threads_per_wave = best.threads_per_wave;
         opt.tiling = (int)(best.flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING));
         opt.hot = (int)(best.flags & (MPS_PLAN_NO_HOT | MPS_PLAN_FORCE_HOT));
+        opt.slab_bytes = (size_t)best.slab_bytes;
         opt.use_plan = true;
         mps_ok(mps_num_partitions(N, nnz, cost, &P), "mps_num_partitions");
     }

@@ -17,6 +17,7 @@
 #include "mpspmm_device.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <new>
 #include <vector>
 
@@ -55,6 +56,46 @@ namespace {
 // Slab of X that stays resident in a 4 MiB L2 next to the streamed data
 // (3 MiB measured best on the power-law benchmark graph; 2 and 2.5 MiB within 5 %).
 constexpr size_t kDefaultSlabBytes = 3u << 20;
+
+// ---------------------------------------------------------------------------
+// Cost model behind the automatic choices (slab size, hot columns), from
+// measurements on MI355X with plans of power-law and uniform graphs of 0.2 to
+// 2 M rows and 60 to 200 M nonzeros, K = 16 to 64.
+//   * A gather costs one L1->L2 request per 128 bytes of a row of X, and the
+//     time per request depends on how much of X the wavefronts that run
+//     together spread their gathers over: 5.3 ps when that is a 3 MiB slab
+//     (the L2 of an XCD serves it), 6.5 ps for 6 MiB, 9.4 ps for 15 MiB,
+//     11.7 ps for 32 MiB, 14 ps for 64 MiB, 16 ps for 128 MiB, 17.5 ps beyond
+//     (power-law graphs; uniform graphs are the same up to 6 MiB and up to a
+//     third slower beyond, which is why larger slabs are left to the tuner).
+//   * Every virtual row costs its fp32 partial row written once and read once:
+//     2.8 ps per element of the row (45 ps at K = 16).
+// ---------------------------------------------------------------------------
+double request_ps(double table_bytes)
+{
+    static const double mib[] = {3, 6, 15, 32, 64, 128, 256};
+    static const double ps[] = {5.3, 6.5, 9.4, 11.7, 14.0, 16.0, 17.5};
+    const double m = table_bytes / (1024.0 * 1024.0);
+    if (m <= mib[0]) return ps[0];
+    for (int i = 1; i < 7; ++i)
+        if (m <= mib[i]) {
+            const double t = std::log2(m / mib[i - 1]) / std::log2(mib[i] / mib[i - 1]);
+            return ps[i - 1] + t * (ps[i] - ps[i - 1]);
+        }
+    return ps[6];
+}
+constexpr double kPartialPsPerElement = 2.8;
+
+// Modelled time (ps) of one product with X cut into slabs of slab_cols columns (num_slabs == 1: untiled).
+double modelled_ps(int n_rows, int nnz, int K, int elem_bytes, int num_slabs, int slab_cols)
+{
+    const double row_bytes = (double)K * elem_bytes;
+    const double requests = std::ceil(row_bytes / 128.0);
+    const double table = (double)(num_slabs > 1 ? slab_cols : n_rows) * row_bytes;
+    double t = (double)nnz * requests * request_ps(table);
+    if (num_slabs > 1) t += (double)num_slabs * n_rows * K * kPartialPsPerElement;
+    return t;
+}
 
 // ---------------------------------------------------------------------------
 // Column-slab tiling plan.
@@ -544,8 +585,16 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             MPS_BUILD_HIP(hipMemcpyAsync(h_deg.data(), t.deg, (size_t)n * sizeof(int), hipMemcpyDeviceToHost, st));
             MPS_BUILD_HIP(hipStreamSynchronize(st));
             pl->hot_nnz = select_hot_columns(h_deg, n, pl->num_slabs, pl->slab_cols, hot_rows, h_slot, h_hot_cols);
-            // worth a second launch and twice the partial rows only if it takes a real share of the gathers
-            if ((double)pl->hot_nnz < 0.15 * (double)nnz && !(flags & MPS_PLAN_FORCE_HOT)) {
+            // Worth a second launch and twice the partial rows?  Measured on MI355X at 64-byte rows,
+            // graphs of 0.1 to 0.5 M rows with 3 to 45 M nonzeros in hot columns: a gather from LDS
+            // saves 2.7 ps against one through L2; the second launch costs 40 us whatever its size
+            // (table fill, tail, more carry records); a virtual row of the hot segments costs 0.4 ps
+            // per element while the partial rows of the plan fit the 256 MiB last-level cache and
+            // 3.6 ps per element once they do not.
+            const double vrows = (double)pl->num_slabs * n;
+            const double partial_bytes = 2.0 * vrows * K * sizeof(float);
+            const double gain_ps = 2.7 * (double)pl->hot_nnz - vrows * K * (partial_bytes > 256.0 * 1048576.0 ? 3.6 : 0.4) - 40e6;
+            if (gain_ps <= 0 && !(flags & MPS_PLAN_FORCE_HOT)) {
                 hot_rows = 0;
                 pl->hot_nnz = 0;
             } else {
@@ -822,22 +871,31 @@ int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes
 {
     if (!num_slabs_out || !slab_cols_out || n_rows < 0 || nnz < 0 || K < 1) return MPS_ERR_INVALID_ARG;
     if (elem_bytes != 4 && elem_bytes != 2) return MPS_ERR_INVALID_ARG;
-    if (slab_bytes == 0) slab_bytes = kDefaultSlabBytes;
     const uint64_t row_b = (uint64_t)K * elem_bytes;
     const uint64_t x_bytes = (uint64_t)n_rows * row_b;
     int slabs = 1, cols = n_rows > 0 ? n_rows : 1;
-    // Worth it when X overflows one XCD's L2 (4 MiB) and the nonzeros of a row
-    // inside one slab still form runs long enough to stream (>= 8 on average).
-    if (x_bytes > (3u << 20) && n_rows > 0) {
-        uint64_t want = (x_bytes + slab_bytes - 1) / slab_bytes;
-        if (want > 4096) want = 4096;
-        uint64_t per = ((uint64_t)n_rows + want - 1) / want;
-        per = (per + 63) / 64 * 64;
-        uint64_t s2 = ((uint64_t)n_rows + per - 1) / per;
-        if ((double)nnz / ((double)n_rows * (double)s2) >= 8.0 &&
-            (uint64_t)s2 * n_rows + 1 + (uint64_t)nnz <= (uint64_t)INT_MAX) {
-            slabs = (int)s2;
-            cols = (int)per;
+    // Candidates: the given slab size, or 3 and 6 MiB.  A candidate must leave the
+    // rows of a slab runs long enough to stream (>= 4 nonzeros per row and slab on
+    // average) and beat the untiled plan by 5 % in the model above.
+    const size_t sizes[2] = {slab_bytes ? slab_bytes : kDefaultSlabBytes, slab_bytes ? 0 : 2 * kDefaultSlabBytes};
+    if (x_bytes > kDefaultSlabBytes && n_rows > 0) {
+        double best = 0.95 * modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows);
+        for (size_t sb : sizes) {
+            if (sb == 0) continue;
+            uint64_t want = (x_bytes + sb - 1) / sb;
+            if (want < 2) continue;
+            if (want > 4096) want = 4096;
+            uint64_t per = ((uint64_t)n_rows + want - 1) / want;
+            per = (per + 63) / 64 * 64;
+            const uint64_t s2 = ((uint64_t)n_rows + per - 1) / per;
+            if (s2 < 2 || (double)nnz / ((double)n_rows * (double)s2) < 4.0) continue;
+            if (s2 * n_rows + 1 + (uint64_t)nnz > (uint64_t)INT_MAX) continue;
+            const double t = modelled_ps(n_rows, nnz, K, elem_bytes, (int)s2, (int)per);
+            if (t < best) {
+                best = t;
+                slabs = (int)s2;
+                cols = (int)per;
+            }
         }
     }
     *num_slabs_out = slabs;
@@ -976,10 +1034,14 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     mps_tune_result cand[16];
     int n_cand = 0;
     const int costs[] = {16, 24, 32, 48, 64, 96, 128, 256};
-    for (int c : costs) cand[n_cand++] = {c, max_tpw, 0u, 0.f};
-    if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, 0u, 0.f};
-    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f};
-    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f};
+    for (int c : costs) cand[n_cand++] = {c, max_tpw, 0u, 0.f, 0};
+    if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, 0u, 0.f, 0};
+    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f, 0};
+    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f, 0};
+    // slab sizes the model does not pick on its own: larger slabs pay on skewed graphs
+    for (unsigned long long mib : {3ull, 6ull, 12ull, 24ull})
+        if ((unsigned long long)n_rows * K * elem_bytes > 2 * (mib << 20))
+            cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_HOT, 0.f, mib << 20};
     hipEvent_t e0 = nullptr, e1 = nullptr;
     MPS_HIP_TRY(hipEventCreate(&e0));
     hipError_t he = hipEventCreate(&e1);
@@ -987,15 +1049,19 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
         (void)hipEventDestroy(e0);
         return MPS_ERR_HIP + (int)he;
     }
-    mps_tune_result best{0, 0, 0u, 0.f};
+    mps_tune_result best{0, 0, 0u, 0.f, 0};
     int tried = 0;
     const int cap = (tried_out && n_tried_io) ? *n_tried_io : 0;
     rc = MPS_OK;
     for (int ci = 0; ci < n_cand; ++ci) {
         mps_tune_result &c = cand[ci];
         mps_plan *pl = nullptr;
-        rc = mps_plan_create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, c.cost, c.threads_per_wave, c.flags, 0,
-                             stream, &pl);
+        rc = mps_plan_create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, c.cost, c.threads_per_wave, c.flags,
+                             (size_t)c.slab_bytes, stream, &pl);
+        if ((c.flags & MPS_PLAN_FORCE_TILING) && (rc == MPS_ERR_UNSORTED || rc == MPS_ERR_UNSUPPORTED)) {
+            rc = MPS_OK;  // this matrix cannot be tiled that way: not a candidate
+            continue;
+        }
         if (rc != MPS_OK) break;
         const unsigned all = MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE;
         for (int i = 0; i < 2 && rc == MPS_OK; ++i) rc = mps_plan_spmm_phases(pl, d_X, d_Y, all, stream);

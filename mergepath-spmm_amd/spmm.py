@@ -62,7 +62,7 @@ def autotune(csr, X, repeats=5):
     matrix and K (mps_plan_autotune) - the sweep the reference's users run by
     hand over its <cost> and <threads_per_warp> arguments
     (src/MergePathSpMM.cu:121-122).  Returns (best, tried): dicts with cost,
-    threads_per_wave, flags, ms."""
+    threads_per_wave, flags, ms, slab_bytes."""
     K = X.shape[1]
     eb = 4 if csr.val.dtype == torch.float32 else 2
     Y = torch.empty_like(X)
@@ -72,7 +72,8 @@ def autotune(csr, X, repeats=5):
     check(_cabi.lib().mps_plan_autotune(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz, int(K),
                                         eb, _ptr(X), _ptr(Y), int(repeats), _stream(), ctypes.byref(best), tried,
                                         ctypes.byref(n)), "mps_plan_autotune")
-    as_dict = lambda r: {"cost": r.cost, "threads_per_wave": r.threads_per_wave, "flags": r.flags, "ms": r.ms}
+    as_dict = lambda r: {"cost": r.cost, "threads_per_wave": r.threads_per_wave, "flags": r.flags, "ms": r.ms,
+                         "slab_bytes": r.slab_bytes}
     return as_dict(best), [as_dict(tried[i]) for i in range(min(n.value, 32))]
 
 

@@ -48,7 +48,7 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     for cost, tpw, extra in ((32, 16, ()), ("default", 64, ()), (7, 1, ("--no-plan",)), (128, 0, ("--no-plan",)),
                              (16, 16, ("--tiling", "force", "--slab-bytes", 65536, "--hot", "off")),
-                             (16, 16, ("--tiling", "force", "--slab-bytes", 65536))):
+                             (16, 16, ("--tiling", "force", "--slab-bytes", 65536, "--hot", "force"))):
         dump = tmp_path / "y.bin"
         out = run("MergePathSpMM", graph_file, K, cost, tpw, 3, "--dump", dump, *extra)
         assert out.splitlines()[0] == "Total number of rows: %d and non-zeros: %d" % (rp.size - 1, ci.size)
@@ -59,7 +59,7 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
         assert j["kernel"] == "merge_path" and j["repeat"] == 3 and j["nnz"] == ci.size
         slabs = j["num_slabs"]
         assert j["plan"] == ("--no-plan" not in extra) and (slabs > 1) == ("force" in extra)
-        hot = "force" in extra and "off" not in extra  # forced slabs are narrower than the LDS table: all columns hot
+        hot = extra[-2:] == ("--hot", "force")  # forced slabs are narrower than the LDS table: all columns hot
         assert (j["hot_rows"] > 0) == hot and ("hot columns: " in out) == hot
         if not hot:  # with hot columns every segment is split on its own
             assert j["P"] == orc.num_partitions(slabs * (rp.size - 1), ci.size, 32 if cost == "default" else cost)  # small graph: 32
@@ -101,7 +101,7 @@ def test_merge_path_driver_auto_cost(pkg, orc, graph_file, tmp_path):
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     dump = tmp_path / "y.bin"
     out = run("MergePathSpMM", graph_file, K, "auto", 0, 2, "--dump", dump)
-    assert out.count("tune: cost") == 11
+    assert out.count("tune: cost") == 11  # the graph is too small for the slab-size candidates
     j = last_json(out)
     assert j["plan"] and j["cost"] in (16, 24, 32, 48, 64, 96, 128, 256)
     Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)

@@ -34,7 +34,8 @@ def test_power_law_config_full_size(pkg, orc, dev):
     (d_X,) = to_dev(dev, X)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     plan = pkg.spmm.Plan(csr, K)
-    assert plan.info.num_slabs > 1
+    # the library's own choice here: 5 slabs of 3 MiB, 1,728 hot columns per slab (over a third of the nonzeros)
+    assert plan.info.num_slabs == 5 and plan.info.hot_rows == 1728 and plan.info.hot_nnz > 0.3 * ci.size
     Yp = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz)
     # the partition of the caller's CSR is the reference split, bit for bit, at this size too

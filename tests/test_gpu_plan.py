@@ -147,7 +147,8 @@ def check_plan_layout(pkg, orc, plan, rp, ci, val):
 @pytest.mark.parametrize("tiling,slab_bytes,cost,tpw,hot",
                          [("off", 0, 16, 0, "auto"), ("force", 16384, 16, 0, "off"), ("force", 4096, 7, 3, "off"),
                           ("force", 1 << 20, 64, 16, "off"), ("force", 8192, 128, 1, "off"),
-                          ("force", 16384, 16, 0, "auto"), ("force", 4096, 7, 3, "force"), ("force", 8192, 128, 1, "auto")])
+                          ("force", 16384, 16, 0, "force"), ("force", 4096, 7, 3, "force"), ("force", 8192, 128, 1, "auto"),
+                          ("force", 8192, 128, 1, "force")])
 def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw, hot):
     rng = np.random.default_rng(cost + slab_bytes)
     n = 500
@@ -157,8 +158,9 @@ def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw,
     plan = pkg.spmm.Plan(csr, 16, cost=cost, threads_per_wave=tpw, tiling=tiling, slab_bytes=slab_bytes, hot=hot)
     if tiling == "force":
         assert plan.info.num_slabs == -(-n // plan.info.slab_cols) and plan.info.slab_cols % 64 == 0
-        # slabs narrower than the LDS table: every referenced column is hot
-        assert plan.info.hot_rows == (0 if hot == "off" else 1728)
+        # slabs narrower than the LDS table: every referenced column is hot, if asked for
+        # (on its own the library does not spend a second launch on a matrix this small)
+        assert plan.info.hot_rows == (1728 if hot == "force" else 0)
     else:
         assert plan.info.num_slabs == 1 and plan.info.hot_rows == 0
     check_plan_layout(pkg, orc, plan, rp, ci, val)
@@ -180,13 +182,12 @@ def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
     X = g.fill_uniform_f32(n * K, 6, -1.0, 1.0).reshape(n, K).astype(dtype)
     csr = make_csr(pkg, dev, rp, ci, val)
     slab_cols = 4096
-    wide = K * val.itemsize > 64 or dtype == np.float16  # wider rows or fp16: hot columns only on request
-    if wide:
-        auto = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize)
-        assert auto.info.hot_rows == 0
-        auto.close()
-    plan = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize,
-                         hot="force" if wide else "auto")
+    # wider rows, fp16, or (here) a matrix whose hot gathers do not outweigh a second launch:
+    # hot columns only on request
+    auto = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize)
+    assert auto.info.hot_rows == 0
+    auto.close()
+    plan = pkg.spmm.Plan(csr, K, cost=24, tiling="force", slab_bytes=slab_cols * K * val.itemsize, hot="force")
     i = plan.info
     assert (i.num_slabs, i.slab_cols, i.hot_rows, i.num_segments) == (3, slab_cols, hot_rows, 6)
     assert 0 < i.hot_nnz < ci.size
@@ -255,7 +256,7 @@ def test_unsorted_rows(pkg, dev):
 
 def test_unsorted_rows_fall_back_to_untiled_in_auto_mode(pkg, orc, dev):
     g = pkg.graphs
-    rp, ci, _ = g.generate("chunglu:n=60000,nnz=6000000,gamma=2.1,dmax=5000", seed=4)
+    rp, ci, _ = g.generate("chunglu:n=120000,nnz=18000000,gamma=2.1,dmax=9000", seed=4)
     n, K = rp.size - 1, 16
     ci = ci.copy()
     lo, hi = rp[10], rp[11]
@@ -327,6 +328,11 @@ def test_tile_shape_heuristic(pkg):
     assert sp.tile_shape(232965, 114604189, 16, 4, 2 << 20)[0] == 8
     assert sp.tile_shape(4096, 32731, 16, 4)[0] == 1  # X fits in L2
     assert sp.tile_shape(1048576, 16086273, 16, 4)[0] == 1  # too few nonzeros per row and slab
+    # 1 M rows: 21 slabs of 3 MiB would cost more in partial rows than they save, 11 of 6 MiB pay ...
+    ns, sc = sp.tile_shape(1000000, 120000000, 16, 4)
+    assert ns == 11 and sc * 16 * 4 <= (6 << 20) + 64 * 64
+    assert sp.tile_shape(1000000, 60000000, 16, 4)[0] == 1  # ... but not with half the nonzeros
+    assert sp.tile_shape(232965, 114604189, 64, 4)[0] == 10  # 256-byte rows: 6 MiB slabs
 
 
 def test_power_law_graph_auto_plan(pkg, orc, dev):
@@ -339,7 +345,7 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
     plan = pkg.spmm.Plan(csr, K, cost=128)
-    assert plan.info.num_slabs == 3
+    assert plan.info.num_slabs == 2 and plan.info.slab_cols * K * 4 < (4 << 20)  # X = 6.4 MB: two slabs that fit an L2
     Y = plan.spmm(d_X)
     torch.cuda.synchronize()
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
@@ -364,9 +370,10 @@ def test_autotune_picks_a_measured_candidate(pkg, orc, dev):
     assert {t["cost"] for t in tried} >= {16, 32, 64, 128, 256}
     assert best["ms"] == min(t["ms"] for t in tried) and best in tried
     c = pkg._cabi
-    tiling = "off" if best["flags"] & c.MPS_PLAN_NO_TILING else "auto"
+    tiling = "off" if best["flags"] & c.MPS_PLAN_NO_TILING else "force" if best["flags"] & c.MPS_PLAN_FORCE_TILING else "auto"
     hot = "off" if best["flags"] & c.MPS_PLAN_NO_HOT else "auto"
-    plan = pkg.spmm.Plan(csr, K, cost=best["cost"], threads_per_wave=best["threads_per_wave"], tiling=tiling, hot=hot)
+    plan = pkg.spmm.Plan(csr, K, cost=best["cost"], threads_per_wave=best["threads_per_wave"], tiling=tiling, hot=hot,
+                         slab_bytes=best["slab_bytes"])
     Y = plan.spmm(d_X)
     torch.cuda.synchronize()
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
