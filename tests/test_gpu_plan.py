@@ -320,21 +320,6 @@ def test_plan_edge_shapes(pkg, orc, dev):
             plan.close()
 
 
-def test_tile_shape_heuristic(pkg):
-    sp = pkg.spmm
-    # config 2: X = 14.9 MB, ~492 nonzeros per row -> 5 slabs of ~3 MiB
-    ns, sc = sp.tile_shape(232965, 114604189, 16, 4)
-    assert ns == 5 and sc * 16 * 4 <= (3 << 20) + 64 * 64 and ns * sc >= 232965
-    assert sp.tile_shape(232965, 114604189, 16, 4, 2 << 20)[0] == 8
-    assert sp.tile_shape(4096, 32731, 16, 4)[0] == 1  # X fits in L2
-    assert sp.tile_shape(1048576, 16086273, 16, 4)[0] == 1  # too few nonzeros per row and slab
-    # 1 M rows: 21 slabs of 3 MiB would cost more in partial rows than they save, 11 of 6 MiB pay ...
-    ns, sc = sp.tile_shape(1000000, 120000000, 16, 4)
-    assert ns == 11 and sc * 16 * 4 <= (6 << 20) + 64 * 64
-    assert sp.tile_shape(1000000, 60000000, 16, 4)[0] == 1  # ... but not with half the nonzeros
-    assert sp.tile_shape(232965, 114604189, 64, 4)[0] == 10  # 256-byte rows: 6 MiB slabs
-
-
 def test_power_law_graph_auto_plan(pkg, orc, dev):
     g = pkg.graphs
     rp, ci, _ = g.generate("chunglu:n=100000,nnz=20000000,gamma=2.1,dmax=9000", seed=2)

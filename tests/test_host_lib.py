@@ -285,3 +285,19 @@ def test_npz_to_csr_tool(pkg, tmp_path, compressed, dtype):
     assert np.array_equal(rp, want_rp) and np.array_equal(ci, want_ci)
     p = subprocess.run([exe, "--graph", str(out), "--output", str(tmp_path / "x.csr")], capture_output=True, text=True)
     assert p.returncode == 1 and "npz_to_csr:" in p.stderr
+
+
+def test_tile_shape_cost_model(pkg):
+    """mps_tile_shape: slab count and width from the library's cost model (host arithmetic only)."""
+    sp = pkg.spmm
+    # config 2: X = 14.9 MB, ~492 nonzeros per row -> 5 slabs of ~3 MiB
+    ns, sc = sp.tile_shape(232965, 114604189, 16, 4)
+    assert ns == 5 and sc * 16 * 4 <= (3 << 20) + 64 * 64 and ns * sc >= 232965
+    assert sp.tile_shape(232965, 114604189, 16, 4, 2 << 20)[0] == 8
+    assert sp.tile_shape(4096, 32731, 16, 4)[0] == 1  # X fits in L2
+    assert sp.tile_shape(1048576, 16086273, 16, 4)[0] == 1  # too few nonzeros per row and slab
+    # 1 M rows: 21 slabs of 3 MiB would cost more in partial rows than they save, 11 of 6 MiB pay ...
+    ns, sc = sp.tile_shape(1000000, 120000000, 16, 4)
+    assert ns == 11 and sc * 16 * 4 <= (6 << 20) + 64 * 64
+    assert sp.tile_shape(1000000, 60000000, 16, 4)[0] == 1  # ... but not with half the nonzeros
+    assert sp.tile_shape(232965, 114604189, 64, 4)[0] == 10  # 256-byte rows: 6 MiB slabs
