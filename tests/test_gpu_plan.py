@@ -340,19 +340,25 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
     assert (Y - Y0).abs().max().item() <= 1e-3
 
 
-def test_autotune_picks_a_measured_candidate(pkg, orc, dev):
+@pytest.mark.parametrize("spec,n_candidates,slab_sizes",
+                         [("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", 11, set()),
+                          # X = 15.4 MB: slabs of 3 and 6 MiB are candidates too (X holds more than two of them)
+                          ("chunglu:n=240000,nnz=6000000,gamma=2.1,dmax=5000", 13, {3 << 20, 6 << 20})])
+def test_autotune_picks_a_measured_candidate(pkg, orc, dev, spec, n_candidates, slab_sizes):
     """mps_plan_autotune: every candidate is timed, the reported best is the
     fastest of them, and a plan built from it gives the right product."""
     g = pkg.graphs
-    rp, ci, _ = g.generate("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", seed=8)
+    rp, ci, _ = g.generate(spec, seed=8)
     n, K = rp.size - 1, 16
     val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
     X = g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
     best, tried = pkg.spmm.autotune(csr, d_X, repeats=3)
-    assert len(tried) == 11 and all(t["ms"] > 0 for t in tried)
+    assert len(tried) == n_candidates and all(t["ms"] > 0 for t in tried)
     assert {t["cost"] for t in tried} >= {16, 32, 64, 128, 256}
+    assert {t["slab_bytes"] for t in tried if t["flags"] & pkg._cabi.MPS_PLAN_FORCE_TILING} == slab_sizes
+    assert all(t["slab_bytes"] == 0 for t in tried if not t["flags"] & pkg._cabi.MPS_PLAN_FORCE_TILING)
     assert best["ms"] == min(t["ms"] for t in tried) and best in tried
     c = pkg._cabi
     tiling = "off" if best["flags"] & c.MPS_PLAN_NO_TILING else "force" if best["flags"] & c.MPS_PLAN_FORCE_TILING else "auto"
