@@ -287,6 +287,37 @@ def test_npz_to_csr_tool(pkg, tmp_path, compressed, dtype):
     assert p.returncode == 1 and "npz_to_csr:" in p.stderr
 
 
+@pytest.mark.parametrize("undirected", [False, True])
+def test_edges_to_csr_tool(pkg, tmp_path, undirected):
+    """Text edge list -> .csr: the recipe of scripts/fetch_dataset.py:10-21 (edge list -> coo -> csr ->
+    two comma lines) for a file with comments, tabs, commas, a weight column and repeated edges."""
+    exe = os.path.join(ROOT, "mergepath-spmm_amd", "csrc", "edges_to_csr")
+    assert os.path.exists(exe), "edges_to_csr is not built"
+    rng = np.random.default_rng(11)
+    src = rng.integers(0, 3000, 50000)
+    dst = rng.integers(0, 3000, 50000)
+    sep = ["\t", " ", ",", "  "]
+    lines = ["# Directed graph: test", "% another comment", ""]
+    for i, (a, b) in enumerate(zip(src, dst)):
+        lines.append("%d%s%d%s" % (a, sep[i % 4], b, " 0.5" if i % 7 == 0 else ""))
+    txt = tmp_path / "g.txt"
+    txt.write_text("\n".join(lines) + ("\n" if undirected else ""))  # with and without a final newline
+    out = tmp_path / "g.csr"
+    p = subprocess.run([exe, "--edges", str(txt), "--output", str(out)] + (["--undirected"] if undirected else []),
+                       capture_output=True, text=True, timeout=60)
+    assert p.returncode == 0, p.stderr
+    if undirected:
+        keep = src != dst
+        src, dst = np.concatenate([src, dst[keep]]), np.concatenate([dst, src[keep]])
+    want_rp, want_ci = reference_conversion(src, dst)
+    assert out.read_text() == ",".join(map(str, want_rp)) + ",\n" + ",".join(map(str, want_ci)) + ","
+    assert p.stdout.startswith("%d rows, %d nonzeros" % (want_rp.size - 1, want_ci.size))
+    bad = tmp_path / "bad.txt"
+    bad.write_text("1 2\n3 x\n")
+    p = subprocess.run([exe, "--edges", str(bad), "--output", str(out)], capture_output=True, text=True)
+    assert p.returncode == 1 and "edges_to_csr:" in p.stderr
+
+
 def test_tile_shape_cost_model(pkg):
     """mps_tile_shape: slab count and width from the library's cost model (host arithmetic only)."""
     sp = pkg.spmm
