@@ -331,7 +331,7 @@ typedef struct mps_plan_info {
     int hot_rows;                  /* rows of X per LDS table (0: no hot launch)  */
     int hot_waves;                 /* wavefronts of the hot launch                */
     long long hot_nnz;             /* nonzeros gathered from LDS                  */
-    int hot_cost;                  /* merge items per partition of the hot segments */
+    int hot_cost;                  /* merge items per partition of the hot segments (64 .. 256 by the amount of hot work, at least cost) */
     int mark_shift;                /* > 0: SLICE_COLS entries are column | row_ends << mark_shift */
     int hot_mark_shift;            /* the same for the entries of the hot wavefronts (column = LDS slot) */
 } mps_plan_info;

@@ -439,7 +439,7 @@ int plan_set_values(mps_plan *pl, const void *d_val, hipStream_t st)
 
 // Static LDS of a hot workgroup (see mp_spmm_kernel) and the rows of X that
 // fit beside it in the 160 KiB of a CU.
-constexpr int kHotCost = 256;  // merge items per partition of a hot segment (at least the plan's cost)
+constexpr int kHotCost = 256;  // most merge items per partition of a hot segment (unless the plan's cost is larger)
 
 size_t hot_static_lds(int vec)
 {
@@ -587,13 +587,13 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             pl->hot_nnz = select_hot_columns(h_deg, n, pl->num_slabs, pl->slab_cols, hot_rows, h_slot, h_hot_cols);
             // Worth a second launch and twice the partial rows?  Measured on MI355X at 64-byte rows,
             // graphs of 0.1 to 0.5 M rows with 3 to 45 M nonzeros in hot columns: a gather from LDS
-            // saves 2.7 ps against one through L2; the second launch costs 40 us whatever its size
-            // (table fill, tail, more carry records); a virtual row of the hot segments costs 0.4 ps
+            // saves 2.7 ps against one through L2; the second launch costs 15 us whatever its size
+            // (table fill, tail, more carry records); a virtual row of the hot segments costs 1.7 ps
             // per element while the partial rows of the plan fit the 256 MiB last-level cache and
-            // 3.6 ps per element once they do not.
+            // 4 ps per element once they do not.
             const double vrows = (double)pl->num_slabs * n;
             const double partial_bytes = 2.0 * vrows * K * sizeof(float);
-            const double gain_ps = 2.7 * (double)pl->hot_nnz - vrows * K * (partial_bytes > 256.0 * 1048576.0 ? 3.6 : 0.4) - 40e6;
+            const double gain_ps = 2.7 * (double)pl->hot_nnz - vrows * K * (partial_bytes > 256.0 * 1048576.0 ? 4.0 : 1.7) - 15e6;
             if (gain_ps <= 0 && !(flags & MPS_PLAN_FORCE_HOT)) {
                 hot_rows = 0;
                 pl->hot_nnz = 0;
@@ -679,22 +679,29 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
     } else {
         // every segment is split on its own and padded to whole wavefronts
         const int S2 = pl->num_segs, S = pl->num_slabs;
-        {
-            const char *e = std::getenv("MPS_HOT_COST");
-            const int v = e ? std::atoi(e) : 0;
-            pl->hot_cost = v > 0 ? v : (pl->cost > kHotCost ? pl->cost : kHotCost);
-        }
         std::vector<int> seg_y((size_t)S2 + 1);
         for (int g = 0; g <= S2; ++g)
             MPS_BUILD_HIP(hipMemcpyAsync(&seg_y[(size_t)g], pl->vrow_ptr + (size_t)g * n, sizeof(int), hipMemcpyDeviceToHost, st));
         MPS_BUILD_HIP(hipStreamSynchronize(st));
+        {
+            // Hot segments take long partitions (nothing to gain from small ones where every
+            // gather costs the same, and a long one hides the start-up loads), but every one
+            // of the 16 wavefronts of the 256 hot workgroups should get a piece: measured on a
+            // 100,000-row graph with 7.4 M hot nonzeros, cost 256 leaves 9 of 16 wavefronts
+            // idle (0.169 ms per product), cost 128 runs at 0.146 ms.
+            const long long hot_items = (long long)S * (n + 1) + (seg_y[(size_t)S] - seg_y[0]);
+            long long fit = hot_items / (16LL * kHotWavesPerBlock * 256);
+            if (fit > kHotCost) fit = kHotCost;
+            if (fit < 64) fit = 64;
+            const char *e = std::getenv("MPS_HOT_COST");
+            const int v = e ? std::atoi(e) : 0;
+            pl->hot_cost = v > 0 ? v : (pl->cost > (int)fit ? pl->cost : (int)fit);
+        }
         std::vector<int> h_seg((size_t)3 * S2 + 1);  // seg_off[S2 + 1], seg_parts[S2], seg_ipt[S2]
         int *seg_off = h_seg.data(), *seg_parts = seg_off + S2 + 1, *seg_ipt = seg_parts + S2;
         long long off = 0;
         for (int g = 0; g < S2; ++g) {
             const long long total = (long long)n + 1 + (seg_y[(size_t)g + 1] - seg_y[(size_t)g]);
-            // hot segments take long partitions: nothing to gain from small ones where
-            // every gather costs the same, and a long one hides the start-up loads
             long long parts = (total - 1) / (g < S ? pl->hot_cost : pl->cost);
             if (parts < 1) parts = 1;
             const long long mult = G;  // whole wavefronts

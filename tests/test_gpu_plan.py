@@ -83,8 +83,10 @@ def check_plan_layout(pkg, orc, plan, rp, ci, val):
     c, i = pkg._cabi, plan.info
     n, nnz = rp.size - 1, ci.size
     if i.hot_rows > 0:
-        assert i.num_segments == 2 * i.num_slabs and i.hot_cost == max(i.cost, 256)
         hot_slot, hot_cols = hot_reference(rp, ci, i.num_slabs, i.slab_cols, i.hot_rows)
+        # one piece (16 partitions) for each of the 16 wavefronts of 256 workgroups, within 64 .. 256 items
+        hot_items = i.num_slabs * (n + 1) + int((hot_slot[ci] >= 0).sum())
+        assert i.num_segments == 2 * i.num_slabs and i.hot_cost == max(i.cost, min(256, max(64, hot_items // 65536)))
         assert np.array_equal(plan.array(c.MPS_PLAN_ARRAY_HOT_COLS), hot_cols)
         assert i.hot_nnz == int((hot_slot[ci] >= 0).sum())
         vrp, perm = segment_major_reference(rp, ci, i.num_slabs, i.slab_cols, hot_slot)
