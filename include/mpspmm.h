@@ -366,7 +366,8 @@ int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsig
  * Builds a plan for each candidate (costs 16 .. 256 with a full wavefront, the
  * default cost with half the partitions per wavefront, without hot columns,
  * without tiling, with slabs of 3, 6, 12 and 24 MiB where X holds more than
- * two of them), runs `repeats` timed products Y = A * X after two warm-ups
+ * two of them and the library's cost model does not put them 50 % behind the
+ * untiled plan), runs `repeats` timed products Y = A * X after two warm-ups
  * (HIP events on the stream) and reports the fastest.  d_Y is overwritten.
  * tried_out (optional) receives every candidate with its time;
  * *n_tried_io is its capacity on entry and the number of candidates on

@@ -1046,9 +1046,17 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f, 0};
     cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f, 0};
     // slab sizes the model does not pick on its own: larger slabs pay on skewed graphs
-    for (unsigned long long mib : {3ull, 6ull, 12ull, 24ull})
-        if ((unsigned long long)n_rows * K * elem_bytes > 2 * (mib << 20))
-            cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_HOT, 0.f, mib << 20};
+    // (not those the model puts 50 % behind the untiled plan: thousands of slabs for a matrix with short rows)
+    const double untiled_ps = modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows);
+    for (unsigned long long mib : {3ull, 6ull, 12ull, 24ull}) {
+        const unsigned long long row_bytes = (unsigned long long)K * elem_bytes;
+        if ((unsigned long long)n_rows * row_bytes <= 2 * (mib << 20)) continue;
+        unsigned long long cols = (mib << 20) / row_bytes / 64 * 64;  // what MPS_PLAN_FORCE_TILING makes of the size
+        if (cols < 64) cols = 64;
+        const unsigned long long slabs = ((unsigned long long)n_rows + cols - 1) / cols;
+        if (modelled_ps(n_rows, nnz, K, elem_bytes, (int)slabs, (int)cols) > 1.5 * untiled_ps) continue;
+        cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_HOT, 0.f, mib << 20};
+    }
     hipEvent_t e0 = nullptr, e1 = nullptr;
     MPS_HIP_TRY(hipEventCreate(&e0));
     hipError_t he = hipEventCreate(&e1);

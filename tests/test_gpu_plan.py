@@ -345,7 +345,7 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
 @pytest.mark.parametrize("spec,n_candidates,slab_sizes",
                          [("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", 11, set()),
                           # X = 15.4 MB: slabs of 3 and 6 MiB are candidates too (X holds more than two of them)
-                          ("chunglu:n=240000,nnz=6000000,gamma=2.1,dmax=5000", 13, {3 << 20, 6 << 20})])
+                          ("chunglu:n=240000,nnz=12000000,gamma=2.1,dmax=5000", 13, {3 << 20, 6 << 20})])
 def test_autotune_picks_a_measured_candidate(pkg, orc, dev, spec, n_candidates, slab_sizes):
     """mps_plan_autotune: every candidate is timed, the reported best is the
     fastest of them, and a plan built from it gives the right product."""
