@@ -285,18 +285,22 @@ __global__ __launch_bounds__(256) void col_histogram_kernel(const int *__restric
     if (e < nnz) atomicAdd(deg + col_idx[e], 1);
 }
 
-// One thread per (slab, row): where the row's nonzeros of that slab start, and
-// how many of them lie in hot columns.
+// Sixteen lanes per (slab, row): where the row's nonzeros of that slab start,
+// and how many of them lie in hot columns.  (One thread per pair would walk a
+// hub row's thousands of nonzeros alone while the rest of the launch waits.)
+constexpr int kSplitLanes = 16;
+
 __global__ __launch_bounds__(256) void hot_count_kernel(const int *__restrict__ row_ptr,
                                                          const int *__restrict__ col_idx, int n_rows,
                                                          int num_slabs, int slab_cols,
                                                          const int *__restrict__ hot_slot, int *__restrict__ first,
                                                          int *__restrict__ counts)
 {
-    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long t = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / kSplitLanes;
+    const int sub = threadIdx.x & (kSplitLanes - 1);
     const long long nv = (long long)num_slabs * n_rows;
-    if (t == nv) counts[2 * nv] = 0;
-    if (t >= nv) return;
+    if (t == nv && sub == 0) counts[2 * nv] = 0;
+    if (t >= nv) return;  // whole 16-lane group
     const int s = (int)(t / n_rows);
     const int r = (int)(t - (long long)s * n_rows);
     const int b = row_ptr[r], e = row_ptr[r + 1];
@@ -311,36 +315,68 @@ __global__ __launch_bounds__(256) void hot_count_kernel(const int *__restrict__ 
     const int f0 = lower((long long)s * slab_cols);
     const int f1 = (s + 1 == num_slabs) ? e : lower((long long)(s + 1) * slab_cols);
     int hot = 0;
-    for (int i = f0; i < f1; ++i) hot += hot_slot[col_idx[i]] >= 0;
-    first[t] = f0;
-    counts[t] = hot;                  // hot segment s
-    counts[nv + t] = (f1 - f0) - hot; // cold segment num_slabs + s
+    for (int i = f0 + sub; i < f1; i += kSplitLanes) hot += hot_slot[col_idx[i]] >= 0;
+#pragma unroll
+    for (int d = kSplitLanes / 2; d > 0; d >>= 1) hot += __shfl_xor(hot, d, kSplitLanes);
+    if (sub == 0) {
+        first[t] = f0;
+        counts[t] = hot;                  // hot segment s
+        counts[nv + t] = (f1 - f0) - hot; // cold segment num_slabs + s
+    }
 }
 
-// One thread per (slab, row): its nonzeros go, in order, to the hot or the cold
-// virtual row; hot ones carry their LDS slot instead of the column id.
+// Sixteen lanes per (slab, row): its nonzeros go, in order, to the hot or the
+// cold virtual row; hot ones carry their LDS slot instead of the column id.
 __global__ __launch_bounds__(256) void hot_scatter_kernel(const int *__restrict__ col_idx, int n_rows, int num_slabs,
                                                            const int *__restrict__ hot_slot,
                                                            const int *__restrict__ first,
                                                            const int *__restrict__ vrow_ptr,
                                                            int *__restrict__ col_out, int *__restrict__ perm)
 {
-    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long t = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / kSplitLanes;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & (kSplitLanes - 1);
     const long long nv = (long long)num_slabs * n_rows;
-    if (t >= nv) return;
-    int dh = vrow_ptr[t], dc = vrow_ptr[nv + t];
-    const int len = (vrow_ptr[t + 1] - dh) + (vrow_ptr[nv + t + 1] - dc);
-    const int f0 = first[t];
-    for (int i = f0; i < f0 + len; ++i) {
-        const int c = col_idx[i];
-        const int slot = hot_slot[c];
-        if (slot >= 0) {
-            col_out[dh] = slot;
-            perm[dh++] = i;
-        } else {
-            col_out[dc] = c;
-            perm[dc++] = i;
+    // lanes of a wavefront whose pair does not exist still take part in the ballots below
+    const bool live = t < nv;
+    int dh = 0, dc = 0, len = 0, f0 = 0;
+    if (live) {
+        dh = vrow_ptr[t];
+        dc = vrow_ptr[nv + t];
+        len = (vrow_ptr[t + 1] - dh) + (vrow_ptr[nv + t + 1] - dc);
+        f0 = first[t];
+    }
+    int longest = len;  // the four groups of a wavefront loop together
+#pragma unroll
+    for (int d = 32; d >= kSplitLanes; d >>= 1) longest = max(longest, __shfl_xor(longest, d, 64));
+    const int group_shift = lane & ~(kSplitLanes - 1);
+    for (int base = 0; base < longest; base += kSplitLanes) {
+        const int k = base + sub;
+        const bool have = k < len;
+        int c = 0, slot = -1;
+        if (have) {
+            c = col_idx[f0 + k];
+            slot = hot_slot[c];
         }
+        const unsigned long long hot_mask = __ballot(have && slot >= 0);
+        const unsigned long long any_mask = __ballot(have);
+        const unsigned mine_hot = (unsigned)(hot_mask >> group_shift) & 0xffffu;
+        const unsigned mine_any = (unsigned)(any_mask >> group_shift) & 0xffffu;
+        const unsigned below = (1u << sub) - 1u;
+        if (have) {
+            const int hot_before = __popc(mine_hot & below);
+            if (slot >= 0) {
+                col_out[dh + hot_before] = slot;
+                perm[dh + hot_before] = f0 + k;
+            } else {
+                const int cold_before = __popc(mine_any & below) - hot_before;
+                col_out[dc + cold_before] = c;
+                perm[dc + cold_before] = f0 + k;
+            }
+        }
+        const int nh = __popc(mine_hot);
+        dh += nh;
+        dc += __popc(mine_any) - nh;
     }
 }
 
@@ -645,11 +681,12 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
         }
         const unsigned row_blocks = (unsigned)((nslab_rows + 1 + 255) / 256);
         if (hot_rows > 0) {
-            hipLaunchKernelGGL(hot_count_kernel, dim3(row_blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n, pl->num_slabs,
+            const unsigned split_blocks = (unsigned)(((nslab_rows + 1) * kSplitLanes + 255) / 256);
+            hipLaunchKernelGGL(hot_count_kernel, dim3(split_blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n, pl->num_slabs,
                                pl->slab_cols, t.hot_slot, t.first, pl->vrow_ptr);
             MPS_BUILD_HIP(hipGetLastError());
             MPS_BUILD_TRY(scan_exclusive_inplace(pl->vrow_ptr, (int)nv + 1, t.sums, st));
-            hipLaunchKernelGGL(hot_scatter_kernel, dim3(row_blocks), dim3(256), 0, st, d_col_idx, n, pl->num_slabs,
+            hipLaunchKernelGGL(hot_scatter_kernel, dim3(split_blocks), dim3(256), 0, st, d_col_idx, n, pl->num_slabs,
                                t.hot_slot, t.first, pl->vrow_ptr, t.col_v, t.perm);
         } else {
             hipLaunchKernelGGL(tile_count_kernel, dim3(row_blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n, pl->num_slabs,
