@@ -151,7 +151,8 @@ __global__ __launch_bounds__(256) void tile_scatter_kernel(const int *__restrict
                                                             int num_slabs, int slab_cols,
                                                             const int *__restrict__ first,
                                                             const int *__restrict__ vrow_ptr,
-                                                            int *__restrict__ col_tiled, int *__restrict__ perm)
+                                                            int *__restrict__ col_tiled, int *__restrict__ perm,
+                                                            int *__restrict__ vrow_of)
 {
     const long long e64 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (e64 >= nnz) return;
@@ -168,6 +169,7 @@ __global__ __launch_bounds__(256) void tile_scatter_kernel(const int *__restrict
     const int dst = vrow_ptr[v] + (e - first[v]);
     col_tiled[dst] = c;
     perm[dst] = e;
+    vrow_of[dst] = (int)v;
 }
 
 // Y[r] = sum over slabs, in slab order, of the partial rows part[s * n_rows + r].
@@ -215,12 +217,20 @@ __global__ __launch_bounds__(256) void slice_count_kernel(const int *__restrict_
 // number of rows that end in front of this nonzero inside its partition: its
 // virtual row minus that of the nonzero before it, or minus the row the
 // partition starts in (coord_x - 1) for the partition's first nonzero.
+// The virtual row of a nonzero comes from vrow_of (tiled plans: the scatter
+// kernels know it) or from a bisection of vrow_ptr.  Its partition needs no
+// search: the merge path passes through (row + 1, y) right before it consumes
+// nonzero y, on diagonal row + 1 + y, and partition p owns the diagonals
+// [p * ipt, (p + 1) * ipt) - of the whole matrix (seg == nullptr), or of the
+// nonzero's segment (seg: seg_off[num_segs + 1], seg_parts[num_segs], seg_ipt[num_segs]).
 __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restrict__ col_v,
                                                              const int *__restrict__ perm,
+                                                             const int *__restrict__ vrow_of,
                                                              const int *__restrict__ vrow_ptr, int n_vrows,
                                                              const int *__restrict__ coord_x,
-                                                             const int *__restrict__ coord_y, int P, int tpw,
-                                                             const int *__restrict__ wave_off, int nnz,
+                                                             const int *__restrict__ coord_y, int tpw,
+                                                             const int *__restrict__ wave_off, int nnz, int ipt,
+                                                             const int *__restrict__ seg, int num_segs, int seg_rows,
                                                              int hot_parts, int hot_mark_shift, int mark_shift,
                                                              int *__restrict__ slice_cols,
                                                              int *__restrict__ slice_src)
@@ -228,12 +238,24 @@ __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restric
     const long long y64 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (y64 >= nnz) return;
     const int y = (int)y64;
-    int lo = 0, hi = P - 1;  // largest p with coord_y[p] <= y
-    while (lo < hi) {
-        int mid = (lo + hi + 1) >> 1;
-        if (coord_y[mid] <= y) lo = mid; else hi = mid - 1;
+    auto row_of = [&](int yy) {  // largest v with vrow_ptr[v] <= yy
+        int a = 0, b = n_vrows - 1;
+        while (a < b) {
+            int mid = (a + b + 1) >> 1;
+            if (vrow_ptr[mid] <= yy) a = mid; else b = mid - 1;
+        }
+        return a;
+    };
+    const int row = vrow_of ? vrow_of[y] : row_of(y);
+    int p;
+    if (seg) {
+        const int g = row / seg_rows;
+        const long long base = (long long)g * seg_rows;
+        const long long d = (row - base) + 1 + (y - vrow_ptr[base]);
+        p = seg[g] + (int)(d / seg[2 * num_segs + 1 + g]);
+    } else {
+        p = (int)(((long long)row + 1 + y) / ipt);
     }
-    const int p = lo;
     const int w = p / tpw, g = p - w * tpw;
     const int k = y - coord_y[p];
     const size_t slot = ((size_t)wave_off[w] + (size_t)(k / kWindow)) * (size_t)(tpw * kWindow) + (size_t)g * kWindow +
@@ -241,17 +263,9 @@ __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restric
     unsigned entry = (unsigned)col_v[y];
     const int shift = p < hot_parts ? hot_mark_shift : mark_shift;
     if (shift > 0) {
-        auto row_of = [&](int yy) {  // largest v with vrow_ptr[v] <= yy
-            int a = 0, b = n_vrows - 1;
-            while (a < b) {
-                int mid = (a + b + 1) >> 1;
-                if (vrow_ptr[mid] <= yy) a = mid; else b = mid - 1;
-            }
-            return a;
-        };
-        const int row = row_of(y);
         int before;
         if (k == 0) before = max(coord_x[p], 1) - 1;
+        else if (vrow_of) before = vrow_of[y - 1];
         else before = vrow_ptr[row] < y ? row : row_of(y - 1);
         entry |= (unsigned)(row - before) << shift;
     }
@@ -331,7 +345,8 @@ __global__ __launch_bounds__(256) void hot_scatter_kernel(const int *__restrict_
                                                            const int *__restrict__ hot_slot,
                                                            const int *__restrict__ first,
                                                            const int *__restrict__ vrow_ptr,
-                                                           int *__restrict__ col_out, int *__restrict__ perm)
+                                                           int *__restrict__ col_out, int *__restrict__ perm,
+                                                           int *__restrict__ vrow_of)
 {
     const long long t = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / kSplitLanes;
     const int lane = threadIdx.x & 63;
@@ -368,10 +383,12 @@ __global__ __launch_bounds__(256) void hot_scatter_kernel(const int *__restrict_
             if (slot >= 0) {
                 col_out[dh + hot_before] = slot;
                 perm[dh + hot_before] = f0 + k;
+                vrow_of[dh + hot_before] = (int)t;
             } else {
                 const int cold_before = __popc(mine_any & below) - hot_before;
                 col_out[dc + cold_before] = c;
                 perm[dc + cold_before] = f0 + k;
+                vrow_of[dc + cold_before] = (int)(nv + t);
             }
         }
         const int nh = __popc(mine_hot);
@@ -502,18 +519,19 @@ int choose_hot_rows(int K, int eb, const SpmmShape &sh, bool force)
 }
 
 struct BuildTmp {
-    int *first = nullptr, *col_v = nullptr, *perm = nullptr, *sums = nullptr, *deg = nullptr, *hot_slot = nullptr,
-        *seg = nullptr;
+    int *first = nullptr, *col_v = nullptr, *perm = nullptr, *vrow = nullptr, *sums = nullptr, *deg = nullptr,
+        *hot_slot = nullptr, *seg = nullptr;
     void drop()
     {
         (void)hipFree(first);
         (void)hipFree(col_v);
         (void)hipFree(perm);
+        (void)hipFree(vrow);
         (void)hipFree(sums);
         (void)hipFree(deg);
         (void)hipFree(hot_slot);
         (void)hipFree(seg);
-        first = col_v = perm = sums = deg = hot_slot = seg = nullptr;
+        first = col_v = perm = vrow = sums = deg = hot_slot = seg = nullptr;
     }
     ~BuildTmp() { drop(); }
 };
@@ -655,6 +673,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
         MPS_BUILD_TRY(tmp_alloc(&t.first, (size_t)nslab_rows));
         MPS_BUILD_TRY(tmp_alloc(&t.col_v, (size_t)nnz));
         MPS_BUILD_TRY(tmp_alloc(&t.perm, (size_t)nnz));
+        MPS_BUILD_TRY(tmp_alloc(&t.vrow, (size_t)nnz));
         int *bad = t.sums + kScanMaxBlocks;
         int zero = 0, h_bad = 0;
         MPS_BUILD_HIP(hipMemcpyAsync(bad, &zero, sizeof(int), hipMemcpyHostToDevice, st));
@@ -669,8 +688,8 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
                 t.drop();
                 return MPS_ERR_UNSORTED;
             }
-            (void)hipFree(t.first); (void)hipFree(t.col_v); (void)hipFree(t.perm);
-            t.first = t.col_v = t.perm = nullptr;
+            (void)hipFree(t.first); (void)hipFree(t.col_v); (void)hipFree(t.perm); (void)hipFree(t.vrow);
+            t.first = t.col_v = t.perm = t.vrow = nullptr;
             (void)hipFree(pl->vrow_ptr);
             pl->vrow_ptr = nullptr;
             pl->num_slabs = 1;
@@ -687,7 +706,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             MPS_BUILD_HIP(hipGetLastError());
             MPS_BUILD_TRY(scan_exclusive_inplace(pl->vrow_ptr, (int)nv + 1, t.sums, st));
             hipLaunchKernelGGL(hot_scatter_kernel, dim3(split_blocks), dim3(256), 0, st, d_col_idx, n, pl->num_slabs,
-                               t.hot_slot, t.first, pl->vrow_ptr, t.col_v, t.perm);
+                               t.hot_slot, t.first, pl->vrow_ptr, t.col_v, t.perm, t.vrow);
         } else {
             hipLaunchKernelGGL(tile_count_kernel, dim3(row_blocks), dim3(256), 0, st, d_row_ptr, d_col_idx, n, pl->num_slabs,
                                pl->slab_cols, t.first, pl->vrow_ptr);
@@ -695,7 +714,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             MPS_BUILD_TRY(scan_exclusive_inplace(pl->vrow_ptr, (int)nv + 1, t.sums, st));
             hipLaunchKernelGGL(tile_scatter_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st,
                                d_row_ptr, d_col_idx, n, nnz, pl->num_slabs, pl->slab_cols, t.first, pl->vrow_ptr, t.col_v,
-                               t.perm);
+                               t.perm, t.vrow);
         }
         MPS_BUILD_HIP(hipGetLastError());
         break;
@@ -844,9 +863,10 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
     }
     if (nnz > 0) {
         hipLaunchKernelGGL(slice_scatter_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st, cols_v,
-                           pl->num_slabs == 1 ? nullptr : t.perm, pl->vrow_ptr, pl->n_vrows, pl->coord_x, pl->coord_y,
-                           pl->P, G, pl->wave_off, nnz, pl->hot_waves * G, pl->hot_mark_shift, pl->mark_shift,
-                           pl->slice_cols, pl->slice_src);
+                           pl->num_slabs == 1 ? nullptr : t.perm, pl->num_slabs == 1 ? nullptr : t.vrow, pl->vrow_ptr,
+                           pl->n_vrows, pl->coord_x, pl->coord_y, G, pl->wave_off, nnz, max_cold_ipt,
+                           hot_rows > 0 ? t.seg : nullptr, pl->num_segs, n, pl->hot_waves * G, pl->hot_mark_shift,
+                           pl->mark_shift, pl->slice_cols, pl->slice_src);
         MPS_BUILD_HIP(hipGetLastError());
     }
     MPS_BUILD_TRY(plan_set_values(pl, d_val, st));
