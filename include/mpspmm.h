@@ -334,6 +334,7 @@ typedef struct mps_plan_info {
     int hot_cost;                  /* merge items per partition of the hot segments (64 .. 256 by the amount of hot work, at least cost) */
     int mark_shift;                /* > 0: SLICE_COLS entries are column | row_ends << mark_shift */
     int hot_mark_shift;            /* the same for the entries of the hot wavefronts (column = LDS slot) */
+    int hot_blocks;                /* workgroups of the hot launch: at most one per CU unless there are more hot segments than CUs */
 } mps_plan_info;
 
 enum {

@@ -41,7 +41,7 @@ class PlanInfo(ctypes.Structure):
                [("total_rounds", ctypes.c_longlong), ("slice_slots", ctypes.c_longlong),
                 ("device_bytes", ctypes.c_size_t), ("num_segments", ctypes.c_int), ("hot_rows", ctypes.c_int),
                 ("hot_waves", ctypes.c_int), ("hot_nnz", ctypes.c_longlong), ("hot_cost", ctypes.c_int), ("mark_shift", ctypes.c_int),
-                ("hot_mark_shift", ctypes.c_int)]
+                ("hot_mark_shift", ctypes.c_int), ("hot_blocks", ctypes.c_int)]
 
 class TuneResult(ctypes.Structure):
     """struct mps_tune_result"""

@@ -322,6 +322,29 @@ def test_plan_edge_shapes(pkg, orc, dev):
             plan.close()
 
 
+@pytest.mark.parametrize("num_slabs", [3, 5, 6, 7, 11])
+def test_hot_launch_never_has_more_workgroups_than_cus(pkg, orc, dev, num_slabs):
+    """One LDS table per CU: a hot launch of 258 workgroups on 256 CUs would run its last two alone."""
+    g = pkg.graphs
+    rp, ci, _ = g.generate("chunglu:n=60000,nnz=40000000,gamma=2.1,dmax=20000", seed=3)
+    n, K = rp.size - 1, 16
+    val = g.fill_uniform_f32(ci.size, 5, 0.0, 1.0)
+    X = g.fill_uniform_f32(n * K, 6, -1.0, 1.0).reshape(n, K)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    slab_cols = -(-(-(-n // num_slabs)) // 64) * 64
+    plan = pkg.spmm.Plan(csr, K, tiling="force", slab_bytes=slab_cols * K * 4, hot="force")
+    i = plan.info
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    assert i.num_slabs == num_slabs and i.hot_rows == 1728
+    assert min(cus, i.hot_waves // 16) - num_slabs < i.hot_blocks <= cus  # all CUs busy, none twice
+    (d_X,) = to_dev(dev, X)
+    Y = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    plan.close()
+
+
 def test_power_law_graph_auto_plan(pkg, orc, dev):
     g = pkg.graphs
     rp, ci, _ = g.generate("chunglu:n=100000,nnz=20000000,gamma=2.1,dmax=9000", seed=2)
