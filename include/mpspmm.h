@@ -74,7 +74,8 @@ int mps_num_partitions(int n_rows, int nnz, int cost, int *P_out);
  * items on; and never fewer than about 512 items per wavefront, i.e. at least
  * 512 / partitions per wavefront for the given K and element size (32 at
  * K = 16 fp32, 128 at K = 64, 512 at K = 256: the carry-out records of a
- * wavefront are 8 K bytes, so wide rows want few of them). */
+ * wavefront are 8 K bytes, so wide rows want few of them); 1,024 items per
+ * wavefront where the rows hold 32 nonzeros or more on average. */
 int mps_default_cost(int n_rows, int nnz, int K, int elem_bytes, int *cost_out);
 
 /* Merge items per partition, src/MergePathSpMM.cu:327-328:

@@ -748,9 +748,15 @@ int mps_default_cost(int n_rows, int nnz, int K, int elem_bytes, int *cost_out)
     if (!cost_out || n_rows < 0 || nnz < 0 || K <= 0 || (elem_bytes != 2 && elem_bytes != 4)) return MPS_ERR_INVALID_ARG;
     const int64_t total = (int64_t)n_rows + 1 + nnz;
     const int by_size = total >= (1 << 27) ? 128 : total >= (1 << 25) ? 64 : 32;
-    // a wavefront should have some 512 merge items whatever number of partitions it holds
+    // A wavefront should have some 512 merge items whatever number of partitions it holds,
+    // twice that where rows are long (32 nonzeros and more on average).  Measured on MI355X:
+    // R-MAT graphs (15 per row) run best at 512 items per wavefront for every K (scale 22, fp16,
+    // K = 64: cost 64 1.23 ms, 128 1.27 ms, 256 1.33 ms); the 232,965-row power-law graph (492
+    // per row) at 1,024 or more (K = 32 fp32: cost 64 0.99 ms, 128 0.93 ms; fp16 K = 64: cost 64
+    // 1.10 ms, 128 0.99 ms), K = 16 fp32 at its 16 x 64 either way.
     const int groups = mps_make_lane_shape(K, elem_bytes).groups;
-    const int by_width = 512 / groups;  // 32 (16 groups) .. 512 (one group)
+    const bool long_rows = n_rows > 0 && (int64_t)nnz >= 32 * (int64_t)n_rows;
+    const int by_width = (long_rows ? 1024 : 512) / groups;  // 32 (16 groups, short rows) .. 1024 (one group, long rows)
     *cost_out = by_size > by_width ? by_size : by_width;
     return MPS_OK;
 }

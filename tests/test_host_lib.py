@@ -57,6 +57,9 @@ def test_num_partitions_matches_oracle(pkg, orc):
     # wide rows: fewer partitions per wavefront, so more items each
     assert dc(1 << 20, 16086273, 64, 4) == 128 and dc(1 << 20, 16086273, 64, 2) == 64 and dc(4096, 32731, 256, 4) == 512
     assert dc(1 << 20, 16086273, 128, 4) == 256
+    # long rows (32 nonzeros and more on average): twice the items per wavefront
+    assert dc(232965, 114604189, 32, 4) == 128 and dc(232965, 114604189, 64, 2) == 128 and dc(232965, 114604189, 64, 4) == 256
+    assert dc(100000, 20000000) == 64 and dc(100000, 3100000) == 32
 
 
 def test_max_threads_per_wave(pkg):
