@@ -95,6 +95,16 @@ struct XOps<half_t, 8> {
 };
 
 template <>
+struct XOps<half_t, 4> {
+    using Raw = half4_t;
+    static __device__ __forceinline__ void fma(float (&acc)[4], float v, const Raw &r)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(v, (float)r[i], acc[i]);
+    }
+};
+
+template <>
 struct XOps<half_t, 1> {
     using Raw = half_t;
     static __device__ __forceinline__ void fma(float (&acc)[1], float v, const Raw &r)
@@ -928,6 +938,10 @@ int launch_spmm_any(const int *row_ptr, const int *col_idx, const T *val, const 
 {
     if (sh.ls.vec == 1)
         return launch_spmm<T, TOut, 1>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, pl, sh, ws, phases, st);
+    if constexpr (sizeof(T) == 2) {
+        if (sh.ls.vec == 4)  // narrow fp16 rows: 8 bytes per lane
+            return launch_spmm<T, TOut, 4>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, pl, sh, ws, phases, st);
+    }
     return launch_spmm<T, TOut, 16 / (int)sizeof(T)>(row_ptr, col_idx, val, X, Y, nnz, K, P, cx, cy, pl, sh, ws,
                                                      phases, st);
 }

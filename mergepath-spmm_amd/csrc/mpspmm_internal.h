@@ -7,7 +7,7 @@
 // group in the comparison kernels); each of its lanes owns `vec` adjacent
 // output columns.
 struct mps_lane_shape {
-    int vec;         // columns per lane: 16 bytes worth (4 fp32 / 8 fp16) or 1
+    int vec;         // columns per lane: 16 bytes worth (4 fp32 / 8 fp16), 4 fp16 for narrow rows, or 1
     int lanes_log2;  // log2(lanes per group), lanes in 4..64
     int groups;      // lane-groups per wavefront = 64 / lanes
     int col_tiles;   // passes over the columns when K > lanes * vec
@@ -17,7 +17,7 @@ static inline mps_lane_shape mps_make_lane_shape(int K, int elem_bytes)
 {
     mps_lane_shape s;
     int vec = 16 / elem_bytes;
-    if (!(K % vec == 0 && K >= 4 * vec)) vec = 1;
+    if (!(K % vec == 0 && K >= 4 * vec)) vec = (K % 4 == 0 && K >= 16) ? 4 : 1;  // fp16, K = 16 .. 28: 8 bytes per lane
     int want = (K + vec - 1) / vec;
     int l2 = 2;
     while ((1 << l2) < want && l2 < 6) ++l2;

@@ -10,7 +10,7 @@ from gpu_util import check_fp16, check_fp32, make_csr, random_csr, to_dev
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("K", [8, 16, 32, 64, 100, 128, 256])
+@pytest.mark.parametrize("K", [8, 16, 20, 28, 32, 64, 100, 128, 256])  # 1, 4 (K = 16 .. 28) or 8 columns per lane
 def test_fp16_against_oracle(pkg, orc, dev, K):
     rng = np.random.default_rng(K)
     n = 700

@@ -64,7 +64,7 @@ def test_num_partitions_matches_oracle(pkg, orc):
 
 def test_max_threads_per_wave(pkg):
     table = {(16, 4): 16, (32, 4): 8, (64, 4): 4, (128, 4): 2, (256, 4): 1, (512, 4): 1, (8, 4): 8, (1, 4): 16,
-             (20, 4): 8, (17, 4): 2, (64, 2): 8, (32, 2): 16, (16, 2): 4, (128, 2): 4}
+             (20, 4): 8, (17, 4): 2, (64, 2): 8, (32, 2): 16, (16, 2): 16, (24, 2): 8, (12, 2): 4, (128, 2): 4}
     for (K, eb), want in table.items():
         assert pkg.graphs.max_threads_per_wave(K, eb) == want, (K, eb)
 
