@@ -285,7 +285,8 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     v = seg * n_rows + r, 2 * num_slabs segments), each is partitioned on
  *     its own, and the plan runs two launches of the same kernel.  Used for
  *     fp32 when a row of X has at most 64 bytes (K = 16; wider rows are
- *     cheaper through L2, fp16 gains nothing) and the gathers taken off the
+ *     cheaper through L2), for fp16 at most 32 bytes (K = 16; at K = 32 the
+ *     half-to-float conversions eat the gain), and when the gathers taken off the
  *     L2 path outweigh the second set of partial rows (on the 232,965-row
  *     power-law graph: from about 15 % of the nonzeros in hot columns);
  *     MPS_PLAN_FORCE_HOT lifts these limits.
@@ -319,7 +320,7 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_NO_TILING 1u    /* never tile                                  */
 #define MPS_PLAN_FORCE_TILING 2u /* tile with slab_bytes slabs whatever the shape */
 #define MPS_PLAN_NO_HOT 4u       /* never keep hot columns' rows of X in LDS     */
-#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros, rows of X are wider than 64 bytes or fp16 */
+#define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
 
 typedef struct mps_plan_info {
     int n_rows, nnz, K, elem_bytes, cost, threads_per_wave;

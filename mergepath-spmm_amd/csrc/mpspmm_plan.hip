@@ -510,8 +510,9 @@ int choose_hot_rows(int K, int eb, const SpmmShape &sh, bool force)
     // half the rows, and the hot launch loses (1.16 against 0.99 ms at K = 32).
     // fp16 rows of 64 bytes (K = 32): 8 conversions and 8 multiply-adds per lane and nonzero make the
     // hot launch ALU-bound; it runs as fast as the L2 path and costs a second set of partial rows
-    // (0.672 ms either way), so it is not used.
-    if (!force && ((size_t)K * eb > 64 || eb != 4)) return 0;
+    // (0.672 ms either way), so it is not used.  fp16 rows of 32 bytes (K = 16) have half the
+    // arithmetic per lane and twice the rows in the table: 0.555 against 0.659 ms.
+    if (!force && (size_t)K * eb > (eb == 4 ? 64u : 32u)) return 0;
     const size_t budget = 160 * 1024 - hot_static_lds(sh.ls.vec) - 2048;
     size_t rows = budget / ((size_t)K * eb);
     rows = rows / 64 * 64;

@@ -174,7 +174,7 @@ def test_plan_layout_matches_numpy(pkg, orc, dev, tiling, slab_bytes, cost, tpw,
 
 
 @pytest.mark.parametrize("K,dtype,hot_rows", [(16, np.float32, 1728), (32, np.float16, 1472), (32, np.float32, 832),
-                                              (64, np.float16, 704)])
+                                              (64, np.float16, 704), (16, np.float16, 3456)])
 def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
     """Slabs wider than the LDS table: part of every slab is hot, part cold."""
     g = pkg.graphs
