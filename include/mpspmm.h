@@ -303,7 +303,10 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *   the library's cost model prefers: gathers get cheaper with smaller slabs,
  *   every slab adds one fp32 partial row per row); num_slabs == 1 means
  *   tiling does not pay (X fits in L2, or a row holds too few nonzeros per
- *   slab).
+ *   slab).  Where X exceeds 24 MiB and rows hold 16 nonzeros or more on
+ *   average, mps_plan_create also looks at the matrix: it counts the nonzeros
+ *   per column and, if they are concentrated in few columns (which then stay
+ *   in L2 by themselves), may take slabs of 12 or 24 MiB instead.
  * mps_plan_create: d_val is fp32 (elem_bytes 4) or fp16 (2); cost and tpw as
  *   for mps_num_partitions / mps_spmm_f32.  Synchronises the stream.
  * mps_plan_set_values: the nonzero values changed, the pattern did not.

@@ -63,38 +63,102 @@ constexpr size_t kDefaultSlabBytes = 3u << 20;
 // 2 M rows and 60 to 200 M nonzeros, K = 16 to 64.
 //   * A gather costs one L1->L2 request per 128 bytes of a row of X, and the
 //     time per request depends on how much of X the wavefronts that run
-//     together spread their gathers over: 5.3 ps when that is a 3 MiB slab
-//     (the L2 of an XCD serves it), 6.5 ps for 6 MiB, 9.4 ps for 15 MiB,
-//     11.7 ps for 32 MiB, 14 ps for 64 MiB, 16 ps for 128 MiB, 17.5 ps beyond
-//     (power-law graphs; uniform graphs are the same up to 6 MiB and up to a
-//     third slower beyond, which is why larger slabs are left to the tuner).
+//     together spread their gathers over, and on how unevenly: with a 3 MiB
+//     slab (the L2 of an XCD serves it) 5 ps whatever the matrix; with 12 MiB
+//     6.8 ps on a power-law graph, whose popular columns stay in L2, and
+//     11.7 ps on a uniform one; the tables below hold both ends.
+//   * Skew is measured as the share of the nonzeros that lie in the busiest
+//     tenth of the columns: 0.11 for a uniform graph, 0.54 to 0.65 for the
+//     power-law graphs (exponent 2.1) measured, 0.41 and 0.31 for exponents
+//     2.6 and 3.0; in between, the two tables are mixed (skew_from_share).  Unknown skew (negative): the power-law table, which
+//     is the optimistic one for the untiled plan and so the cautious one for
+//     tiling, and no slabs beyond 6 MiB.
 //   * Every virtual row costs its fp32 partial row written once and read once:
 //     2.8 ps per element of the row (45 ps at K = 16).
 // ---------------------------------------------------------------------------
-double request_ps(double table_bytes)
+double request_ps(double table_bytes, double skew, bool tiled)
 {
-    static const double mib[] = {3, 6, 15, 32, 64, 128, 256};
-    static const double ps[] = {5.3, 6.5, 9.4, 11.7, 14.0, 16.0, 17.5};
+    // slabs of a tiled plan (measured at 3 .. 24 MiB) and the whole of X in an untiled one
+    // (measured at 15 .. 128 MiB) are not the same curve: keep both
+    static const double mib_t[] = {3, 6, 12, 24, 48, 96, 192, 384};
+    static const double skewed_t[] = {5.3, 6.4, 6.8, 8.8, 11.7, 14.0, 16.0, 17.5};
+    static const double uniform_t[] = {5.0, 6.9, 11.7, 15.0, 17.0, 18.5, 19.0, 19.5};
+    static const double mib_u[] = {3, 6, 15, 32, 64, 128, 256, 512};
+    static const double skewed_u[] = {5.3, 6.5, 9.4, 11.7, 14.0, 16.0, 17.5, 17.5};
+    static const double uniform_u[] = {5.0, 6.9, 13.7, 16.5, 18.5, 19.0, 19.5, 19.5};
+    const double *mib = tiled ? mib_t : mib_u, *skewed = tiled ? skewed_t : skewed_u, *uniform = tiled ? uniform_t : uniform_u;
+    const double w = skew < 0 ? 1.0 : skew;
     const double m = table_bytes / (1024.0 * 1024.0);
-    if (m <= mib[0]) return ps[0];
-    for (int i = 1; i < 7; ++i)
+    auto at = [&](int i) { return w * skewed[i] + (1.0 - w) * uniform[i]; };
+    if (m <= mib[0]) return at(0);
+    for (int i = 1; i < 8; ++i)
         if (m <= mib[i]) {
             const double t = std::log2(m / mib[i - 1]) / std::log2(mib[i] / mib[i - 1]);
-            return ps[i - 1] + t * (ps[i] - ps[i - 1]);
+            return at(i - 1) + t * (at(i) - at(i - 1));
         }
-    return ps[6];
+    return at(7);
 }
 constexpr double kPartialPsPerElement = 2.8;
 
+// share of the nonzeros in the busiest tenth of the columns -> 0 (uniform) .. 1 (as skewed as the measured power-law graphs)
+double skew_from_share(double top_tenth_share)
+{
+    // measured weights of the power-law table at 12 MiB slabs: share 0.63 -> 1, 0.59 -> 0.8, 0.41 -> 0.5, 0.31 -> 0.3, 0.11 -> 0
+    const double s = (top_tenth_share - 0.11) / (0.63 - 0.11);
+    return s <= 0 ? 0 : s >= 1 ? 1 : std::pow(s, 1.3);
+}
+
 // Modelled time (ps) of one product with X cut into slabs of slab_cols columns (num_slabs == 1: untiled).
-double modelled_ps(int n_rows, int nnz, int K, int elem_bytes, int num_slabs, int slab_cols)
+double modelled_ps(int n_rows, int nnz, int K, int elem_bytes, int num_slabs, int slab_cols, double skew)
 {
     const double row_bytes = (double)K * elem_bytes;
     const double requests = std::ceil(row_bytes / 128.0);
     const double table = (double)(num_slabs > 1 ? slab_cols : n_rows) * row_bytes;
-    double t = (double)nnz * requests * request_ps(table);
+    double t = (double)nnz * requests * request_ps(table, skew, num_slabs > 1);
     if (num_slabs > 1) t += (double)num_slabs * n_rows * K * kPartialPsPerElement;
     return t;
+}
+
+// The cheapest of {untiled, slabs of slab_bytes} or, with slab_bytes == 0, of
+// {untiled, 3 MiB, 6 MiB} and, when the skew is known, {12 MiB, 24 MiB}.  A
+// candidate must leave the rows of a slab runs long enough to stream (>= 4
+// nonzeros per row and slab on average) and beat the untiled plan by 5 %.
+void pick_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, double skew, int *num_slabs_out,
+                     int *slab_cols_out)
+{
+    const uint64_t row_b = (uint64_t)K * elem_bytes;
+    const uint64_t x_bytes = (uint64_t)n_rows * row_b;
+    int slabs = 1, cols = n_rows > 0 ? n_rows : 1;
+    size_t sizes[4] = {slab_bytes ? slab_bytes : kDefaultSlabBytes, 0, 0, 0};
+    if (!slab_bytes) {
+        sizes[1] = 2 * kDefaultSlabBytes;
+        if (skew >= 0) {
+            sizes[2] = 4 * kDefaultSlabBytes;
+            sizes[3] = 8 * kDefaultSlabBytes;
+        }
+    }
+    if (x_bytes > kDefaultSlabBytes && n_rows > 0) {
+        double best = 0.95 * modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows, skew);
+        for (size_t sb : sizes) {
+            if (sb == 0) continue;
+            uint64_t want = (x_bytes + sb - 1) / sb;
+            if (want < 2) continue;
+            if (want > 4096) want = 4096;
+            uint64_t per = ((uint64_t)n_rows + want - 1) / want;
+            per = (per + 63) / 64 * 64;
+            const uint64_t s2 = ((uint64_t)n_rows + per - 1) / per;
+            if (s2 < 2 || (double)nnz / ((double)n_rows * (double)s2) < 4.0) continue;
+            if (s2 * n_rows + 1 + (uint64_t)nnz > (uint64_t)INT_MAX) continue;
+            const double t = modelled_ps(n_rows, nnz, K, elem_bytes, (int)s2, (int)per, skew);
+            if (t < best) {
+                best = t;
+                slabs = (int)s2;
+                cols = (int)per;
+            }
+        }
+    }
+    *num_slabs_out = slabs;
+    *slab_cols_out = cols;
 }
 
 // ---------------------------------------------------------------------------
@@ -601,8 +665,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             pl->num_slabs = (int)slabs;
             pl->slab_cols = (int)cols;
         } else {
-            rc = mps_tile_shape(n, nnz, K, eb, slab_bytes, &pl->num_slabs, &pl->slab_cols);
-            if (rc != MPS_OK) return rc;
+            pick_tile_shape(n, nnz, K, eb, slab_bytes, -1.0, &pl->num_slabs, &pl->slab_cols);
         }
     }
     BuildTmp t;
@@ -624,21 +687,48 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
         }                                                       \
     } while (0)
 
+    // Nonzeros per column, on the host (once, for whoever needs it below).
+    std::vector<int> h_deg;
+    auto column_histogram = [&]() -> int {
+        if (!h_deg.empty()) return MPS_OK;
+        h_deg.resize((size_t)n);
+        MPS_BUILD_TRY(tmp_alloc(&t.deg, (size_t)n));
+        MPS_BUILD_HIP(hipMemsetAsync(t.deg, 0, (size_t)n * sizeof(int), st));
+        hipLaunchKernelGGL(col_histogram_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st, d_col_idx,
+                           nnz, t.deg);
+        MPS_BUILD_HIP(hipGetLastError());
+        MPS_BUILD_HIP(hipMemcpyAsync(h_deg.data(), t.deg, (size_t)n * sizeof(int), hipMemcpyDeviceToHost, st));
+        MPS_BUILD_HIP(hipStreamSynchronize(st));
+        return MPS_OK;
+    };
+
+    // 1b. Slabs of 12 and 24 MiB pay on skewed matrices only: where X is large enough for them
+    // to matter, measure the skew (share of the nonzeros in the busiest tenth of the columns)
+    // and choose again.
+    if (!(flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING)) && slab_bytes == 0 && n >= 10 &&
+        (uint64_t)n * K * eb > 8 * kDefaultSlabBytes && (long long)nnz >= 16LL * n) {
+        MPS_BUILD_TRY(column_histogram());
+        std::vector<int> d(h_deg);
+        const size_t tenth = d.size() / 10;
+        std::nth_element(d.begin(), d.begin() + (long)tenth, d.end(), [](int a, int b) { return a > b; });
+        long long top = 0;
+        for (size_t i = 0; i < tenth; ++i) top += d[i];
+        pick_tile_shape(n, nnz, K, eb, 0, skew_from_share((double)top / (double)nnz), &pl->num_slabs, &pl->slab_cols);
+    }
+
     // 2. hot columns of every slab (tiled plans, shapes the hot kernel supports)
     int hot_rows = 0;
     std::vector<int> h_hot_cols;
     if (pl->num_slabs > 1 && !(flags & MPS_PLAN_NO_HOT)) {
         hot_rows = choose_hot_rows(K, eb, pl->shape, (flags & MPS_PLAN_FORCE_HOT) != 0);
+        // Slabs beyond the L2 live on the hits of their popular columns; taking exactly those
+        // columns out leaves the cold launch with the misses (500,000-row power-law graph,
+        // 3 slabs of 10 MiB: 0.81 ms with hot columns, 0.79 ms without).
+        if (!(flags & MPS_PLAN_FORCE_HOT) && (uint64_t)pl->slab_cols * K * eb > (4u << 20)) hot_rows = 0;
         if (2LL * pl->num_slabs * n + 1 + nnz > INT_MAX) hot_rows = 0;
         if (hot_rows > 0) {
-            std::vector<int> h_deg((size_t)n), h_slot;
-            MPS_BUILD_TRY(tmp_alloc(&t.deg, (size_t)n));
-            MPS_BUILD_HIP(hipMemsetAsync(t.deg, 0, (size_t)n * sizeof(int), st));
-            hipLaunchKernelGGL(col_histogram_kernel, dim3((unsigned)(((long long)nnz + 255) / 256)), dim3(256), 0, st,
-                               d_col_idx, nnz, t.deg);
-            MPS_BUILD_HIP(hipGetLastError());
-            MPS_BUILD_HIP(hipMemcpyAsync(h_deg.data(), t.deg, (size_t)n * sizeof(int), hipMemcpyDeviceToHost, st));
-            MPS_BUILD_HIP(hipStreamSynchronize(st));
+            std::vector<int> h_slot;
+            MPS_BUILD_TRY(column_histogram());
             pl->hot_nnz = select_hot_columns(h_deg, n, pl->num_slabs, pl->slab_cols, hot_rows, h_slot, h_hot_cols);
             // Worth a second launch and twice the partial rows?  Measured on MI355X at 64-byte rows,
             // graphs of 0.1 to 0.5 M rows with 3 to 45 M nonzeros in hot columns: a gather from LDS
@@ -961,35 +1051,7 @@ int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes
 {
     if (!num_slabs_out || !slab_cols_out || n_rows < 0 || nnz < 0 || K < 1) return MPS_ERR_INVALID_ARG;
     if (elem_bytes != 4 && elem_bytes != 2) return MPS_ERR_INVALID_ARG;
-    const uint64_t row_b = (uint64_t)K * elem_bytes;
-    const uint64_t x_bytes = (uint64_t)n_rows * row_b;
-    int slabs = 1, cols = n_rows > 0 ? n_rows : 1;
-    // Candidates: the given slab size, or 3 and 6 MiB.  A candidate must leave the
-    // rows of a slab runs long enough to stream (>= 4 nonzeros per row and slab on
-    // average) and beat the untiled plan by 5 % in the model above.
-    const size_t sizes[2] = {slab_bytes ? slab_bytes : kDefaultSlabBytes, slab_bytes ? 0 : 2 * kDefaultSlabBytes};
-    if (x_bytes > kDefaultSlabBytes && n_rows > 0) {
-        double best = 0.95 * modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows);
-        for (size_t sb : sizes) {
-            if (sb == 0) continue;
-            uint64_t want = (x_bytes + sb - 1) / sb;
-            if (want < 2) continue;
-            if (want > 4096) want = 4096;
-            uint64_t per = ((uint64_t)n_rows + want - 1) / want;
-            per = (per + 63) / 64 * 64;
-            const uint64_t s2 = ((uint64_t)n_rows + per - 1) / per;
-            if (s2 < 2 || (double)nnz / ((double)n_rows * (double)s2) < 4.0) continue;
-            if (s2 * n_rows + 1 + (uint64_t)nnz > (uint64_t)INT_MAX) continue;
-            const double t = modelled_ps(n_rows, nnz, K, elem_bytes, (int)s2, (int)per);
-            if (t < best) {
-                best = t;
-                slabs = (int)s2;
-                cols = (int)per;
-            }
-        }
-    }
-    *num_slabs_out = slabs;
-    *slab_cols_out = cols;
+    pick_tile_shape(n_rows, nnz, K, elem_bytes, slab_bytes, -1.0, num_slabs_out, slab_cols_out);
     return MPS_OK;
 }
 
@@ -1131,14 +1193,14 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f, 0};
     // slab sizes the model does not pick on its own: larger slabs pay on skewed graphs
     // (not those the model puts 50 % behind the untiled plan: thousands of slabs for a matrix with short rows)
-    const double untiled_ps = modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows);
+    const double untiled_ps = modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows, -1.0);
     for (unsigned long long mib : {3ull, 6ull, 12ull, 24ull}) {
         const unsigned long long row_bytes = (unsigned long long)K * elem_bytes;
         if ((unsigned long long)n_rows * row_bytes <= 2 * (mib << 20)) continue;
         unsigned long long cols = (mib << 20) / row_bytes / 64 * 64;  // what MPS_PLAN_FORCE_TILING makes of the size
         if (cols < 64) cols = 64;
         const unsigned long long slabs = ((unsigned long long)n_rows + cols - 1) / cols;
-        if (modelled_ps(n_rows, nnz, K, elem_bytes, (int)slabs, (int)cols) > 1.5 * untiled_ps) continue;
+        if (modelled_ps(n_rows, nnz, K, elem_bytes, (int)slabs, (int)cols, -1.0) > 1.5 * untiled_ps) continue;
         cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_HOT, 0.f, mib << 20};
     }
     hipEvent_t e0 = nullptr, e1 = nullptr;

@@ -60,6 +60,27 @@ def test_power_law_config_full_size(pkg, orc, dev):
     assert ((lhs - rhs).abs() <= bound).all()
 
 
+@pytest.mark.parametrize("spec,big_slabs", [("chunglu:n=1000000,nnz=60000000,gamma=2.1,dmax=30000", True),
+                                            ("er:n=1000000,deg=60", False)])
+def test_slab_size_follows_the_skew_of_the_matrix(pkg, orc, dev, spec, big_slabs):
+    """X of 64 MB: a power-law matrix gets slabs far beyond the L2 (its popular columns stay
+    cached), a uniform one slabs of at most 6 MiB; both plans give the right product."""
+    K = 16
+    rp, ci, val, X = workload(pkg, spec, K)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, K)
+    i = plan.info
+    slab_bytes = i.slab_cols * K * 4
+    assert i.num_slabs > 1 and i.hot_rows == 0
+    assert (slab_bytes > (8 << 20)) == big_slabs and (big_slabs or slab_bytes <= (6 << 20) + 4096)
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    plan.close()
+
+
 @pytest.mark.parametrize("K", [16, 256])
 def test_rmat_config_full_size(pkg, orc, dev, K):
     # config 4: R-MAT scale 20, edge factor 16, deduplicated; ends of the K sweep
