@@ -68,6 +68,11 @@ def main():
                          "(column-slab tiling where it pays / never / always)")
     ap.add_argument("--hot", default="auto", choices=["auto", "off", "force"],
                     help="hot columns of a tiled plan (their rows of X in LDS): where they pay / never / always")
+    ap.add_argument("--rowblock", default="auto", choices=["auto", "off", "force"],
+                    help="row-block plan (rows summed in LDS, popular columns' rows of X in LDS tables): where the "
+                         "library picks it / never / always")
+    ap.add_argument("--rb-steps", type=int, default=0, help="steps (LDS tables) of a row-block plan (0 = library default)")
+    ap.add_argument("--rb-table-rows", type=int, default=0, help="rows per LDS table of a row-block plan (0 = what fits)")
     ap.add_argument("--slab-bytes", type=int, default=0, help="slab size for tiling (0 = library default)")
     ap.add_argument("--tpw", type=int, default=0, help="partitions per wavefront (0 = full wavefront)")
     ap.add_argument("--seed", type=int, default=1)
@@ -112,7 +117,9 @@ def main():
     plan = None
     if args.mode != "plain":
         tiling = {"auto": "auto", "untiled": "off", "tiled": "force"}[args.mode]
-        plan = sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes, hot=args.hot)
+        plan_kw = dict(cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes, hot=args.hot,
+                       rowblock=args.rowblock, rowblock_steps=args.rb_steps, rowblock_table_rows=args.rb_table_rows)
+        plan = sp.Plan(csr, K, **plan_kw)
         P = plan.info.num_partitions
     else:
         sched = sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
@@ -177,7 +184,7 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     if plan is not None:
-        sp.Plan(csr, K, cost=cost, threads_per_wave=args.tpw, tiling=tiling, slab_bytes=args.slab_bytes, hot=args.hot).close()
+        sp.Plan(csr, K, **plan_kw).close()
     else:
         sp.generate_mp_sched(csr.row_ptr, nnz, cost=cost)
     torch.cuda.synchronize()
@@ -207,6 +214,10 @@ def main():
                    "max_row_degree": int(max_deg), "cost": cost, "partitions": P,
                    "threads_per_wave": args.tpw or g.max_threads_per_wave(K, eb), "seed": args.seed,
                    "layout": "plain CSR, no plan" if plan is None else
+                   ("row-block plan: %d blocks, %d steps x %d table rows, %.1f %% of the nonzeros from LDS, %.0f MB"
+                    % (plan.info.rowblock_blocks, plan.info.rowblock_steps, plan.info.rowblock_table_rows,
+                       100.0 * plan.info.hot_nnz / max(nnz, 1), plan.info.device_bytes / 1e6))
+                   if plan.info.rowblock_steps > 0 else
                    ("plan: %d column slab(s) of %d, sliced, %.0f MB" % (plan.info.num_slabs, plan.info.slab_cols,
                                                                        plan.info.device_bytes / 1e6)) +
                    ("" if plan is None or plan.info.hot_rows == 0 else

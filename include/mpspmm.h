@@ -298,6 +298,22 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *     by side, so that a wavefront stages a round with one contiguous load.
  *   - The workspace (partial rows, carry-out records).
  *
+ * Row-block plans (fp32, K = 16: a row of X is 64 bytes, half a cache line, so
+ * every gather through L2 costs a full request for half its payload).  For
+ * matrices whose rows are long (hundreds of nonzeros on average) the plan is
+ * built differently: rows are cut into contiguous blocks of about equal
+ * nonzero count, one per 1,024-thread workgroup, whose output rows are summed
+ * in LDS and written to Y once -- no partial rows, no carry-out records, one
+ * kernel.  Columns are dealt to `steps` steps: the steps * table_rows columns
+ * with the most nonzeros are gathered from a per-step LDS table of rows of X,
+ * the others through L2, a contiguous range of column ids per step.  Inside a
+ * (block, step) the nonzeros are cut into 16 equal runs (one per wavefront)
+ * and a wavefront's hot and cold nonzeros are each dealt evenly to its 16
+ * lane-groups.  Results are deterministic.  The layout is built on the host
+ * (the CSR arrays are copied back once, at creation).  mps_plan_create picks
+ * this kind of plan by itself where its model says it wins;
+ * MPS_PLAN_NO_ROWBLOCK / MPS_PLAN_FORCE_ROWBLOCK override that.
+ *
  * mps_tile_shape: the slab count and width mps_plan_create chooses for an X
  *   of n_rows x K elements (slab_bytes = 0: slabs of 3 or 6 MiB, whichever
  *   the library's cost model prefers: gathers get cheaper with smaller slabs,
@@ -324,6 +340,10 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_FORCE_TILING 2u /* tile with slab_bytes slabs whatever the shape */
 #define MPS_PLAN_NO_HOT 4u       /* never keep hot columns' rows of X in LDS     */
 #define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
+#define MPS_PLAN_NO_ROWBLOCK 16u    /* never build a row-block plan (see below)  */
+#define MPS_PLAN_FORCE_ROWBLOCK 32u /* row-block plan whatever the matrix looks like (fp32, K = 16 only) */
+#define MPS_PLAN_NO_SOURCES 64u     /* do not keep the original nonzero index of every slot: saves 4 bytes per
+                                       nonzero of device memory; mps_plan_set_values then returns MPS_ERR_UNSUPPORTED */
 
 typedef struct mps_plan_info {
     int n_rows, nnz, K, elem_bytes, cost, threads_per_wave;
@@ -340,7 +360,24 @@ typedef struct mps_plan_info {
     int mark_shift;                /* > 0: SLICE_COLS entries are column | row_ends << mark_shift */
     int hot_mark_shift;            /* the same for the entries of the hot wavefronts (column = LDS slot) */
     int hot_blocks;                /* workgroups of the hot launch: at most one per CU unless there are more hot segments than CUs */
+    /* row-block plans (rowblock_steps > 0); the fields above that describe slabs, partitions and slices are then 0 / 1 */
+    int rowblock_steps;            /* T: steps, one LDS table each                */
+    int rowblock_table_rows;       /* H: rows of X per LDS table                  */
+    int rowblock_blocks;           /* row blocks = workgroups                     */
+    int rowblock_acc_rows;         /* rows of LDS accumulators per workgroup      */
+    long long rowblock_hot_slots;  /* entries of the hot stream incl. padding     */
+    long long rowblock_cold_slots; /* entries of the cold stream incl. padding    */
 } mps_plan_info;
+
+/* Optional parameters of mps_plan_create_ex; zero means "the library chooses". */
+typedef struct mps_plan_options {
+    unsigned flags;          /* MPS_PLAN_*                                       */
+    size_t slab_bytes;       /* column-slab size of a tiled plan                 */
+    int rowblock_steps;      /* T of a row-block plan                            */
+    int rowblock_table_rows; /* H of a row-block plan                            */
+    int rowblock_block_rows; /* most rows per row block                          */
+    int rowblock_blocks_per_round; /* row blocks are made in multiples of this (0: the number of CUs) */
+} mps_plan_options;
 
 enum {
     MPS_PLAN_ARRAY_VROW_PTR = 0,   /* int[num_slabs * n_rows + 1]                 */
@@ -350,7 +387,16 @@ enum {
     MPS_PLAN_ARRAY_SLICE_COLS = 4, /* int[slice_slots]                            */
     MPS_PLAN_ARRAY_SLICE_SRC = 5,  /* int[slice_slots]: original nonzero index, -1 = padding */
     MPS_PLAN_ARRAY_SLICE_VALS = 6, /* elem_bytes * slice_slots                    */
-    MPS_PLAN_ARRAY_HOT_COLS = 7    /* int[num_slabs * hot_rows]: column of each LDS slot, -1 = unused */
+    MPS_PLAN_ARRAY_HOT_COLS = 7,   /* int[num_slabs * hot_rows]: column of each LDS slot, -1 = unused */
+    /* row-block plans */
+    MPS_PLAN_ARRAY_RB_BLOCK_ROW = 8,  /* int[blocks + 1]: first row of every block  */
+    MPS_PLAN_ARRAY_RB_HOT_COLS = 9,   /* int[steps * table_rows]: column of each table slot, -1 = unused */
+    MPS_PLAN_ARRAY_RB_META = 10,      /* int[blocks * steps * 16 * 4]: {hot entries, cold entries, first local row, 0} per wavefront */
+    MPS_PLAN_ARRAY_RB_WAVE_BASE = 11, /* long long[blocks * 16 * 2]: first round of each wavefront's hot / cold stream */
+    MPS_PLAN_ARRAY_RB_HOT = 12,       /* 8 bytes x hot slots: {index | rows_advanced << bits, value} */
+    MPS_PLAN_ARRAY_RB_COLD = 13,      /* 8 bytes x cold slots                       */
+    MPS_PLAN_ARRAY_RB_HOT_SRC = 14,   /* int[hot slots]: original nonzero index, -1 = padding */
+    MPS_PLAN_ARRAY_RB_COLD_SRC = 15   /* int[cold slots]                            */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,
@@ -358,6 +404,9 @@ int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes
 int mps_plan_create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz,
                     int K, int elem_bytes, int cost, int tpw, unsigned flags, size_t slab_bytes,
                     void *stream, mps_plan **plan_out);
+int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz,
+                       int K, int elem_bytes, int cost, int tpw, const mps_plan_options *options,
+                       void *stream, mps_plan **plan_out);
 void mps_plan_destroy(mps_plan *plan);
 int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info);
 int mps_plan_set_values(mps_plan *plan, const void *d_val, void *stream);
@@ -365,6 +414,19 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
 int mps_plan_spmm_f32(const mps_plan *plan, const float *d_X, float *d_Y, void *stream);
 int mps_plan_spmm_f16(const mps_plan *plan, const uint16_t *d_X, uint16_t *d_Y, void *stream);
 int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsigned phases, void *stream);
+
+/* The layout of a row-block plan, built from host arrays without a GPU: what
+ * mps_plan_create_ex uploads.  For inspection, tests and callers that prepare
+ * plans offline.  options: rowblock_* fields as for mps_plan_create_ex
+ * (rowblock_blocks_per_round 0 = 256).  mps_rowblock_layout_array hands out a
+ * pointer into the layout (valid until it is freed) for MPS_PLAN_ARRAY_RB_*. */
+typedef struct mps_rowblock_layout mps_rowblock_layout;
+int mps_rowblock_layout_build(const int *row_ptr, const int *col_idx, const float *val, int n_rows, int nnz,
+                              int K, const mps_plan_options *options, mps_rowblock_layout **layout_out);
+int mps_rowblock_layout_info(const mps_rowblock_layout *layout, mps_plan_info *info);
+int mps_rowblock_layout_array(const mps_rowblock_layout *layout, int which, const void **data_out,
+                              size_t *bytes_out);
+void mps_rowblock_layout_free(mps_rowblock_layout *layout);
 
 /* Parameter sweep for one matrix and K — what the reference leaves to the
  * user's hand (cost and partitions per warp are command-line arguments,

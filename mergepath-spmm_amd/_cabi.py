@@ -30,8 +30,13 @@ MPS_PLAN_NO_TILING = 1
 MPS_PLAN_FORCE_TILING = 2
 MPS_PLAN_NO_HOT = 4
 MPS_PLAN_FORCE_HOT = 8
+MPS_PLAN_NO_ROWBLOCK = 16
+MPS_PLAN_FORCE_ROWBLOCK = 32
+MPS_PLAN_NO_SOURCES = 64
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
- MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS) = range(8)
+ MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
+ MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
+ MPS_PLAN_ARRAY_RB_HOT, MPS_PLAN_ARRAY_RB_COLD, MPS_PLAN_ARRAY_RB_HOT_SRC, MPS_PLAN_ARRAY_RB_COLD_SRC) = range(16)
 
 
 class PlanInfo(ctypes.Structure):
@@ -41,7 +46,18 @@ class PlanInfo(ctypes.Structure):
                [("total_rounds", ctypes.c_longlong), ("slice_slots", ctypes.c_longlong),
                 ("device_bytes", ctypes.c_size_t), ("num_segments", ctypes.c_int), ("hot_rows", ctypes.c_int),
                 ("hot_waves", ctypes.c_int), ("hot_nnz", ctypes.c_longlong), ("hot_cost", ctypes.c_int), ("mark_shift", ctypes.c_int),
-                ("hot_mark_shift", ctypes.c_int), ("hot_blocks", ctypes.c_int)]
+                ("hot_mark_shift", ctypes.c_int), ("hot_blocks", ctypes.c_int),
+                ("rowblock_steps", ctypes.c_int), ("rowblock_table_rows", ctypes.c_int),
+                ("rowblock_blocks", ctypes.c_int), ("rowblock_acc_rows", ctypes.c_int),
+                ("rowblock_hot_slots", ctypes.c_longlong), ("rowblock_cold_slots", ctypes.c_longlong)]
+
+
+class PlanOptions(ctypes.Structure):
+    """struct mps_plan_options"""
+    _fields_ = [("flags", ctypes.c_uint), ("slab_bytes", ctypes.c_size_t), ("rowblock_steps", ctypes.c_int),
+                ("rowblock_table_rows", ctypes.c_int), ("rowblock_block_rows", ctypes.c_int),
+                ("rowblock_blocks_per_round", ctypes.c_int)]
+
 
 class TuneResult(ctypes.Structure):
     """struct mps_tune_result"""
@@ -87,6 +103,12 @@ PROTOTYPES = {
                                  ctypes.c_uint, _vp]),
     "mps_tile_shape": (_i, [_i, _i, _i, _i, _sz, c_int_p, c_int_p]),
     "mps_plan_create": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_uint, _sz, _vp, ctypes.POINTER(_vp)]),
+    "mps_plan_create_ex": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.POINTER(PlanOptions), _vp,
+                                ctypes.POINTER(_vp)]),
+    "mps_rowblock_layout_build": (_i, [_vp, _vp, _vp, _i, _i, _i, ctypes.POINTER(PlanOptions), ctypes.POINTER(_vp)]),
+    "mps_rowblock_layout_info": (_i, [_vp, _vp]),
+    "mps_rowblock_layout_array": (_i, [_vp, _i, ctypes.POINTER(_vp), ctypes.POINTER(_sz)]),
+    "mps_rowblock_layout_free": (None, [_vp]),
     "mps_plan_destroy": (None, [_vp]),
     "mps_plan_get_info": (_i, [_vp, _vp]),
     "mps_plan_set_values": (_i, [_vp, _vp, _vp]),

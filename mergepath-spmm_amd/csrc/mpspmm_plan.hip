@@ -15,6 +15,7 @@
 //      group);
 //   4. the workspace of the SpMM (per-slab partial rows, carry-out records).
 #include "mpspmm_device.hpp"
+#include "mpspmm_rowblock.hpp"
 
 #include <algorithm>
 #include <cmath>
@@ -49,6 +50,8 @@ struct mps_plan {
     int mark_shift = 0, hot_mark_shift = 0;  // row marks sit above this bit of a column entry (0: none)
     int *hot_block_wave = nullptr;  // [hot_blocks + 1] first wave of every hot workgroup
     int hot_blocks = 0;
+    bool keep_sources = true;       // slice_src is kept (mps_plan_set_values works)
+    mps_rb::DevicePlan *rb = nullptr;  // row-block plan: everything above about slabs and slices is unused
 };
 
 namespace {
@@ -516,6 +519,7 @@ int dev_alloc(mps_plan *pl, T **p, size_t count)
 void plan_free(mps_plan *pl)
 {
     if (!pl) return;
+    mps_rb::destroy(pl->rb);
     (void)hipFree(pl->vrow_ptr);
     (void)hipFree(pl->coord_x);
     (void)hipFree(pl->coord_y);
@@ -986,6 +990,13 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
         MPS_BUILD_HIP(hipGetLastError());
     }
     MPS_BUILD_TRY(plan_set_values(pl, d_val, st));
+    if (!pl->keep_sources) {
+        // only mps_plan_set_values reads the source indices again
+        MPS_BUILD_HIP(hipStreamSynchronize(st));
+        (void)hipFree(pl->slice_src);
+        pl->slice_src = nullptr;
+        pl->device_bytes -= (slots ? slots : 1) * sizeof(int);
+    }
 
     // 6. workspace
     pl->part_bytes = part_bytes_for(n, pl->num_segs, K);
@@ -1009,6 +1020,10 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     if (pl->n_rows == 0) return MPS_OK;
     if (!X || !Y) return MPS_ERR_INVALID_ARG;
     if (!aligned_to(X, 16) || !aligned_to(Y, 16)) return MPS_ERR_ALIGNMENT;
+    if (pl->rb) {
+        if constexpr (sizeof(T) == 4) return mps_rb::spmm(pl->rb, X, Y, phases, st);
+        else return MPS_ERR_INVALID_ARG;
+    }
     const T *vals = static_cast<const T *>(pl->slice_vals);
     void *carry = static_cast<char *>(pl->workspace) + pl->part_bytes;
     PlanLaunch how;
@@ -1042,6 +1057,18 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     return MPS_OK;
 }
 
+// Row-block plan or not.  Forced: yes.  Otherwise only for what the kernel is built for (fp32,
+// K = 16) and where it was measured to win on MI355X: long rows (the LDS tables are loaded once
+// per block and step, so a block must hold many nonzeros per table) and an X beyond the L2.
+bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, unsigned flags)
+{
+    if (flags & MPS_PLAN_FORCE_ROWBLOCK) return true;
+    if (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT)) return false;
+    if (elem_bytes != 4 || K != 16 || n_rows < 1) return false;
+    if ((uint64_t)n_rows * 64 <= (4u << 20) || n_rows > (1 << 22)) return false;
+    return (long long)nnz >= 128LL * n_rows;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1059,12 +1086,27 @@ int mps_plan_create(const int *d_row_ptr, const int *d_col_idx, const void *d_va
                     int elem_bytes, int cost, int tpw, unsigned flags, size_t slab_bytes, void *stream,
                     mps_plan **plan_out)
 {
+    mps_plan_options opt{};
+    opt.flags = flags;
+    opt.slab_bytes = slab_bytes;
+    return mps_plan_create_ex(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, cost, tpw, &opt, stream, plan_out);
+}
+
+int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n_rows, int nnz, int K,
+                       int elem_bytes, int cost, int tpw, const mps_plan_options *options, void *stream,
+                       mps_plan **plan_out)
+{
     if (!plan_out) return MPS_ERR_INVALID_ARG;
     *plan_out = nullptr;
     if (!d_row_ptr || n_rows < 0 || nnz < 0 || K < 1 || cost <= 0 || tpw < 0) return MPS_ERR_INVALID_ARG;
     if (elem_bytes != 4 && elem_bytes != 2) return MPS_ERR_INVALID_ARG;
     if (nnz > 0 && (!d_col_idx || !d_val)) return MPS_ERR_INVALID_ARG;
     if ((long long)n_rows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
+    mps_plan_options opt{};
+    if (options) opt = *options;
+    const unsigned flags = opt.flags;
+    const size_t slab_bytes = opt.slab_bytes;
+    if ((flags & MPS_PLAN_FORCE_ROWBLOCK) && (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING))) return MPS_ERR_INVALID_ARG;
     mps_plan *pl = new (std::nothrow) mps_plan;
     if (!pl) return MPS_ERR_UNSUPPORTED;
     pl->n_rows = n_rows;
@@ -1072,6 +1114,29 @@ int mps_plan_create(const int *d_row_ptr, const int *d_col_idx, const void *d_va
     pl->K = K;
     pl->elem_bytes = elem_bytes;
     pl->cost = cost;
+    pl->keep_sources = !(flags & MPS_PLAN_NO_SOURCES);
+    if (rowblock_wanted(n_rows, nnz, K, elem_bytes, flags)) {
+        if (elem_bytes != 4 || K != 16 || n_rows < 1) {
+            plan_free(pl);
+            return MPS_ERR_UNSUPPORTED;
+        }
+        mps_rb::BuildParams bp;
+        bp.steps = opt.rowblock_steps;
+        bp.table_rows = opt.rowblock_table_rows;
+        bp.block_rows = opt.rowblock_block_rows;
+        bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
+        bp.keep_src = pl->keep_sources;
+        int rc = mps_rb::create(d_row_ptr, d_col_idx, static_cast<const float *>(d_val), n_rows, nnz, K, bp,
+                                static_cast<hipStream_t>(stream), &pl->rb);
+        if (rc != MPS_OK) {
+            plan_free(pl);
+            return rc;
+        }
+        pl->device_bytes = mps_rb::device_bytes_of(pl->rb);
+        make_spmm_shape(n_rows, K, 1, 0, elem_bytes, pl->shape);
+        *plan_out = pl;
+        return MPS_OK;
+    }
     int rc;
     try {
         rc = plan_build(pl, d_row_ptr, d_col_idx, d_val, flags, slab_bytes, tpw, static_cast<hipStream_t>(stream));
@@ -1112,12 +1177,30 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->mark_shift = plan->mark_shift;
     info->hot_mark_shift = plan->hot_mark_shift;
     info->hot_blocks = plan->hot_blocks;
+    info->rowblock_steps = info->rowblock_table_rows = info->rowblock_blocks = info->rowblock_acc_rows = 0;
+    info->rowblock_hot_slots = info->rowblock_cold_slots = 0;
+    if (plan->rb) {
+        const mps_rb::Layout &L = mps_rb::layout_of(plan->rb);
+        info->num_slabs = 1;
+        info->slab_cols = plan->n_rows;
+        info->hot_nnz = L.hot_nnz;
+        info->mark_shift = L.cold_bits;
+        info->hot_mark_shift = L.hot_bits;
+        info->rowblock_steps = L.steps;
+        info->rowblock_table_rows = L.table_rows;
+        info->rowblock_blocks = L.num_blocks;
+        info->rowblock_acc_rows = L.acc_rows;
+        info->rowblock_hot_slots = L.hot_rounds * mps_rb::kRoundEntries;
+        info->rowblock_cold_slots = L.cold_rounds * mps_rb::kRoundEntries;
+    }
     return MPS_OK;
 }
 
 int mps_plan_set_values(mps_plan *plan, const void *d_val, void *stream)
 {
     if (!plan || (plan->nnz > 0 && !d_val)) return MPS_ERR_INVALID_ARG;
+    if (!plan->keep_sources) return MPS_ERR_UNSUPPORTED;
+    if (plan->rb) return mps_rb::set_values(plan->rb, static_cast<const float *>(d_val), static_cast<hipStream_t>(stream));
     return plan_set_values(plan, d_val, static_cast<hipStream_t>(stream));
 }
 
@@ -1133,14 +1216,19 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
     case MPS_PLAN_ARRAY_COORD_Y: src = plan->coord_y; have = ((size_t)plan->P + 1) * sizeof(int); break;
     case MPS_PLAN_ARRAY_WAVE_OFF: src = plan->wave_off; have = ((size_t)plan->shape.num_waves + 1) * sizeof(int); break;
     case MPS_PLAN_ARRAY_SLICE_COLS: src = plan->slice_cols; have = slots * sizeof(int); break;
-    case MPS_PLAN_ARRAY_SLICE_SRC: src = plan->slice_src; have = slots * sizeof(int); break;
+    case MPS_PLAN_ARRAY_SLICE_SRC: src = plan->slice_src; have = plan->slice_src ? slots * sizeof(int) : 0; break;
     case MPS_PLAN_ARRAY_SLICE_VALS: src = plan->slice_vals; have = slots * (size_t)plan->elem_bytes; break;
     case MPS_PLAN_ARRAY_HOT_COLS:
         src = plan->hot_cols;
         have = (size_t)(plan->hot_rows > 0 ? plan->num_slabs : 0) * (size_t)plan->hot_rows * sizeof(int);
         break;
-    default: return MPS_ERR_INVALID_ARG;
+    default:
+        if (!plan->rb) return MPS_ERR_INVALID_ARG;
+        src = mps_rb::device_array(plan->rb, which, &have);
+        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_COLD_SRC)) return MPS_ERR_INVALID_ARG;
+        break;
     }
+    if (plan->rb && which < MPS_PLAN_ARRAY_RB_BLOCK_ROW) return MPS_ERR_INVALID_ARG;
     if (bytes != have) return MPS_ERR_INVALID_ARG;
     if (have == 0) return MPS_OK;
     MPS_HIP_TRY(hipMemcpy(host_dst, src, have, hipMemcpyDeviceToHost));

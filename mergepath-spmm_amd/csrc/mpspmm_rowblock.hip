@@ -1,0 +1,515 @@
+// Row-block plans, device side: the kernel that walks the layout of
+// mpspmm_rowblock.hpp, and the plan object's device arrays.
+//
+// Same arithmetic as the reference kernel (src/MergePathSpMM.cu:426-477: one
+// fp32 accumulator per output column, a rounded product added per nonzero in
+// row order within a run), with explicit values in place of the degree product
+// (:450,:459-460); what differs is that the rows of X of the popular columns
+// are gathered from LDS, and that a block's output rows are summed in LDS
+// instead of through atomics on Y (:445,:477).
+#include "mpspmm_device.hpp"
+#include "mpspmm_rowblock.hpp"
+
+#include <new>
+
+namespace mps_rb {
+
+struct DevicePlan {
+    Layout host;  // the small tables stay filled; the streams are released after the upload
+    Entry *hot = nullptr, *cold = nullptr;
+    int *hot_src = nullptr, *cold_src = nullptr;
+    long long *wave_base = nullptr;
+    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr;
+    float *hot_x = nullptr;  // [T][H][16] rows of X of the hot columns, gathered per product
+    size_t lds_bytes = 0;
+    size_t device_bytes = 0;
+    size_t hot_slots = 0, cold_slots = 0;
+};
+
+namespace {
+
+// hot_x[t][slot][:] = X[hot_cols[t][slot]][:]  (zeros for unused slots)
+__global__ __launch_bounds__(256) void rb_gather_hot_kernel(const int *__restrict__ hot_cols,
+                                                             const float4 *__restrict__ X4,
+                                                             float4 *__restrict__ hot_x4, int slots)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= slots * 4) return;
+    const int c = hot_cols[i >> 2];
+    hot_x4[i] = c >= 0 ? X4[(size_t)c * 4 + (i & 3)] : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+constexpr int kThreads = kWaveSlots * 64;
+constexpr int kPrefetch = (kMaxTableRows * 4 + kThreads - 1) / kThreads;  // float4 per thread of one table
+
+// A lane's 16 bytes of a round: its entry of the lane-group's two windows {word A, value A, word B, value B}.
+__device__ __forceinline__ uint4 load_round(const Entry *p)
+{
+    typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+    u4_t t = __builtin_nontemporal_load(reinterpret_cast<const u4_t *>(p));
+    return make_uint4(t[0], t[1], t[2], t[3]);
+}
+
+__device__ __forceinline__ void add4(float4 &a, const float4 &b)
+{
+    a.x += b.x;
+    a.y += b.y;
+    a.z += b.z;
+    a.w += b.w;
+}
+
+// One lane-group's position in one of its two streams.
+struct Walk {
+    int row;     // block-local row of the nonzeros being summed
+    float a[4];  // sums of the current row
+};
+
+// Lane j of a lane-group (4 lanes) holds entry j of the group's window.  The other lanes read
+// it through a quad permute folded into the instruction that uses it (DPP): no LDS staging, no
+// separate move.  `word`/`val` were written long before (the window's load), so the two wait
+// states that a DPP read needs after a write of its source have passed.
+#define RB_QUAD(j) "quad_perm:[" #j "," #j "," #j "," #j "] row_mask:0xf bank_mask:0xf"
+template <int J>
+__device__ __forceinline__ unsigned and_from_lane(unsigned word, unsigned mask)
+{
+    unsigned r;
+    if constexpr (J == 0) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(0) : "=v"(r) : "v"(word), "v"(mask));
+    if constexpr (J == 1) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(1) : "=v"(r) : "v"(word), "v"(mask));
+    if constexpr (J == 2) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(2) : "=v"(r) : "v"(word), "v"(mask));
+    if constexpr (J == 3) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(3) : "=v"(r) : "v"(word), "v"(mask));
+    return r;
+}
+// a += val[lane J of the group] * x   (one fused multiply-add per column, as the compiler's fmaf)
+template <int J>
+__device__ __forceinline__ void fma_from_lane(float (&a)[4], float val, const float4 &x)
+{
+#define RB_FMAC(j)                                                                          \
+    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[0]) : "v"(val), "v"(x.x));         \
+    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[1]) : "v"(val), "v"(x.y));         \
+    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[2]) : "v"(val), "v"(x.z));         \
+    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[3]) : "v"(val), "v"(x.w));
+    if constexpr (J == 0) { RB_FMAC(0) }
+    if constexpr (J == 1) { RB_FMAC(1) }
+    if constexpr (J == 2) { RB_FMAC(2) }
+    if constexpr (J == 3) { RB_FMAC(3) }
+#undef RB_FMAC
+}
+#undef RB_QUAD
+
+// rounds (two windows per lane-group each) that a wavefront needs for n windows dealt to its 16 lane-groups
+__device__ __forceinline__ int rounds_of(int n) { return ((n >> 4) + ((n & 15) != 0) + 1) >> 1; }
+
+template <typename TOut>
+__global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restrict__ hot, const Entry *__restrict__ cold,
+                                                            const long long *__restrict__ wave_base,
+                                                            const int4 *__restrict__ meta,
+                                                            const int *__restrict__ block_row,
+                                                            const float4 *__restrict__ hot_x4,
+                                                            const float4 *__restrict__ X4, TOut *__restrict__ Y, int T,
+                                                            int H, int acc_rows, int hot_bits, int cold_bits)
+{
+    extern __shared__ __align__(16) char smem[];
+    float *table = reinterpret_cast<float *>(smem);                         // [H][16]
+    float *acc = table + (size_t)H * 16;                                    // [acc_rows][16]
+    float4 *stage = reinterpret_cast<float4 *>(acc + (size_t)acc_rows * 16);  // [16 waves][64]: the tails
+    float *slots = reinterpret_cast<float *>(stage + kWaveSlots * 64);      // [16 waves][16]
+    int *slot_row = reinterpret_cast<int *>(slots + kWaveSlots * 16);       // [16]
+    int *crows = slot_row + kWaveSlots;                                     // [16 waves][16 groups]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 2, s = lane & 3;
+    const int b = blockIdx.x;
+    const int row0 = block_row[b], nrows = block_row[b + 1] - row0;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 *table4 = reinterpret_cast<float4 *>(table);
+    float4 *acc4 = reinterpret_cast<float4 *>(acc);
+    const int4 *meta_b = meta + (size_t)b * T * kWaveSlots;
+
+    for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4;
+    if (tid < kWaveSlots * 16) slots[tid] = 0.f;
+    for (int i = tid; i < H * 4; i += kThreads) table4[i] = hot_x4[i];
+
+#define RB_PRE_LOAD(k) const float4 pre##k = tid + k * kThreads < H * 4 ? pre_src[tid + k * kThreads] : zero4;
+#define RB_PRE_STORE(k) if (tid + k * kThreads < H * 4) table4[tid + k * kThreads] = pre##k;
+    static_assert(kPrefetch == 6, "one RB_PRE_LOAD / RB_PRE_STORE per float4 of a table that a thread moves");
+
+    {
+        // ---- every wavefront walks its runs
+        long long cur_h = wave_base[((size_t)b * kWaveSlots + wave) * 2];
+        long long cur_c = wave_base[((size_t)b * kWaveSlots + wave) * 2 + 1];
+        float4 *st4 = stage + wave * 64;
+        float4 *my_slot4 = reinterpret_cast<float4 *>(slots + wave * 16) + s;
+        int *my_crows = crows + wave * 16;
+        // the masks live in vector registers (the DPP form of v_and takes no scalar operand); the
+        // empty asm keeps the compiler from re-creating them from scalars at every use
+        unsigned hmask = (1u << hot_bits) - 1u, cmask = (1u << cold_bits) - 1u, hot_hi = ~hmask, cold_hi = ~cmask;
+        asm volatile("" : "+v"(hmask), "+v"(cmask), "+v"(hot_hi), "+v"(cold_hi));
+        int4 m = meta_b[wave];
+        __syncthreads();
+
+        for (int t = 0; t < T; ++t) {
+            const int nh = __builtin_amdgcn_readfirstlane(m.x), nc = __builtin_amdgcn_readfirstlane(m.y);
+            const int first_row = __builtin_amdgcn_readfirstlane(m.z);
+            // next step's counts: in flight while this step is walked
+            const int4 m_next = meta_b[(size_t)min(t + 1, T - 1) * kWaveSlots + wave];
+            int slot_first = 0;  // wave 0 adds the slots after the barrier: the first rows of all runs of this step
+            if (wave == 0) slot_first = meta_b[(size_t)t * kWaveSlots + min(g, kWaves - 1)].z;
+
+            const int rounds_h = rounds_of(nh), rounds_c = rounds_of(nc);
+            const int full_h = nh >> 5, full_c = nc >> 5;  // rounds in which every lane-group holds two windows
+            const int len_h = (nh >> 4) + (g < (nh & 15)), len_c = (nc >> 4) + (g < (nc & 15));  // windows of this lane-group
+            Walk wh, wc;
+            wh.row = wc.row = first_row;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) wh.a[i] = wc.a[i] = 0.f;
+
+            // A window (four nonzeros) lies in one row; its first entry says how many rows the
+            // group's run advanced in front of it.  A finished row is added to its LDS
+            // accumulator there and then, with a plain read-add-write: among the lane-groups of
+            // this wavefront only this one adds to that row while the runs are walked (the others
+            // that hold a part of it keep it until after the walk, see tails below), and no other
+            // wavefront adds to it directly - except for the first row of the wavefront's run,
+            // which goes to the wavefront's slot instead.  (A run's first window counts its rows
+            // from the wavefront's first row: the sums that this "row end" adds are zeros.)
+            auto row_end = [&](Walk &w, unsigned adv) {
+                float4 *dst = w.row == first_row ? my_slot4 : acc4 + (size_t)w.row * 4 + s;
+                float4 o = *dst;
+                o.x += w.a[0];
+                o.y += w.a[1];
+                o.z += w.a[2];
+                o.w += w.a[3];
+                *dst = o;
+                w.row += (int)adv;
+                w.a[0] = w.a[1] = w.a[2] = w.a[3] = 0.f;
+            };
+            auto hot_gather = [&](unsigned word, float4 (&x)[kWin]) {
+                x[0] = table4[and_from_lane<0>(word, hmask) * 4 + s];
+                x[1] = table4[and_from_lane<1>(word, hmask) * 4 + s];
+                x[2] = table4[and_from_lane<2>(word, hmask) * 4 + s];
+                x[3] = table4[and_from_lane<3>(word, hmask) * 4 + s];
+            };
+            auto cold_gather = [&](unsigned word, float4 (&x)[kWin]) {
+                const char *xb = reinterpret_cast<const char *>(X4);
+                x[0] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<0>(word, cmask) << 6) | (unsigned)(s << 4)));
+                x[1] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<1>(word, cmask) << 6) | (unsigned)(s << 4)));
+                x[2] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<2>(word, cmask) << 6) | (unsigned)(s << 4)));
+                x[3] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<3>(word, cmask) << 6) | (unsigned)(s << 4)));
+            };
+            auto window = [&](Walk &w, unsigned word, unsigned valbits, const float4 (&x)[kWin], unsigned himask, int bits) {
+                const unsigned hi = and_from_lane<0>(word, himask);
+                if (hi != 0) row_end(w, hi >> bits);
+                const float v = __uint_as_float(valbits);
+                fma_from_lane<0>(w.a, v, x[0]);
+                fma_from_lane<1>(w.a, v, x[1]);
+                fma_from_lane<2>(w.a, v, x[2]);
+                fma_from_lane<3>(w.a, v, x[3]);
+            };
+            // The two windows (A, B) of a round.  have_a / have_b: the lane-group holds them (always, except in
+            // the last round of a run).
+            auto pair = [&](Walk &w, const uint4 &cu, const float4 (&xa)[kWin], const float4 (&xb)[kWin], unsigned himask,
+                            int bits, bool have_a, bool have_b) {
+                if (have_a) window(w, cu.x, cu.y, xa, himask, bits);
+                if (have_b) window(w, cu.z, cu.w, xb, himask, bits);
+            };
+
+            const Entry *hp = hot + (size_t)cur_h * kRoundEntries + 2 * lane;
+            const Entry *cp = cold + (size_t)cur_c * kRoundEntries + 2 * lane;
+            uint4 nx_h = make_uint4(0u, 0u, 0u, 0u), nx_c = nx_h;
+            if (rounds_h > 0) nx_h = load_round(hp);
+            if (rounds_c > 0) nx_c = load_round(cp);
+            int rh = 0, rc = 0;  // rounds done
+            // The rounds in which every lane-group holds two windows: the hot and the cold ones are
+            // spread evenly over max(full_h, full_c) passes (a cold round in every pass whose
+            // share of the cold rounds crosses a whole number, likewise for hot), so that the
+            // gathers through L2 and the gathers from LDS both run all the time instead of one
+            // after the other.
+            const int passes = max(full_h, full_c);
+            int due_h = (wave * passes) >> 4, due_c = ((wave + 8) * passes) >> 4;  // wavefronts start at different points
+            for (int pass = 0; pass < passes; ++pass) {
+                due_h += full_h;
+                due_c += full_c;
+                const bool do_h = due_h >= passes && rh < full_h, do_c = due_c >= passes && rc < full_c;
+                const uint4 cu_c = nx_c;
+                float4 xca[kWin], xcb[kWin];
+                if (do_c) {
+                    due_c -= passes;
+                    cold_gather(cu_c.x, xca);
+                    cold_gather(cu_c.z, xcb);
+                    // after the gathers: what waits for them does not wait for this
+                    ++rc;
+                    if (rc < rounds_c) nx_c = load_round(cp + (size_t)rc * kRoundEntries);
+                }
+                if (do_h) {
+                    due_h -= passes;
+                    const uint4 cu_h = nx_h;
+                    float4 xha[kWin], xhb[kWin];
+                    ++rh;
+                    if (rh < rounds_h) nx_h = load_round(hp + (size_t)rh * kRoundEntries);
+                    hot_gather(cu_h.x, xha);
+                    hot_gather(cu_h.z, xhb);
+                    pair(wh, cu_h, xha, xhb, hot_hi, hot_bits, true, true);
+                }
+                if (do_c) pair(wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
+            }
+            // what the rounding of the shares left over
+            for (; rh < full_h; ++rh) {
+                const uint4 cu_h = nx_h;
+                float4 xha[kWin], xhb[kWin];
+                if (rh + 1 < rounds_h) nx_h = load_round(hp + (size_t)(rh + 1) * kRoundEntries);
+                hot_gather(cu_h.x, xha);
+                hot_gather(cu_h.z, xhb);
+                pair(wh, cu_h, xha, xhb, hot_hi, hot_bits, true, true);
+            }
+            for (; rc < full_c; ++rc) {
+                const uint4 cu_c = nx_c;
+                float4 xca[kWin], xcb[kWin];
+                cold_gather(cu_c.x, xca);
+                cold_gather(cu_c.z, xcb);
+                if (rc + 1 < rounds_c) nx_c = load_round(cp + (size_t)(rc + 1) * kRoundEntries);
+                pair(wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
+            }
+            // the last round of a run: lane-groups hold two, one or none of its windows (the rest is padding)
+            if (rc < rounds_c) {
+                float4 xca[kWin], xcb[kWin];
+                cold_gather(nx_c.x, xca);
+                cold_gather(nx_c.z, xcb);
+                pair(wc, nx_c, xca, xcb, cold_hi, cold_bits, 2 * rc < len_c, 2 * rc + 1 < len_c);
+            }
+            if (rh < rounds_h) {
+                float4 xha[kWin], xhb[kWin];
+                hot_gather(nx_h.x, xha);
+                hot_gather(nx_h.z, xhb);
+                pair(wh, nx_h, xha, xhb, hot_hi, hot_bits, 2 * rh < len_h, 2 * rh + 1 < len_h);
+            }
+            cur_h += rounds_h;
+            cur_c += rounds_c;
+
+            // Tails: what every lane-group still holds for the last row of its run.  Neighbouring
+            // groups can end in the same row (one that is longer than a run), so the first group of
+            // every stretch of equal rows adds the stretch up in group order and adds the total.
+            auto tails = [&](const Walk &w, int len) {
+                const int row = len > 0 ? w.row : -1;
+                st4[lane] = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
+                if (s == 0) my_crows[g] = row;
+                wave_lds_sync();
+                const int prev = g > 0 ? my_crows[g - 1] : -2;
+                if (row >= 0 && prev != row) {
+                    float4 sum = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
+                    for (int k = g + 1; k < kGroups && my_crows[k] == row; ++k) add4(sum, st4[k * 4 + s]);
+                    float4 *dst = row == first_row ? my_slot4 : acc4 + (size_t)row * 4 + s;
+                    float4 o = *dst;
+                    add4(o, sum);
+                    *dst = o;
+                }
+                wave_lds_sync();
+            };
+            tails(wh, len_h);
+            tails(wc, len_c);
+            m = m_next;
+
+            __syncthreads();  // every gather from this step's table and every add of this step is done
+            if (wave == 0) {
+                // Shared rows: slot q holds what wavefront q held back for the first row of its run.
+                // Equal rows are adjacent (first rows never decrease); the first lane-group of
+                // such a stretch adds its slots in wavefront order.
+                const int q = g;
+                if (s == 0) slot_row[q] = slot_first;
+                wave_lds_sync();
+                const bool leader = q < kWaves && (q == 0 || slot_row[q - 1] != slot_first);
+                if (leader) {
+                    float4 sum = zero4;
+                    for (int k = q; k < kWaves && slot_row[k] == slot_first; ++k)
+                        add4(sum, *reinterpret_cast<const float4 *>(slots + k * 16 + s * 4));
+                    float4 *dst = acc4 + (size_t)slot_first * 4 + s;
+                    float4 o = *dst;
+                    add4(o, sum);
+                    *dst = o;
+                }
+                wave_lds_sync();
+                *reinterpret_cast<float4 *>(slots + lane * 4) = zero4;
+            }
+            if (t + 1 < T) {
+                const float4 *pre_src = hot_x4 + (size_t)(t + 1) * H * 4;
+                RB_PRE_LOAD(0) RB_PRE_LOAD(1) RB_PRE_LOAD(2) RB_PRE_LOAD(3) RB_PRE_LOAD(4) RB_PRE_LOAD(5)
+                RB_PRE_STORE(0) RB_PRE_STORE(1) RB_PRE_STORE(2) RB_PRE_STORE(3) RB_PRE_STORE(4) RB_PRE_STORE(5)
+            }
+            __syncthreads();
+        }
+    }
+#undef RB_PRE_LOAD
+#undef RB_PRE_STORE
+
+    // the block's rows, once
+    for (int i = tid; i < nrows * 4; i += kThreads) {
+        const float4 v = acc4[i];
+        const float a[4] = {v.x, v.y, v.z, v.w};
+        store_acc<4, true>(Y + (size_t)row0 * 16 + (size_t)i * 4, a);
+    }
+}
+
+template <typename T>
+int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
+{
+    const size_t bytes = (src.size() ? src.size() : 1) * sizeof(T);
+    MPS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(dst), bytes));
+    dp->device_bytes += bytes;
+    if (!src.empty()) MPS_HIP_TRY(hipMemcpyAsync(*dst, src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice, st));
+    return MPS_OK;
+}
+
+template <typename T>
+void release(std::vector<T> &v)
+{
+    std::vector<T>().swap(v);
+}
+
+}  // namespace
+
+void destroy(DevicePlan *dp)
+{
+    if (!dp) return;
+    (void)hipFree(dp->hot);
+    (void)hipFree(dp->cold);
+    (void)hipFree(dp->hot_src);
+    (void)hipFree(dp->cold_src);
+    (void)hipFree(dp->wave_base);
+    (void)hipFree(dp->meta);
+    (void)hipFree(dp->block_row);
+    (void)hipFree(dp->hot_cols);
+    (void)hipFree(dp->hot_x);
+    delete dp;
+}
+
+// Copies the CSR arrays to the host, builds the layout there and uploads it.
+int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n, int nnz, int K, const BuildParams &bp_in,
+           hipStream_t st, DevicePlan **out)
+{
+    *out = nullptr;
+    DevicePlan *dp = new (std::nothrow) DevicePlan;
+    if (!dp) return MPS_ERR_UNSUPPORTED;
+    int rc = MPS_OK;
+    auto fail = [&](int code) {
+        destroy(dp);
+        return code;
+    };
+    try {
+        BuildParams bp = bp_in;
+        if (bp.num_cus <= 0) {
+            int dev = 0, cus = 256;
+            hipError_t e = hipGetDevice(&dev);
+            if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            bp.num_cus = cus;
+        }
+        std::vector<int> rp((size_t)n + 1), ci((size_t)nnz);
+        std::vector<float> val((size_t)nnz);
+        hipError_t e = hipMemcpyAsync(rp.data(), d_row_ptr, rp.size() * sizeof(int), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(ci.data(), d_col_idx, ci.size() * sizeof(int), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(val.data(), d_val, val.size() * sizeof(float), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+        // the builder indexes by column id: refuse what mps_csr_validate would refuse
+        if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
+        for (int r = 0; r < n; ++r)
+            if (rp[(size_t)r] > rp[(size_t)r + 1]) return fail(MPS_ERR_INVALID_CSR);
+        for (int i = 0; i < nnz; ++i)
+            if (ci[(size_t)i] < 0 || ci[(size_t)i] >= n) return fail(MPS_ERR_INVALID_CSR);
+        rc = build_layout(rp.data(), ci.data(), val.data(), n, nnz, K, bp, dp->host);
+        if (rc != MPS_OK) return fail(rc);
+    } catch (const std::bad_alloc &) {
+        return fail(MPS_ERR_UNSUPPORTED);
+    }
+    Layout &L = dp->host;
+    dp->hot_slots = L.hot.size();
+    dp->cold_slots = L.cold.size();
+    if ((rc = upload(dp, &dp->hot, L.hot, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->cold, L.cold, st)) != MPS_OK) return fail(rc);
+    if (bp_in.keep_src) {
+        if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
+        if ((rc = upload(dp, &dp->cold_src, L.cold_src, st)) != MPS_OK) return fail(rc);
+    }
+    if ((rc = upload(dp, &dp->wave_base, L.wave_base, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->meta, L.meta, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->block_row, L.block_row, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->hot_cols, L.hot_cols, st)) != MPS_OK) return fail(rc);
+    {
+        const size_t bytes = (size_t)L.steps * L.table_rows * 16 * sizeof(float);
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&dp->hot_x), bytes);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+        dp->device_bytes += bytes;
+    }
+    dp->lds_bytes = (size_t)(L.table_rows + L.acc_rows) * 64 + kStageBytes + kSlotBytes;
+    {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+    }
+    release(L.hot);
+    release(L.cold);
+    release(L.hot_src);
+    release(L.cold_src);
+    *out = dp;
+    return MPS_OK;
+}
+
+int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStream_t st)
+{
+    const Layout &L = dp->host;
+    if (!(phases & MPS_PHASE_MAIN)) return MPS_OK;
+    const int slots = L.steps * L.table_rows;
+    hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
+                       reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
+    hipLaunchKernelGGL((rb_spmm_kernel<float>), dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot,
+                       dp->cold, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta), dp->block_row,
+                       reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X), Y, L.steps,
+                       L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+namespace {
+__global__ __launch_bounds__(256) void rb_set_values_kernel(const float *__restrict__ val, const int *__restrict__ src,
+                                                             size_t slots, Entry *__restrict__ entries)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= slots) return;
+    const int e = src[i];
+    if (e >= 0) entries[i].val = val[e];
+}
+}  // namespace
+
+int set_values(DevicePlan *dp, const float *d_val, hipStream_t st)
+{
+    if (!dp->hot_src || !dp->cold_src) return MPS_ERR_UNSUPPORTED;
+    if (dp->hot_slots)
+        hipLaunchKernelGGL(rb_set_values_kernel, dim3((unsigned)((dp->hot_slots + 255) / 256)), dim3(256), 0, st, d_val,
+                           dp->hot_src, dp->hot_slots, dp->hot);
+    if (dp->cold_slots)
+        hipLaunchKernelGGL(rb_set_values_kernel, dim3((unsigned)((dp->cold_slots + 255) / 256)), dim3(256), 0, st, d_val,
+                           dp->cold_src, dp->cold_slots, dp->cold);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+const Layout &layout_of(const DevicePlan *dp) { return dp->host; }
+
+const void *device_array(const DevicePlan *dp, int which, size_t *bytes)
+{
+    const Layout &L = dp->host;
+    switch (which) {
+    case MPS_PLAN_ARRAY_RB_BLOCK_ROW: *bytes = L.block_row.size() * sizeof(int); return dp->block_row;
+    case MPS_PLAN_ARRAY_RB_HOT_COLS: *bytes = L.hot_cols.size() * sizeof(int); return dp->hot_cols;
+    case MPS_PLAN_ARRAY_RB_META: *bytes = L.meta.size() * sizeof(int); return dp->meta;
+    case MPS_PLAN_ARRAY_RB_WAVE_BASE: *bytes = L.wave_base.size() * sizeof(long long); return dp->wave_base;
+    case MPS_PLAN_ARRAY_RB_HOT: *bytes = dp->hot_slots * sizeof(Entry); return dp->hot;
+    case MPS_PLAN_ARRAY_RB_COLD: *bytes = dp->cold_slots * sizeof(Entry); return dp->cold;
+    case MPS_PLAN_ARRAY_RB_HOT_SRC: *bytes = dp->hot_src ? dp->hot_slots * sizeof(int) : 0; return dp->hot_src;
+    case MPS_PLAN_ARRAY_RB_COLD_SRC: *bytes = dp->cold_src ? dp->cold_slots * sizeof(int) : 0; return dp->cold_src;
+    default: *bytes = 0; return nullptr;
+    }
+}
+size_t device_bytes_of(const DevicePlan *dp) { return dp->device_bytes; }
+
+}  // namespace mps_rb

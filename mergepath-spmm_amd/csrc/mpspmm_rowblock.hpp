@@ -1,0 +1,121 @@
+// Row-block plans: layout shared by the host-side builder
+// (mpspmm_rowblock_host.cpp) and the device side (mpspmm_rowblock.hip).
+// Not installed.
+//
+// The reference walks every merge-path partition with one accumulator per
+// output column and gathers the dense row of every nonzero from memory
+// (src/MergePathSpMM.cu:426-477).  On MI355X that gather is what limits a
+// matrix with long rows: a 64-byte row of X is one L1->L2 request however it
+// is scheduled.  A row-block plan keeps the arithmetic and changes where the
+// operands live:
+//
+//   * The rows of the matrix are cut into NB contiguous blocks of about equal
+//     nonzero count, one per 1,024-thread workgroup (one workgroup per CU).
+//     A block's output rows are accumulated in LDS (fp32) and written to Y
+//     once: no partial rows in memory, no carry-out records, no second kernel.
+//   * The columns are dealt to T steps.  The T * H columns with the most
+//     nonzeros are "hot": step t keeps the rows of X of its H hot columns in
+//     an LDS table, and their nonzeros gather from there.  The other columns
+//     are "cold": step t owns a contiguous range of column ids (equal cold
+//     nonzero counts per step), gathered through L2, so that the CUs of an
+//     XCD, which walk the steps at about the same pace, share a few hundred
+//     KiB of X at a time.
+//   * Within (block, step) the nonzeros in row order (a row's hot ones, then
+//     its cold ones) are cut into 15 equal runs, one per wavefront that walks
+//     nonzeros (the 16th wavefront of a workgroup only touches the streams
+//     ahead of the others, so that their loads find them in L2); a
+//     wavefront's hot nonzeros are then dealt evenly and in order to its 16
+//     lane-groups, and so are its cold ones.  Every lane-group therefore walks
+//     two short streams (hot: LDS gathers, cold: L2 gathers) of the same
+//     length as its neighbours': no divergence, no padding beyond whole
+//     4-entry windows.
+//   * An entry is 8 bytes: {index | rows_advanced << index_bits, value}.
+//     index is the LDS table slot (hot) or the column id (cold);
+//     rows_advanced is how many block-local rows lie between this nonzero and
+//     the previous one of the same lane-group stream (for the first one:
+//     between it and the first row of the wavefront's run).
+//   * When the row changes, a lane-group adds its partial sums to the row's
+//     LDS accumulator (plain read-add-write).  That is safe because a row is
+//     added to directly only by the lane-group in whose stream it begins: the
+//     partial sums of a lane-group's first row (which may have begun in the
+//     stream before) are held back and added after the walk, in lane-group
+//     order, by the first lane-group of every stretch of equal rows.  Only
+//     the first row of a wavefront's run can be shared with another
+//     wavefront: what is held back for it goes to a per-wavefront slot, and
+//     the slots are added in wavefront order after the step's barrier.
+//     Results do not depend on timing.
+#ifndef MPSPMM_ROWBLOCK_HPP
+#define MPSPMM_ROWBLOCK_HPP
+
+#include <cstdint>
+#include <vector>
+
+namespace mps_rb {
+
+constexpr int kWaves = 16;         // wavefronts of a workgroup, each walks nonzeros
+constexpr int kWaveSlots = 16;     // stride of the per-wavefront tables
+constexpr int kGroups = 16;        // lane-groups per wavefront (4 lanes x 4 columns, K = 16 fp32)
+constexpr int kWin = 4;            // entries of a window: one per lane of a lane-group
+constexpr int kPair = 2;           // windows of a lane-group per round: a lane loads its entry of both with one 16-byte load
+constexpr int kRoundEntries = kGroups * kWin * kPair;  // 128 entries = 1 KiB per round
+constexpr int kLdsBytes = 160 * 1024;
+constexpr int kStageBytes = kWaveSlots * 64 * 16;  // 64 float4 per wavefront: what its lane-groups hold at the end of their runs
+// shared-row slots [16][16] floats, their rows [16], tail rows [16][16]
+constexpr int kSlotBytes = kWaveSlots * 16 * 4 + kWaveSlots * 4 + kWaveSlots * 16 * 4;
+constexpr int kMaxTableRows = 1536;  // six 16-byte pieces per thread when a table is moved
+
+struct Entry {
+    uint32_t word;  // index | rows_advanced << index_bits
+    float val;
+};
+
+struct Layout {
+    int n = 0, nnz = 0, K = 16;
+    int steps = 0;        // T
+    int table_rows = 0;   // H
+    int acc_rows = 0;     // rows of LDS accumulators per workgroup (>= rows of every block)
+    int num_blocks = 0;   // NB
+    int hot_bits = 0, cold_bits = 0;
+    long long hot_nnz = 0;
+    long long hot_rounds = 0, cold_rounds = 0;
+    std::vector<int> block_row;         // [NB + 1]
+    std::vector<int> hot_cols;          // [T][H] column of every table slot, -1 = unused
+    std::vector<int> cold_begin;        // [T + 1] column-id range of every step's cold columns
+    std::vector<int> meta;              // [NB][T][16][4] {hot entries, cold entries, first local row, 0}; [..][15] unused
+    std::vector<long long> wave_base;   // [NB * 16][2] first round of the wavefront's hot / cold stream; [..][15]: where the block's streams end
+    std::vector<Entry> hot, cold;       // rounds of 64 entries
+    std::vector<int> hot_src, cold_src; // original nonzero index per entry slot, -1 = padding (optional)
+};
+
+struct BuildParams {
+    int steps = 0;       // 0 = choose
+    int table_rows = 0;  // 0 = what fits in LDS beside the accumulators
+    int block_rows = 0;  // 0 = choose; otherwise the most rows a block may hold
+    int num_cus = 256;
+    bool keep_src = true;
+};
+
+// Host arrays in, layout out.  Returns an mps_status.
+int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,
+                 const BuildParams &bp, Layout &out);
+
+// Steps the library picks for a matrix when the caller names none.
+int default_steps(int n, long long nnz, int table_rows);
+
+#ifdef MPSPMM_DEVICE_HPP
+// Device side (mpspmm_rowblock.hip), for translation units that include the HIP runtime.
+struct DevicePlan;
+int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n, int nnz, int K, const BuildParams &bp,
+           hipStream_t st, DevicePlan **out);
+void destroy(DevicePlan *dp);
+int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStream_t st);
+int set_values(DevicePlan *dp, const float *d_val, hipStream_t st);
+const Layout &layout_of(const DevicePlan *dp);
+size_t device_bytes_of(const DevicePlan *dp);
+// Device array `which` (MPS_PLAN_ARRAY_RB_*) and its size in bytes; nullptr if the plan does not hold it.
+const void *device_array(const DevicePlan *dp, int which, size_t *bytes);
+#endif
+
+}  // namespace mps_rb
+
+#endif

@@ -1,0 +1,457 @@
+// Host-side builder of row-block plans (layout described in
+// mpspmm_rowblock.hpp).  Pure host code: no GPU is touched here.
+#include "mpspmm_rowblock.hpp"
+
+#include <algorithm>
+#include <atomic>
+#include <cstring>
+#include <new>
+
+#include "mpspmm.h"
+#include "mpspmm_hostpar.hpp"
+
+namespace mps_rb {
+
+namespace {
+
+using mps_host::parallel_for;
+
+int bits_for(long long v)  // bits that hold the values 0..v
+{
+    int b = 1;
+    while ((v >> b) != 0) ++b;
+    return b;
+}
+
+// Contiguous row blocks of at most `cap` rows and (except for a single row
+// that is longer) at most `target` nonzeros each, taken greedily.
+int greedy_blocks(const int *rp, int n, int cap, long long target, std::vector<int> *out)
+{
+    int count = 0, r = 0;
+    if (out) out->assign(1, 0);
+    while (r < n) {
+        const int hi = (int)std::min<long long>(n, (long long)r + cap);
+        // furthest e in (r, hi] with rp[e] - rp[r] <= target
+        const long long limit = (long long)rp[r] + target;
+        int e = (int)(std::upper_bound(rp + r + 1, rp + hi + 1, limit,
+                                       [](long long lim, int v) { return lim < (long long)v; }) -
+                      rp) - 1;
+        if (e <= r) e = r + 1;
+        r = e;
+        ++count;
+        if (out) out->push_back(r);
+    }
+    return count;
+}
+
+// i-th element of a list of len entries dealt evenly and in order to 16
+// lane-groups: the first len % 16 groups hold one entry more.
+inline void deal(int len, int i, int *g, int *j)
+{
+    const int base = len / kGroups, rem = len % kGroups, big = base + 1;
+    if (i < rem * big) {
+        *g = i / big;
+        *j = i - *g * big;
+    } else {
+        const int i2 = i - rem * big;
+        *g = rem + i2 / base;
+        *j = i2 % base;
+    }
+}
+
+// rounds (two windows per lane-group each) that a wavefront needs for n windows dealt to its 16 lane-groups
+inline int rounds_for(int n) { return (n / kGroups + (n % kGroups != 0) + kPair - 1) / kPair; }
+
+inline int windows_of(int entries) { return (entries + kWin - 1) / kWin; }
+
+struct ColumnMap {
+    std::vector<int16_t> step;  // per column
+    std::vector<int16_t> slot;  // per column: table slot, -1 = cold
+};
+
+// Everything about one (block, step): where each wavefront's run starts.
+struct StepSplit {
+    int first_row[kWaves];
+    int hstart[kWaves + 1], cstart[kWaves + 1];
+};
+
+// cnt_t: [lr * 2 + kind] nonzeros of local row lr in this step (kind 0 hot, 1 cold).  The step's
+// windows in row order (a row's hot windows, then its cold ones) are cut into 15 equal runs.
+void split_step(const int *cnt_t, int nr, StepSplit &sp)
+{
+    long long E = 0;
+    for (int i = 0; i < 2 * nr; ++i) E += windows_of(cnt_t[i]);
+    long long S[kWaves + 1];
+    for (int w = 0; w <= kWaves; ++w) S[w] = (long long)w * E / kWaves;
+    long long q = 0;
+    int hq = 0, cq = 0, wp = 0;
+    for (int lr = 0; lr < nr && wp < kWaves; ++lr) {
+        const int h = windows_of(cnt_t[2 * lr]), c = windows_of(cnt_t[2 * lr + 1]);
+        while (wp < kWaves && S[wp] < q + h + c) {
+            const long long d = S[wp] - q;
+            sp.first_row[wp] = lr;
+            if (d < h) {
+                sp.hstart[wp] = hq + (int)d;
+                sp.cstart[wp] = cq;
+            } else {
+                sp.hstart[wp] = hq + h;
+                sp.cstart[wp] = cq + (int)(d - h);
+            }
+            ++wp;
+        }
+        q += h + c;
+        hq += h;
+        cq += c;
+    }
+    // runs that start at the very end (nothing left for them)
+    int hot_total = 0, cold_total = 0;
+    for (int lr = 0; lr < nr; ++lr) {
+        hot_total += windows_of(cnt_t[2 * lr]);
+        cold_total += windows_of(cnt_t[2 * lr + 1]);
+    }
+    for (; wp < kWaves; ++wp) {
+        sp.first_row[wp] = wp > 0 ? sp.first_row[wp - 1] : 0;
+        sp.hstart[wp] = hot_total;
+        sp.cstart[wp] = cold_total;
+    }
+    sp.hstart[kWaves] = hot_total;
+    sp.cstart[kWaves] = cold_total;
+}
+
+void count_block(const int *rp, const int *ci, const ColumnMap &cm, int r0, int nr, int T, std::vector<int> &cnt)
+{
+    cnt.assign((size_t)T * nr * 2, 0);
+    for (int lr = 0; lr < nr; ++lr)
+        for (int e = rp[r0 + lr]; e < rp[r0 + lr + 1]; ++e) {
+            const int c = ci[e];
+            ++cnt[((size_t)cm.step[c] * nr + lr) * 2 + (cm.slot[c] < 0)];
+        }
+}
+
+}  // namespace
+
+int default_steps(int n, long long nnz, int table_rows)
+{
+    // Measured on MI355X with the 232,965-row power-law benchmark graph (492 nonzeros per row):
+    // more steps put more nonzeros on the LDS path, but every step costs two barriers and a table
+    // load per workgroup.  Keep about 24 table loads per workgroup and never more hot slots than
+    // there are columns.
+    if (table_rows < 1) table_rows = 1;
+    long long t = 24;
+    const long long most = ((long long)n + table_rows - 1) / table_rows;
+    if (t > most) t = most;
+    (void)nnz;
+    return (int)std::max<long long>(t, 1);
+}
+
+int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp,
+                 Layout &L)
+{
+    if (!rp || n < 1 || nnz < 0 || (nnz > 0 && (!ci || !val))) return MPS_ERR_INVALID_ARG;
+    if (K != 16) return MPS_ERR_UNSUPPORTED;
+    const int cold_bits = bits_for(n > 1 ? n - 1 : 1);
+    if (cold_bits > 22) return MPS_ERR_UNSUPPORTED;
+    const int num_cus = bp.num_cus > 0 ? bp.num_cus : 256;
+    L = Layout();
+    L.n = n;
+    L.nnz = nnz;
+    L.K = K;
+    L.cold_bits = cold_bits;
+
+    // ---- 1. row blocks: about equal nonzero counts, as few rounds of workgroups as the LDS allows
+    const int budget_rows = (kLdsBytes - kStageBytes - kSlotBytes - 256) / 64;  // table rows + accumulator rows
+    int cap_limit = std::min(1024, 1 << (32 - cold_bits));                      // rows_advanced must fit above the index
+    if (bp.table_rows > 0) cap_limit = std::min(cap_limit, budget_rows - bp.table_rows);
+    if (cap_limit < 4) return MPS_ERR_INVALID_ARG;
+    int cap = bp.block_rows > 0 ? std::min(bp.block_rows, cap_limit) : cap_limit;
+    if (cap < 1) cap = 1;
+    for (int m = 1;; ++m) {
+        const long long most = (long long)num_cus * m;
+        if (((long long)n + cap - 1) / cap > most) continue;
+        long long lo = std::max<long long>(1, ((long long)nnz + most - 1) / most), hi = std::max<long long>(nnz, 1);
+        if (greedy_blocks(rp, n, cap, hi, nullptr) > most) continue;  // cannot happen: rows alone fit
+        while (lo < hi) {
+            const long long mid = lo + (hi - lo) / 2;
+            if (greedy_blocks(rp, n, cap, mid, nullptr) <= most) hi = mid; else lo = mid + 1;
+        }
+        greedy_blocks(rp, n, cap, lo, &L.block_row);
+        break;
+    }
+    L.num_blocks = (int)L.block_row.size() - 1;
+    int most_rows = 1;
+    for (int b = 0; b < L.num_blocks; ++b) most_rows = std::max(most_rows, L.block_row[b + 1] - L.block_row[b]);
+    L.acc_rows = (most_rows + 3) / 4 * 4;
+
+    // ---- 2. table size, steps
+    int H = bp.table_rows > 0 ? bp.table_rows : std::min(kMaxTableRows, budget_rows - L.acc_rows);
+    if (H > kMaxTableRows) H = kMaxTableRows;
+    int T = bp.steps > 0 ? bp.steps : default_steps(n, nnz, H);
+    if (T > 4096) T = 4096;
+    if (bp.table_rows <= 0) {
+        // no more slots than columns to put in them
+        const int need = (n + T - 1) / T;
+        if (H > need) H = need;
+        H = (H + 3) / 4 * 4;
+    }
+    if (H < 1 || (long long)(H + L.acc_rows) * 64 + kStageBytes + kSlotBytes > kLdsBytes) return MPS_ERR_INVALID_ARG;
+    L.table_rows = H;
+    L.steps = T;
+    L.hot_bits = bits_for(H > 1 ? H - 1 : 1);
+
+    // ---- 3. nonzeros per column; hot columns by rank, cold columns by id range
+    std::vector<std::atomic<int>> deg((size_t)n);
+    for (auto &d : deg) d.store(0, std::memory_order_relaxed);
+    parallel_for(nnz, 1 << 20, [&](int64_t a, int64_t b) {
+        for (int64_t e = a; e < b; ++e) deg[(size_t)ci[e]].fetch_add(1, std::memory_order_relaxed);
+    });
+    auto d_of = [&](int c) { return deg[(size_t)c].load(std::memory_order_relaxed); };
+    std::vector<int> cand;
+    cand.reserve((size_t)n);
+    for (int c = 0; c < n; ++c)
+        if (d_of(c) > 0) cand.push_back(c);
+    const size_t R = std::min<size_t>((size_t)T * H, cand.size());
+    auto hotter = [&](int a, int b) {
+        const int da = d_of(a), db = d_of(b);
+        return da != db ? da > db : a < b;
+    };
+    if (R < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)R, cand.end(), hotter);
+    std::sort(cand.begin(), cand.begin() + (long)R, hotter);
+    ColumnMap cm;
+    cm.step.assign((size_t)n, 0);
+    cm.slot.assign((size_t)n, -1);
+    L.hot_cols.assign((size_t)T * H, -1);
+    L.hot_nnz = 0;
+    for (size_t k = 0; k < R; ++k) {
+        const int c = cand[k];
+        const int t = (int)(k % (size_t)T), slot = (int)(k / (size_t)T);
+        cm.step[(size_t)c] = (int16_t)t;
+        cm.slot[(size_t)c] = (int16_t)slot;
+        L.hot_cols[(size_t)t * H + slot] = c;
+        L.hot_nnz += d_of(c);
+    }
+    {
+        const long long cold_total = (long long)nnz - L.hot_nnz;
+        long long cum = 0;
+        L.cold_begin.assign((size_t)T + 1, n);
+        int t_prev = -1;
+        for (int c = 0; c < n; ++c) {
+            if (cm.slot[(size_t)c] >= 0) continue;
+            int t = cold_total > 0 ? (int)std::min<long long>(T - 1, cum * T / cold_total) : 0;
+            cm.step[(size_t)c] = (int16_t)t;
+            for (int u = t_prev + 1; u <= t; ++u) L.cold_begin[(size_t)u] = c;
+            t_prev = std::max(t_prev, t);
+            cum += d_of(c);
+        }
+    }
+
+    // ---- 4. pass 1: windows and first rows of every wavefront's runs
+    const int NB = L.num_blocks;
+    L.meta.assign((size_t)NB * T * kWaveSlots * 4, 0);
+    std::vector<long long> rounds((size_t)NB * kWaveSlots * 2, 0);
+    parallel_for(NB, 1, [&](int64_t b0, int64_t b1) {
+        std::vector<int> cnt;
+        for (int64_t b = b0; b < b1; ++b) {
+            const int r0 = L.block_row[(size_t)b], nr = L.block_row[(size_t)b + 1] - r0;
+            count_block(rp, ci, cm, r0, nr, T, cnt);
+            for (int t = 0; t < T; ++t) {
+                StepSplit sp;
+                split_step(cnt.data() + (size_t)t * nr * 2, nr, sp);
+                for (int w = 0; w < kWaves; ++w) {
+                    int *m = &L.meta[(((size_t)b * T + t) * kWaveSlots + w) * 4];
+                    m[0] = sp.hstart[w + 1] - sp.hstart[w];
+                    m[1] = sp.cstart[w + 1] - sp.cstart[w];
+                    m[2] = sp.first_row[w];
+                    rounds[((size_t)b * kWaveSlots + w) * 2 + 0] += rounds_for(m[0]);
+                    rounds[((size_t)b * kWaveSlots + w) * 2 + 1] += rounds_for(m[1]);
+                }
+            }
+        }
+    });
+
+    // ---- 5. where every wavefront's streams start
+    L.wave_base.assign((size_t)NB * kWaveSlots * 2, 0);
+    long long hr = 0, cr = 0;
+    for (size_t i = 0; i < (size_t)NB * kWaveSlots; ++i) {
+        L.wave_base[2 * i] = hr;
+        L.wave_base[2 * i + 1] = cr;
+        hr += rounds[2 * i];
+        cr += rounds[2 * i + 1];
+    }
+    L.hot_rounds = hr;
+    L.cold_rounds = cr;
+    const Entry empty{0u, 0.f};
+    L.hot.assign((size_t)hr * kRoundEntries, empty);
+    L.cold.assign((size_t)cr * kRoundEntries, empty);
+    if (bp.keep_src) {
+        L.hot_src.assign(L.hot.size(), -1);
+        L.cold_src.assign(L.cold.size(), -1);
+    }
+
+    // ---- 6. pass 2: place the entries
+    parallel_for(NB, 1, [&](int64_t b0, int64_t b1) {
+        std::vector<int> cnt, off, s_src;
+        std::vector<uint32_t> s_idx;
+        std::vector<float> s_val;
+        for (int64_t b = b0; b < b1; ++b) {
+            const int r0 = L.block_row[(size_t)b], nr = L.block_row[(size_t)b + 1] - r0;
+            const int e0 = rp[r0], ne = rp[r0 + nr] - e0;
+            count_block(rp, ci, cm, r0, nr, T, cnt);
+            off.resize(cnt.size() + 1);
+            off[0] = 0;
+            for (size_t i = 0; i < cnt.size(); ++i) off[i + 1] = off[i] + cnt[i];
+            std::vector<int> t_begin((size_t)T + 1);
+            for (int t = 0; t <= T; ++t) t_begin[(size_t)t] = off[(size_t)t * nr * 2];
+            s_idx.resize((size_t)ne);
+            s_val.resize((size_t)ne);
+            s_src.resize((size_t)ne);
+            for (int lr = 0; lr < nr; ++lr)
+                for (int e = rp[r0 + lr]; e < rp[r0 + lr + 1]; ++e) {
+                    const int c = ci[e];
+                    const int slot = cm.slot[(size_t)c];
+                    const int k = slot < 0;
+                    const int pos = off[((size_t)cm.step[(size_t)c] * nr + lr) * 2 + k]++;
+                    s_idx[(size_t)pos] = (uint32_t)(k ? c : slot);
+                    s_val[(size_t)pos] = val[e];
+                    s_src[(size_t)pos] = e;
+                }
+            long long round_off[kWaves][2];
+            for (int w = 0; w < kWaves; ++w)
+                for (int k = 0; k < 2; ++k) round_off[w][k] = L.wave_base[((size_t)b * kWaveSlots + w) * 2 + k];
+            for (int t = 0; t < T; ++t) {
+                const int *m0 = &L.meta[((size_t)b * T + t) * kWaveSlots * 4];
+                const int *cnt_t = cnt.data() + (size_t)t * nr * 2;
+                long long E = 0;
+                for (int i = 0; i < 2 * nr; ++i) E += windows_of(cnt_t[i]);
+                int w = 0;
+                long long w_end = E / kWaves;  // first window of run w + 1
+                int placed[2] = {0, 0}, last_row[2] = {0, 0};
+                long long q = 0;           // windows so far
+                size_t p = (size_t)t_begin[(size_t)t];  // sorted nonzeros so far
+                for (int lr = 0; lr < nr; ++lr)
+                    for (int k = 0; k < 2; ++k) {
+                        int left = cnt_t[2 * lr + k];
+                        while (left > 0) {
+                            while (q >= w_end) {
+                                ++w;
+                                w_end = (long long)(w + 1) * E / kWaves;
+                                placed[0] = placed[1] = 0;
+                            }
+                            const int *m = m0 + w * 4;
+                            int g, j;
+                            deal(m[k], placed[k], &g, &j);
+                            const int prev = j == 0 ? m[2] : last_row[k];
+                            const uint32_t adv = (uint32_t)(lr - prev);
+                            last_row[k] = lr;
+                            ++placed[k];
+                            // round j / 2; inside it lane (g, e) holds entry e of the group's two windows side by side
+                            const size_t dst = (size_t)(round_off[w][k] + j / kPair) * kRoundEntries + (size_t)g * kWin * kPair + (size_t)(j % kPair);
+                            const int take = left < kWin ? left : kWin;
+                            std::vector<Entry> &out = k ? L.cold : L.hot;
+                            for (int e = 0; e < kWin; ++e) {
+                                // padding repeats the window's last nonzero with value 0
+                                const size_t src = p + (size_t)(e < take ? e : take - 1);
+                                Entry en;
+                                en.word = s_idx[src] | (e == 0 ? adv << (k ? L.cold_bits : L.hot_bits) : 0u);
+                                en.val = e < take ? s_val[src] : 0.f;
+                                out[dst + (size_t)e * kPair] = en;
+                                if (bp.keep_src && e < take) (k ? L.cold_src : L.hot_src)[dst + (size_t)e * kPair] = s_src[src];
+                            }
+                            p += (size_t)take;
+                            left -= take;
+                            ++q;
+                        }
+                    }
+                for (int ww = 0; ww < kWaves; ++ww)
+                    for (int k = 0; k < 2; ++k) round_off[ww][k] += rounds_for(m0[ww * 4 + k]);
+            }
+        }
+    });
+    return MPS_OK;
+}
+
+}  // namespace mps_rb
+
+struct mps_rowblock_layout {
+    mps_rb::Layout L;
+};
+
+extern "C" {
+
+int mps_rowblock_layout_build(const int *row_ptr, const int *col_idx, const float *val, int n_rows, int nnz, int K,
+                              const mps_plan_options *options, mps_rowblock_layout **layout_out)
+{
+    if (!layout_out) return MPS_ERR_INVALID_ARG;
+    *layout_out = nullptr;
+    mps_rb::BuildParams bp;
+    if (options) {
+        bp.steps = options->rowblock_steps;
+        bp.table_rows = options->rowblock_table_rows;
+        bp.block_rows = options->rowblock_block_rows;
+        bp.num_cus = options->rowblock_blocks_per_round;
+        bp.keep_src = !(options->flags & MPS_PLAN_NO_SOURCES);
+    }
+    if (bp.num_cus <= 0) bp.num_cus = 256;
+    mps_rowblock_layout *h = new (std::nothrow) mps_rowblock_layout;
+    if (!h) return MPS_ERR_UNSUPPORTED;
+    int rc;
+    try {
+        rc = mps_rb::build_layout(row_ptr, col_idx, val, n_rows, nnz, K, bp, h->L);
+    } catch (const std::bad_alloc &) {
+        rc = MPS_ERR_UNSUPPORTED;
+    }
+    if (rc != MPS_OK) {
+        delete h;
+        return rc;
+    }
+    *layout_out = h;
+    return MPS_OK;
+}
+
+int mps_rowblock_layout_info(const mps_rowblock_layout *layout, mps_plan_info *info)
+{
+    if (!layout || !info) return MPS_ERR_INVALID_ARG;
+    const mps_rb::Layout &L = layout->L;
+    std::memset(info, 0, sizeof(*info));
+    info->n_rows = L.n;
+    info->nnz = L.nnz;
+    info->K = L.K;
+    info->elem_bytes = 4;
+    info->num_slabs = 1;
+    info->slab_cols = L.n;
+    info->hot_nnz = L.hot_nnz;
+    info->mark_shift = L.cold_bits;
+    info->hot_mark_shift = L.hot_bits;
+    info->rowblock_steps = L.steps;
+    info->rowblock_table_rows = L.table_rows;
+    info->rowblock_blocks = L.num_blocks;
+    info->rowblock_acc_rows = L.acc_rows;
+    info->rowblock_hot_slots = L.hot_rounds * mps_rb::kRoundEntries;
+    info->rowblock_cold_slots = L.cold_rounds * mps_rb::kRoundEntries;
+    return MPS_OK;
+}
+
+int mps_rowblock_layout_array(const mps_rowblock_layout *layout, int which, const void **data_out, size_t *bytes_out)
+{
+    if (!layout || !data_out || !bytes_out) return MPS_ERR_INVALID_ARG;
+    const mps_rb::Layout &L = layout->L;
+    auto give = [&](const auto &v) {
+        *data_out = v.data();
+        *bytes_out = v.size() * sizeof(v[0]);
+        return (int)MPS_OK;
+    };
+    switch (which) {
+    case MPS_PLAN_ARRAY_RB_BLOCK_ROW: return give(L.block_row);
+    case MPS_PLAN_ARRAY_RB_HOT_COLS: return give(L.hot_cols);
+    case MPS_PLAN_ARRAY_RB_META: return give(L.meta);
+    case MPS_PLAN_ARRAY_RB_WAVE_BASE: return give(L.wave_base);
+    case MPS_PLAN_ARRAY_RB_HOT: return give(L.hot);
+    case MPS_PLAN_ARRAY_RB_COLD: return give(L.cold);
+    case MPS_PLAN_ARRAY_RB_HOT_SRC: return give(L.hot_src);
+    case MPS_PLAN_ARRAY_RB_COLD_SRC: return give(L.cold_src);
+    default: return MPS_ERR_INVALID_ARG;
+    }
+}
+
+void mps_rowblock_layout_free(mps_rowblock_layout *layout) { delete layout; }
+
+}  // extern "C"

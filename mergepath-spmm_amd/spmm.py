@@ -174,7 +174,9 @@ class Plan:
     and the workspace.  The counterpart of what the reference sets up once
     before its repeat loop (src/MergePathSpMM.cu:192-220)."""
 
-    def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto"):
+    def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
+                 rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
+                 rowblock_blocks_per_round=0, keep_sources=True):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -182,10 +184,15 @@ class Plan:
         eb = 4 if self.dtype == torch.float32 else 2
         flags = {"auto": 0, "off": _cabi.MPS_PLAN_NO_TILING, "force": _cabi.MPS_PLAN_FORCE_TILING}[tiling]
         flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_HOT, "force": _cabi.MPS_PLAN_FORCE_HOT}[hot]
-        check(_cabi.lib().mps_plan_create(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
-                                          int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
-                                          int(threads_per_wave), flags, int(slab_bytes), _stream(),
-                                          ctypes.byref(self._h)), "mps_plan_create")
+        flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_ROWBLOCK, "force": _cabi.MPS_PLAN_FORCE_ROWBLOCK}[rowblock]
+        if not keep_sources:
+            flags |= _cabi.MPS_PLAN_NO_SOURCES
+        opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
+                                int(rowblock_block_rows), int(rowblock_blocks_per_round))
+        check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
+                                             int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
+                                             int(threads_per_wave), ctypes.byref(opt), _stream(),
+                                             ctypes.byref(self._h)), "mps_plan_create_ex")
         self.K, self.n_rows = int(K), csr.n_rows
         info = _cabi.PlanInfo()
         check(_cabi.lib().mps_plan_get_info(self._h, ctypes.byref(info)), "mps_plan_get_info")
@@ -220,6 +227,14 @@ class Plan:
             _cabi.MPS_PLAN_ARRAY_SLICE_SRC: (slots, np.int32),
             _cabi.MPS_PLAN_ARRAY_SLICE_VALS: (slots, np.float32 if i.elem_bytes == 4 else np.float16),
             _cabi.MPS_PLAN_ARRAY_HOT_COLS: (i.num_slabs * i.hot_rows, np.int32),
+            _cabi.MPS_PLAN_ARRAY_RB_BLOCK_ROW: (i.rowblock_blocks + 1, np.int32),
+            _cabi.MPS_PLAN_ARRAY_RB_HOT_COLS: (i.rowblock_steps * i.rowblock_table_rows, np.int32),
+            _cabi.MPS_PLAN_ARRAY_RB_META: (i.rowblock_blocks * i.rowblock_steps * 64, np.int32),
+            _cabi.MPS_PLAN_ARRAY_RB_WAVE_BASE: (i.rowblock_blocks * 32, np.int64),
+            _cabi.MPS_PLAN_ARRAY_RB_HOT: (2 * int(i.rowblock_hot_slots), np.uint32),
+            _cabi.MPS_PLAN_ARRAY_RB_COLD: (2 * int(i.rowblock_cold_slots), np.uint32),
+            _cabi.MPS_PLAN_ARRAY_RB_HOT_SRC: (int(i.rowblock_hot_slots), np.int32),
+            _cabi.MPS_PLAN_ARRAY_RB_COLD_SRC: (int(i.rowblock_cold_slots), np.int32),
         }
         n, dt = shapes[which]
         out = np.empty(n, dtype=dt)
@@ -286,3 +301,45 @@ def spmm_nz_splitting(csr, X, parts, out=None):
                                            csr.nnz, K, _ptr(parts.part_ptr), _ptr(parts.part2node),
                                            parts.num_parts, _stream()), "mps_nzsplit_spmm_f32")
     return Y
+
+
+class RowBlockLayout:
+    """The layout of a row-block plan, built on the host (mps_rowblock_layout_build): no GPU needed."""
+
+    def __init__(self, row_ptr, col_idx, val, K=16, steps=0, table_rows=0, block_rows=0, blocks_per_round=0,
+                 keep_sources=True):
+        import numpy as np
+        self._np = np
+        self._h = ctypes.c_void_p()
+        rp = np.ascontiguousarray(row_ptr, dtype=np.int32)
+        ci = np.ascontiguousarray(col_idx, dtype=np.int32)
+        v = np.ascontiguousarray(val, dtype=np.float32)
+        opt = _cabi.PlanOptions(0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES, 0, int(steps), int(table_rows),
+                                int(block_rows), int(blocks_per_round))
+        check(_cabi.lib().mps_rowblock_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size,
+                                                    int(K), ctypes.byref(opt), ctypes.byref(self._h)),
+              "mps_rowblock_layout_build")
+        self.info = _cabi.PlanInfo()
+        check(_cabi.lib().mps_rowblock_layout_info(self._h, ctypes.byref(self.info)), "mps_rowblock_layout_info")
+
+    def array(self, which, dtype):
+        """Copy of one of the layout's arrays (MPS_PLAN_ARRAY_RB_*) as a numpy array of `dtype`."""
+        np = self._np
+        data, nbytes = ctypes.c_void_p(), ctypes.c_size_t()
+        check(_cabi.lib().mps_rowblock_layout_array(self._h, int(which), ctypes.byref(data), ctypes.byref(nbytes)),
+              "mps_rowblock_layout_array")
+        if nbytes.value == 0:
+            return np.zeros(0, dtype=dtype)
+        buf = (ctypes.c_char * nbytes.value).from_address(data.value)
+        return np.frombuffer(buf, dtype=dtype).copy()
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            _cabi.lib().mps_rowblock_layout_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

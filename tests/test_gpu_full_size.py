@@ -34,16 +34,22 @@ def test_power_law_config_full_size(pkg, orc, dev):
     (d_X,) = to_dev(dev, X)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     plan = pkg.spmm.Plan(csr, K)
-    # the library's own choice here: 5 slabs of 3 MiB, 1,728 hot columns per slab (over a third of the nonzeros)
-    assert plan.info.num_slabs == 5 and plan.info.hot_rows == 1728 and plan.info.hot_nnz > 0.3 * ci.size
+    # the library's own choice here: a row-block plan (rows summed in LDS, more than half of the nonzeros
+    # gathered from LDS tables), one block per CU
+    assert plan.info.rowblock_steps > 0 and plan.info.rowblock_blocks % 256 == 0 and plan.info.hot_nnz > 0.5 * ci.size
     Yp = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    # without row blocks: 5 slabs of 3 MiB, 1,728 hot columns per slab (over a third of the nonzeros)
+    slab_plan = pkg.spmm.Plan(csr, K, rowblock="off")
+    assert slab_plan.info.num_slabs == 5 and slab_plan.info.hot_rows == 1728 and slab_plan.info.hot_nnz > 0.3 * ci.size
+    Ys = slab_plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    slab_plan.close()
     sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz)
     # the partition of the caller's CSR is the reference split, bit for bit, at this size too
     xs, ys = orc.partition_coords(rp, ci.size, sched.P)
     assert np.array_equal(sched.coord_x.cpu().numpy(), xs) and np.array_equal(sched.coord_y.cpu().numpy(), ys)
     Yc = pkg.spmm.spmm_merge_path(csr, d_X, sched, out=torch.full_like(d_X, float("nan")))
     torch.cuda.synchronize()
-    for Y in (Yp, Yc):
+    for Y in (Yp, Ys, Yc):
         check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
     assert torch.equal(Yp, plan.spmm(d_X))  # same bits on a second launch
     # all-ones features: every column of Y is the row sum of the values

@@ -354,11 +354,16 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
-    plan = pkg.spmm.Plan(csr, K, cost=128)
+    plan = pkg.spmm.Plan(csr, K, cost=128, rowblock="off")
     assert plan.info.num_slabs == 2 and plan.info.slab_cols * K * 4 < (4 << 20)  # X = 6.4 MB: two slabs that fit an L2
     Y = plan.spmm(d_X)
     torch.cuda.synchronize()
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    # the library's own choice for rows this long (200 nonzeros on average): a row-block plan
+    auto = pkg.spmm.Plan(csr, K)
+    assert auto.info.rowblock_steps > 0
+    check_fp32(auto.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    auto.close()
     # the plain path on the caller's CSR agrees to rounding
     sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz, cost=128)
     Y0 = pkg.spmm.spmm_merge_path(csr, d_X, sched)

@@ -1,0 +1,130 @@
+"""Row-block plans on the GPU, through the C ABI: parity with the fp64 CPU loop
+(the oracle), bit-identical repeats, value refresh, edge shapes."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import check_fp32, make_csr, random_csr, to_dev
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # n, max_deg, hubs, steps, table_rows, block_rows, blocks_per_round
+    (300, 40, ((5, 280), (150, 300)), 3, 16, 64, 4),
+    (97, 12, (), 2, 8, 0, 2),
+    (513, 60, ((0, 500), (512, 400)), 5, 32, 40, 8),
+    (64, 64, ((10, 64),), 1, 64, 0, 1),
+    (200, 5, (), 4, 4, 16, 256),
+    (5000, 200, ((17, 4800), (4999, 3000)), 6, 256, 0, 64),
+    (20000, 64, ((0, 15000),), 8, 0, 0, 0),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_rowblock_plan_matches_fp64_loop(pkg, orc, dev, case):
+    n, max_deg, hubs, steps, table_rows, block_rows, per_round = case
+    rng = np.random.default_rng(hash(case) % (2 ** 32))
+    rp, ci = random_csr(rng, n, max_deg, p_empty=0.25, hub_rows=hubs)
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=steps, rowblock_table_rows=table_rows,
+                         rowblock_block_rows=block_rows, rowblock_blocks_per_round=per_round)
+    assert plan.info.rowblock_steps == steps
+    Y = torch.full_like(d_X, float("nan"))
+    plan.spmm(d_X, out=Y)
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    # repeats give the same bits, whatever Y held
+    Y2 = torch.zeros_like(d_X)
+    for _ in range(3):
+        plan.spmm(d_X, out=Y2)
+    torch.cuda.synchronize()
+    assert torch.equal(Y, Y2)
+
+
+def test_rowblock_plan_closed_forms(pkg, dev):
+    # identity: Y = X; all-ones features: row sums
+    n = 1000
+    rp = np.arange(n + 1, dtype=np.int32)
+    ci = np.arange(n, dtype=np.int32)
+    val = np.ones(n, dtype=np.float32)
+    rng = np.random.default_rng(1)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=3, rowblock_table_rows=100, rowblock_blocks_per_round=8)
+    assert np.array_equal(plan.spmm(d_X).cpu().numpy(), X)
+    rp2, ci2 = random_csr(rng, n, 50, hub_rows=((3, 900),))
+    v2 = rng.random(ci2.size).astype(np.float32)
+    csr2 = make_csr(pkg, dev, rp2, ci2, v2)
+    ones = torch.ones((n, 16), dtype=torch.float32, device=dev)
+    plan2 = pkg.spmm.Plan(csr2, 16, rowblock="force", rowblock_steps=4, rowblock_table_rows=64, rowblock_blocks_per_round=8)
+    Y = plan2.spmm(ones).cpu().numpy().astype(np.float64)
+    sums = np.add.reduceat(np.concatenate([v2.astype(np.float64), [0.0]]), np.minimum(rp2[:-1], v2.size))
+    sums[np.diff(rp2) == 0] = 0.0
+    assert np.allclose(Y, sums[:, None], rtol=1e-5, atol=1e-6)
+
+
+def test_rowblock_plan_set_values_and_sources(pkg, orc, dev):
+    rng = np.random.default_rng(9)
+    n = 800
+    rp, ci = random_csr(rng, n, 70, hub_rows=((1, 700),))
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=3, rowblock_table_rows=48, rowblock_blocks_per_round=8)
+    val2 = rng.random(ci.size).astype(np.float32)
+    (d_v2,) = to_dev(dev, val2)
+    plan.set_values(d_v2)
+    ref, scale = orc.spmm_f64(rp, ci, val2, X, want_abs=True)
+    check_fp32(plan.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    lean = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=3, rowblock_table_rows=48, rowblock_blocks_per_round=8,
+                         keep_sources=False)
+    assert lean.info.device_bytes < plan.info.device_bytes
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        lean.set_values(d_v2)
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+    # the device arrays are what the host-side builder makes
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=3, table_rows=48, blocks_per_round=8)
+    C = pkg._cabi
+    for which, dt in ((C.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32), (C.MPS_PLAN_ARRAY_RB_META, np.int32),
+                      (C.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32), (C.MPS_PLAN_ARRAY_RB_COLD, np.uint32),
+                      (C.MPS_PLAN_ARRAY_RB_HOT_SRC, np.int32)):
+        assert np.array_equal(lean.array(which) if which != C.MPS_PLAN_ARRAY_RB_HOT_SRC else plan.array(which),
+                              lay.array(which, dt))
+
+
+def test_rowblock_plan_rejects_other_shapes(pkg, dev):
+    rng = np.random.default_rng(2)
+    rp, ci = random_csr(rng, 100, 10)
+    val = rng.random(ci.size).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        pkg.spmm.Plan(csr, 32, rowblock="force")
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+    bad = make_csr(pkg, dev, rp, np.where(np.arange(ci.size) == 3, 100, ci).astype(np.int32), val)
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        pkg.spmm.Plan(bad, 16, rowblock="force")
+    assert e.value.status == pkg._cabi.MPS_ERR_INVALID_CSR
+
+
+def test_rowblock_plan_power_law_graph(pkg, orc, dev):
+    # the benchmark graph's shape at a tenth of its size; the library picks the plan kind and its parameters
+    rp, ci, _ = pkg.graphs.generate("chunglu:n=60000,nnz=12000000,gamma=2.1,dmax=8000", seed=3)
+    n, nnz = rp.size - 1, ci.size
+    val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
+    X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16, rowblock="force")
+    assert plan.info.rowblock_blocks > 0 and plan.info.hot_nnz > 0
+    Y = plan.spmm(d_X)
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    Y2 = plan.spmm(d_X)
+    assert torch.equal(Y, Y2)

@@ -1,0 +1,170 @@
+"""Row-block plan layout, checked on the CPU: the host-side builder
+(mps_rowblock_layout_build) against a Python walk that decodes the streams the
+way the kernel does (rows_advanced marks, per-step tables, shared-row slots),
+and against the structure the layout promises.  No GPU, no oracle needed: the
+product of the walk is compared with a dense fp64 product."""
+import numpy as np
+import pytest
+
+from tests.gpu_util import random_csr
+
+G, WAVES, WSLOTS, WIN = 16, 16, 16, 4
+
+
+def dealt_len(n, g):
+    return n // G + (1 if g < n % G else 0)
+
+
+def rounds_for(n):
+    """rounds (two windows per lane-group each) a wavefront needs for n windows dealt to its 16 lane-groups"""
+    return (n // G + (1 if n % G else 0) + 1) // 2
+
+
+def walk_layout(pkg, lay, X, n):
+    """Y = A @ X from the layout alone, in the order the kernel uses; also returns the
+    original nonzero indices seen (from the source arrays)."""
+    C = pkg._cabi
+    i = lay.info
+    T, H, NB = i.rowblock_steps, i.rowblock_table_rows, i.rowblock_blocks
+    hot_bits, cold_bits = i.hot_mark_shift, i.mark_shift
+    brow = lay.array(C.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
+    hot_cols = lay.array(C.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32).reshape(T, H)
+    meta = lay.array(C.MPS_PLAN_ARRAY_RB_META, np.int32).reshape(NB, T, WSLOTS, 4)
+    base = lay.array(C.MPS_PLAN_ARRAY_RB_WAVE_BASE, np.int64).reshape(NB, WSLOTS, 2)
+    streams = [lay.array(C.MPS_PLAN_ARRAY_RB_HOT, np.uint32).reshape(-1, 2),
+               lay.array(C.MPS_PLAN_ARRAY_RB_COLD, np.uint32).reshape(-1, 2)]
+    srcs = [lay.array(C.MPS_PLAN_ARRAY_RB_HOT_SRC, np.int32), lay.array(C.MPS_PLAN_ARRAY_RB_COLD_SRC, np.int32)]
+    bits = [hot_bits, cold_bits]
+    Y = np.zeros((n, X.shape[1]), dtype=np.float64)
+    seen = []
+    assert brow[0] == 0 and brow[-1] == n and (np.diff(brow) > 0).all()
+    assert (np.diff(brow) <= i.rowblock_acc_rows).all()
+    for b in range(NB):
+        row0, nr = int(brow[b]), int(brow[b + 1] - brow[b])
+        acc = np.zeros((i.rowblock_acc_rows, X.shape[1]))
+        cur = base[b].copy()
+        for t in range(T):
+            table = np.where(hot_cols[t][:, None] >= 0, X[np.maximum(hot_cols[t], 0)], 0.0)
+            firsts = meta[b, t, :WAVES, 2]
+            assert (np.diff(firsts) >= 0).all(), "first rows of the wavefronts' runs must not decrease"
+            slots = np.zeros((WAVES, X.shape[1]))
+            for w in range(WAVES):
+                first_row = int(firsts[w])
+                for k in range(2):
+                    nk = int(meta[b, t, w, k])  # windows of this wavefront's run
+                    for g in range(G):
+                        row, part, any_entry = first_row, np.zeros(X.shape[1]), False
+                        for jw in range(dealt_len(nk, g)):
+                            # round jw // 2; lane (g, e) holds entry e of the group's two windows side by side
+                            slot0 = (int(cur[w, k]) + jw // 2) * (G * WIN * 2) + g * WIN * 2 + jw % 2
+                            adv = int(streams[k][slot0, 0]) >> bits[k]
+                            if adv:
+                                (slots[w] if row == first_row else acc[row]).__iadd__(part)
+                                part = np.zeros(X.shape[1])
+                                row += adv
+                            assert 0 <= row < nr
+                            real = 0
+                            for e in range(WIN):
+                                word, vbits = int(streams[k][slot0 + 2 * e, 0]), streams[k][slot0 + 2 * e, 1]
+                                val = float(np.array([vbits], dtype=np.uint32).view(np.float32)[0])
+                                idx = word & ((1 << bits[k]) - 1)
+                                assert e == 0 or (word >> bits[k]) == 0, "only a window's first entry advances rows"
+                                x = table[idx] if k == 0 else X[idx]
+                                if k == 0:
+                                    assert hot_cols[t, idx] >= 0
+                                src = int(srcs[k][slot0 + 2 * e])
+                                if src >= 0:
+                                    assert real == e, "a window's nonzeros come first, padding after them"
+                                    real += 1
+                                    seen.append(src)
+                                else:
+                                    assert val == 0.0, "padding carries the value 0"
+                                part = part + val * x
+                            assert real >= 1
+                            any_entry = True
+                        if any_entry:
+                            (slots[w] if row == first_row else acc[row]).__iadd__(part)
+                    cur[w, k] += rounds_for(nk)
+            for w in range(WAVES):
+                acc[int(firsts[w])] += slots[w]
+        for k in range(2):
+            for w in range(WAVES - 1):
+                assert cur[w, k] == base[b, w + 1, k], "a wavefront's streams end where the next one's begin"
+        Y[row0:row0 + nr] = acc[:nr]
+    return Y, np.array(seen, dtype=np.int64)
+
+
+CASES = [
+    # n, max_deg, hubs, steps, table_rows, block_rows, blocks_per_round
+    (300, 40, ((5, 280), (150, 300)), 3, 16, 64, 4),
+    (97, 12, (), 2, 8, 0, 2),
+    (513, 60, ((0, 500), (512, 400)), 5, 32, 40, 8),
+    (64, 64, ((10, 64),), 1, 64, 0, 1),
+    (200, 5, (), 4, 4, 16, 256),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_layout_walk_reproduces_the_product(pkg, case):
+    n, max_deg, hubs, steps, table_rows, block_rows, per_round = case
+    rng = np.random.default_rng(hash(case) % (2 ** 32))
+    rp, ci = random_csr(rng, n, max_deg, p_empty=0.25, hub_rows=hubs)
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, K=16, steps=steps, table_rows=table_rows, block_rows=block_rows,
+                                  blocks_per_round=per_round)
+    assert lay.info.rowblock_steps == steps and lay.info.rowblock_table_rows == table_rows
+    Y, seen = walk_layout(pkg, lay, X.astype(np.float64), n)
+    # every nonzero exactly once
+    assert np.array_equal(np.sort(seen), np.arange(ci.size))
+    A = np.zeros((n, n))
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    A[rows, ci] = val
+    ref = A @ X.astype(np.float64)
+    assert np.allclose(Y, ref, rtol=1e-12, atol=1e-12)
+    # padding slots hold no source
+    C = pkg._cabi
+    for which in (C.MPS_PLAN_ARRAY_RB_HOT_SRC, C.MPS_PLAN_ARRAY_RB_COLD_SRC):
+        src = lay.array(which, np.int32)
+        assert ((src >= 0).sum() + 0) <= ci.size
+    hot_src = lay.array(C.MPS_PLAN_ARRAY_RB_HOT_SRC, np.int32)
+    assert (hot_src >= 0).sum() == lay.info.hot_nnz
+
+
+def test_hot_columns_are_the_busiest_and_dealt_round_robin(pkg):
+    rng = np.random.default_rng(3)
+    n = 400
+    rp, ci = random_csr(rng, n, 80, p_empty=0.1, hub_rows=((7, 390),))
+    val = np.ones(ci.size, dtype=np.float32)
+    T, H = 4, 20
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=T, table_rows=H, blocks_per_round=4)
+    hot_cols = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32).reshape(T, H)
+    deg = np.bincount(ci, minlength=n)
+    order = sorted(range(n), key=lambda c: (-deg[c], c))[:T * H]
+    for k, c in enumerate(order):
+        assert hot_cols[k % T, k // T] == c
+    assert lay.info.hot_nnz == deg[order].sum()
+
+
+def test_blocks_balance_nonzeros(pkg):
+    rng = np.random.default_rng(5)
+    n = 4000
+    rp, ci = random_csr(rng, n, 30, p_empty=0.3, hub_rows=((100, 3000), (2000, 2500), (3999, 1000)))
+    val = np.ones(ci.size, dtype=np.float32)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=2, table_rows=64, blocks_per_round=16)
+    brow = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
+    assert brow.size - 1 == 16
+    per_block = rp[brow[1:]] - rp[brow[:-1]]
+    # no block holds more than the average plus the longest row
+    assert per_block.max() <= ci.size / 16 + np.diff(rp).max()
+
+
+def test_rejects_what_it_is_not_built_for(pkg):
+    rp = np.array([0, 1, 2], dtype=np.int32)
+    ci = np.array([0, 1], dtype=np.int32)
+    val = np.ones(2, dtype=np.float32)
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        pkg.spmm.RowBlockLayout(rp, ci, val, K=32)
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+    with pytest.raises(pkg._cabi.MpsError):
+        pkg.spmm.RowBlockLayout(rp, ci, val, K=16, table_rows=100000)
