@@ -237,6 +237,24 @@ int mps_spmm_f16(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_v
                  const int *d_coord_x, const int *d_coord_y, int tpw, void *d_workspace,
                  size_t workspace_bytes, void *stream);
 
+/* mps_spmm_f32 for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc) and have
+ * no workspace to hand over.  No counterpart in the reference.  The carry-out
+ * records live in an array that is part of the library's device image (one
+ * copy per GPU, MPS_STATIC_SCRATCH_MIB MiB, held until the process ends), so
+ * the call allocates and frees nothing.  Same kernels, same bits as
+ * mps_spmm_f32.  MPS_ERR_WORKSPACE when the records of P partitions do not
+ * fit (mps_spmm_workspace_bytes(P, K, tpw, 4) > mps_static_scratch_bytes()):
+ * at K = 16 that is beyond about 4 million partitions.  All calls on one GPU
+ * share the array: calls that overlap there (different streams or threads)
+ * race.  Nothing has to be cleared between calls: every record a call reads
+ * it has written itself. */
+#define MPS_STATIC_SCRATCH_MIB 32
+int mps_static_scratch_bytes(size_t *bytes_out);
+int mps_spmm_f32_static(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
+                        const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
+                        const int *d_coord_x, const int *d_coord_y, int tpw, void *stream);
+
 /* The same two entry points with the kernels selectable, for per-kernel
  * timing: phases bit 0 = the main kernel, bit 1 = the carry-out fix-up. */
 #define MPS_PHASE_MAIN 1u

@@ -19,6 +19,8 @@
 // sliced copy of the matrix.
 #include "mpspmm_device.hpp"
 
+#include <mutex>
+
 namespace {
 
 // ---------------------------------------------------------------------------
@@ -376,6 +378,36 @@ int spmm_entry(const int *row_ptr, const int *col_idx, const T *val, const T *X,
                                  static_cast<hipStream_t>(stream));
 }
 
+// ---------------------------------------------------------------------------
+// Carry-out records in device memory that the library never allocates: a
+// file-scope array, one copy per GPU, for callers that must not call hipMalloc.
+// `scratch` is a host-side stand-in for the array; its device address is looked
+// up once per device (hipGetSymbolAddress) and only that address is handed to
+// kernels.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = (size_t)MPS_STATIC_SCRATCH_MIB << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices];  // per device, nullptr until first use there
+
+int static_scratch(void **ptr_out)
+{
+    int dev = 0;
+    MPS_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return MPS_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        MPS_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return MPS_ERR_HIP + (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr_out = g_scratch_ptr[dev];
+    return MPS_OK;
+}
+
 }  // namespace
 
 // ===========================================================================
@@ -479,6 +511,28 @@ int mps_spmm_f32(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
 {
     return spmm_entry<float>(d_row_ptr, d_col_idx, d_val, d_X, d_Y, n_rows, nnz, K, P, d_coord_x, d_coord_y,
                              tpw, d_workspace, workspace_bytes, MPS_PHASE_MAIN | MPS_PHASE_FIXUP, stream);
+}
+
+int mps_static_scratch_bytes(size_t *bytes_out)
+{
+    if (!bytes_out) return MPS_ERR_INVALID_ARG;
+    *bytes_out = kStaticScratchBytes;
+    return MPS_OK;
+}
+
+int mps_spmm_f32_static(const int *d_row_ptr, const int *d_col_idx, const float *d_val, const float *d_X,
+                        float *d_Y, int n_rows, int nnz, int K, int P, const int *d_coord_x,
+                        const int *d_coord_y, int tpw, void *stream)
+{
+    // sizes first: a request beyond the array must fail before anything touches the device
+    SpmmShape sh;
+    int rc = make_spmm_shape(n_rows > 0 ? n_rows : 1, K, P, tpw, 4, sh);
+    if (rc != MPS_OK) return rc;
+    if (carry_bytes_for(sh.num_waves, K) > kStaticScratchBytes) return MPS_ERR_WORKSPACE;
+    void *ws = nullptr;
+    if ((rc = static_scratch(&ws)) != MPS_OK) return rc;
+    return spmm_entry<float>(d_row_ptr, d_col_idx, d_val, d_X, d_Y, n_rows, nnz, K, P, d_coord_x, d_coord_y,
+                             tpw, ws, kStaticScratchBytes, MPS_PHASE_MAIN | MPS_PHASE_FIXUP, stream);
 }
 
 int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16_t *d_val,
