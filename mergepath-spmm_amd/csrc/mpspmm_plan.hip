@@ -1058,14 +1058,20 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
 }
 
 // Row-block plan or not.  Forced: yes.  Otherwise only for what the kernel is built for (fp32,
-// K = 16) and where it was measured to win on MI355X: long rows (the LDS tables are loaded once
-// per block and step, so a block must hold many nonzeros per table) and an X beyond the L2.
+// K = 16) and where it was measured to win on MI355X against the slab plans: long rows (the
+// LDS tables are loaded once per block and step, so a block must hold many nonzeros per
+// table), an X of 12 MiB or more (232,965 rows: 0.53 against 0.58 ms, and 0.35 against
+// 0.38 ms at half the nonzeros; 500,000 rows: 0.73 against 0.75 ms; but 100,000 rows, whose X
+// two slabs cover: 0.175 against 0.140 ms) and columns skewed enough for the tables to serve a
+// quarter of the nonzeros (uniform 232,965-row matrix, 10 %: 0.49 against 0.41 ms) - the
+// last is known only once the builder has counted the columns, see kMinHotShare.
+constexpr double kMinHotShare = 0.25;
 bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, unsigned flags)
 {
     if (flags & MPS_PLAN_FORCE_ROWBLOCK) return true;
     if (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT)) return false;
     if (elem_bytes != 4 || K != 16 || n_rows < 1) return false;
-    if ((uint64_t)n_rows * 64 <= (4u << 20) || n_rows > (1 << 22)) return false;
+    if ((uint64_t)n_rows * 64 < (12u << 20) || n_rows > (1 << 22)) return false;
     return (long long)nnz >= 128LL * n_rows;
 }
 
@@ -1126,16 +1132,20 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.block_rows = opt.rowblock_block_rows;
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
+        bp.min_hot_share = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 0.0 : kMinHotShare;
         int rc = mps_rb::create(d_row_ptr, d_col_idx, static_cast<const float *>(d_val), n_rows, nnz, K, bp,
                                 static_cast<hipStream_t>(stream), &pl->rb);
-        if (rc != MPS_OK) {
+        if (rc == MPS_OK) {
+            pl->device_bytes = mps_rb::device_bytes_of(pl->rb);
+            make_spmm_shape(n_rows, K, 1, 0, elem_bytes, pl->shape);
+            *plan_out = pl;
+            return MPS_OK;
+        }
+        if (rc != mps_rb::kNotWorthwhile) {
             plan_free(pl);
             return rc;
         }
-        pl->device_bytes = mps_rb::device_bytes_of(pl->rb);
-        make_spmm_shape(n_rows, K, 1, 0, elem_bytes, pl->shape);
-        *plan_out = pl;
-        return MPS_OK;
+        // columns too evenly used for LDS tables to pay: the slab plan below
     }
     int rc;
     try {

@@ -285,27 +285,37 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restri
             cur_h += rounds_h;
             cur_c += rounds_c;
 
-            // Tails: what every lane-group still holds for the last row of its run.  Neighbouring
-            // groups can end in the same row (one that is longer than a run), so the first group of
-            // every stretch of equal rows adds the stretch up in group order and adds the total.
+            // Tails: what every lane-group still holds for the last row of its run.  A group whose
+            // neighbours end in other rows adds its sums to the row at once.  Neighbouring groups
+            // can also end in the same row (one that is longer than a run): then the first group of
+            // the stretch of equal rows adds the stretch up in group order, through LDS, and adds
+            // the total.
             auto tails = [&](const Walk &w, int len) {
                 const int row = len > 0 ? w.row : -1;
-                st4[lane] = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
-                if (s == 0) my_crows[g] = row;
-                wave_lds_sync();
-                const int prev = g > 0 ? my_crows[g - 1] : -2;
-                if (row >= 0 && prev != row) {
-                    float4 sum = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
-                    for (int k = g + 1; k < kGroups && my_crows[k] == row; ++k) add4(sum, st4[k * 4 + s]);
+                const int prev = __shfl_up(row, 4, 64), next = __shfl_down(row, 4, 64);
+                const bool first = g == 0 || prev != row;
+                const bool shared = row >= 0 && ((g > 0 && prev == row) || (g < kGroups - 1 && next == row));
+                float4 sum = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
+                if (__any(shared)) {
+                    st4[lane] = sum;
+                    if (s == 0) my_crows[g] = row;
+                    wave_lds_sync();
+                    if (shared && first)
+                        for (int k = g + 1; k < kGroups && my_crows[k] == row; ++k) add4(sum, st4[k * 4 + s]);
+                    wave_lds_sync();
+                }
+                if (row >= 0 && first) {
                     float4 *dst = row == first_row ? my_slot4 : acc4 + (size_t)row * 4 + s;
                     float4 o = *dst;
                     add4(o, sum);
                     *dst = o;
                 }
-                wave_lds_sync();
             };
             tails(wh, len_h);
             tails(wc, len_c);
+            // the next table: on its way while the wavefronts gather at the barrier
+            const float4 *pre_src = hot_x4 + (size_t)min(t + 1, T - 1) * H * 4;
+            RB_PRE_LOAD(0) RB_PRE_LOAD(1) RB_PRE_LOAD(2) RB_PRE_LOAD(3) RB_PRE_LOAD(4) RB_PRE_LOAD(5)
             m = m_next;
 
             __syncthreads();  // every gather from this step's table and every add of this step is done
@@ -330,8 +340,6 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restri
                 *reinterpret_cast<float4 *>(slots + lane * 4) = zero4;
             }
             if (t + 1 < T) {
-                const float4 *pre_src = hot_x4 + (size_t)(t + 1) * H * 4;
-                RB_PRE_LOAD(0) RB_PRE_LOAD(1) RB_PRE_LOAD(2) RB_PRE_LOAD(3) RB_PRE_LOAD(4) RB_PRE_LOAD(5)
                 RB_PRE_STORE(0) RB_PRE_STORE(1) RB_PRE_STORE(2) RB_PRE_STORE(3) RB_PRE_STORE(4) RB_PRE_STORE(5)
             }
             __syncthreads();

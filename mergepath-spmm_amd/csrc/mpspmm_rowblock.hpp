@@ -93,7 +93,10 @@ struct BuildParams {
     int block_rows = 0;  // 0 = choose; otherwise the most rows a block may hold
     int num_cus = 256;
     bool keep_src = true;
+    double min_hot_share = 0.0;  // give up (kNotWorthwhile) when the tables would serve a smaller share of the nonzeros
 };
+
+constexpr int kNotWorthwhile = -1;  // build_layout: the matrix is not skewed enough for min_hot_share
 
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,

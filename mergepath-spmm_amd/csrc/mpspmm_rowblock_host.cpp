@@ -132,12 +132,12 @@ void count_block(const int *rp, const int *ci, const ColumnMap &cm, int r0, int 
 
 int default_steps(int n, long long nnz, int table_rows)
 {
-    // Measured on MI355X with the 232,965-row power-law benchmark graph (492 nonzeros per row):
-    // more steps put more nonzeros on the LDS path, but every step costs two barriers and a table
-    // load per workgroup.  Keep about 24 table loads per workgroup and never more hot slots than
-    // there are columns.
+    // Measured on MI355X with power-law graphs of 233,000 to 500,000 rows and 260 to 490 nonzeros per
+    // row: 16 to 24 steps run within 2 % of each other (more steps put more nonzeros on the LDS path,
+    // but every step costs two barriers, a table load per workgroup and more padded windows); 16 makes
+    // the smallest plan.  Never more table slots than columns.
     if (table_rows < 1) table_rows = 1;
-    long long t = 24;
+    long long t = 16;
     const long long most = ((long long)n + table_rows - 1) / table_rows;
     if (t > most) t = most;
     (void)nnz;
@@ -229,6 +229,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         L.hot_cols[(size_t)t * H + slot] = c;
         L.hot_nnz += d_of(c);
     }
+    if ((double)L.hot_nnz < bp.min_hot_share * (double)nnz) return kNotWorthwhile;
     {
         const long long cold_total = (long long)nnz - L.hot_nnz;
         long long cum = 0;

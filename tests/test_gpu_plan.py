@@ -359,11 +359,14 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
     Y = plan.spmm(d_X)
     torch.cuda.synchronize()
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
-    # the library's own choice for rows this long (200 nonzeros on average): a row-block plan
+    # an X this small (two slabs cover it) gets no row-block plan unless asked for
     auto = pkg.spmm.Plan(csr, K)
-    assert auto.info.rowblock_steps > 0
-    check_fp32(auto.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    assert auto.info.rowblock_steps == 0 and auto.info.num_slabs == 2
     auto.close()
+    forced = pkg.spmm.Plan(csr, K, rowblock="force")
+    assert forced.info.rowblock_steps > 0
+    check_fp32(forced.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    forced.close()
     # the plain path on the caller's CSR agrees to rounding
     sched = pkg.spmm.generate_mp_sched(csr.row_ptr, csr.nnz, cost=128)
     Y0 = pkg.spmm.spmm_merge_path(csr, d_X, sched)

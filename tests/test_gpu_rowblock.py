@@ -128,3 +128,22 @@ def test_rowblock_plan_power_law_graph(pkg, orc, dev):
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
     Y2 = plan.spmm(d_X)
     assert torch.equal(Y, Y2)
+
+
+def test_uniform_matrix_falls_back_to_slabs(pkg, orc, dev):
+    # long rows and a large X, but columns used evenly: LDS tables would serve a tenth of the nonzeros,
+    # so the library builds the column-slab plan instead (and a forced row-block plan still works)
+    rp, ci, _ = pkg.graphs.generate("er:n=200000,deg=130", seed=5)
+    n, nnz = rp.size - 1, ci.size
+    assert nnz >= 128 * n
+    val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
+    X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16)
+    assert plan.info.rowblock_steps == 0 and plan.info.num_slabs > 1
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(plan.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    forced = pkg.spmm.Plan(csr, 16, rowblock="force")
+    assert forced.info.rowblock_steps > 0 and forced.info.hot_nnz < 0.25 * nnz
+    check_fp32(forced.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
