@@ -194,6 +194,13 @@ int mps_csr_validate(const int *d_row_ptr, const int *d_col_idx, int n_rows, int
 int mps_partition(const int *d_row_ptr, int n_rows, int nnz, int P, int *d_coord_x,
                   int *d_coord_y, void *stream);
 
+/* The same coordinates computed on the host (row_ptr, coord_x, coord_y are host
+ * arrays), for callers without a GPU at hand and for checking the device
+ * result: the host code of the reference, MergePathSearch and the diagonals of
+ * generate_mp_sched (src/MergePathSpMM.cu:280-297, :327-334), on the host
+ * thread pool.  Bit-exact with mps_partition. */
+int mps_partition_host(const int *row_ptr, int n_rows, int nnz, int P, int *coord_x, int *coord_y);
+
 /* The six per-partition arrays of generate_mp_sched
  * (src/MergePathSpMM.cu:300-385), including its zero-means-none encoding,
  * derived on the device from the coordinates of mps_partition.  Each output
@@ -360,6 +367,9 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
 #define MPS_PLAN_NO_ROWBLOCK 16u    /* never build a row-block plan (see below)  */
 #define MPS_PLAN_FORCE_ROWBLOCK 32u /* row-block plan whatever the matrix looks like (fp32, K = 16 only) */
+#define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
+                                       CSR arrays (what a matrix gets anyway whose column ids and row-end counts do not
+                                       fit 32 bits together) */
 #define MPS_PLAN_NO_SOURCES 64u     /* do not keep the original nonzero index of every slot: saves 4 bytes per
                                        nonzero of device memory; mps_plan_set_values then returns MPS_ERR_UNSUPPORTED */
 

@@ -33,6 +33,7 @@ MPS_PLAN_FORCE_HOT = 8
 MPS_PLAN_NO_ROWBLOCK = 16
 MPS_PLAN_FORCE_ROWBLOCK = 32
 MPS_PLAN_NO_SOURCES = 64
+MPS_PLAN_NO_ROW_MARKS = 128
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
@@ -93,6 +94,7 @@ PROTOTYPES = {
     "mps_degree_values_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "mps_csr_validate": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "mps_partition": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
+    "mps_partition_host": (_i, [_vp, _i, _i, _i, _vp, _vp]),
     "mps_schedule_legacy": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mps_spmm_workspace_bytes": (_i, [_i, _i, _i, _i, ctypes.POINTER(_sz)]),
     "mps_spmm_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _sz, _vp]),

@@ -20,24 +20,14 @@
         if (e_ != hipSuccess) return MPS_ERR_HIP + (int)e_;     \
     } while (0)
 
-#ifndef MPS_HOT_WPB
-#define MPS_HOT_WPB 16
-#endif
-#ifndef MPS_HOT_RPL
-#define MPS_HOT_RPL 1
-#endif
-#ifndef MPS_MAIN_KERNEL_ATTR
-#define MPS_MAIN_KERNEL_ATTR
-#endif
-
 namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kBlock = 64 * kWavesPerBlock;
 constexpr int kWindow = 16;  // nonzeros staged per lane-group per round
 constexpr int kXcds = 8;     // accelerator dies of an MI355X, each with its own L2
-constexpr int kHotRoundsPerLoad = MPS_HOT_RPL;  // rounds of the sliced arrays a hot wavefront loads at a time
-constexpr int kHotWavesPerBlock = MPS_HOT_WPB;  // workgroup of the LDS-resident ("hot") launch of a plan
+constexpr int kHotRoundsPerLoad = 1;    // rounds of the sliced arrays a hot wavefront loads at a time
+constexpr int kHotWavesPerBlock = 16;   // workgroup of the LDS-resident ("hot") launch of a plan
 
 using half_t = _Float16;
 typedef half_t half8_t __attribute__((ext_vector_type(8)));
@@ -256,14 +246,14 @@ __device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T 
 // HOT = true: the column part of an entry is a row slot of the table of X rows
 //   that the workgroup keeps in LDS (see below).
 template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED, bool HOT, bool MARKS, int RPL>
-__global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) MPS_MAIN_KERNEL_ATTR void mp_spmm_kernel(
+__global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) void mp_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
     const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
     const int *__restrict__ coord_y, const int *__restrict__ wave_off, int nnz, int K, int P,
     int lanes_log2, int tpw, int wave_begin, int wave_end, int row_shift, int *__restrict__ ws_head_row,
     float *__restrict__ ws_head, float *__restrict__ ws_tail, const int *__restrict__ hot_cols,
-    const int *__restrict__ seg_part_off, int hot_rows, const int *__restrict__ hot_block_wave, int hot_blocks,
-    int mark_shift)
+    const int *__restrict__ seg_part_off, int num_hot_segs, int hot_rows, const int *__restrict__ hot_block_wave,
+    int hot_blocks, int mark_shift)
 {
     static_assert(!MARKS || SLICED, "row marks live in the sliced arrays");
     static_assert(!HOT || MARKS, "the hot launch reads marked entries");
@@ -297,7 +287,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) MP
         if (w0 >= w_stop) return;  // whole block
         w = w0 + wib;
         const int p0 = w0 * tpw;
-        int lo = 0, hi = seg_part_off[-1] - 1;  // the number of hot segments is stored in front of the table
+        int lo = 0, hi = num_hot_segs - 1;
         while (lo < hi) {  // largest hot segment g with seg_part_off[g] <= p0
             int mid = (lo + hi + 1) >> 1;
             if (seg_part_off[mid] <= p0) lo = mid; else hi = mid - 1;
@@ -826,18 +816,9 @@ inline size_t carry_bytes_for(int num_waves, int K)
     return rows * sizeof(int) + 2 * (size_t)num_waves * K * sizeof(float);
 }
 
-// Gathers in flight per lane between waits.  Fewer means fewer registers and
-// more resident wavefronts, which is what keeps the L1's request queue full;
-// 4 measured best on MI355X.  MPS_GATHER_BATCH=2|4|8 overrides it for tuning.
-inline int gather_batch()
-{
-    static int b = [] {
-        const char *e = std::getenv("MPS_GATHER_BATCH");
-        int v = e ? std::atoi(e) : 0;
-        return (v == 8 || v == 2) ? v : 4;
-    }();
-    return b;
-}
+// Gathers in flight per lane between waits: 4 (fewer registers mean more resident wavefronts,
+// which is what keeps the L1's request queue full; 2 and 8 measured the same or worse on MI355X).
+constexpr int kGatherBatch = 4;
 
 // What a plan adds to a launch: sliced arrays, and optionally the hot launch.
 struct PlanLaunch {
@@ -845,7 +826,8 @@ struct PlanLaunch {
     int hot_waves = 0;                  // waves [0, hot_waves) gather from LDS
     int hot_rows = 0;                   // rows of X per hot table
     const int *hot_cols = nullptr;      // [hot segments][hot_rows] column ids, -1 = unused slot
-    const int *seg_part_off = nullptr;  // first partition of every hot segment; [-1] holds their number
+    const int *seg_part_off = nullptr;  // first partition of every hot segment
+    int num_hot_segs = 0;
     const int *hot_block_wave = nullptr;  // [hot_blocks + 1] wave range of every hot workgroup
     int hot_blocks = 0;
     size_t hot_lds_bytes = 0;
@@ -865,7 +847,6 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
     float *ws_tail = ws_head + (size_t)W * K;
     const int *wave_off = pl.wave_off;
     if (phases & MPS_PHASE_MAIN) {
-        const int batch = gather_batch();
 #define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED, HOT, MARKS, WB, WE, WPB, LDS, SHIFT)                                \
     do {                                                                                                          \
         const int nblocks_ = (HOT) ? pl.hot_blocks : ((WE) - (WB) + (WPB)-1) / (WPB);                             \
@@ -873,16 +854,15 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
         hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED, HOT, MARKS, (HOT) ? kHotRoundsPerLoad : 1>), grid_, \
                            dim3(64 * (WPB)), LDS, st, row_ptr, col_idx, val, X, Y, cx, cy, wave_off, nnz, K, P,   \
                            sh.ls.lanes_log2, sh.tpw, WB, WE, sh.row_shift, ws_head_row, ws_head, ws_tail,         \
-                           pl.hot_cols, pl.seg_part_off, pl.hot_rows, pl.hot_block_wave, pl.hot_blocks, SHIFT);   \
+                           pl.hot_cols, pl.seg_part_off, pl.num_hot_segs, pl.hot_rows, pl.hot_block_wave,         \
+                           pl.hot_blocks, SHIFT);                                                                 \
     } while (0)
         if (pl.hot_waves > 0) {
             // hot launch: only built for power-of-two pitches and vector lanes (VEC > 1)
             if constexpr (VEC > 1) {
                 if (pl.hot_mark_shift <= 0) return MPS_ERR_INVALID_ARG;
-                auto kern = mp_spmm_kernel<T, TOut, VEC, true, 4, true, true, true, kHotRoundsPerLoad>;
-                MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.hot_lds_bytes));
-                MPS_LAUNCH_MAIN(true, 4, true, true, true, 0, pl.hot_waves, kHotWavesPerBlock, pl.hot_lds_bytes,
+                // (the kernel's dynamic LDS limit was raised when the plan was made: allow_hot_lds)
+                MPS_LAUNCH_MAIN(true, kGatherBatch, true, true, true, 0, pl.hot_waves, kHotWavesPerBlock, pl.hot_lds_bytes,
                                 pl.hot_mark_shift);
             } else {
                 return MPS_ERR_UNSUPPORTED;
@@ -891,24 +871,14 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
         const int cold_begin = pl.hot_waves;
         if (cold_begin < W) {
             if (wave_off && pl.mark_shift > 0) {
-                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, 4, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
-                else MPS_LAUNCH_MAIN(false, 4, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+                else MPS_LAUNCH_MAIN(false, kGatherBatch, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
             } else if (wave_off) {
-                if (sh.row_shift >= 0) {
-                    if (batch == 8) MPS_LAUNCH_MAIN(true, 8, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
-                    else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
-                    else MPS_LAUNCH_MAIN(true, 4, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
-                } else {
-                    MPS_LAUNCH_MAIN(false, 4, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
-                }
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
+                else MPS_LAUNCH_MAIN(false, kGatherBatch, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
             } else {
-                if (sh.row_shift >= 0) {
-                    if (batch == 8) MPS_LAUNCH_MAIN(true, 8, false, false, false, 0, W, kWavesPerBlock, 0, 0);
-                    else if (batch == 2) MPS_LAUNCH_MAIN(true, 2, false, false, false, 0, W, kWavesPerBlock, 0, 0);
-                    else MPS_LAUNCH_MAIN(true, 4, false, false, false, 0, W, kWavesPerBlock, 0, 0);
-                } else {
-                    MPS_LAUNCH_MAIN(false, 4, false, false, false, 0, W, kWavesPerBlock, 0, 0);
-                }
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, false, false, false, 0, W, kWavesPerBlock, 0, 0);
+                else MPS_LAUNCH_MAIN(false, kGatherBatch, false, false, false, 0, W, kWavesPerBlock, 0, 0);
             }
         }
 #undef MPS_LAUNCH_MAIN
@@ -929,6 +899,31 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
         MPS_HIP_TRY(hipGetLastError());
     }
     return MPS_OK;
+}
+
+// Raises the dynamic LDS limit of the hot instantiation that launch_spmm<T, TOut, VEC> uses; called once
+// per plan, so that a product launches kernels only (it may run under stream capture).
+template <typename T, typename TOut, int VEC>
+int allow_hot_lds_for(size_t bytes)
+{
+    if constexpr (VEC > 1) {
+        auto kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, true, kHotRoundsPerLoad>;
+        MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)bytes));
+        return MPS_OK;
+    } else {
+        return MPS_ERR_UNSUPPORTED;
+    }
+}
+
+template <typename T, typename TOut>
+int allow_hot_lds(const SpmmShape &sh, size_t bytes)
+{
+    if (sh.ls.vec == 1) return allow_hot_lds_for<T, TOut, 1>(bytes);
+    if constexpr (sizeof(T) == 2) {
+        if (sh.ls.vec == 4) return allow_hot_lds_for<T, TOut, 4>(bytes);
+    }
+    return allow_hot_lds_for<T, TOut, 16 / (int)sizeof(T)>(bytes);
 }
 
 template <typename T, typename TOut>

@@ -714,6 +714,31 @@ int mps_items_per_partition(int n_rows, int nnz, int P, int *ipt_out)
     return MPS_OK;
 }
 
+int mps_partition_host(const int *row_ptr, int n_rows, int nnz, int P, int *coord_x, int *coord_y)
+{
+    if (!row_ptr || !coord_x || !coord_y || n_rows < 0 || nnz < 0 || P < 1) return MPS_ERR_INVALID_ARG;
+    int ipt = 0;
+    int rc = mps_items_per_partition(n_rows, nnz, P, &ipt);
+    if (rc != MPS_OK) return rc;
+    const int num_rows = n_rows + 1;  // the search runs over all of row_ptr, row_ptr[0] included (:333-334)
+    const int64_t total = (int64_t)num_rows + nnz;
+    parallel_for((int64_t)P + 1, 4096, [&](int64_t a, int64_t b) {
+        for (int64_t i = a; i < b; ++i) {
+            const int64_t d64 = (int64_t)ipt * i;
+            const int diagonal = (int)(d64 < total ? d64 : total);
+            // smallest x with row_ptr[x] + x >= diagonal: what the bisection of :283-295 finds
+            int lo = diagonal > nnz ? diagonal - nnz : 0, hi = diagonal < num_rows ? diagonal : num_rows;
+            while (lo < hi) {
+                const int mid = (int)(((int64_t)lo + hi) >> 1);
+                if (row_ptr[mid] <= diagonal - mid - 1) lo = mid + 1; else hi = mid;
+            }
+            coord_x[i] = lo < num_rows ? lo : num_rows;
+            coord_y[i] = diagonal - lo;
+        }
+    });
+    return MPS_OK;
+}
+
 int mps_max_threads_per_wave(int K, int elem_bytes, int *tpw_out)
 {
     if (!tpw_out || K < 1 || (elem_bytes != 4 && elem_bytes != 2)) return MPS_ERR_INVALID_ARG;

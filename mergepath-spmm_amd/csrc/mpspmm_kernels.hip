@@ -52,44 +52,37 @@ __global__ __launch_bounds__(256) void mp_partition_kernel(const int *__restrict
     coord_y[i] = diagonal - x_min;
 }
 
-// The six arrays of generate_mp_sched (src/MergePathSpMM.cu:336-376), from the
-// coordinates, zero-means-none encoding included.
+// The six per-partition arrays that generate_mp_sched hands to the reference
+// kernels (src/MergePathSpMM.cu:336-376), derived from the boundary
+// coordinates.  Partition i covers rows first..last; it has a head piece when
+// it starts inside row `first` (its first nonzero, y_begin, is not the row's
+// first one) and a tail piece when it stops inside row `last`.  The reference
+// stores a piece as (nonzero index, count) and writes index 0 for "no piece",
+// so a piece that would start at nonzero 0 is reported as absent; partition 0
+// never has a head.  A partition that lies inside a single row is all head.
 __global__ __launch_bounds__(256) void mp_schedule_legacy_kernel(
     const int *__restrict__ row_ptr, int P, const int *__restrict__ coord_x,
-    const int *__restrict__ coord_y, int *__restrict__ feature_start_all,
-    int *__restrict__ feature_start_num, int *__restrict__ feature_end_all,
-    int *__restrict__ feature_end_num, int *__restrict__ start_row_all, int *__restrict__ end_row_all)
+    const int *__restrict__ coord_y, int *__restrict__ head_at_out, int *__restrict__ head_count_out,
+    int *__restrict__ tail_at_out, int *__restrict__ tail_count_out, int *__restrict__ first_row_out,
+    int *__restrict__ last_row_out)
 {
-    int core_id = blockIdx.x * blockDim.x + threadIdx.x;
-    if (core_id >= P) return;
-    int start = coord_x[core_id] - 1;
-    int end = coord_x[core_id + 1] - 1;
-    if (start < 0) start = 0;
-    int num_features = 0;
-    int feature_start = coord_y[core_id];
-    if (row_ptr[start] == feature_start) feature_start = 0;
-    if (core_id == 0) feature_start = 0;
-    int feature_end = coord_y[core_id + 1];
-    if (row_ptr[end] == feature_end) feature_end = 0;
-    if (feature_start != 0) {
-        if (start == end && feature_end != 0) {
-            num_features = feature_end - feature_start;
-            feature_end = 0;
-        } else {
-            num_features = row_ptr[start + 1] - feature_start;
-        }
-    }
-    int num_features_end = 0;
-    if (feature_end != 0) {
-        num_features_end = feature_end - row_ptr[end];
-        feature_end = row_ptr[end];
-    }
-    feature_start_all[core_id] = feature_start;
-    feature_end_all[core_id] = feature_end;
-    feature_start_num[core_id] = num_features;
-    feature_end_num[core_id] = num_features_end;
-    start_row_all[core_id] = start;
-    end_row_all[core_id] = end;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= P) return;
+    const int first = max(coord_x[i] - 1, 0), last = coord_x[i + 1] - 1;
+    const int y_begin = coord_y[i], y_end = coord_y[i + 1];
+    const int last_begin = row_ptr[last];
+    const bool head = i != 0 && y_begin != row_ptr[first] && y_begin != 0;
+    bool tail = y_end != last_begin && y_end != 0;
+    const bool one_row = head && tail && first == last;
+    int head_count = 0;
+    if (head) head_count = (one_row ? y_end : row_ptr[first + 1]) - y_begin;
+    if (one_row) tail = false;
+    head_at_out[i] = head ? y_begin : 0;
+    head_count_out[i] = head_count;
+    tail_at_out[i] = tail ? last_begin : 0;
+    tail_count_out[i] = tail ? y_end - last_begin : 0;
+    first_row_out[i] = first;
+    last_row_out[i] = last;
 }
 
 // ---------------------------------------------------------------------------

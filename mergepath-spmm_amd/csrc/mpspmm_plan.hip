@@ -44,7 +44,7 @@ struct mps_plan {
     int hot_waves = 0;         // wavefronts [0, hot_waves) belong to hot segments
     long long hot_nnz = 0;     // nonzeros whose column is hot
     int *hot_cols = nullptr;   // [num_slabs][hot_rows] column ids by slot, -1 = unused
-    int *seg_table = nullptr;  // [0] = num_slabs, [1 + g] = first partition of hot segment g (g <= num_slabs)
+    int *seg_table = nullptr;  // [g] = first partition of hot segment g (g <= num_slabs)
     size_t hot_lds_bytes = 0;
     int hot_cost = 0;               // merge items per partition in the hot segments
     int mark_shift = 0, hot_mark_shift = 0;  // row marks sit above this bit of a column entry (0: none)
@@ -651,6 +651,9 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
 {
     const int n = pl->n_rows, nnz = pl->nnz, K = pl->K, eb = pl->elem_bytes;
     int rc;
+    // The histogram, the hot-column tables and the row marks all index by column id: a column
+    // beyond the matrix (it is square) would write out of bounds or corrupt the marks.
+    if ((rc = mps_csr_validate(d_row_ptr, d_col_idx, n, n, nnz, st)) != MPS_OK) return rc;
     // lane shape and partitions per wavefront do not depend on the partition count
     if ((rc = make_spmm_shape(n, K, 1, tpw, eb, pl->shape)) != MPS_OK) return rc;
     const int G = pl->shape.tpw;
@@ -844,9 +847,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             long long fit = hot_items / (16LL * kHotWavesPerBlock * 256);
             if (fit > kHotCost) fit = kHotCost;
             if (fit < 64) fit = 64;
-            const char *e = std::getenv("MPS_HOT_COST");
-            const int v = e ? std::atoi(e) : 0;
-            pl->hot_cost = v > 0 ? v : (pl->cost > (int)fit ? pl->cost : (int)fit);
+            pl->hot_cost = pl->cost > (int)fit ? pl->cost : (int)fit;
         }
         std::vector<int> h_seg((size_t)3 * S2 + 1);  // seg_off[S2 + 1], seg_parts[S2], seg_ipt[S2]
         int *seg_off = h_seg.data(), *seg_parts = seg_off + S2 + 1, *seg_ipt = seg_parts + S2;
@@ -878,24 +879,24 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
                            pl->vrow_ptr, n, S2, t.seg, t.seg + S2 + 1, t.seg + 2 * S2 + 1, pl->P, pl->coord_x, pl->coord_y);
         MPS_BUILD_HIP(hipGetLastError());
         // what the hot kernel needs: slot -> column lists, and where the hot segments start
-        std::vector<int> h_table((size_t)S + 2);
-        h_table[0] = S;
-        for (int g = 0; g <= S; ++g) h_table[(size_t)g + 1] = seg_off[g];
+        std::vector<int> h_table((size_t)S + 1);
+        for (int g = 0; g <= S; ++g) h_table[(size_t)g] = seg_off[g];
         MPS_BUILD_TRY(dev_alloc(pl, &pl->seg_table, h_table.size()));
         MPS_BUILD_HIP(hipMemcpyAsync(pl->seg_table, h_table.data(), h_table.size() * sizeof(int), hipMemcpyHostToDevice, st));
         MPS_BUILD_TRY(dev_alloc(pl, &pl->hot_cols, h_hot_cols.size()));
         MPS_BUILD_HIP(hipMemcpyAsync(pl->hot_cols, h_hot_cols.data(), h_hot_cols.size() * sizeof(int), hipMemcpyHostToDevice, st));
         MPS_BUILD_HIP(hipStreamSynchronize(st));
         pl->hot_lds_bytes = (size_t)hot_rows * K * eb;
+        // the hot launch's dynamic LDS limit, once (not at every product): tiled plans write fp32 partial rows
+        const int lds_rc = eb == 4 ? (allow_hot_lds<float, float>(pl->shape, pl->hot_lds_bytes))
+                                   : (allow_hot_lds<half_t, float>(pl->shape, pl->hot_lds_bytes));
+        MPS_BUILD_TRY(lds_rc);
         // Hot workgroups: one LDS table per CU at a time, so a few long-lived
         // workgroups per CU, each with a contiguous share of one segment's waves.
         int dev = 0, cus = 256;
         MPS_BUILD_HIP(hipGetDevice(&dev));
         MPS_BUILD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        const char *e = std::getenv("MPS_HOT_BLOCKS_PER_CU");
-        int per_cu = e ? std::atoi(e) : 1;
-        if (per_cu < 1 || per_cu > 64) per_cu = 1;
-        const long long target = (long long)cus * per_cu;
+        const long long target = cus;
         // Workgroups per segment in proportion to its wavefronts, never more than `target` in
         // all: one workgroup too many would run alone after all the others (6 segments at 43
         // workgroups each on 256 CUs took 0.66 instead of 0.55 ms).  Largest remainders first.
@@ -944,10 +945,8 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
     // many values must fit above the column (or LDS slot) bits of an entry.
     auto bits_for = [](long long v) { int b = 1; while ((v >> b) != 0) ++b; return b; };  // values 0..v
     {
-        const char *e = std::getenv("MPS_ROW_MARKS");
-        const bool want = !(e && std::atoi(e) == 0);
         const int col_bits = bits_for(n > 1 ? n - 1 : 1);
-        pl->mark_shift = (want && nnz > 0 && col_bits + bits_for(max_cold_ipt) <= 32) ? col_bits : 0;
+        pl->mark_shift = (!(flags & MPS_PLAN_NO_ROW_MARKS) && nnz > 0 && col_bits + bits_for(max_cold_ipt) <= 32) ? col_bits : 0;
         if (hot_rows > 0) {
             const int slot_bits = bits_for(hot_rows - 1);
             if (slot_bits + bits_for(max_hot_ipt) > 32) {
@@ -1031,7 +1030,8 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     how.hot_waves = pl->hot_waves;
     how.hot_rows = pl->hot_rows;
     how.hot_cols = pl->hot_cols;
-    how.seg_part_off = pl->seg_table ? pl->seg_table + 1 : nullptr;
+    how.seg_part_off = pl->seg_table;
+    how.num_hot_segs = pl->hot_rows > 0 ? pl->num_slabs : 0;
     how.hot_lds_bytes = pl->hot_lds_bytes;
     how.hot_block_wave = pl->hot_block_wave;
     how.hot_blocks = pl->hot_blocks;

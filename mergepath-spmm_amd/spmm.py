@@ -123,12 +123,13 @@ def num_partitions(n_rows, nnz, cost):
     return p.value
 
 
-def generate_mp_sched(row_ptr, nnz, cost=None, P=None):
-    """Merge-path split of (row_ptr, 0..nnz-1) into P partitions, on the device."""
+def generate_mp_sched(row_ptr, nnz, cost=None, P=None, K=16, elem_bytes=4):
+    """Merge-path split of (row_ptr, 0..nnz-1) into P partitions, on the device.  Without cost or P the
+    library's default cost for feature width K and element size elem_bytes is used."""
     _need(row_ptr, torch.int32, "row_ptr")
     n_rows = int(row_ptr.numel()) - 1
     if P is None:
-        P = num_partitions(n_rows, nnz, default_cost(n_rows, nnz) if cost is None else cost)
+        P = num_partitions(n_rows, nnz, default_cost(n_rows, nnz, K, elem_bytes) if cost is None else cost)
     cx = torch.empty(P + 1, dtype=torch.int32, device=row_ptr.device)
     cy = torch.empty(P + 1, dtype=torch.int32, device=row_ptr.device)
     check(_cabi.lib().mps_partition(_ptr(row_ptr), n_rows, int(nnz), int(P), _ptr(cx), _ptr(cy), _stream()),
@@ -176,7 +177,7 @@ class Plan:
 
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
-                 rowblock_blocks_per_round=0, keep_sources=True):
+                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -187,6 +188,8 @@ class Plan:
         flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_ROWBLOCK, "force": _cabi.MPS_PLAN_FORCE_ROWBLOCK}[rowblock]
         if not keep_sources:
             flags |= _cabi.MPS_PLAN_NO_SOURCES
+        if not row_marks:
+            flags |= _cabi.MPS_PLAN_NO_ROW_MARKS
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
                                 int(rowblock_block_rows), int(rowblock_blocks_per_round))
         check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,

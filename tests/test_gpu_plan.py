@@ -215,11 +215,10 @@ def test_hot_columns_layout_and_result(pkg, orc, dev, K, dtype, hot_rows):
     assert torch.equal(Y, Y2)
 
 
-def test_plan_without_row_marks(pkg, orc, dev, monkeypatch):
-    """MPS_ROW_MARKS=0 at plan creation: plain column ids in the sliced array, and
-    the kernel follows row_ptr as it does on the caller's CSR arrays (the path a
-    matrix takes whose column ids and row-end counts do not fit 32 bits together)."""
-    monkeypatch.setenv("MPS_ROW_MARKS", "0")
+def test_plan_without_row_marks(pkg, orc, dev):
+    """MPS_PLAN_NO_ROW_MARKS: plain column ids in the sliced array, and the kernel
+    follows row_ptr as it does on the caller's CSR arrays (the path a matrix takes
+    whose column ids and row-end counts do not fit 32 bits together)."""
     rng = np.random.default_rng(77)
     n, K = 700, 16
     rp, ci = random_csr(rng, n, 30, hub_rows=[(0, 650), (350, 400)])
@@ -229,14 +228,13 @@ def test_plan_without_row_marks(pkg, orc, dev, monkeypatch):
     (d_X,) = to_dev(dev, X)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     for tiling, slab_bytes in (("off", 0), ("force", 16384)):
-        plan = pkg.spmm.Plan(csr, K, cost=12, tiling=tiling, slab_bytes=slab_bytes, hot="off")
+        plan = pkg.spmm.Plan(csr, K, cost=12, tiling=tiling, slab_bytes=slab_bytes, hot="off", row_marks=False)
         assert plan.info.mark_shift == 0 and plan.info.hot_rows == 0
         check_plan_layout(pkg, orc, plan, rp, ci, val)
         Y = plan.spmm(d_X)
         torch.cuda.synchronize()
         check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
         plan.close()
-    monkeypatch.delenv("MPS_ROW_MARKS")
     plan = pkg.spmm.Plan(csr, K, cost=12, tiling="off")
     assert plan.info.mark_shift == 10  # 700 columns: 10 bits
     plan.close()
@@ -411,12 +409,19 @@ def test_plan_spmm_in_a_hip_graph(pkg, orc, dev):
     g = pkg.graphs
     K = 16
     for spec, kwargs in (("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", dict(tiling="force", slab_bytes=4096 * K * 4)),
+                         # with the hot launch (LDS tables) and its cold companion
+                         ("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000",
+                          dict(tiling="force", slab_bytes=4096 * K * 4, hot="force")),
+                         # a row-block plan: gather kernel + main kernel
+                         ("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", dict(rowblock="force", rowblock_steps=5)),
                          ("er:n=4096,deg=8", dict())):
         rp, ci, _ = g.generate(spec, seed=8)
         n = rp.size - 1
         val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
         csr = make_csr(pkg, dev, rp, ci, val)
         plan = pkg.spmm.Plan(csr, K, **kwargs)
+        assert (plan.info.hot_rows > 0) == (kwargs.get("hot") == "force")
+        assert (plan.info.rowblock_steps > 0) == (kwargs.get("rowblock") == "force")
         X = torch.from_numpy(g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)).to(dev)
         Y = torch.full_like(X, float("nan"))
         eager = plan.spmm(X).clone()
@@ -446,3 +451,16 @@ def test_plan_spmm_in_a_hip_graph(pkg, orc, dev):
         ref, scale = orc.spmm_f64(rp, ci, val, X.cpu().numpy(), want_abs=True)
         check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
         plan.close()
+
+
+def test_plan_refuses_columns_beyond_the_matrix(pkg, dev):
+    rng = np.random.default_rng(4)
+    rp, ci = random_csr(rng, 500, 20)
+    val = rng.random(ci.size).astype(np.float32)
+    bad = ci.copy()
+    bad[7] = 500  # one past the last row of X
+    csr = make_csr(pkg, dev, rp, bad, val)
+    for kwargs in (dict(), dict(tiling="force", slab_bytes=64 * 16 * 4), dict(tiling="force", slab_bytes=64 * 16 * 4, hot="force")):
+        with pytest.raises(pkg._cabi.MpsError) as e:
+            pkg.spmm.Plan(csr, 16, cost=8, **kwargs)
+        assert e.value.status == pkg._cabi.MPS_ERR_INVALID_CSR

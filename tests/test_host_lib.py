@@ -62,6 +62,36 @@ def test_num_partitions_matches_oracle(pkg, orc):
     assert dc(100000, 20000000) == 64 and dc(100000, 3100000) == 32
 
 
+def test_partition_host_matches_oracle(pkg, orc):
+    """mps_partition_host (the host twin of the device partitioner) against the oracle's literal
+    search, on random CSRs with empty rows and hubs, for partition counts below, at and above the
+    number of merge items, and on the hand-worked examples."""
+    from tests.gpu_util import random_csr
+    L = pkg._cabi.lib()
+    rng = np.random.default_rng(12)
+
+    def host(rp, nnz, P):
+        rp = np.ascontiguousarray(rp, dtype=np.int32)
+        x, y = np.empty(P + 1, dtype=np.int32), np.empty(P + 1, dtype=np.int32)
+        pkg._cabi.check(L.mps_partition_host(rp.ctypes.data, rp.size - 1, int(nnz), int(P), x.ctypes.data, y.ctypes.data),
+                        "mps_partition_host")
+        return x, y
+
+    for _ in range(60):
+        n = int(rng.integers(1, 400))
+        rp, ci = random_csr(rng, n, int(rng.integers(1, 40)), p_empty=0.3, hub_rows=((int(rng.integers(0, n)), n),))
+        for P in (1, 3, 17, 1024, n + ci.size + 1, 2 * (n + ci.size) + 7):
+            x, y = host(rp, ci.size, P)
+            xs, ys = orc.partition_coords(rp, ci.size, P)
+            assert np.array_equal(x, xs) and np.array_equal(y, ys)
+    # hand-worked coordinates (P used directly)
+    x, y = host([0, 0, 5, 5, 6, 14, 15], 15, 5)
+    assert list(zip(x, y)) == [(0, 0), (2, 3), (4, 6), (5, 10), (6, 14), (7, 15)]
+    x, y = host([0, 3, 3, 4, 9], 9, 3)
+    assert list(zip(x, y)) == [(0, 0), (2, 3), (4, 6), (5, 9)]
+    assert L.mps_partition_host(None, 3, 3, 4, None, None) == pkg._cabi.MPS_ERR_INVALID_ARG
+
+
 def test_max_threads_per_wave(pkg):
     table = {(16, 4): 16, (32, 4): 8, (64, 4): 4, (128, 4): 2, (256, 4): 1, (512, 4): 1, (8, 4): 8, (1, 4): 16,
              (20, 4): 8, (17, 4): 2, (64, 2): 8, (32, 2): 16, (16, 2): 16, (24, 2): 8, (12, 2): 4, (128, 2): 4}
