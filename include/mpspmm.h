@@ -267,6 +267,7 @@ int mps_spmm_f32_static(const int *d_row_ptr, const int *d_col_idx, const float 
 #define MPS_PHASE_MAIN 1u
 #define MPS_PHASE_FIXUP 2u
 #define MPS_PHASE_REDUCE 4u /* plans with column slabs only */
+#define MPS_PHASE_PREPARE 8u /* row-block plans only: the small kernel that gathers the hot columns' rows of X */
 int mps_spmm_f32_phases(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
                         const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
                         const int *d_coord_x, const int *d_coord_y, int tpw,
@@ -356,7 +357,8 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *   Calls on one plan share its workspace: do not overlap them on different
  *   streams.
  * mps_plan_spmm_phases: the same with the kernels selectable, for timing
- *   (MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE).
+ *   (MPS_PHASE_PREPARE | MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE;
+ *   a phase the plan's kind does not have launches nothing).
  * mps_plan_copy_array: copies one of the plan's device arrays to the host
  *   (bytes must equal its size), for inspection and tests. */
 typedef struct mps_plan mps_plan;

@@ -24,6 +24,7 @@ MPS_ERR_HIP = 1000
 MPS_PHASE_MAIN = 1
 MPS_PHASE_FIXUP = 2
 MPS_PHASE_REDUCE = 4
+MPS_PHASE_PREPARE = 8
 MPS_WEIGHT_DEGREE_PRODUCT = 0
 MPS_WEIGHT_GCN = 1
 MPS_PLAN_NO_TILING = 1

@@ -1247,14 +1247,14 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
 
 int mps_plan_spmm_f32(const mps_plan *plan, const float *d_X, float *d_Y, void *stream)
 {
-    return plan_spmm<float>(plan, d_X, d_Y, MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE,
+    return plan_spmm<float>(plan, d_X, d_Y, MPS_PHASE_PREPARE | MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE,
                             static_cast<hipStream_t>(stream));
 }
 
 int mps_plan_spmm_f16(const mps_plan *plan, const uint16_t *d_X, uint16_t *d_Y, void *stream)
 {
     return plan_spmm<half_t>(plan, reinterpret_cast<const half_t *>(d_X), reinterpret_cast<half_t *>(d_Y),
-                             MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE, static_cast<hipStream_t>(stream));
+                             MPS_PHASE_PREPARE | MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE, static_cast<hipStream_t>(stream));
 }
 
 int mps_plan_spmm_phases(const mps_plan *plan, const void *d_X, void *d_Y, unsigned phases, void *stream)
@@ -1322,7 +1322,7 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
             continue;
         }
         if (rc != MPS_OK) break;
-        const unsigned all = MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE;
+        const unsigned all = MPS_PHASE_PREPARE | MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE;
         for (int i = 0; i < 2 && rc == MPS_OK; ++i) rc = mps_plan_spmm_phases(pl, d_X, d_Y, all, stream);
         if (rc == MPS_OK) he = hipEventRecord(e0, st);
         for (int i = 0; i < repeats && rc == MPS_OK; ++i) rc = mps_plan_spmm_phases(pl, d_X, d_Y, all, stream);

@@ -465,11 +465,12 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
 int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStream_t st)
 {
     const Layout &L = dp->host;
-    if (!(phases & MPS_PHASE_MAIN)) return MPS_OK;
     const int slots = L.steps * L.table_rows;
-    hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
-                       reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
-    hipLaunchKernelGGL((rb_spmm_kernel<float>), dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot,
+    if (phases & MPS_PHASE_PREPARE)
+        hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
+                           reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
+    if (phases & MPS_PHASE_MAIN)
+        hipLaunchKernelGGL((rb_spmm_kernel<float>), dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot,
                        dp->cold, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta), dp->block_row,
                        reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X), Y, L.steps,
                        L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits);
