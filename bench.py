@@ -59,7 +59,8 @@ def plan_signature(workload, info):
     if info.rowblock_steps > 0:
         return "%s|rowblock|steps=%d|table_rows=%d|blocks=%d" % (workload, info.rowblock_steps, info.rowblock_table_rows,
                                                                   info.rowblock_blocks)
-    return "%s|slabs=%d|cost=%d|hot_rows=%d" % (workload, info.num_slabs, info.cost, info.hot_rows)
+    return "%s|slabs=%d|cost=%d|hot_rows=%d|resident_cols=%d" % (workload, info.num_slabs, info.cost, info.hot_rows,
+                                                                 info.resident_cols)
 
 
 def measured_traffic(signature):
@@ -130,6 +131,9 @@ def layout_text(w, plan):
                 % (i.rowblock_blocks, i.rowblock_steps, i.rowblock_table_rows, 100.0 * i.hot_nnz / max(w.nnz, 1),
                    i.device_bytes / 1e6))
     text = "plan: %d column slab(s) of %d, sliced, %.0f MB" % (i.num_slabs, i.slab_cols, i.device_bytes / 1e6)
+    if i.resident_cols:
+        text += ", streaming hint on gathers outside the %d busiest columns (%.1f %% of the nonzeros)" % (
+            i.resident_cols, 100.0 * (1.0 - i.resident_nnz / max(w.nnz, 1)))
     if i.hot_rows:
         text += ", %d hot columns per slab in LDS (%.1f %% of the nonzeros)" % (i.hot_rows, 100.0 * i.hot_nnz / max(w.nnz, 1))
     return text
@@ -168,6 +172,9 @@ def main():
                          "library picks it / never / always")
     ap.add_argument("--rb-steps", type=int, default=0, help="steps (LDS tables) of a row-block plan (0 = library default)")
     ap.add_argument("--rb-table-rows", type=int, default=0, help="rows per LDS table of a row-block plan (0 = what fits)")
+    ap.add_argument("--resident", default="auto", choices=["auto", "off"],
+                    help="untiled plans: streaming hint on the gathers of unpopular columns where the library picks it / never")
+    ap.add_argument("--resident-bytes", type=int, default=0, help="rows of X gathered without the hint (0 = library default)")
     ap.add_argument("--slab-bytes", type=int, default=0, help="slab size for tiling (0 = library default)")
     ap.add_argument("--tpw", type=int, default=0, help="partitions per wavefront (0 = full wavefront)")
     ap.add_argument("--seed", type=int, default=1)
@@ -207,7 +214,8 @@ def main():
         cost = args.cost if args.cost > 0 else sp.default_cost(wl.n, wl.nnz, wl.K, wl.eb)
         kw = dict(cost=cost, threads_per_wave=args.tpw, tiling={"auto": "auto", "untiled": "off", "tiled": "force", "plain": "auto"}[args.mode],
                   slab_bytes=args.slab_bytes, hot=args.hot, rowblock=args.rowblock, rowblock_steps=args.rb_steps,
-                  rowblock_table_rows=args.rb_table_rows, keep_sources=False)
+                  rowblock_table_rows=args.rb_table_rows, keep_sources=False, resident=args.resident,
+                  resident_bytes=args.resident_bytes)
         kw.update(overrides)
         return sp.Plan(wl.csr, wl.K, **kw), cost
 

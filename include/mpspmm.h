@@ -369,6 +369,7 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
 #define MPS_PLAN_NO_ROWBLOCK 16u    /* never build a row-block plan (see below)  */
 #define MPS_PLAN_FORCE_ROWBLOCK 32u /* row-block plan whatever the matrix looks like (fp32, K = 16 only) */
+#define MPS_PLAN_NO_RESIDENT 256u    /* untiled plans: no streaming hint on the gathers of unpopular columns (see below) */
 #define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
                                        CSR arrays (what a matrix gets anyway whose column ids and row-end counts do not
                                        fit 32 bits together) */
@@ -397,6 +398,9 @@ typedef struct mps_plan_info {
     int rowblock_acc_rows;         /* rows of LDS accumulators per workgroup      */
     long long rowblock_hot_slots;  /* entries of the hot stream incl. padding     */
     long long rowblock_cold_slots; /* entries of the cold stream incl. padding    */
+    /* resident columns (resident_cols > 0): SLICE_COLS entries are column | streamed << mark_shift | row_ends << (mark_shift + 1) */
+    int resident_cols;             /* columns whose rows of X are gathered without the streaming hint */
+    long long resident_nnz;        /* nonzeros in them                            */
 } mps_plan_info;
 
 /* Optional parameters of mps_plan_create_ex; zero means "the library chooses". */
@@ -407,6 +411,7 @@ typedef struct mps_plan_options {
     int rowblock_table_rows; /* H of a row-block plan                            */
     int rowblock_block_rows; /* most rows per row block                          */
     int rowblock_blocks_per_round; /* row blocks are made in multiples of this (0: the number of CUs) */
+    size_t resident_bytes;   /* rows of X (of the busiest columns) that an untiled plan gathers without the streaming hint; set: whatever the size of X and the skew */
 } mps_plan_options;
 
 enum {

@@ -35,6 +35,7 @@ MPS_PLAN_NO_ROWBLOCK = 16
 MPS_PLAN_FORCE_ROWBLOCK = 32
 MPS_PLAN_NO_SOURCES = 64
 MPS_PLAN_NO_ROW_MARKS = 128
+MPS_PLAN_NO_RESIDENT = 256
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
@@ -51,14 +52,15 @@ class PlanInfo(ctypes.Structure):
                 ("hot_mark_shift", ctypes.c_int), ("hot_blocks", ctypes.c_int),
                 ("rowblock_steps", ctypes.c_int), ("rowblock_table_rows", ctypes.c_int),
                 ("rowblock_blocks", ctypes.c_int), ("rowblock_acc_rows", ctypes.c_int),
-                ("rowblock_hot_slots", ctypes.c_longlong), ("rowblock_cold_slots", ctypes.c_longlong)]
+                ("rowblock_hot_slots", ctypes.c_longlong), ("rowblock_cold_slots", ctypes.c_longlong),
+                ("resident_cols", ctypes.c_int), ("resident_nnz", ctypes.c_longlong)]
 
 
 class PlanOptions(ctypes.Structure):
     """struct mps_plan_options"""
     _fields_ = [("flags", ctypes.c_uint), ("slab_bytes", ctypes.c_size_t), ("rowblock_steps", ctypes.c_int),
                 ("rowblock_table_rows", ctypes.c_int), ("rowblock_block_rows", ctypes.c_int),
-                ("rowblock_blocks_per_round", ctypes.c_int)]
+                ("rowblock_blocks_per_round", ctypes.c_int), ("resident_bytes", ctypes.c_size_t)]
 
 
 class TuneResult(ctypes.Structure):

@@ -143,6 +143,25 @@ __device__ __forceinline__ void store_acc(half_t *p, const float (&acc)[VEC])
     }
 }
 
+// A row piece of X read through a buffer descriptor, with or without the streaming hint (AUX bit 1,
+// "nt": the line is the first to leave the caches again).  Two plain global loads on the two sides of
+// a branch get folded into one by the compiler, which then drops the hint; buffer loads that differ
+// in their cache-policy operand stay two instructions.
+template <typename Raw, int AUX>
+__device__ __forceinline__ Raw buffer_load_raw(__amdgpu_buffer_rsrc_t rsrc, unsigned off)
+{
+    if constexpr (sizeof(Raw) == 16) {
+        return __builtin_bit_cast(Raw, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, AUX));
+    } else if constexpr (sizeof(Raw) == 8) {
+        return __builtin_bit_cast(Raw, __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)off, 0, AUX));
+    } else if constexpr (sizeof(Raw) == 4) {
+        return __builtin_bit_cast(Raw, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, AUX));
+    } else {
+        static_assert(sizeof(Raw) == 2, "rows of X are read 2, 4, 8 or 16 bytes at a time");
+        return __builtin_bit_cast(Raw, __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)off, 0, AUX));
+    }
+}
+
 // Address of the VEC columns a lane owns in row `c` of X.  POW2: the row
 // pitch is a power of two and the matrix is below 4 GiB, so the byte offset
 // is one shift-or in 32 bits (the load then takes its base from SGPRs).
@@ -162,6 +181,13 @@ struct Gather {
             size_t off = (size_t)c * row_bytes + col_byte;
             return *reinterpret_cast<const Raw *>(xb + off);
         }
+    }
+    // POW2 only: row c with the streaming hint (streamed) or without, through the buffer descriptor of X
+    __device__ __forceinline__ Raw load_hinted(__amdgpu_buffer_rsrc_t rsrc, int c, bool streamed) const
+    {
+        static_assert(POW2, "32-bit offsets");
+        const unsigned off = ((unsigned)c << row_shift) | col_byte;
+        return streamed ? buffer_load_raw<Raw, 2>(rsrc, off) : buffer_load_raw<Raw, 0>(rsrc, off);
     }
 };
 
@@ -239,13 +265,17 @@ __device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T 
 //   (wave_off[w] + round) * tpw * 16 elements into the arrays, so the whole
 //   wavefront stages a round with one contiguous, fully coalesced load per
 //   array; wave_off[w + 1] - wave_off[w] is the number of rounds of wave w.
-// MARKS = true (sliced arrays only): every column entry also says how many
+// MARKS = 1 (sliced arrays only): every column entry also says how many
 //   rows end in front of its nonzero, entry = column | ends << mark_shift, so
 //   the kernel never reads row_ptr while it works through a partition: no load
 //   of its own sits between the window prefetch and the gathers.
+// MARKS = 2: entry = column | streamed << mark_shift | ends << (mark_shift + 1);
+//   streamed = 1 marks a column outside the set of popular columns whose rows
+//   of X are meant to stay in L2: its row is gathered with the streaming hint,
+//   so that it does not push a popular row out.
 // HOT = true: the column part of an entry is a row slot of the table of X rows
 //   that the workgroup keeps in LDS (see below).
-template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED, bool HOT, bool MARKS, int RPL>
+template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED, bool HOT, int MARKS, int RPL>
 __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) void mp_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
     const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
@@ -257,6 +287,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
 {
     static_assert(!MARKS || SLICED, "row marks live in the sliced arrays");
     static_assert(!HOT || MARKS, "the hot launch reads marked entries");
+    static_assert(MARKS != 2 || POW2, "streamed entries need the 32-bit offsets of a power-of-two pitch");
     constexpr int WPB = HOT ? kHotWavesPerBlock : kWavesPerBlock;
     using XO = XOps<T, VEC>;
     using Raw = typename XO::Raw;
@@ -316,9 +347,16 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
     const Gather<T, VEC, POW2> gx{reinterpret_cast<const char *>(X), (size_t)K * sizeof(T),
                                   col_ok ? (unsigned)(kcol * sizeof(T)) : 0u, row_shift};
 
-    auto gather = [&](int c) -> Raw {
+    // all of X below 4 GiB (what POW2 promises), 32-bit elements, no swizzle
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(X), 0, 0xffffffff, 0x00020000);
+    // the row of X that a column entry names
+    auto gather = [&](int entry, unsigned mask, int shift) -> Raw {
+        const int c = MARKS ? (int)((unsigned)entry & mask) : entry;
         if constexpr (HOT) {
             return *reinterpret_cast<const Raw *>(s_hot + (((unsigned)c << row_shift) | gx.col_byte));
+        } else if constexpr (MARKS == 2) {
+            return gx.load_hinted(x_rsrc, c, (((unsigned)entry >> shift) & 1u) != 0);
         } else {
             return gx.load(c);
         }
@@ -372,12 +410,11 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
     // rows that end in front of nonzero idx (entry: what the column array holds for it)
     auto finish_rows = [&](int idx, int entry) {
         if constexpr (MARKS) {
-            for (unsigned e = (unsigned)entry >> mark_shift; e != 0; --e) emit();
+            for (unsigned e = (unsigned)entry >> (mark_shift + (MARKS == 2 ? 1 : 0)); e != 0; --e) emit();
         } else {
             while (idx == row_end) emit();
         }
     };
-    auto column_of = [&](int entry) { return MARKS ? (int)((unsigned)entry & mark_mask) : entry; };
 
     int wbase = y_begin;
     // sliced staging: lane l moves elements [4l, 4l + 4) of the wave's round block
@@ -397,7 +434,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
                 for (int j = 0; j < BATCH; ++j) {
                     ent[j] = s_col[b + j];
                     av[j] = s_val[b + j];
-                    xr[j] = gather(column_of(ent[j]));
+                    xr[j] = gather(ent[j], mark_mask, mark_shift);
                 }
 #pragma unroll
                 for (int j = 0; j < BATCH; ++j) {
@@ -414,7 +451,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
                 for (int j = 0; j < BATCH; ++j) {
                     if (b + j < nvalid) {
                         ent[j] = s_col[b + j];
-                        xr[j] = gather(column_of(ent[j]));
+                        xr[j] = gather(ent[j], mark_mask, mark_shift);
                     }
                 }
 #pragma unroll
@@ -833,6 +870,7 @@ struct PlanLaunch {
     size_t hot_lds_bytes = 0;
     int mark_shift = 0;      // > 0: entries of the (cold) sliced column array carry row marks above this bit
     int hot_mark_shift = 0;  // the same for the hot waves
+    bool streamed_flag = false;  // the bit at mark_shift says "gather with the streaming hint", row marks sit one bit higher
 };
 
 template <typename T, typename TOut, int VEC>
@@ -847,7 +885,7 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
     float *ws_tail = ws_head + (size_t)W * K;
     const int *wave_off = pl.wave_off;
     if (phases & MPS_PHASE_MAIN) {
-#define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED, HOT, MARKS, WB, WE, WPB, LDS, SHIFT)                                \
+#define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED, HOT, MARKS, WB, WE, WPB, LDS, SHIFT)  /* MARKS: 0, 1 or 2 */                                \
     do {                                                                                                          \
         const int nblocks_ = (HOT) ? pl.hot_blocks : ((WE) - (WB) + (WPB)-1) / (WPB);                             \
         dim3 grid_((nblocks_ + kXcds - 1) / kXcds * kXcds, sh.ls.col_tiles);                                      \
@@ -862,7 +900,7 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
             if constexpr (VEC > 1) {
                 if (pl.hot_mark_shift <= 0) return MPS_ERR_INVALID_ARG;
                 // (the kernel's dynamic LDS limit was raised when the plan was made: allow_hot_lds)
-                MPS_LAUNCH_MAIN(true, kGatherBatch, true, true, true, 0, pl.hot_waves, kHotWavesPerBlock, pl.hot_lds_bytes,
+                MPS_LAUNCH_MAIN(true, kGatherBatch, true, true, 1, 0, pl.hot_waves, kHotWavesPerBlock, pl.hot_lds_bytes,
                                 pl.hot_mark_shift);
             } else {
                 return MPS_ERR_UNSUPPORTED;
@@ -870,15 +908,18 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
         }
         const int cold_begin = pl.hot_waves;
         if (cold_begin < W) {
-            if (wave_off && pl.mark_shift > 0) {
-                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
-                else MPS_LAUNCH_MAIN(false, kGatherBatch, true, false, true, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+            if (wave_off && pl.mark_shift > 0 && pl.streamed_flag) {
+                if (sh.row_shift < 0) return MPS_ERR_INVALID_ARG;  // plans set the flag for power-of-two pitches only
+                MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, 2, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+            } else if (wave_off && pl.mark_shift > 0) {
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, 1, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
+                else MPS_LAUNCH_MAIN(false, kGatherBatch, true, false, 1, cold_begin, W, kWavesPerBlock, 0, pl.mark_shift);
             } else if (wave_off) {
-                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
-                else MPS_LAUNCH_MAIN(false, kGatherBatch, true, false, false, cold_begin, W, kWavesPerBlock, 0, 0);
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, true, false, 0, cold_begin, W, kWavesPerBlock, 0, 0);
+                else MPS_LAUNCH_MAIN(false, kGatherBatch, true, false, 0, cold_begin, W, kWavesPerBlock, 0, 0);
             } else {
-                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, false, false, false, 0, W, kWavesPerBlock, 0, 0);
-                else MPS_LAUNCH_MAIN(false, kGatherBatch, false, false, false, 0, W, kWavesPerBlock, 0, 0);
+                if (sh.row_shift >= 0) MPS_LAUNCH_MAIN(true, kGatherBatch, false, false, 0, 0, W, kWavesPerBlock, 0, 0);
+                else MPS_LAUNCH_MAIN(false, kGatherBatch, false, false, 0, 0, W, kWavesPerBlock, 0, 0);
             }
         }
 #undef MPS_LAUNCH_MAIN
@@ -907,7 +948,7 @@ template <typename T, typename TOut, int VEC>
 int allow_hot_lds_for(size_t bytes)
 {
     if constexpr (VEC > 1) {
-        auto kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, true, kHotRoundsPerLoad>;
+        auto kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, 1, kHotRoundsPerLoad>;
         MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         (int)bytes));
         return MPS_OK;

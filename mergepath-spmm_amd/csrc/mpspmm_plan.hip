@@ -48,6 +48,9 @@ struct mps_plan {
     size_t hot_lds_bytes = 0;
     int hot_cost = 0;               // merge items per partition in the hot segments
     int mark_shift = 0, hot_mark_shift = 0;  // row marks sit above this bit of a column entry (0: none)
+    bool streamed_flag = false;  // untiled plans: bit mark_shift of an entry marks a column outside the resident set
+    int resident_cols = 0;       // columns whose rows of X are gathered without the streaming hint
+    long long resident_nnz = 0;  // nonzeros in them
     int *hot_block_wave = nullptr;  // [hot_blocks + 1] first wave of every hot workgroup
     int hot_blocks = 0;
     bool keep_sources = true;       // slice_src is kept (mps_plan_set_values works)
@@ -59,6 +62,9 @@ namespace {
 // Slab of X that stays resident in a 4 MiB L2 next to the streamed data
 // (3 MiB measured best on the power-law benchmark graph; 2 and 2.5 MiB within 5 %).
 constexpr size_t kDefaultSlabBytes = 3u << 20;
+constexpr size_t kDefaultResidentBytes = 10u << 20;  // rows of X that an untiled plan shields from streamed gathers
+constexpr uint64_t kResidentMinXBytes = 192ull << 20;  // ... when X is this large
+constexpr double kResidentMinShare = 0.4;               // ... and the shielded columns hold this share of the nonzeros
 
 // ---------------------------------------------------------------------------
 // Cost model behind the automatic choices (slab size, hot columns), from
@@ -290,6 +296,7 @@ __global__ __launch_bounds__(256) void slice_count_kernel(const int *__restrict_
 // nonzero y, on diagonal row + 1 + y, and partition p owns the diagonals
 // [p * ipt, (p + 1) * ipt) - of the whole matrix (seg == nullptr), or of the
 // nonzero's segment (seg: seg_off[num_segs + 1], seg_parts[num_segs], seg_ipt[num_segs]).
+// streamed (optional, int per column, 0 or 1): goes into bit shift of the entry, the row marks one bit higher.
 __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restrict__ col_v,
                                                              const int *__restrict__ perm,
                                                              const int *__restrict__ vrow_of,
@@ -299,6 +306,7 @@ __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restric
                                                              const int *__restrict__ wave_off, int nnz, int ipt,
                                                              const int *__restrict__ seg, int num_segs, int seg_rows,
                                                              int hot_parts, int hot_mark_shift, int mark_shift,
+                                                             const int *__restrict__ streamed,
                                                              int *__restrict__ slice_cols,
                                                              int *__restrict__ slice_src)
 {
@@ -334,7 +342,8 @@ __global__ __launch_bounds__(256) void slice_scatter_kernel(const int *__restric
         if (k == 0) before = max(coord_x[p], 1) - 1;
         else if (vrow_of) before = vrow_of[y - 1];
         else before = vrow_ptr[row] < y ? row : row_of(y - 1);
-        entry |= (unsigned)(row - before) << shift;
+        if (streamed) entry |= ((unsigned)streamed[col_v[y]] << shift) | ((unsigned)(row - before) << (shift + 1));
+        else entry |= (unsigned)(row - before) << shift;
     }
     slice_cols[slot] = (int)entry;
     slice_src[slot] = perm ? perm[y] : y;
@@ -647,7 +656,7 @@ long long select_hot_columns(const std::vector<int> &deg, int n, int num_slabs, 
 
 // Builds everything; temporaries are released before returning.
 int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const void *d_val, unsigned flags,
-               size_t slab_bytes, int tpw, hipStream_t st)
+               size_t slab_bytes, size_t resident_bytes, int tpw, hipStream_t st)
 {
     const int n = pl->n_rows, nnz = pl->nnz, K = pl->K, eb = pl->elem_bytes;
     int rc;
@@ -955,6 +964,47 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
             }
             pl->hot_mark_shift = slot_bits;
         }
+        // Resident columns (untiled plans): the columns with the most nonzeros, as many as fit
+        // resident_bytes, are gathered as usual; the entries of all other columns carry a flag and are
+        // gathered with the streaming hint, so that the popular rows of X outlive in the caches the rows
+        // that are used once or twice.  Measured on MI355X (R-MAT, 16 nonzeros per row, 1 and 4 M rows):
+        // the hint makes a gather that misses dearer, so it pays only where the resident columns hold a
+        // good share of the nonzeros and X is beyond the 256 MiB last-level cache: X of 256 MiB to 1 GiB
+        // with 8 to 12 MiB resident (47 to 73 % of the nonzeros) runs 10 to 18 % faster, X of 64 and
+        // 128 MiB up to 10 % slower, 0.5 MiB resident (13 to 27 % of the nonzeros) 30 to 60 % slower.
+        const uint64_t row_bytes = (uint64_t)K * eb;
+        const uint64_t budget = resident_bytes ? resident_bytes : kDefaultResidentBytes;
+        const long long fit = (long long)(budget / row_bytes);
+        if (pl->mark_shift > 0 && pl->num_slabs == 1 && hot_rows == 0 && !(flags & MPS_PLAN_NO_RESIDENT) && fit >= 1 &&
+            fit < n && ((uint64_t)n * row_bytes >= kResidentMinXBytes || resident_bytes) && pl->shape.row_shift >= 0 &&
+            col_bits + 1 + bits_for(max_cold_ipt) <= 32) {
+            MPS_BUILD_TRY(column_histogram());
+            std::vector<int> d(h_deg);
+            std::nth_element(d.begin(), d.begin() + (long)fit, d.end(), [](int a, int b) { return a > b; });
+            const int thr = d[(size_t)fit];  // the (fit + 1)-th largest count: columns above it are resident
+            long long above = 0, above_nnz = 0, thr_cols = 0;
+            for (int c = 0; c < n; ++c) {
+                const int x = h_deg[(size_t)c];
+                above += x > thr;
+                above_nnz += x > thr ? x : 0;
+                thr_cols += x == thr;
+            }
+            long long ties = thr > 0 ? std::min(fit - above, thr_cols) : 0;  // columns with exactly thr nonzeros that still fit
+            if (resident_bytes || (double)(above_nnz + ties * thr) >= kResidentMinShare * (double)nnz) {
+                for (int c = 0; c < n; ++c) {
+                    int &x = h_deg[(size_t)c];
+                    const bool in = x > thr || (x == thr && ties > 0 && ties-- > 0);  // ties in column order
+                    if (in) {
+                        ++pl->resident_cols;
+                        pl->resident_nnz += x;
+                    }
+                    x = in ? 0 : 1;  // from here on: the streamed flag of the column
+                }
+                MPS_BUILD_HIP(hipMemcpyAsync(t.deg, h_deg.data(), (size_t)n * sizeof(int), hipMemcpyHostToDevice, st));
+                MPS_BUILD_HIP(hipStreamSynchronize(st));
+                pl->streamed_flag = true;
+            }
+        }
     }
 
     // 5. slices
@@ -985,7 +1035,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
                            pl->num_slabs == 1 ? nullptr : t.perm, pl->num_slabs == 1 ? nullptr : t.vrow, pl->vrow_ptr,
                            pl->n_vrows, pl->coord_x, pl->coord_y, G, pl->wave_off, nnz, max_cold_ipt,
                            hot_rows > 0 ? t.seg : nullptr, pl->num_segs, n, pl->hot_waves * G, pl->hot_mark_shift,
-                           pl->mark_shift, pl->slice_cols, pl->slice_src);
+                           pl->mark_shift, pl->streamed_flag ? t.deg : nullptr, pl->slice_cols, pl->slice_src);
         MPS_BUILD_HIP(hipGetLastError());
     }
     MPS_BUILD_TRY(plan_set_values(pl, d_val, st));
@@ -1037,6 +1087,7 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     how.hot_blocks = pl->hot_blocks;
     how.mark_shift = pl->mark_shift;
     how.hot_mark_shift = pl->hot_mark_shift;
+    how.streamed_flag = pl->streamed_flag;
     if (pl->num_segs == 1)
         return launch_spmm_any<T, T>(pl->vrow_ptr, pl->slice_cols, vals, X, Y, pl->nnz, pl->K, pl->P, pl->coord_x,
                                      pl->coord_y, how, pl->shape, carry, phases, st);
@@ -1149,7 +1200,8 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     }
     int rc;
     try {
-        rc = plan_build(pl, d_row_ptr, d_col_idx, d_val, flags, slab_bytes, tpw, static_cast<hipStream_t>(stream));
+        rc = plan_build(pl, d_row_ptr, d_col_idx, d_val, flags, slab_bytes, opt.resident_bytes, tpw,
+                        static_cast<hipStream_t>(stream));
     } catch (const std::bad_alloc &) {  // host-side tables of the build
         rc = MPS_ERR_UNSUPPORTED;
     }
@@ -1186,6 +1238,8 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->hot_cost = plan->hot_cost;
     info->mark_shift = plan->mark_shift;
     info->hot_mark_shift = plan->hot_mark_shift;
+    info->resident_cols = plan->resident_cols;
+    info->resident_nnz = plan->resident_nnz;
     info->hot_blocks = plan->hot_blocks;
     info->rowblock_steps = info->rowblock_table_rows = info->rowblock_blocks = info->rowblock_acc_rows = 0;
     info->rowblock_hot_slots = info->rowblock_cold_slots = 0;

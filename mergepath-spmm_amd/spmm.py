@@ -177,7 +177,7 @@ class Plan:
 
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
-                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True):
+                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -190,8 +190,10 @@ class Plan:
             flags |= _cabi.MPS_PLAN_NO_SOURCES
         if not row_marks:
             flags |= _cabi.MPS_PLAN_NO_ROW_MARKS
+        if resident == "off":
+            flags |= _cabi.MPS_PLAN_NO_RESIDENT
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
-                                int(rowblock_block_rows), int(rowblock_blocks_per_round))
+                                int(rowblock_block_rows), int(rowblock_blocks_per_round), int(resident_bytes))
         check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
                                              int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
                                              int(threads_per_wave), ctypes.byref(opt), _stream(),

@@ -141,6 +141,10 @@ def test_rmat_config_full_size(pkg, orc, dev, K):
     (d_X,) = to_dev(dev, X)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     plan = pkg.spmm.Plan(csr, K)
+    # X of 256 MiB and more (beyond the last-level cache): the 10 MiB of busiest columns stay plain gathers,
+    # the rest is gathered with the streaming hint
+    assert plan.info.num_slabs == 1 and (plan.info.resident_cols > 0) == (K >= 64)
+    assert plan.info.resident_cols == 0 or plan.info.resident_nnz > 0.4 * ci.size
     Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     torch.cuda.synchronize()
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
@@ -184,6 +188,7 @@ def test_fp16_config_full_size(pkg, orc, dev):
     (d_X,) = to_dev(dev, X)
     ref, scale = orc.spmm_f64_f16in(rp, ci, val, X, want_abs=True)
     plan = pkg.spmm.Plan(csr, K)
+    assert plan.info.resident_cols == (10 << 20) // 128 and plan.info.resident_nnz > 0.6 * ci.size
     Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     torch.cuda.synchronize()
     Yh = Y.cpu().numpy().astype(np.float64)

@@ -137,7 +137,16 @@ def check_plan_layout(pkg, orc, plan, rp, ci, val):
     assert (i.hot_mark_shift > 0) == (i.hot_rows > 0)
     cols_u = cols.astype(np.int64) & 0xFFFFFFFF
     got_col = np.where(shift > 0, cols_u & ((1 << shift) - 1), cols_u)
-    got_ends = np.where(shift > 0, cols_u >> shift, 0)
+    # plans with resident columns: one flag bit (gather with the streaming hint) between column and row ends
+    flag_bits = 1 if i.resident_cols > 0 else 0
+    got_ends = np.where(shift > 0, cols_u >> (shift + flag_bits), 0)
+    if flag_bits:
+        deg = np.bincount(ci, minlength=n)
+        order = sorted(range(n), key=lambda col: (-deg[col], col))[:i.resident_cols]
+        assert all(deg[col] > 0 for col in order) and i.resident_nnz == int(deg[order].sum())
+        streamed = np.ones(n, dtype=np.int64)
+        streamed[order] = 0
+        assert np.array_equal(((cols_u >> shift) & 1)[live], streamed[want_cols[want_src[live]]])
     inv = np.empty(nnz, dtype=np.int64)
     inv[perm] = np.arange(nnz)  # original nonzero -> virtual position
     vpos = inv[want_src[live]]
@@ -238,6 +247,60 @@ def test_plan_without_row_marks(pkg, orc, dev):
     plan = pkg.spmm.Plan(csr, K, cost=12, tiling="off")
     assert plan.info.mark_shift == 10  # 700 columns: 10 bits
     plan.close()
+
+
+@pytest.mark.parametrize("K,dtype", [(16, np.float32), (4, np.float32), (2, np.float32), (1, np.float32), (64, np.float16),
+                                     (4, np.float16), (2, np.float16), (1, np.float16), (256, np.float32)])
+def test_resident_columns_layout_and_result(pkg, orc, dev, K, dtype):
+    """Untiled plan with resident columns (resident_bytes set, so that a small matrix gets them): the busiest
+    columns' entries are plain, all others carry the streamed flag and are gathered with the streaming hint;
+    the product has the same bits as without the flag (same partition, same order of summation).  The widths
+    cover the 16-, 8-, 4- and 2-byte gathers of both element types."""
+    rng = np.random.default_rng(1234 + K)
+    n = 900
+    rp, ci = random_csr(rng, n, 24, hub_rows=[(3, 800), (500, 650)])
+    half = dtype == np.float16
+    val = rng.random(ci.size).astype(dtype)
+    X = (rng.random((n, K)) * 2 - 1).astype(dtype)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    row_bytes = K * (2 if half else 4)
+    want = 40
+    plan = pkg.spmm.Plan(csr, K, cost=12, tiling="off", resident_bytes=want * row_bytes)
+    assert plan.info.resident_cols == want and plan.info.num_slabs == 1 and plan.info.mark_shift == 10
+    check_plan_layout(pkg, orc, plan, rp, ci, val)
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    plain = pkg.spmm.Plan(csr, K, cost=12, tiling="off", resident="off")
+    assert plain.info.resident_cols == 0
+    Y0 = plain.spmm(d_X)
+    torch.cuda.synchronize()
+    assert torch.equal(Y, Y0)
+    if half:
+        ref, scale = orc.spmm_f64_f16in(rp, ci, val, X, want_abs=True)
+        check_fp16(Y.cpu().numpy(), ref, scale)
+    else:
+        ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+        check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    # new values through the kept source indices
+    val2 = rng.random(ci.size).astype(dtype)
+    plan.set_values(to_dev(dev, val2)[0])
+    plain.set_values(to_dev(dev, val2)[0])
+    assert torch.equal(plan.spmm(d_X), plain.spmm(d_X))
+    plan.close()
+    plain.close()
+
+
+def test_resident_columns_are_chosen_for_large_skewed_inputs_only(pkg, dev):
+    """Without resident_bytes the library flags streamed gathers only where they were measured to pay: X of
+    192 MiB or more and at least 40 % of the nonzeros in the 10 MiB of busiest columns; a pitch that is not a
+    power of two (64-bit offsets) never gets them."""
+    rng = np.random.default_rng(5)
+    rp, ci = random_csr(rng, 600, 20)
+    val = rng.random(ci.size).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    assert pkg.spmm.Plan(csr, 16, tiling="off").info.resident_cols == 0           # small X
+    assert pkg.spmm.Plan(csr, 20, tiling="off", resident_bytes=800).info.resident_cols == 0  # 80-byte pitch
+    assert pkg.spmm.Plan(csr, 16, tiling="off", resident_bytes=64 * 10).info.resident_cols == 10
 
 
 def test_unsorted_rows(pkg, dev):
