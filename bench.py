@@ -86,7 +86,7 @@ def measured_traffic(signature):
 class Workload:
     """One benchmark configuration resident on the device."""
 
-    def __init__(self, pkg, name, spec, K, dt, seed, torch, dev):
+    def __init__(self, pkg, name, spec, K, dt, seed, torch, dev, values="uniform"):
         g, sp = pkg.graphs, pkg.spmm
         self.name, self.spec, self.K, self.dt = name, spec, K, dt
         self.f16 = dt == "f16"
@@ -95,11 +95,18 @@ class Workload:
         self.rp, self.ci, self.max_deg = g.generate(spec, seed=seed)
         self.n, self.nnz = self.rp.size - 1, self.ci.size
         fill = g.fill_uniform_f16 if self.f16 else g.fill_uniform_f32
-        self.val = fill(self.nnz, 11, 0.0, 1.0)
         self.X = fill(self.n * K, 13, -1.0, 1.0).reshape(self.n, K)
+        d_rp, d_ci = torch.from_numpy(self.rp).to(dev), torch.from_numpy(self.ci).to(dev)
+        if values == "uniform":
+            self.val = fill(self.nnz, 11, 0.0, 1.0)
+            d_val = torch.from_numpy(self.val).to(dev)
+        else:
+            # the reference's implicit edge weight (or the GCN norm) as an explicit array, made on the device
+            d_val = sp.degree_values(d_rp, d_ci, mode="product" if values == "degree" else "gcn",
+                                     dtype=torch.float16 if self.f16 else torch.float32)
+            self.val = d_val.cpu().numpy()
         self.gen_s = time.time() - t0
-        self.csr = sp.CsrDevice(torch.from_numpy(self.rp).to(dev), torch.from_numpy(self.ci).to(dev),
-                                torch.from_numpy(self.val).to(dev))
+        self.csr = sp.CsrDevice(d_rp, d_ci, d_val)
         self.d_X = torch.from_numpy(self.X).to(dev)
         self.d_Y = torch.full_like(self.d_X, float("nan"))
         self.csr.validate()
@@ -175,6 +182,11 @@ def main():
     ap.add_argument("--resident", default="auto", choices=["auto", "off"],
                     help="untiled plans: streaming hint on the gathers of unpopular columns where the library picks it / never")
     ap.add_argument("--resident-bytes", type=int, default=0, help="rows of X gathered without the hint (0 = library default)")
+    ap.add_argument("--values", default="uniform", choices=["uniform", "degree", "gcn"],
+                    help="edge values: U[0,1), or the reference's deg(r) * deg(c), or 1 / sqrt(deg(r) * deg(c)), as a value array")
+    ap.add_argument("--weights", default="none", choices=["none", "degree", "gcn"],
+                    help="plan with degree weights: the same weights formed from one factor per node, no value array "
+                         "(fp32; the check then compares with the value array of the same weights)")
     ap.add_argument("--slab-bytes", type=int, default=0, help="slab size for tiling (0 = library default)")
     ap.add_argument("--tpw", type=int, default=0, help="partitions per wavefront (0 = full wavefront)")
     ap.add_argument("--seed", type=int, default=1)
@@ -208,14 +220,19 @@ def main():
     if args.dtype:
         dt, custom = args.dtype, True
     name = "custom" if custom else args.workload
-    w = Workload(pkg, name, spec, K, dt, args.seed, torch, dev)
+    if args.weights != "none":
+        args.values, custom = args.weights, True
+    elif args.values != "uniform":
+        custom = True
+    name = "custom" if custom else args.workload
+    w = Workload(pkg, name, spec, K, dt, args.seed, torch, dev, values=args.values)
 
     def make_plan(wl, **overrides):
         cost = args.cost if args.cost > 0 else sp.default_cost(wl.n, wl.nnz, wl.K, wl.eb)
         kw = dict(cost=cost, threads_per_wave=args.tpw, tiling={"auto": "auto", "untiled": "off", "tiled": "force", "plain": "auto"}[args.mode],
                   slab_bytes=args.slab_bytes, hot=args.hot, rowblock=args.rowblock, rowblock_steps=args.rb_steps,
                   rowblock_table_rows=args.rb_table_rows, keep_sources=False, resident=args.resident,
-                  resident_bytes=args.resident_bytes)
+                  resident_bytes=args.resident_bytes, weights=None if args.weights == "none" else args.weights)
         kw.update(overrides)
         return sp.Plan(wl.csr, wl.K, **kw), cost
 
@@ -307,6 +324,7 @@ def main():
         "config": {"workload": name, "spec": spec, "n_rows": int(w.n), "nnz": int(w.nnz), "K": K,
                    "max_row_degree": int(w.max_deg), "cost": cost, "partitions": P,
                    "threads_per_wave": args.tpw or g.max_threads_per_wave(K, w.eb), "seed": args.seed,
+                   "values": args.values, "weights": "value array" if args.weights == "none" else "one factor per node (no value array)",
                    "layout": layout_text(w, plan), "plan_signature": signature,
                    "plan_bytes": int(info.device_bytes) if info is not None else 0, "csr_bytes": int(csr_bytes)},
         "gbs_algorithmic_per_step": round(w.b_alg / (ms_per_step * 1e6), 2),

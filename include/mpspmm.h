@@ -360,7 +360,21 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *   (MPS_PHASE_PREPARE | MPS_PHASE_MAIN | MPS_PHASE_FIXUP | MPS_PHASE_REDUCE;
  *   a phase the plan's kind does not have launches nothing).
  * mps_plan_copy_array: copies one of the plan's device arrays to the host
- *   (bytes must equal its size), for inspection and tests. */
+ *   (bytes must equal its size), for inspection and tests.
+ *
+ * Degree weights (mps_plan_options.degree_weights, fp32 only): the reference
+ * forms the weight of nonzero (r, c) from the degrees of r and c inside its
+ * kernel instead of reading a value array (src/MergePathSpMM.cu:183-185, :450,
+ * :459-460).  A plan with degree weights does the same without a value per
+ * nonzero: it keeps one factor per node (the degree, or 1 / sqrt(degree)),
+ * scales X by the column factor into a buffer of its own before the kernels
+ * (MPS_PHASE_PREPARE), adds up rows of that buffer (the sliced arrays hold
+ * column entries only) and multiplies every finished row by its row factor
+ * where it is written.  Y = D A_pattern D X with the factors applied in that
+ * order: within rounding of the product with mps_degree_values_f32's array
+ * (row sums differ by a few ulp), half the sparse bytes per nonzero.
+ * mps_plan_set_values returns MPS_ERR_UNSUPPORTED on such a plan; row-block
+ * plans are not built for it. */
 typedef struct mps_plan mps_plan;
 
 #define MPS_PLAN_NO_TILING 1u    /* never tile                                  */
@@ -411,6 +425,8 @@ typedef struct mps_plan_options {
     int rowblock_table_rows; /* H of a row-block plan                            */
     int rowblock_block_rows; /* most rows per row block                          */
     int rowblock_blocks_per_round; /* row blocks are made in multiples of this (0: the number of CUs) */
+    int degree_weights;      /* 0: values from d_val.  1: the weight of nonzero (r, c) is deg(r) * deg(c), 2: 1 / sqrt(deg(r) * deg(c))
+                                (MPS_WEIGHT_DEGREE_PRODUCT + 1, MPS_WEIGHT_GCN + 1): d_val is not read, see "degree weights" below */
     size_t resident_bytes;   /* rows of X (of the busiest columns) that an untiled plan gathers without the streaming hint; set: whatever the size of X and the skew */
 } mps_plan_options;
 

@@ -60,7 +60,8 @@ class PlanOptions(ctypes.Structure):
     """struct mps_plan_options"""
     _fields_ = [("flags", ctypes.c_uint), ("slab_bytes", ctypes.c_size_t), ("rowblock_steps", ctypes.c_int),
                 ("rowblock_table_rows", ctypes.c_int), ("rowblock_block_rows", ctypes.c_int),
-                ("rowblock_blocks_per_round", ctypes.c_int), ("resident_bytes", ctypes.c_size_t)]
+                ("rowblock_blocks_per_round", ctypes.c_int), ("degree_weights", ctypes.c_int),
+                ("resident_bytes", ctypes.c_size_t)]
 
 
 class TuneResult(ctypes.Structure):

@@ -244,13 +244,17 @@ __device__ __forceinline__ Win load_slice_vals(const half_t *p, Win w)
     w.v = make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
     return w;
 }
+__device__ __forceinline__ int4 load_slice_cols(const int *__restrict__ cols, size_t e0)
+{
+    typedef int i4_t __attribute__((ext_vector_type(4)));
+    i4_t t = __builtin_nontemporal_load(reinterpret_cast<const i4_t *>(cols + e0));
+    return make_int4(t[0], t[1], t[2], t[3]);
+}
 template <typename T>
 __device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T *__restrict__ vals, size_t e0)
 {
-    typedef int i4_t __attribute__((ext_vector_type(4)));
     Win w;
-    i4_t t = __builtin_nontemporal_load(reinterpret_cast<const i4_t *>(cols + e0));
-    w.c = make_int4(t[0], t[1], t[2], t[3]);
+    w.c = load_slice_cols(cols, e0);
     return load_slice_vals(vals + e0, w);
 }
 
@@ -275,7 +279,13 @@ __device__ __forceinline__ Win load_slice(const int *__restrict__ cols, const T 
 //   so that it does not push a popular row out.
 // HOT = true: the column part of an entry is a row slot of the table of X rows
 //   that the workgroup keeps in LDS (see below).
-template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED, bool HOT, int MARKS, int RPL>
+// PATTERN = 1: every nonzero counts 1 (val is not read): rows of X are added
+//   up.  PATTERN = 2: also, a finished row r is multiplied by row_scale[r]
+//   where it is written to Y (the carry records stay unscaled, the fix-up
+//   kernel scales).  Plans with degree weights use them: X arrives scaled by
+//   the column factor; the row factor is row_scale (2, untiled plans) or is
+//   applied when the partial rows are summed (1, tiled plans).
+template <typename T, typename TOut, int VEC, bool POW2, int BATCH, bool SLICED, bool HOT, int MARKS, int RPL, int PATTERN = 0>
 __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) void mp_spmm_kernel(
     const int *__restrict__ row_ptr, const int *__restrict__ col_idx, const T *__restrict__ val,
     const T *__restrict__ X, TOut *__restrict__ Y, const int *__restrict__ coord_x,
@@ -283,9 +293,10 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
     int lanes_log2, int tpw, int wave_begin, int wave_end, int row_shift, int *__restrict__ ws_head_row,
     float *__restrict__ ws_head, float *__restrict__ ws_tail, const int *__restrict__ hot_cols,
     const int *__restrict__ seg_part_off, int num_hot_segs, int hot_rows, const int *__restrict__ hot_block_wave,
-    int hot_blocks, int mark_shift)
+    int hot_blocks, int mark_shift, const float *__restrict__ row_scale)
 {
     static_assert(!MARKS || SLICED, "row marks live in the sliced arrays");
+    static_assert(!PATTERN || MARKS, "pattern mode is built for plans with row marks");
     static_assert(!HOT || MARKS, "the hot launch reads marked entries");
     static_assert(MARKS != 2 || POW2, "streamed entries need the 32-bit offsets of a power-of-two pitch");
     constexpr int WPB = HOT ? kHotWavesPerBlock : kWavesPerBlock;
@@ -389,6 +400,10 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
     int head_row = -1;
+    [[maybe_unused]] float cur_scale = 1.f;  // PATTERN = 2: row_scale of the row in progress
+    if constexpr (PATTERN == 2) {
+        if (part_ok && x - 1 < x_end) cur_scale = row_scale[x - 1];
+    }
 
     auto emit = [&]() {
         const int row = x - 1;
@@ -397,7 +412,15 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
 #pragma unroll
             for (int i = 0; i < VEC; ++i) my_head[i] = acc[i];
         } else if (col_ok) {
+            if constexpr (PATTERN == 2) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[i] *= cur_scale;
+            }
             store_acc<VEC, !HOT>(Y + (size_t)row * K + kcol, acc);
+        }
+        if constexpr (PATTERN == 2) {
+            // the factor of the row that starts now, requested a whole row ahead of its use
+            if (x < x_end) cur_scale = row_scale[x];
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
@@ -433,7 +456,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
 #pragma unroll
                 for (int j = 0; j < BATCH; ++j) {
                     ent[j] = s_col[b + j];
-                    av[j] = s_val[b + j];
+                    av[j] = PATTERN ? 1.0f : s_val[b + j];
                     xr[j] = gather(ent[j], mark_mask, mark_shift);
                 }
 #pragma unroll
@@ -458,7 +481,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
                 for (int j = 0; j < BATCH; ++j) {
                     if (b + j < nvalid) {
                         finish_rows(wbase + b + j, ent[j]);
-                        XO::fma(acc, s_val[b + j], xr[j]);
+                        XO::fma(acc, PATTERN ? 1.0f : s_val[b + j], xr[j]);
                     }
                 }
             }
@@ -481,8 +504,10 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
         auto load_rounds = [&](int r0) {
 #pragma unroll
             for (int h = 0; h < RPL; ++h)
-                if (stager && r0 + h < round_end)
-                    nx[h] = load_slice<T>(col_idx, val, (size_t)(r0 + h) * round_elems + 4 * lane);
+                if (stager && r0 + h < round_end) {
+                    if constexpr (PATTERN) nx[h].c = load_slice_cols(col_idx, (size_t)(r0 + h) * round_elems + 4 * lane);
+                    else nx[h] = load_slice<T>(col_idx, val, (size_t)(r0 + h) * round_elems + 4 * lane);
+                }
         };
         load_rounds(round);
         while (round < round_end) {
@@ -495,7 +520,7 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
                 const int nvalid = min(kWindow, y_end - wbase);  // <= 0 for a group that is done
                 if (stager) {
                     *reinterpret_cast<int4 *>(s_col_wave + 4 * lane) = cu[0].c;
-                    *reinterpret_cast<float4 *>(s_val_wave + 4 * lane) = cu[0].v;
+                    if constexpr (!PATTERN) *reinterpret_cast<float4 *>(s_val_wave + 4 * lane) = cu[0].v;
                 }
                 wave_lds_sync();
                 consume(nvalid);
@@ -554,7 +579,9 @@ __global__ __launch_bounds__(64 * (HOT ? kHotWavesPerBlock : kWavesPerBlock)) vo
                     if (kc == 0) ws_head_row[w] = hr;
                     first = false;
                 } else if (kc_ok) {
-                    Y[(size_t)hr * K + kc] = (TOut)v;
+                    float f = 1.f;
+                    if constexpr (PATTERN == 2) f = row_scale[hr];
+                    Y[(size_t)hr * K + kc] = (TOut)(v * f);
                 }
                 carry = t;
             } else {
@@ -581,7 +608,8 @@ template <typename TOut>
 __global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ ws_head_row,
                                                         const float *__restrict__ ws_head,
                                                         const float *__restrict__ ws_tail,
-                                                        TOut *__restrict__ Y, int num_waves, int K)
+                                                        TOut *__restrict__ Y, int num_waves, int K,
+                                                        const float *__restrict__ row_scale)
 {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long w64 = idx / K;
@@ -613,6 +641,7 @@ __global__ __launch_bounds__(256) void mp_fixup_kernel(const int *__restrict__ w
         if (done) break;
         j -= 4;
     }
+    if (row_scale) sum *= row_scale[hr];
     Y[(size_t)hr * K + k] = (TOut)sum;
 }
 
@@ -628,7 +657,8 @@ template <typename TOut>
 __global__ __launch_bounds__(256) void mp_fixup_wide_kernel(const int *__restrict__ ws_head_row,
                                                              const float *__restrict__ ws_head,
                                                              const float *__restrict__ ws_tail,
-                                                             TOut *__restrict__ Y, int num_waves, int K)
+                                                             TOut *__restrict__ Y, int num_waves, int K,
+                                                             const float *__restrict__ row_scale)
 {
     const int lane = threadIdx.x & 63;
     const int lpr = K >> 2;      // lanes per record
@@ -724,6 +754,13 @@ __global__ __launch_bounds__(256) void mp_fixup_wide_kernel(const int *__restric
         if (slot * lpr == src_lane && slot < slots) add(sum, v);
     }
     if (mine) {
+        if (row_scale) {
+            const float f = row_scale[hr];
+            sum.x *= f;
+            sum.y *= f;
+            sum.z *= f;
+            sum.w *= f;
+        }
         TOut *out = Y + (size_t)hr * K + 4 * q;
         out[0] = (TOut)sum.x;
         out[1] = (TOut)sum.y;
@@ -870,6 +907,8 @@ struct PlanLaunch {
     size_t hot_lds_bytes = 0;
     int mark_shift = 0;      // > 0: entries of the (cold) sliced column array carry row marks above this bit
     int hot_mark_shift = 0;  // the same for the hot waves
+    bool pattern = false;             // every nonzero counts 1, val is not read (plans with degree weights)
+    const float *row_scale = nullptr; // pattern: factor of every finished row (nullptr: none, e.g. partial rows of a tiled plan)
     bool streamed_flag = false;  // the bit at mark_shift says "gather with the streaming hint", row marks sit one bit higher
 };
 
@@ -884,16 +923,37 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
     float *ws_head = reinterpret_cast<float *>(ws_head_row + rows);
     float *ws_tail = ws_head + (size_t)W * K;
     const int *wave_off = pl.wave_off;
+    if (pl.pattern && (sizeof(T) != 4 || !wave_off || pl.mark_shift <= 0)) return MPS_ERR_UNSUPPORTED;
     if (phases & MPS_PHASE_MAIN) {
 #define MPS_LAUNCH_MAIN(POW2, BATCH, SLICED, HOT, MARKS, WB, WE, WPB, LDS, SHIFT)  /* MARKS: 0, 1 or 2 */                                \
     do {                                                                                                          \
         const int nblocks_ = (HOT) ? pl.hot_blocks : ((WE) - (WB) + (WPB)-1) / (WPB);                             \
         dim3 grid_((nblocks_ + kXcds - 1) / kXcds * kXcds, sh.ls.col_tiles);                                      \
+        if constexpr ((MARKS) != 0 && sizeof(T) == 4) {                                                           \
+            if (pl.pattern && pl.row_scale) {                                                                     \
+                hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED, HOT, MARKS,                 \
+                                                   (HOT) ? kHotRoundsPerLoad : 1, 2>), grid_,                     \
+                                   dim3(64 * (WPB)), LDS, st, row_ptr, col_idx, val, X, Y, cx, cy, wave_off, nnz, \
+                                   K, P, sh.ls.lanes_log2, sh.tpw, WB, WE, sh.row_shift, ws_head_row, ws_head,    \
+                                   ws_tail, pl.hot_cols, pl.seg_part_off, pl.num_hot_segs, pl.hot_rows,           \
+                                   pl.hot_block_wave, pl.hot_blocks, SHIFT, pl.row_scale);                        \
+                break;                                                                                            \
+            }                                                                                                     \
+            if (pl.pattern) {                                                                                     \
+                hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED, HOT, MARKS,                 \
+                                                   (HOT) ? kHotRoundsPerLoad : 1, 1>), grid_,                     \
+                                   dim3(64 * (WPB)), LDS, st, row_ptr, col_idx, val, X, Y, cx, cy, wave_off, nnz, \
+                                   K, P, sh.ls.lanes_log2, sh.tpw, WB, WE, sh.row_shift, ws_head_row, ws_head,    \
+                                   ws_tail, pl.hot_cols, pl.seg_part_off, pl.num_hot_segs, pl.hot_rows,           \
+                                   pl.hot_block_wave, pl.hot_blocks, SHIFT, nullptr);                             \
+                break;                                                                                            \
+            }                                                                                                     \
+        }                                                                                                         \
         hipLaunchKernelGGL((mp_spmm_kernel<T, TOut, VEC, POW2, BATCH, SLICED, HOT, MARKS, (HOT) ? kHotRoundsPerLoad : 1>), grid_, \
                            dim3(64 * (WPB)), LDS, st, row_ptr, col_idx, val, X, Y, cx, cy, wave_off, nnz, K, P,   \
                            sh.ls.lanes_log2, sh.tpw, WB, WE, sh.row_shift, ws_head_row, ws_head, ws_tail,         \
                            pl.hot_cols, pl.seg_part_off, pl.num_hot_segs, pl.hot_rows, pl.hot_block_wave,         \
-                           pl.hot_blocks, SHIFT);                                                                 \
+                           pl.hot_blocks, SHIFT, nullptr);                                                        \
     } while (0)
         if (pl.hot_waves > 0) {
             // hot launch: only built for power-of-two pitches and vector lanes (VEC > 1)
@@ -930,12 +990,12 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
             const int per_wave = 64 / (K / 4);  // records per wavefront
             const long long fix_waves = ((long long)W + per_wave - 1) / per_wave;
             hipLaunchKernelGGL((mp_fixup_wide_kernel<TOut>), dim3((unsigned)((fix_waves + 3) / 4)), dim3(256), 0, st,
-                               ws_head_row, ws_head, ws_tail, Y, W, K);
+                               ws_head_row, ws_head, ws_tail, Y, W, K, pl.row_scale);
         } else {
             long long threads = (long long)W * K;
             unsigned blocks = (unsigned)((threads + 255) / 256);
             hipLaunchKernelGGL((mp_fixup_kernel<TOut>), dim3(blocks), dim3(256), 0, st, ws_head_row, ws_head, ws_tail,
-                               Y, W, K);
+                               Y, W, K, pl.row_scale);
         }
         MPS_HIP_TRY(hipGetLastError());
     }
@@ -951,6 +1011,12 @@ int allow_hot_lds_for(size_t bytes)
         auto kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, 1, kHotRoundsPerLoad>;
         MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         (int)bytes));
+        if constexpr (sizeof(T) == 4) {
+            // hot columns come with tiled plans, whose partial rows are scaled when they are summed
+            auto pattern_kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, 1, kHotRoundsPerLoad, 1>;
+            MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(pattern_kern),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        }
         return MPS_OK;
     } else {
         return MPS_ERR_UNSUPPORTED;

@@ -54,6 +54,11 @@ struct mps_plan {
     int *hot_block_wave = nullptr;  // [hot_blocks + 1] first wave of every hot workgroup
     int hot_blocks = 0;
     bool keep_sources = true;       // slice_src is kept (mps_plan_set_values works)
+    // degree weights (weights != 0): no value arrays; X is scaled by col_scale into xs before the kernels,
+    // which add up rows of xs; finished rows are scaled by row_scale
+    int weights = 0;                // 0: values from val; else 1 + MPS_WEIGHT_*
+    float *col_scale = nullptr, *row_scale = nullptr;  // [n_rows] each
+    float *xs = nullptr;            // [n_rows * K]
     mps_rb::DevicePlan *rb = nullptr;  // row-block plan: everything above about slabs and slices is unused
 };
 
@@ -248,7 +253,8 @@ __global__ __launch_bounds__(256) void tile_scatter_kernel(const int *__restrict
 // Y[r] = sum over slabs, in slab order, of the partial rows part[s * n_rows + r].
 template <typename TOut, int VEC>
 __global__ __launch_bounds__(256) void tile_reduce_kernel(const float *__restrict__ part, TOut *__restrict__ Y,
-                                                           int n_rows, int K, int num_slabs)
+                                                           int n_rows, int K, int num_slabs,
+                                                           const float *__restrict__ row_scale)
 {
     const size_t per_slab = (size_t)n_rows * K;
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
@@ -265,9 +271,47 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const float *__restric
             acc[0] += p[0];
         }
     }
+    if (row_scale) {  // plans with degree weights: the row factor
+        const float f = row_scale[i / (size_t)K];
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) acc[u] *= f;
+    }
     store_acc<VEC>(Y + i, acc);
 }
 
+
+// Degree weights as two factors per node: the weight of nonzero (r, c) is row_scale[r] * col_scale[c].
+// Product mode: both the degree as a float (src/MergePathSpMM.cu:183-185, :450, :459 multiply them per
+// nonzero).  GCN mode: 1 / sqrt(degree), 0 for an empty row.
+__global__ __launch_bounds__(256) void degree_scales_kernel(const int *__restrict__ row_ptr, int n, int mode,
+                                                             float *__restrict__ row_scale,
+                                                             float *__restrict__ col_scale)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float d = (float)(row_ptr[i + 1] - row_ptr[i]);
+    const float f = mode == MPS_WEIGHT_GCN ? (d > 0.f ? 1.0f / sqrtf(d) : 0.f) : d;
+    row_scale[i] = f;
+    col_scale[i] = f;
+}
+
+// xs[c][:] = col_scale[c] * X[c][:], four columns per thread (K % 4 == 0) or one.
+template <int VEC>
+__global__ __launch_bounds__(256) void scale_rows_kernel(const float *__restrict__ X,
+                                                          const float *__restrict__ col_scale,
+                                                          float *__restrict__ xs, int n, int K)
+{
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (i >= (size_t)n * K) return;
+    const float f = col_scale[i / (size_t)K];
+    if constexpr (VEC == 4) {
+        float4 t = *reinterpret_cast<const float4 *>(X + i);
+        t.x *= f; t.y *= f; t.z *= f; t.w *= f;
+        *reinterpret_cast<float4 *>(xs + i) = t;
+    } else {
+        xs[i] = f * X[i];
+    }
+}
 
 // Rounds of wavefront w: the longest nonzero run among its partitions, in windows.
 __global__ __launch_bounds__(256) void slice_count_kernel(const int *__restrict__ coord_y, int P, int tpw,
@@ -540,6 +584,9 @@ void plan_free(mps_plan *pl)
     (void)hipFree(pl->hot_cols);
     (void)hipFree(pl->seg_table);
     (void)hipFree(pl->hot_block_wave);
+    (void)hipFree(pl->col_scale);
+    (void)hipFree(pl->row_scale);
+    (void)hipFree(pl->xs);
     delete pl;
 }
 
@@ -1021,7 +1068,24 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
     const size_t slots = (size_t)total_rounds * (size_t)(G * kWindow);
     MPS_BUILD_TRY(dev_alloc(pl, &pl->slice_cols, slots));
     MPS_BUILD_TRY(dev_alloc(pl, &pl->slice_src, slots));
-    {
+    if (pl->weights) {
+        // no value array: the kernels add up rows of xs = col_scale * X and scale finished rows
+        if (pl->mark_shift <= 0 || (hot_rows > 0 && pl->hot_mark_shift <= 0)) {
+            t.drop();
+            return MPS_ERR_UNSUPPORTED;
+        }
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->col_scale, (size_t)n));
+        // two spare entries: the merge path ends at row coordinate n + 1, and the kernel asks for the
+        // factor of the row that would start there
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->row_scale, (size_t)n + 2));
+        MPS_BUILD_HIP(hipMemsetAsync(pl->row_scale, 0, ((size_t)n + 2) * sizeof(float), st));
+        MPS_BUILD_TRY(dev_alloc(pl, &pl->xs, (size_t)n * K));
+        if (n > 0) {
+            hipLaunchKernelGGL(degree_scales_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, d_row_ptr, n,
+                               pl->weights - 1, pl->row_scale, pl->col_scale);
+            MPS_BUILD_HIP(hipGetLastError());
+        }
+    } else {
         unsigned char *sv = nullptr;
         MPS_BUILD_TRY(dev_alloc(pl, &sv, (slots ? slots : 1) * (size_t)eb));
         pl->slice_vals = sv;
@@ -1038,7 +1102,7 @@ int plan_build(mps_plan *pl, const int *d_row_ptr, const int *d_col_idx, const v
                            pl->mark_shift, pl->streamed_flag ? t.deg : nullptr, pl->slice_cols, pl->slice_src);
         MPS_BUILD_HIP(hipGetLastError());
     }
-    MPS_BUILD_TRY(plan_set_values(pl, d_val, st));
+    if (!pl->weights) MPS_BUILD_TRY(plan_set_values(pl, d_val, st));
     if (!pl->keep_sources) {
         // only mps_plan_set_values reads the source indices again
         MPS_BUILD_HIP(hipStreamSynchronize(st));
@@ -1088,6 +1152,25 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     how.mark_shift = pl->mark_shift;
     how.hot_mark_shift = pl->hot_mark_shift;
     how.streamed_flag = pl->streamed_flag;
+    if (pl->weights) {
+        if constexpr (sizeof(T) == 4) {
+            if (phases & MPS_PHASE_PREPARE) {
+                const size_t elems = (size_t)pl->n_rows * pl->K;
+                if (pl->K % 4 == 0)
+                    hipLaunchKernelGGL((scale_rows_kernel<4>), dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, st, X,
+                                       pl->col_scale, pl->xs, pl->n_rows, pl->K);
+                else
+                    hipLaunchKernelGGL((scale_rows_kernel<1>), dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st, X,
+                                       pl->col_scale, pl->xs, pl->n_rows, pl->K);
+                MPS_HIP_TRY(hipGetLastError());
+            }
+            X = pl->xs;
+            how.pattern = true;
+            how.row_scale = pl->num_segs == 1 ? pl->row_scale : nullptr;  // tiled plans: the reduce kernel scales
+        } else {
+            return MPS_ERR_UNSUPPORTED;
+        }
+    }
     if (pl->num_segs == 1)
         return launch_spmm_any<T, T>(pl->vrow_ptr, pl->slice_cols, vals, X, Y, pl->nnz, pl->K, pl->P, pl->coord_x,
                                      pl->coord_y, how, pl->shape, carry, phases, st);
@@ -1099,10 +1182,10 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
         const size_t per_slab = (size_t)pl->n_rows * pl->K;
         if (pl->K % 4 == 0)
             hipLaunchKernelGGL((tile_reduce_kernel<T, 4>), dim3((unsigned)((per_slab / 4 + 255) / 256)), dim3(256), 0, st,
-                               part, Y, pl->n_rows, pl->K, pl->num_segs);
+                               part, Y, pl->n_rows, pl->K, pl->num_segs, pl->row_scale);
         else
             hipLaunchKernelGGL((tile_reduce_kernel<T, 1>), dim3((unsigned)((per_slab + 255) / 256)), dim3(256), 0, st, part,
-                               Y, pl->n_rows, pl->K, pl->num_segs);
+                               Y, pl->n_rows, pl->K, pl->num_segs, pl->row_scale);
         MPS_HIP_TRY(hipGetLastError());
     }
     return MPS_OK;
@@ -1157,10 +1240,17 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     *plan_out = nullptr;
     if (!d_row_ptr || n_rows < 0 || nnz < 0 || K < 1 || cost <= 0 || tpw < 0) return MPS_ERR_INVALID_ARG;
     if (elem_bytes != 4 && elem_bytes != 2) return MPS_ERR_INVALID_ARG;
-    if (nnz > 0 && (!d_col_idx || !d_val)) return MPS_ERR_INVALID_ARG;
-    if ((long long)n_rows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
     mps_plan_options opt{};
     if (options) opt = *options;
+    if (opt.degree_weights < 0 || opt.degree_weights > 2) return MPS_ERR_INVALID_ARG;
+    if (nnz > 0 && (!d_col_idx || (!d_val && !opt.degree_weights))) return MPS_ERR_INVALID_ARG;
+    if ((long long)n_rows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
+    if (opt.degree_weights) {
+        // built for fp32 and the slab kernels; the source indices serve new values only
+        if (elem_bytes != 4 || (opt.flags & MPS_PLAN_FORCE_ROWBLOCK)) return MPS_ERR_UNSUPPORTED;
+        opt.flags |= MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_NO_SOURCES;
+        opt.flags &= ~MPS_PLAN_NO_ROW_MARKS;
+    }
     const unsigned flags = opt.flags;
     const size_t slab_bytes = opt.slab_bytes;
     if ((flags & MPS_PLAN_FORCE_ROWBLOCK) && (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING))) return MPS_ERR_INVALID_ARG;
@@ -1172,6 +1262,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     pl->elem_bytes = elem_bytes;
     pl->cost = cost;
     pl->keep_sources = !(flags & MPS_PLAN_NO_SOURCES);
+    pl->weights = opt.degree_weights;
     if (rowblock_wanted(n_rows, nnz, K, elem_bytes, flags)) {
         if (elem_bytes != 4 || K != 16 || n_rows < 1) {
             plan_free(pl);
@@ -1263,7 +1354,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
 int mps_plan_set_values(mps_plan *plan, const void *d_val, void *stream)
 {
     if (!plan || (plan->nnz > 0 && !d_val)) return MPS_ERR_INVALID_ARG;
-    if (!plan->keep_sources) return MPS_ERR_UNSUPPORTED;
+    if (!plan->keep_sources || plan->weights) return MPS_ERR_UNSUPPORTED;
     if (plan->rb) return mps_rb::set_values(plan->rb, static_cast<const float *>(d_val), static_cast<hipStream_t>(stream));
     return plan_set_values(plan, d_val, static_cast<hipStream_t>(stream));
 }
@@ -1281,7 +1372,7 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
     case MPS_PLAN_ARRAY_WAVE_OFF: src = plan->wave_off; have = ((size_t)plan->shape.num_waves + 1) * sizeof(int); break;
     case MPS_PLAN_ARRAY_SLICE_COLS: src = plan->slice_cols; have = slots * sizeof(int); break;
     case MPS_PLAN_ARRAY_SLICE_SRC: src = plan->slice_src; have = plan->slice_src ? slots * sizeof(int) : 0; break;
-    case MPS_PLAN_ARRAY_SLICE_VALS: src = plan->slice_vals; have = slots * (size_t)plan->elem_bytes; break;
+    case MPS_PLAN_ARRAY_SLICE_VALS: src = plan->slice_vals; have = plan->slice_vals ? slots * (size_t)plan->elem_bytes : 0; break;
     case MPS_PLAN_ARRAY_HOT_COLS:
         src = plan->hot_cols;
         have = (size_t)(plan->hot_rows > 0 ? plan->num_slabs : 0) * (size_t)plan->hot_rows * sizeof(int);

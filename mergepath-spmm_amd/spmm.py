@@ -177,7 +177,7 @@ class Plan:
 
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
-                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0):
+                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -193,8 +193,10 @@ class Plan:
         if resident == "off":
             flags |= _cabi.MPS_PLAN_NO_RESIDENT
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
-                                int(rowblock_block_rows), int(rowblock_blocks_per_round), int(resident_bytes))
-        check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), _ptr(csr.val), csr.n_rows, csr.nnz,
+                                int(rowblock_block_rows), int(rowblock_blocks_per_round),
+                                {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes))
+        check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), None if weights else _ptr(csr.val),
+                                             csr.n_rows, csr.nnz,
                                              int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
                                              int(threads_per_wave), ctypes.byref(opt), _stream(),
                                              ctypes.byref(self._h)), "mps_plan_create_ex")
@@ -320,7 +322,7 @@ class RowBlockLayout:
         ci = np.ascontiguousarray(col_idx, dtype=np.int32)
         v = np.ascontiguousarray(val, dtype=np.float32)
         opt = _cabi.PlanOptions(0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES, 0, int(steps), int(table_rows),
-                                int(block_rows), int(blocks_per_round))
+                                int(block_rows), int(blocks_per_round), 0, 0)
         check(_cabi.lib().mps_rowblock_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size,
                                                     int(K), ctypes.byref(opt), ctypes.byref(self._h)),
               "mps_rowblock_layout_build")

@@ -303,6 +303,56 @@ def test_resident_columns_are_chosen_for_large_skewed_inputs_only(pkg, dev):
     assert pkg.spmm.Plan(csr, 16, tiling="off", resident_bytes=64 * 10).info.resident_cols == 10
 
 
+@pytest.mark.parametrize("mode", ["degree", "gcn"])
+@pytest.mark.parametrize("K,tiling,slab_bytes,hot", [(16, "off", 0, "off"), (16, "force", 8192, "off"), (16, "force", 8192, "force"),
+                                                     (20, "off", 0, "off"), (4, "force", 2048, "off"), (1, "off", 0, "off"),
+                                                     (64, "off", 0, "off")])
+def test_degree_weight_plans(pkg, orc, dev, mode, K, tiling, slab_bytes, hot):
+    """Plans that form the reference's implicit edge weight deg(r) * deg(c) (src/MergePathSpMM.cu:450,459-460;
+    or the GCN norm) from one factor per node instead of a value array: against the fp64 row loop over the
+    oracle's weight array, for untiled, tiled and hot-column plans; with X = 1 (the reference's input,
+    src/MergePathSpMM.cu:180-182) the product mode is exact integer arithmetic."""
+    rng = np.random.default_rng(99 + K)
+    n = 800
+    rp, ci = random_csr(rng, n, 20, hub_rows=[(1, 700), (400, 300)])
+    w = orc.degree_values(rp, ci, mode="product" if mode == "degree" else "gcn")
+    X = (rng.random((n, K)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, np.zeros(ci.size, dtype=np.float32))  # values must not be read
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, K, cost=12, tiling=tiling, slab_bytes=slab_bytes, hot=hot, weights=mode)
+    assert (plan.info.num_slabs > 1) == (tiling == "force") and (plan.info.hot_rows > 0) == (hot == "force")
+    assert plan.info.rowblock_steps == 0
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, w, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    assert torch.equal(Y, plan.spmm(d_X))
+    if mode == "degree":
+        deg = np.diff(rp).astype(np.int64)
+        rows = np.repeat(np.arange(n), deg)
+        want = deg * np.bincount(rows, weights=deg[ci], minlength=n).astype(np.int64)
+        assert want.max() < 2 ** 24
+        Y1 = plan.spmm(torch.ones_like(d_X)).cpu().numpy()
+        assert np.array_equal(Y1, np.repeat(want[:, None], K, axis=1).astype(np.float32))
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        plan.set_values(csr.val)
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+    plan.close()
+
+
+def test_degree_weight_plans_are_fp32_slab_plans(pkg, dev):
+    rng = np.random.default_rng(8)
+    rp, ci = random_csr(rng, 300, 12)
+    half = make_csr(pkg, dev, rp, ci, np.zeros(ci.size, dtype=np.float16))
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        pkg.spmm.Plan(half, 16, weights="degree")
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+    full = make_csr(pkg, dev, rp, ci, np.zeros(ci.size, dtype=np.float32))
+    with pytest.raises(pkg._cabi.MpsError) as e:
+        pkg.spmm.Plan(full, 16, weights="degree", rowblock="force")
+    assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+
+
 def test_unsorted_rows(pkg, dev):
     n = 130  # two 64-column slabs
     rp = np.concatenate([[0, 3, 5], np.full(n - 2, 5)]).astype(np.int32)
