@@ -226,6 +226,9 @@ def main():
         custom = True
     name = "custom" if custom else args.workload
     w = Workload(pkg, name, spec, K, dt, args.seed, torch, dev, values=args.values)
+    if args.weights != "none":
+        # no value per nonzero is read; two factors per node are
+        w.b_alg = algorithmic_bytes(w.n, w.nnz, K, 0, w.eb) + 8 * w.n
 
     def make_plan(wl, **overrides):
         cost = args.cost if args.cost > 0 else sp.default_cost(wl.n, wl.nnz, wl.K, wl.eb)

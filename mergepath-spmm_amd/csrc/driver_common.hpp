@@ -8,12 +8,15 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <chrono>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <iostream>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "mpspmm.h"
@@ -54,6 +57,8 @@ struct Options {
     int hot = 0;                // --hot off|force (default: where it pays)
     int weights = -1;           // --weights explicit|degree|gcn: seeded values (default), or from degrees on the device
     bool ones = false;          // --features ones: all features 1.0, as the reference sets them (src/MergePathSpMM.cu:180-182)
+    bool cpu = false;           // --cpu: time the host row loop on the same inputs and compare the results
+    bool factors = false;       // --factors (with --weights degree|gcn, fp32): a plan with degree weights, no value array
 };
 
 // Strips the optional trailing flags; returns the positional arguments.
@@ -64,6 +69,8 @@ inline std::vector<std::string> split_args(int argc, char **argv, Options &opt)
         std::string a = argv[i];
         if (a == "--dump" && i + 1 < argc) opt.dump_path = argv[++i];
         else if (a == "--print") opt.print_matrix = true;
+        else if (a == "--cpu") opt.cpu = true;
+        else if (a == "--factors") opt.factors = true;
         else if (a == "--no-plan") opt.use_plan = false;
         else if (a == "--slab-bytes" && i + 1 < argc) opt.slab_bytes = std::strtoull(argv[++i], nullptr, 10);
         else if (a == "--tiling" && i + 1 < argc) {
@@ -219,6 +226,72 @@ double finish_output(const std::vector<T> &Y, int n_rows, int K, const Options &
         }
     }
     return sum;
+}
+
+// CPU baseline of the drivers (--cpu): the row loop the reference checks its kernels against
+// (test/compare.h:18-31), in fp32 like the device (fp32 accumulation for half inputs too), rows dealt
+// to the host threads in contiguous blocks of equal nonzero count.  Prints the time of one product,
+// the threads used and present, and how far the device result is from it; returns the JSON fields.
+template <typename T>
+std::string cpu_baseline(const int *rp, const int *ci, const std::vector<T> &val, const std::vector<T> &X,
+                         const std::vector<T> &Y_gpu, int n_rows, int nnz, int K, double gpu_us)
+{
+    const unsigned present = std::max(1u, std::thread::hardware_concurrency());
+    // the host share of a one-GPU box is 16 cores; more threads than that only queue
+    const unsigned threads = std::min(present, 16u);
+    std::vector<float> Y((size_t)n_rows * K);
+    std::vector<int> first(threads + 1, n_rows);
+    first[0] = 0;
+    for (unsigned t = 1; t < threads; ++t) {
+        const long long want = (long long)nnz * t / threads;
+        first[t] = (int)(std::lower_bound(rp, rp + n_rows + 1, (int)want) - rp);
+        if (first[t] > n_rows) first[t] = n_rows;
+    }
+    auto pass = [&]() {
+        std::vector<std::thread> pool;
+        for (unsigned t = 0; t < threads; ++t)
+            pool.emplace_back([&, t] {
+                std::vector<float> acc((size_t)K);
+                for (int r = first[t]; r < first[t + 1]; ++r) {
+                    std::fill(acc.begin(), acc.end(), 0.f);
+                    for (int e = rp[r]; e < rp[r + 1]; ++e) {
+                        const float a = (float)to_double(val[(size_t)e]);
+                        const T *x = X.data() + (size_t)ci[e] * K;
+                        for (int k = 0; k < K; ++k) acc[(size_t)k] += a * (float)to_double(x[k]);
+                    }
+                    std::copy(acc.begin(), acc.end(), Y.begin() + (size_t)r * K);
+                }
+            });
+        for (auto &th : pool) th.join();
+    };
+    pass();  // warm
+    int passes = 0;
+    double spent = 0;
+    while (passes < 20 && spent < 5.0) {
+        const auto t0 = std::chrono::steady_clock::now();
+        pass();
+        spent += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        ++passes;
+    }
+    const double cpu_us = spent / passes * 1e6;
+    double max_diff = 0, num = 0, den = 0;
+    for (size_t i = 0; i < Y.size(); ++i) {
+        const double d = to_double(Y_gpu[i]) - (double)Y[i];
+        max_diff = std::max(max_diff, std::fabs(d));
+        num += d * d;
+        den += (double)Y[i] * (double)Y[i];
+    }
+    const double rel = den > 0 ? std::sqrt(num / den) : std::sqrt(num);
+    const double gflops = 2.0 * nnz * K / (cpu_us * 1e3);
+    std::printf("cpu baseline: %.1f us per product (%.2f GFLOP/s) on %u of %u host threads, %d passes; device is %.1fx faster\n",
+                cpu_us, gflops, threads, present, passes, gpu_us > 0 ? cpu_us / gpu_us : 0.0);
+    std::printf("device against the cpu row loop: max |diff| %.3e, relative Frobenius %.3e\n", max_diff, rel);
+    char buf[256];
+    std::snprintf(buf, sizeof buf,
+                  ", \"cpu_us\": %.1f, \"cpu_gflops\": %.3f, \"cpu_threads\": %u, \"cpu_threads_present\": %u, "
+                  "\"max_abs_diff_vs_cpu\": %.3e, \"rel_fro_vs_cpu\": %.3e",
+                  cpu_us, gflops, threads, present, max_diff, rel);
+    return buf;
 }
 
 // <cost>: a number, or "default" / 0 for the library's choice (resolved once the graph is known)

@@ -80,7 +80,12 @@ int mergepath_main(int argc, char **argv)
     d_X.upload(h_X.data());
     mps_ok(mps_csr_validate(d_rp.p, d_ci.p, N, N, nnz, nullptr), "mps_csr_validate");
     // the reference's implicit weight deg(row) * deg(col) (:450,459), written out once
-    if (opt.weights >= 0) mps_ok(Elem<T>::degree_values(d_rp.p, d_ci.p, N, nnz, opt.weights, d_val.p), "mps_degree_values");
+    if (opt.weights >= 0) {
+        mps_ok(Elem<T>::degree_values(d_rp.p, d_ci.p, N, nnz, opt.weights, d_val.p), "mps_degree_values");
+        if (opt.cpu) d_val.download(h_val.data());
+    }
+    if (opt.factors && (opt.weights < 0 || sizeof(T) != 4 || !opt.use_plan || tune))
+        die("--factors needs --weights degree|gcn, fp32 and a plan");
 
     if (tune) {
         mps_tune_result best{}, tried[32];
@@ -112,9 +117,13 @@ int mergepath_main(int argc, char **argv)
     Timing t;
     if (opt.use_plan) {
         hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        mps_plan_options popt{};
+        popt.flags = (unsigned)(opt.tiling | opt.hot) | MPS_PLAN_NO_SOURCES;  // the values never change here
+        popt.slab_bytes = opt.slab_bytes;
+        popt.degree_weights = opt.factors ? opt.weights + 1 : 0;
         prep = time_launches(0, 1, [&] {
-            mps_ok(mps_plan_create(d_rp.p, d_ci.p, d_val.p, N, nnz, K, (int)sizeof(T), cost, threads_per_wave,
-                                   (unsigned)(opt.tiling | opt.hot), opt.slab_bytes, nullptr, &plan), "mps_plan_create");
+            mps_ok(mps_plan_create_ex(d_rp.p, d_ci.p, opt.factors ? nullptr : d_val.p, N, nnz, K, (int)sizeof(T), cost,
+                                      threads_per_wave, &popt, nullptr, &plan), "mps_plan_create_ex");
         });
         mps_ok(mps_plan_get_info(plan, &info), "mps_plan_get_info");
         P = info.num_partitions;
@@ -133,9 +142,17 @@ int mergepath_main(int argc, char **argv)
 
     std::printf("partitions: %d (cost %d), threads_per_wave %d, max row degree %d\n", P, cost, threads_per_wave,
                 gr.max_degree);
-    if (plan)
+    if (plan && info.rowblock_steps > 0)
+        std::printf("plan: %d row blocks, %d steps of %d table rows, %lld of %d nonzeros (%.1f %%) gathered from LDS, %.1f MB of device memory\n",
+                    info.rowblock_blocks, info.rowblock_steps, info.rowblock_table_rows, info.hot_nnz, nnz,
+                    nnz ? 100.0 * (double)info.hot_nnz / nnz : 0.0, info.device_bytes / 1e6);
+    else if (plan)
         std::printf("plan: %d column slab(s) of %d columns, %lld sliced rounds, %.1f MB of device memory\n", info.num_slabs,
                     info.slab_cols, info.total_rounds, info.device_bytes / 1e6);
+    if (plan && info.resident_cols > 0)
+        std::printf("resident columns: %d (%.1f %% of the nonzeros); gathers of the other columns carry the streaming hint\n",
+                    info.resident_cols, nnz ? 100.0 * (double)info.resident_nnz / nnz : 0.0);
+    if (opt.factors) std::printf("degree weights: one factor per node, no value array\n");
     if (plan && info.hot_rows > 0)
         std::printf("hot columns: %d rows of X per slab in LDS, %lld of %d nonzeros (%.1f %%), %d of %d wavefronts\n",
                     info.hot_rows, info.hot_nnz, nnz, nnz ? 100.0 * (double)info.hot_nnz / nnz : 0.0, info.hot_waves,
@@ -143,11 +160,15 @@ int mergepath_main(int argc, char **argv)
     std::printf("preprocessing: %.2f us, once per matrix (not in the launch time below)\n", prep.avg_us);
     char extra[256];
     std::snprintf(extra, sizeof extra,
-                  ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan\": %s, \"num_slabs\": %d, \"hot_rows\": %d, \"prep_us\": %.3f",
+                  ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan\": %s, \"num_slabs\": %d, \"hot_rows\": %d, "
+                  "\"rowblock_steps\": %d, \"resident_cols\": %d, \"prep_us\": %.3f",
                   P, cost, threads_per_wave, plan ? "true" : "false", plan ? info.num_slabs : 1, plan ? info.hot_rows : 0,
-                  prep.avg_us);
+                  plan ? info.rowblock_steps : 0, plan ? info.resident_cols : 0, prep.avg_us);
     mps_plan_destroy(plan);
-    report("merge_path", Elem<T>::name, N, nnz, K, (int)sizeof(T), (int)sizeof(T), repeats, t, checksum, extra);
+    std::string more = extra;
+    if (opt.cpu)
+        more += cpu_baseline<T>(mps_graph_row_ptr(gr.g), mps_graph_col_idx(gr.g), h_val, h_X, h_Y, N, nnz, K, t.avg_us);
+    report("merge_path", Elem<T>::name, N, nnz, K, opt.factors ? 0 : (int)sizeof(T), (int)sizeof(T), repeats, t, checksum, more);
     return 0;
 }
 

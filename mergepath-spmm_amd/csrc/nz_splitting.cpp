@@ -44,6 +44,8 @@ int main(int argc, char **argv)
     std::printf("neighbour groups: %d (part_size %d)\n", num_parts, part_size);
     char extra[128];
     std::snprintf(extra, sizeof extra, ", \"part_size\": %d, \"num_parts\": %d", part_size, num_parts);
-    report("nz_splitting", "fp32", N, nnz, K, 4, 4, repeats, t, checksum, extra);
+    std::string more = extra;
+    if (opt.cpu) more += cpu_baseline<float>(mps_graph_row_ptr(gr.g), mps_graph_col_idx(gr.g), h_val, h_X, h_Y, N, nnz, K, t.avg_us);
+    report("nz_splitting", "fp32", N, nnz, K, 4, 4, repeats, t, checksum, more);
     return 0;
 }

@@ -38,6 +38,8 @@ int main(int argc, char **argv)
     double checksum = finish_output(h_Y, N, K, opt);
     char extra[128];
     std::snprintf(extra, sizeof extra, ", \"num_warps\": %d", num_warps);
-    report("row_wise", "fp32", N, nnz, K, 4, 4, repeats, t, checksum, extra);
+    std::string more = extra;
+    if (opt.cpu) more += cpu_baseline<float>(mps_graph_row_ptr(gr.g), mps_graph_col_idx(gr.g), h_val, h_X, h_Y, N, nnz, K, t.avg_us);
+    report("row_wise", "fp32", N, nnz, K, 4, 4, repeats, t, checksum, more);
     return 0;
 }

@@ -95,6 +95,35 @@ def test_merge_path_driver_reference_setting(pkg, orc, graph_file, tmp_path):
     assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
 
 
+def test_drivers_time_the_cpu_row_loop_beside_the_device(pkg, graph_file):
+    """--cpu: the host row loop (test/compare.h:18-31 in fp32) timed on the same inputs, with the threads used
+    and present, and the distance of the device result from it."""
+    for prog, args in (("MergePathSpMM", (16, 32, 16, 2)), ("MergePathSpMM_fp16", (32, 64, 16, 2)),
+                       ("row_wise", (16, 512, 2)), ("nz_splitting", (16, 32, 2))):
+        out = run(prog, graph_file, *args, "--cpu")
+        j = last_json(out)
+        assert "cpu baseline: " in out and j["cpu_us"] > 0 and 1 <= j["cpu_threads"] <= j["cpu_threads_present"]
+        assert j["rel_fro_vs_cpu"] <= (2e-3 if prog.endswith("fp16") else 1e-5)
+
+
+def test_merge_path_driver_degree_weights_from_factors(pkg, orc, graph_file, tmp_path):
+    """--weights degree --factors: the plan forms the weights from one factor per node; same result, within
+    rounding, as with the value array of the same weights."""
+    K = 16
+    dumps = []
+    for extra in ((), ("--factors",)):
+        dump = tmp_path / ("y%d.bin" % len(extra))
+        out = run("MergePathSpMM", graph_file, K, 32, 16, 2, "--dump", dump, "--weights", "degree", "--cpu", *extra)
+        assert ("degree weights: one factor per node" in out) == bool(extra)
+        assert last_json(out)["rel_fro_vs_cpu"] <= 1e-5
+        dumps.append(np.fromfile(dump, dtype=np.float32).reshape(-1, K))
+    rp, ci, _, X = inputs(pkg, graph_file, K)
+    ref, scale = orc.spmm_f64(rp, ci, orc.degree_values(rp, ci), X, want_abs=True)
+    for Y in dumps:
+        assert (np.abs(Y - ref) <= 1e-5 * scale + 1e-6).all()
+    run("MergePathSpMM_fp16", graph_file, K, 32, 16, 1, "--weights", "degree", "--factors", expect=1)
+
+
 def test_merge_path_driver_auto_cost(pkg, orc, graph_file, tmp_path):
     K = 16
     rp, ci, val, X = inputs(pkg, graph_file, K)
