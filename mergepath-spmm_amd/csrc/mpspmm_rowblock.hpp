@@ -20,29 +20,31 @@
 //     nonzero counts per step), gathered through L2, so that the CUs of an
 //     XCD, which walk the steps at about the same pace, share a few hundred
 //     KiB of X at a time.
-//   * Within (block, step) the nonzeros in row order (a row's hot ones, then
-//     its cold ones) are cut into 15 equal runs, one per wavefront that walks
-//     nonzeros (the 16th wavefront of a workgroup only touches the streams
-//     ahead of the others, so that their loads find them in L2); a
-//     wavefront's hot nonzeros are then dealt evenly and in order to its 16
-//     lane-groups, and so are its cold ones.  Every lane-group therefore walks
-//     two short streams (hot: LDS gathers, cold: L2 gathers) of the same
-//     length as its neighbours': no divergence, no padding beyond whole
-//     4-entry windows.
+//   * Within (block, step) the nonzeros are grouped into windows of 4 entries
+//     of one row (a row's last hot window and last cold window of the step
+//     are padded: value 0, the last index repeated).  The windows in row order
+//     (a row's hot ones, then its cold ones) are cut into 16 equal runs, one
+//     per wavefront; a wavefront's hot windows are then dealt evenly and in
+//     order to its 16 lane-groups, and so are its cold ones.  Every lane-group
+//     therefore walks two short streams (hot: LDS gathers, cold: L2 gathers)
+//     of the same length as its neighbours': no divergence.  A round of a
+//     stream holds two windows per lane-group, side by side, so that a lane
+//     reads its entry of both with one 16-byte load.
 //   * An entry is 8 bytes: {index | rows_advanced << index_bits, value}.
 //     index is the LDS table slot (hot) or the column id (cold);
-//     rows_advanced is how many block-local rows lie between this nonzero and
-//     the previous one of the same lane-group stream (for the first one:
-//     between it and the first row of the wavefront's run).
+//     rows_advanced, in a window's first entry only, is how many block-local
+//     rows lie between this window and the previous one of the same
+//     lane-group stream (for the first one: between it and the first row of
+//     the wavefront's run).
 //   * When the row changes, a lane-group adds its partial sums to the row's
 //     LDS accumulator (plain read-add-write).  That is safe because a row is
-//     added to directly only by the lane-group in whose stream it begins: the
-//     partial sums of a lane-group's first row (which may have begun in the
-//     stream before) are held back and added after the walk, in lane-group
+//     added to directly only by the lane-group in whose stream it ends.  The
+//     sums a lane-group holds at the end of its run (its last row may go on
+//     in the next group's stream) are combined after the walk, in lane-group
 //     order, by the first lane-group of every stretch of equal rows.  Only
 //     the first row of a wavefront's run can be shared with another
-//     wavefront: what is held back for it goes to a per-wavefront slot, and
-//     the slots are added in wavefront order after the step's barrier.
+//     wavefront: its sums go to a per-wavefront slot, and the slots are added
+//     by one wavefront, in wavefront order, after the step's barrier.
 //     Results do not depend on timing.
 #ifndef MPSPMM_ROWBLOCK_HPP
 #define MPSPMM_ROWBLOCK_HPP

@@ -76,7 +76,7 @@ struct StepSplit {
 };
 
 // cnt_t: [lr * 2 + kind] nonzeros of local row lr in this step (kind 0 hot, 1 cold).  The step's
-// windows in row order (a row's hot windows, then its cold ones) are cut into 15 equal runs.
+// windows in row order (a row's hot windows, then its cold ones) are cut into 16 equal runs.
 void split_step(const int *cnt_t, int nr, StepSplit &sp)
 {
     long long E = 0;
