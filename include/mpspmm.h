@@ -482,11 +482,12 @@ void mps_rowblock_layout_free(mps_rowblock_layout *layout);
 /* Parameter sweep for one matrix and K — what the reference leaves to the
  * user's hand (cost and partitions per warp are command-line arguments,
  * src/MergePathSpMM.cu:121-122, and its README reports the best of a sweep).
- * Builds a plan for each candidate (costs 16 .. 256 with a full wavefront, the
- * default cost with half the partitions per wavefront, without hot columns,
- * without tiling, with slabs of 3, 6, 12 and 24 MiB where X holds more than
- * two of them and the library's cost model does not put them 50 % behind the
- * untiled plan), runs `repeats` timed products Y = A * X after two warm-ups
+ * Builds a plan for each candidate (slab plans: costs 16 .. 256 with a full
+ * wavefront, the default cost with half the partitions per wavefront, without
+ * hot columns, without tiling, with slabs of 3, 6, 12 and 24 MiB where X holds
+ * more than two of them and the library's cost model does not put them 50 %
+ * behind the untiled plan; one row-block plan for fp32, K = 16 and rows of 32
+ * nonzeros and more on average), runs `repeats` timed products Y = A * X after two warm-ups
  * (HIP events on the stream) and reports the fastest.  d_Y is overwritten.
  * tried_out (optional) receives every candidate with its time;
  * *n_tried_io is its capacity on entry and the number of candidates on

@@ -97,7 +97,7 @@ int mergepath_main(int argc, char **argv)
                         tried[i].threads_per_wave, tried[i].flags, tried[i].slab_bytes, tried[i].ms * 1e3);
         cost = best.cost;
         threads_per_wave = best.threads_per_wave;
-        opt.tiling = (int)(best.flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING));
+        opt.tiling = (int)(best.flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_ROWBLOCK));
         opt.hot = (int)(best.flags & (MPS_PLAN_NO_HOT | MPS_PLAN_FORCE_HOT));
         opt.slab_bytes = (size_t)best.slab_bytes;
         opt.use_plan = true;

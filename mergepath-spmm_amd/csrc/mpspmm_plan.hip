@@ -1427,13 +1427,17 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     if ((rc = mps_default_cost(n_rows, nnz, K, elem_bytes, &dflt)) != MPS_OK) return rc;
     // what the reference's authors swept by hand: cost and partitions per wave
     // (src/MergePathSpMM.cu:121-122), plus this library's own switch
-    mps_tune_result cand[16];
+    // (slab plans: a row-block plan has neither a cost nor partitions per wavefront, it is one candidate of its own)
+    mps_tune_result cand[20];
     int n_cand = 0;
+    const unsigned slab = MPS_PLAN_NO_ROWBLOCK;
     const int costs[] = {16, 24, 32, 48, 64, 96, 128, 256};
-    for (int c : costs) cand[n_cand++] = {c, max_tpw, 0u, 0.f, 0};
-    if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, 0u, 0.f, 0};
-    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_HOT, 0.f, 0};
-    cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_NO_TILING, 0.f, 0};
+    for (int c : costs) cand[n_cand++] = {c, max_tpw, slab, 0.f, 0};
+    if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, slab, 0.f, 0};
+    cand[n_cand++] = {dflt, max_tpw, slab | MPS_PLAN_NO_HOT, 0.f, 0};
+    cand[n_cand++] = {dflt, max_tpw, slab | MPS_PLAN_NO_TILING, 0.f, 0};
+    if (elem_bytes == 4 && K == 16 && n_rows >= 1 && (long long)nnz >= 32LL * n_rows)
+        cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_ROWBLOCK, 0.f, 0};
     // slab sizes the model does not pick on its own: larger slabs pay on skewed graphs
     // (not those the model puts 50 % behind the untiled plan: thousands of slabs for a matrix with short rows)
     const double untiled_ps = modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows, -1.0);
@@ -1444,7 +1448,7 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
         if (cols < 64) cols = 64;
         const unsigned long long slabs = ((unsigned long long)n_rows + cols - 1) / cols;
         if (modelled_ps(n_rows, nnz, K, elem_bytes, (int)slabs, (int)cols, -1.0) > 1.5 * untiled_ps) continue;
-        cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_HOT, 0.f, mib << 20};
+        cand[n_cand++] = {dflt, max_tpw, slab | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_HOT, 0.f, mib << 20};
     }
     hipEvent_t e0 = nullptr, e1 = nullptr;
     MPS_HIP_TRY(hipEventCreate(&e0));
@@ -1462,8 +1466,8 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
         mps_plan *pl = nullptr;
         rc = mps_plan_create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, c.cost, c.threads_per_wave, c.flags,
                              (size_t)c.slab_bytes, stream, &pl);
-        if ((c.flags & MPS_PLAN_FORCE_TILING) && (rc == MPS_ERR_UNSORTED || rc == MPS_ERR_UNSUPPORTED)) {
-            rc = MPS_OK;  // this matrix cannot be tiled that way: not a candidate
+        if ((c.flags & (MPS_PLAN_FORCE_TILING | MPS_PLAN_FORCE_ROWBLOCK)) && (rc == MPS_ERR_UNSORTED || rc == MPS_ERR_UNSUPPORTED)) {
+            rc = MPS_OK;  // this matrix cannot be tiled or blocked that way: not a candidate
             continue;
         }
         if (rc != MPS_OK) break;
