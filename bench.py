@@ -59,8 +59,8 @@ def plan_signature(workload, info):
     if info.rowblock_steps > 0:
         return "%s|rowblock|steps=%d|table_rows=%d|blocks=%d" % (workload, info.rowblock_steps, info.rowblock_table_rows,
                                                                   info.rowblock_blocks)
-    return "%s|slabs=%d|cost=%d|hot_rows=%d|resident_cols=%d" % (workload, info.num_slabs, info.cost, info.hot_rows,
-                                                                 info.resident_cols)
+    return "%s|slabs=%d|cost=%d|tpw=%d|hot_rows=%d|resident_cols=%d" % (workload, info.num_slabs, info.cost,
+                                                                        info.threads_per_wave, info.hot_rows, info.resident_cols)
 
 
 def measured_traffic(signature):
@@ -181,6 +181,9 @@ def main():
     ap.add_argument("--rb-table-rows", type=int, default=0, help="rows per LDS table of a row-block plan (0 = what fits)")
     ap.add_argument("--resident", default="auto", choices=["auto", "off"],
                     help="untiled plans: streaming hint on the gathers of unpopular columns where the library picks it / never")
+    ap.add_argument("--column-tiles", default="auto", choices=["auto", "off"],
+                    help="untiled plans with rows of X of 512 bytes and more: passes over 128-byte column tiles where the "
+                         "library picks them / never")
     ap.add_argument("--resident-bytes", type=int, default=0, help="rows of X gathered without the hint (0 = library default)")
     ap.add_argument("--values", default="uniform", choices=["uniform", "degree", "gcn"],
                     help="edge values: U[0,1), or the reference's deg(r) * deg(c), or 1 / sqrt(deg(r) * deg(c)), as a value array")
@@ -235,7 +238,8 @@ def main():
         kw = dict(cost=cost, threads_per_wave=args.tpw, tiling={"auto": "auto", "untiled": "off", "tiled": "force", "plain": "auto"}[args.mode],
                   slab_bytes=args.slab_bytes, hot=args.hot, rowblock=args.rowblock, rowblock_steps=args.rb_steps,
                   rowblock_table_rows=args.rb_table_rows, keep_sources=False, resident=args.resident,
-                  resident_bytes=args.resident_bytes, weights=None if args.weights == "none" else args.weights)
+                  resident_bytes=args.resident_bytes, weights=None if args.weights == "none" else args.weights,
+                  column_tiles=args.column_tiles == "auto")
         kw.update(overrides)
         return sp.Plan(wl.csr, wl.K, **kw), cost
 

@@ -383,6 +383,7 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
 #define MPS_PLAN_NO_ROWBLOCK 16u    /* never build a row-block plan (see below)  */
 #define MPS_PLAN_FORCE_ROWBLOCK 32u /* row-block plan whatever the matrix looks like (fp32, K = 16 only) */
+#define MPS_PLAN_NO_COLUMN_TILES 512u /* untiled plans with rows of X of 512 bytes and more: no passes over 128-byte column tiles */
 #define MPS_PLAN_NO_RESIDENT 256u    /* untiled plans: no streaming hint on the gathers of unpopular columns (see below) */
 #define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
                                        CSR arrays (what a matrix gets anyway whose column ids and row-end counts do not

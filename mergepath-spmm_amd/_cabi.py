@@ -36,6 +36,7 @@ MPS_PLAN_FORCE_ROWBLOCK = 32
 MPS_PLAN_NO_SOURCES = 64
 MPS_PLAN_NO_ROW_MARKS = 128
 MPS_PLAN_NO_RESIDENT = 256
+MPS_PLAN_NO_COLUMN_TILES = 512
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,

@@ -177,7 +177,7 @@ class Plan:
 
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
-                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None):
+                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None, column_tiles=True):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -192,6 +192,8 @@ class Plan:
             flags |= _cabi.MPS_PLAN_NO_ROW_MARKS
         if resident == "off":
             flags |= _cabi.MPS_PLAN_NO_RESIDENT
+        if not column_tiles:
+            flags |= _cabi.MPS_PLAN_NO_COLUMN_TILES
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
                                 int(rowblock_block_rows), int(rowblock_blocks_per_round),
                                 {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes))

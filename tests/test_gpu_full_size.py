@@ -141,10 +141,11 @@ def test_rmat_config_full_size(pkg, orc, dev, K):
     (d_X,) = to_dev(dev, X)
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     plan = pkg.spmm.Plan(csr, K)
-    # X of 256 MiB and more (beyond the last-level cache): the 10 MiB of busiest columns stay plain gathers,
-    # the rest is gathered with the streaming hint
-    assert plan.info.num_slabs == 1 and (plan.info.resident_cols > 0) == (K >= 64)
+    # K = 64, X of 256 MiB (beyond the last-level cache): the 10 MiB of busiest columns stay plain gathers, the rest
+    # is gathered with the streaming hint.  K = 128 and 256: 8-lane groups and one pass per 128 bytes of row pitch.
+    assert plan.info.num_slabs == 1 and (plan.info.resident_cols > 0) == (K == 64)
     assert plan.info.resident_cols == 0 or plan.info.resident_nnz > 0.4 * ci.size
+    assert plan.info.threads_per_wave == (8 if K >= 128 else 64 // (K // 4)) and (K < 128 or plan.info.cost == 64)
     Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     torch.cuda.synchronize()
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)

@@ -290,6 +290,45 @@ def test_resident_columns_layout_and_result(pkg, orc, dev, K, dtype):
     plain.close()
 
 
+@pytest.mark.parametrize("K,dtype,tiles", [(128, np.float32, True), (256, np.float32, True), (256, np.float16, True),
+                                           (64, np.float32, False), (160, np.float32, True), (136, np.float32, False)])
+def test_column_tiles_for_wide_rows(pkg, orc, dev, K, dtype, tiles):
+    """Untiled plans for short matrix rows and rows of X of 512 bytes or more (a multiple of 128): lane-groups of 8
+    lanes, one pass per 128 bytes of row pitch, the caller's merge items per wavefront kept (cost scaled by the
+    groups per wavefront).  Same product as with full rows (other partition: equal within rounding) and as the
+    oracle; explicit partitions per wavefront or MPS_PLAN_NO_COLUMN_TILES keep full rows."""
+    rng = np.random.default_rng(4321 + K)
+    n = 1200
+    rp, ci = random_csr(rng, n, 28, hub_rows=[(7, 900)])
+    half = dtype == np.float16
+    val = rng.random(ci.size).astype(dtype)
+    X = (rng.random((n, K)) * 2 - 1).astype(dtype)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    eb = 2 if half else 4
+    full = pkg.spmm.Plan(csr, K, cost=96, column_tiles=False)
+    plan = pkg.spmm.Plan(csr, K, cost=96)
+    assert full.info.threads_per_wave == pkg.graphs.max_threads_per_wave(K, eb) and full.info.cost == 96
+    if tiles:
+        assert plan.info.threads_per_wave == 8 and plan.info.cost == max(16, 96 * full.info.threads_per_wave // 8)
+    else:
+        assert plan.info.threads_per_wave == full.info.threads_per_wave and plan.info.cost == 96
+    assert pkg.spmm.Plan(csr, K, cost=96, threads_per_wave=1).info.threads_per_wave == 1
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    Y0 = full.spmm(d_X)
+    torch.cuda.synchronize()
+    if half:
+        ref, scale = orc.spmm_f64_f16in(rp, ci, val, X, want_abs=True)
+        check_fp16(Y.cpu().numpy(), ref, scale)
+        check_fp16(Y0.cpu().numpy(), ref, scale)
+    else:
+        ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+        check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+        check_fp32(Y0.cpu().numpy(), ref, scale, rel_elem=False)
+    assert torch.equal(Y, plan.spmm(d_X))
+    check_plan_layout(pkg, orc, plan, rp, ci, val)
+
+
 def test_resident_columns_are_chosen_for_large_skewed_inputs_only(pkg, dev):
     """Without resident_bytes the library flags streamed gathers only where they were measured to pay: X of
     192 MiB or more and at least 40 % of the nonzeros in the 10 MiB of busiest columns; a pitch that is not a
