@@ -445,10 +445,13 @@ enum {
     MPS_PLAN_ARRAY_RB_HOT_COLS = 9,   /* int[steps * table_rows]: column of each table slot, -1 = unused */
     MPS_PLAN_ARRAY_RB_META = 10,      /* int[blocks * steps * 16 * 4]: {hot entries, cold entries, first local row, 0} per wavefront */
     MPS_PLAN_ARRAY_RB_WAVE_BASE = 11, /* long long[blocks * 16 * 2]: first round of each wavefront's hot / cold stream */
-    MPS_PLAN_ARRAY_RB_HOT = 12,       /* 8 bytes x hot slots: {index | rows_advanced << bits, value} */
+    MPS_PLAN_ARRAY_RB_HOT = 12,       /* 8 bytes x hot slots: {index | rows_advanced << bits, value}; host layouts only (a device plan holds RB_HOT_PACKED) */
     MPS_PLAN_ARRAY_RB_COLD = 13,      /* 8 bytes x cold slots                       */
     MPS_PLAN_ARRAY_RB_HOT_SRC = 14,   /* int[hot slots]: original nonzero index, -1 = padding */
-    MPS_PLAN_ARRAY_RB_COLD_SRC = 15   /* int[cold slots]                            */
+    MPS_PLAN_ARRAY_RB_COLD_SRC = 15,  /* int[cold slots]                            */
+    MPS_PLAN_ARRAY_RB_HOT_PACKED = 16 /* 12 bytes x (hot slots / 2), what the device reads: per round and lane {value A, value B,
+                                         half A | half B << 16}, half = table slot | piece << 11; the 5-bit pieces of a window's
+                                         entries 0 and 1 are the low and the high half of its rows_advanced */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,

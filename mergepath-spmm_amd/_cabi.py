@@ -40,7 +40,8 @@ MPS_PLAN_NO_COLUMN_TILES = 512
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
- MPS_PLAN_ARRAY_RB_HOT, MPS_PLAN_ARRAY_RB_COLD, MPS_PLAN_ARRAY_RB_HOT_SRC, MPS_PLAN_ARRAY_RB_COLD_SRC) = range(16)
+ MPS_PLAN_ARRAY_RB_HOT, MPS_PLAN_ARRAY_RB_COLD, MPS_PLAN_ARRAY_RB_HOT_SRC, MPS_PLAN_ARRAY_RB_COLD_SRC,
+ MPS_PLAN_ARRAY_RB_HOT_PACKED) = range(17)
 
 
 class PlanInfo(ctypes.Structure):

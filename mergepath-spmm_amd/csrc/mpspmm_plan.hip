@@ -1403,7 +1403,7 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
     default:
         if (!plan->rb) return MPS_ERR_INVALID_ARG;
         src = mps_rb::device_array(plan->rb, which, &have);
-        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_COLD_SRC)) return MPS_ERR_INVALID_ARG;
+        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_HOT_PACKED)) return MPS_ERR_INVALID_ARG;
         break;
     }
     if (plan->rb && which < MPS_PLAN_ARRAY_RB_BLOCK_ROW) return MPS_ERR_INVALID_ARG;

@@ -10,13 +10,16 @@
 #include "mpspmm_device.hpp"
 #include "mpspmm_rowblock.hpp"
 
+#include <type_traits>
+
 #include <new>
 
 namespace mps_rb {
 
 struct DevicePlan {
     Layout host;  // the small tables stay filled; the streams are released after the upload
-    Entry *hot = nullptr, *cold = nullptr;
+    uint32_t *hot = nullptr;  // the hot stream in packed form (12 bytes per lane and round)
+    Entry *cold = nullptr;
     int *hot_src = nullptr, *cold_src = nullptr;
     long long *wave_base = nullptr;
     int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr;
@@ -46,7 +49,7 @@ constexpr int kPrefetch = (kMaxTableRows * 4 + kThreads - 1) / kThreads;  // flo
 
 // The entry streams are read through buffer descriptors: the base of a wavefront's run of rounds in scalar
 // registers, a 32-bit offset per lane, and the cache policy as an operand of the load.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const Entry *base)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_rsrc(const void *base)
 {
     const unsigned long long a = (unsigned long long)base;  // the same in all lanes
     const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
@@ -62,6 +65,15 @@ __device__ __forceinline__ uint4 load_round(__amdgpu_buffer_rsrc_t r, unsigned o
     const u4_t t = keep ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0)
                         : __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 2);
     return make_uint4(t[0], t[1], t[2], t[3]);
+}
+
+// The same from the packed hot stream: 12 bytes {value A, value B, half A | half B << 16}.
+__device__ __forceinline__ uint4 load_round_packed(__amdgpu_buffer_rsrc_t r, unsigned off, bool keep)
+{
+    typedef unsigned u3_t __attribute__((ext_vector_type(3)));
+    const u3_t t = keep ? __builtin_amdgcn_raw_buffer_load_b96(r, (int)off, 0, 0)
+                        : __builtin_amdgcn_raw_buffer_load_b96(r, (int)off, 0, 2);
+    return make_uint4(t[2] & 0xffffu, t[0], t[2] >> 16, t[1]);
 }
 
 __device__ __forceinline__ void add4(float4 &a, const float4 &b)
@@ -114,7 +126,7 @@ __device__ __forceinline__ void fma_from_lane(float (&a)[4], float val, const fl
 __device__ __forceinline__ int rounds_of(int n) { return ((n >> 4) + ((n & 15) != 0) + 1) >> 1; }
 
 template <typename TOut>
-__global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restrict__ hot, const Entry *__restrict__ cold,
+__global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__restrict__ hot, const Entry *__restrict__ cold,
                                                             const long long *__restrict__ wave_base,
                                                             const int4 *__restrict__ meta,
                                                             const int *__restrict__ block_row,
@@ -157,6 +169,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restri
         int *my_crows = crows + wave * 16;
         // the masks live in vector registers (the DPP form of v_and takes no scalar operand); the
         // empty asm keeps the compiler from re-creating them from scalars at every use
+        hot_bits = kPackedSlotBits;  // the halves of the packed hot stream: table slot below, a piece of rows_advanced above
         unsigned hmask = (1u << hot_bits) - 1u, cmask = (1u << cold_bits) - 1u, hot_hi = ~hmask, cold_hi = ~cmask;
         asm volatile("" : "+v"(hmask), "+v"(cmask), "+v"(hot_hi), "+v"(cold_hi));
         int4 m = meta_b[wave];
@@ -210,9 +223,16 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restri
                 x[2] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<2>(word, cmask) << 6) | (unsigned)(s << 4)));
                 x[3] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<3>(word, cmask) << 6) | (unsigned)(s << 4)));
             };
-            auto window = [&](Walk &w, unsigned word, unsigned valbits, const float4 (&x)[kWin], unsigned himask, int bits) {
-                const unsigned hi = and_from_lane<0>(word, himask);
-                if (hi != 0) row_end(w, hi >> bits);
+            // is_hot: a hot window, whose rows_advanced lies in two pieces above the slots of its entries 0 and 1
+            auto window = [&](auto is_hot, Walk &w, unsigned word, unsigned valbits, const float4 (&x)[kWin], unsigned himask,
+                              int bits) {
+                if constexpr (decltype(is_hot)::value) {
+                    const unsigned lo = and_from_lane<0>(word, himask), hi = and_from_lane<1>(word, himask);
+                    if ((lo | hi) != 0) row_end(w, (lo >> kPackedSlotBits) | (hi >> (kPackedSlotBits - kPackedPieceBits)));
+                } else {
+                    const unsigned hi = and_from_lane<0>(word, himask);
+                    if (hi != 0) row_end(w, hi >> bits);
+                }
                 const float v = __uint_as_float(valbits);
                 fma_from_lane<0>(w.a, v, x[0]);
                 fma_from_lane<1>(w.a, v, x[1]);
@@ -221,20 +241,36 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restri
             };
             // The two windows (A, B) of a round.  have_a / have_b: the lane-group holds them (always, except in
             // the last round of a run).
-            auto pair = [&](Walk &w, const uint4 &cu, const float4 (&xa)[kWin], const float4 (&xb)[kWin], unsigned himask,
-                            int bits, bool have_a, bool have_b) {
-                if (have_a) window(w, cu.x, cu.y, xa, himask, bits);
-                if (have_b) window(w, cu.z, cu.w, xb, himask, bits);
+            auto pair = [&](auto is_hot, Walk &w, const uint4 &cu, const float4 (&xa)[kWin], const float4 (&xb)[kWin],
+                            unsigned himask, int bits, bool have_a, bool have_b) {
+                if (have_a) window(is_hot, w, cu.x, cu.y, xa, himask, bits);
+                if (have_b) window(is_hot, w, cu.z, cu.w, xb, himask, bits);
             };
+            constexpr std::true_type kHot{};
+            constexpr std::false_type kCold{};
 
-            const __amdgpu_buffer_rsrc_t hp = stream_rsrc(hot + (size_t)cur_h * kRoundEntries);
-            const __amdgpu_buffer_rsrc_t cp = stream_rsrc(cold + (size_t)cur_c * kRoundEntries);
             const bool keep = t >= keep_from;
+            // a round of the hot stream: 768 bytes (packed), of the cold stream: 1 KiB
+            constexpr unsigned kHotRoundBytes = kPackedRoundWords * 4u;
+            const __amdgpu_buffer_rsrc_t hp = stream_rsrc(hot + (size_t)cur_h * kPackedRoundWords);
+            const unsigned hoff = (unsigned)lane * 12u;
+            auto load_hot = [&](int r) { return load_round_packed(hp, hoff + (unsigned)r * kHotRoundBytes, keep); };
+            const __amdgpu_buffer_rsrc_t cp = stream_rsrc(cold + (size_t)cur_c * kRoundEntries);
             const unsigned loff = (unsigned)lane * 16u;
             uint4 nx_h = make_uint4(0u, 0u, 0u, 0u), nx_c = nx_h;
-            if (rounds_h > 0) nx_h = load_round(hp, loff, keep);
+            if (rounds_h > 0) nx_h = load_hot(0);
             if (rounds_c > 0) nx_c = load_round(cp, loff, keep);
             int rh = 0, rc = 0;  // rounds done
+            // Round rh / rc has been taken: the next one is requested.  (Two rounds ahead instead of one: 1.5 %
+            // slower on the 232,965-row power-law matrix; a round's load is not what the walk waits for.)
+            auto advance_h = [&]() {
+                ++rh;
+                if (rh < rounds_h) nx_h = load_hot(rh);
+            };
+            auto advance_c = [&]() {
+                ++rc;
+                if (rc < rounds_c) nx_c = load_round(cp, loff + (unsigned)rc * 1024u, keep);
+            };
             // The rounds in which every lane-group holds two windows: the hot and the cold ones are
             // spread evenly over max(full_h, full_c) passes (a cold round in every pass whose
             // share of the cold rounds crosses a whole number, likewise for hot), so that the
@@ -253,50 +289,48 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const Entry *__restri
                     cold_gather(cu_c.x, xca);
                     cold_gather(cu_c.z, xcb);
                     // after the gathers: what waits for them does not wait for this
-                    ++rc;
-                    if (rc < rounds_c) nx_c = load_round(cp, loff + (unsigned)rc * 1024u, keep);
+                    advance_c();
                 }
                 if (do_h) {
                     due_h -= passes;
                     const uint4 cu_h = nx_h;
                     float4 xha[kWin], xhb[kWin];
-                    ++rh;
-                    if (rh < rounds_h) nx_h = load_round(hp, loff + (unsigned)rh * 1024u, keep);
+                    advance_h();
                     hot_gather(cu_h.x, xha);
                     hot_gather(cu_h.z, xhb);
-                    pair(wh, cu_h, xha, xhb, hot_hi, hot_bits, true, true);
+                    pair(kHot, wh, cu_h, xha, xhb, hot_hi, 0, true, true);
                 }
-                if (do_c) pair(wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
+                if (do_c) pair(kCold, wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
             }
             // what the rounding of the shares left over
-            for (; rh < full_h; ++rh) {
+            while (rh < full_h) {
                 const uint4 cu_h = nx_h;
                 float4 xha[kWin], xhb[kWin];
-                if (rh + 1 < rounds_h) nx_h = load_round(hp, loff + (unsigned)(rh + 1) * 1024u, keep);
+                advance_h();
                 hot_gather(cu_h.x, xha);
                 hot_gather(cu_h.z, xhb);
-                pair(wh, cu_h, xha, xhb, hot_hi, hot_bits, true, true);
+                pair(kHot, wh, cu_h, xha, xhb, hot_hi, 0, true, true);
             }
-            for (; rc < full_c; ++rc) {
+            while (rc < full_c) {
                 const uint4 cu_c = nx_c;
                 float4 xca[kWin], xcb[kWin];
                 cold_gather(cu_c.x, xca);
                 cold_gather(cu_c.z, xcb);
-                if (rc + 1 < rounds_c) nx_c = load_round(cp, loff + (unsigned)(rc + 1) * 1024u, keep);
-                pair(wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
+                advance_c();
+                pair(kCold, wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
             }
             // the last round of a run: lane-groups hold two, one or none of its windows (the rest is padding)
             if (rc < rounds_c) {
                 float4 xca[kWin], xcb[kWin];
                 cold_gather(nx_c.x, xca);
                 cold_gather(nx_c.z, xcb);
-                pair(wc, nx_c, xca, xcb, cold_hi, cold_bits, 2 * rc < len_c, 2 * rc + 1 < len_c);
+                pair(kCold, wc, nx_c, xca, xcb, cold_hi, cold_bits, 2 * rc < len_c, 2 * rc + 1 < len_c);
             }
             if (rh < rounds_h) {
                 float4 xha[kWin], xhb[kWin];
                 hot_gather(nx_h.x, xha);
                 hot_gather(nx_h.z, xhb);
-                pair(wh, nx_h, xha, xhb, hot_hi, hot_bits, 2 * rh < len_h, 2 * rh + 1 < len_h);
+                pair(kHot, wh, nx_h, xha, xhb, hot_hi, 0, 2 * rh < len_h, 2 * rh + 1 < len_h);
             }
             cur_h += rounds_h;
             cur_c += rounds_c;
@@ -454,11 +488,12 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         // previous pass and lose it again before the next pass gets there.  Measured on MI355X, 232,965-row
         // power-law matrix, 1.07 GB of streams in 16 steps of 67 MB: 0, 2, 3, 4, 5, 16 steps kept: 0.500, 0.482,
         // 0.484, 0.493, 0.503, 0.516 ms per product.
-        const size_t per_step = (dp->hot_slots + dp->cold_slots) * sizeof(Entry) / (size_t)(L.steps > 0 ? L.steps : 1);
+        const size_t hot_bytes = L.hot_packed.size() * sizeof(uint32_t);
+        const size_t per_step = (hot_bytes + dp->cold_slots * sizeof(Entry)) / (size_t)(L.steps > 0 ? L.steps : 1);
         const size_t keep = per_step > 0 ? kStreamKeepBytes / per_step : (size_t)L.steps;
         dp->keep_from = keep >= (size_t)L.steps ? 0 : L.steps - (int)keep;
     }
-    if ((rc = upload(dp, &dp->hot, L.hot, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->hot, L.hot_packed, st)) != MPS_OK) return fail(rc);
     if ((rc = upload(dp, &dp->cold, L.cold, st)) != MPS_OK) return fail(rc);
     if (bp_in.keep_src) {
         if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
@@ -482,6 +517,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
     release(L.hot);
+    release(L.hot_packed);
     release(L.cold);
     release(L.hot_src);
     release(L.cold_src);
@@ -498,9 +534,9 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
                            reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
     if (phases & MPS_PHASE_MAIN)
         hipLaunchKernelGGL((rb_spmm_kernel<float>), dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot,
-                       dp->cold, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta), dp->block_row,
-                       reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X), Y, L.steps,
-                       L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from);
+                           dp->cold, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta), dp->block_row,
+                           reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X), Y, L.steps,
+                           L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from);
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
 }
@@ -514,13 +550,26 @@ __global__ __launch_bounds__(256) void rb_set_values_kernel(const float *__restr
     const int e = src[i];
     if (e >= 0) entries[i].val = val[e];
 }
+
+// The same for the packed hot stream: entry slot i is value (i % 2) of lane (i % 128) / 2 of round i / 128.
+__global__ __launch_bounds__(256) void rb_set_values_packed_kernel(const float *__restrict__ val,
+                                                                    const int *__restrict__ src, size_t slots,
+                                                                    uint32_t *__restrict__ packed)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= slots) return;
+    const int e = src[i];
+    if (e < 0) return;
+    const size_t round = i / kRoundEntries, within = i % kRoundEntries;
+    packed[(round * 64 + within / kPair) * 3 + within % kPair] = __float_as_uint(val[e]);
+}
 }  // namespace
 
 int set_values(DevicePlan *dp, const float *d_val, hipStream_t st)
 {
     if (!dp->hot_src || !dp->cold_src) return MPS_ERR_UNSUPPORTED;
     if (dp->hot_slots)
-        hipLaunchKernelGGL(rb_set_values_kernel, dim3((unsigned)((dp->hot_slots + 255) / 256)), dim3(256), 0, st, d_val,
+        hipLaunchKernelGGL(rb_set_values_packed_kernel, dim3((unsigned)((dp->hot_slots + 255) / 256)), dim3(256), 0, st, d_val,
                            dp->hot_src, dp->hot_slots, dp->hot);
     if (dp->cold_slots)
         hipLaunchKernelGGL(rb_set_values_kernel, dim3((unsigned)((dp->cold_slots + 255) / 256)), dim3(256), 0, st, d_val,
@@ -539,7 +588,8 @@ const void *device_array(const DevicePlan *dp, int which, size_t *bytes)
     case MPS_PLAN_ARRAY_RB_HOT_COLS: *bytes = L.hot_cols.size() * sizeof(int); return dp->hot_cols;
     case MPS_PLAN_ARRAY_RB_META: *bytes = L.meta.size() * sizeof(int); return dp->meta;
     case MPS_PLAN_ARRAY_RB_WAVE_BASE: *bytes = L.wave_base.size() * sizeof(long long); return dp->wave_base;
-    case MPS_PLAN_ARRAY_RB_HOT: *bytes = dp->hot_slots * sizeof(Entry); return dp->hot;
+    case MPS_PLAN_ARRAY_RB_HOT: *bytes = 0; return nullptr;  // host layouts only
+    case MPS_PLAN_ARRAY_RB_HOT_PACKED: *bytes = dp->hot_slots / kPair * 12; return dp->hot;
     case MPS_PLAN_ARRAY_RB_COLD: *bytes = dp->cold_slots * sizeof(Entry); return dp->cold;
     case MPS_PLAN_ARRAY_RB_HOT_SRC: *bytes = dp->hot_src ? dp->hot_slots * sizeof(int) : 0; return dp->hot_src;
     case MPS_PLAN_ARRAY_RB_COLD_SRC: *bytes = dp->cold_src ? dp->cold_slots * sizeof(int) : 0; return dp->cold_src;

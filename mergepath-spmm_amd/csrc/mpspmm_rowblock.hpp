@@ -71,6 +71,17 @@ struct Entry {
     float val;
 };
 
+// Packed hot stream, what the device reads: the table slot of a hot entry needs 11 bits (kMaxTableRows <= 2048) and a
+// window advances fewer than 1,024 rows (a block holds at most 1,024), so a lane's share of a round shrinks from 16
+// to 12 bytes:
+//   {value A, value B, half A | half B << 16},  half = slot | piece << kPackedSlotBits,
+// where the 5-bit pieces of a window's entries 0 and 1 are the low and the high half of its rows_advanced (entries
+// 2 and 3 carry 0).  A round is then 64 x 12 = 768 bytes; rounds and lanes keep their order.
+constexpr int kPackedSlotBits = 11;
+constexpr int kPackedPieceBits = 5;
+constexpr uint32_t kPackedAdvMax = (1u << (2 * kPackedPieceBits)) - 1u;
+constexpr int kPackedRoundWords = 64 * 3;
+
 struct Layout {
     int n = 0, nnz = 0, K = 16;
     int steps = 0;        // T
@@ -87,6 +98,7 @@ struct Layout {
     std::vector<long long> wave_base;   // [NB * 16][2] first round of the wavefront's hot / cold stream; [..][15]: where the block's streams end
     std::vector<Entry> hot, cold;       // rounds of 64 entries
     std::vector<int> hot_src, cold_src; // original nonzero index per entry slot, -1 = padding (optional)
+    std::vector<uint32_t> hot_packed;   // the hot stream in packed form
 };
 
 struct BuildParams {
@@ -103,6 +115,9 @@ constexpr int kNotWorthwhile = -1;  // build_layout: the matrix is not skewed en
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,
                  const BuildParams &bp, Layout &out);
+
+// Fills out.hot_packed from out.hot; false if the packed form cannot hold it (no layout of build_layout does that).
+bool pack_hot_stream(Layout &out);
 
 // Steps the library picks for a matrix when the caller names none.
 int default_steps(int n, long long nnz, int table_rows);

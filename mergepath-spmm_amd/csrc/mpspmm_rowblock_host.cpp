@@ -367,7 +367,39 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             }
         }
     });
-    return MPS_OK;
+    // what the device reads instead of L.hot (blocks hold at most 1,024 rows and tables at most 2,048: it always fits)
+    return pack_hot_stream(L) ? MPS_OK : MPS_ERR_UNSUPPORTED;
+}
+
+bool pack_hot_stream(Layout &L)
+{
+    L.hot_packed.clear();
+    if (L.hot_bits > kPackedSlotBits) return false;
+    const size_t rounds = L.hot.size() / kRoundEntries;
+    const uint32_t slot_mask = (1u << L.hot_bits) - 1u, piece_mask = (1u << kPackedPieceBits) - 1u;
+    std::atomic<bool> fits{true};
+    L.hot_packed.resize(rounds * kPackedRoundWords);
+    parallel_for((int64_t)rounds, 256, [&](int64_t r0, int64_t r1) {
+        for (int64_t r = r0; r < r1; ++r)
+            for (int lane = 0; lane < 64; ++lane) {
+                // lane (g, e) holds entry e of its lane-group's two windows (A, B) side by side; entry 0 of a window
+                // holds its rows_advanced, of which entry 0 keeps the low piece and entry 1 gets the high one
+                const int e = lane % kWin, lane0 = lane - e;
+                uint32_t halves[kPair];
+                uint32_t *dst = &L.hot_packed[((size_t)r * 64 + (size_t)lane) * 3];
+                for (int which = 0; which < kPair; ++which) {
+                    const Entry &en = L.hot[(size_t)r * kRoundEntries + (size_t)lane * kPair + (size_t)which];
+                    const uint32_t adv = L.hot[(size_t)r * kRoundEntries + (size_t)lane0 * kPair + (size_t)which].word >> L.hot_bits;
+                    if (adv > kPackedAdvMax) fits.store(false, std::memory_order_relaxed);
+                    const uint32_t piece = e == 0 ? (adv & piece_mask) : e == 1 ? ((adv >> kPackedPieceBits) & piece_mask) : 0u;
+                    halves[which] = (en.word & slot_mask) | (piece << kPackedSlotBits);
+                    std::memcpy(dst + which, &en.val, 4);
+                }
+                dst[2] = halves[0] | (halves[1] << 16);
+            }
+    });
+    if (!fits.load()) L.hot_packed.clear();
+    return fits.load();
 }
 
 }  // namespace mps_rb
@@ -449,6 +481,7 @@ int mps_rowblock_layout_array(const mps_rowblock_layout *layout, int which, cons
     case MPS_PLAN_ARRAY_RB_COLD: return give(L.cold);
     case MPS_PLAN_ARRAY_RB_HOT_SRC: return give(L.hot_src);
     case MPS_PLAN_ARRAY_RB_COLD_SRC: return give(L.cold_src);
+    case MPS_PLAN_ARRAY_RB_HOT_PACKED: return give(L.hot_packed);
     default: return MPS_ERR_INVALID_ARG;
     }
 }

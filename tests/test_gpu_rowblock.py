@@ -98,6 +98,41 @@ def test_rowblock_plan_set_values_and_sources(pkg, orc, dev):
                               lay.array(which, dt))
 
 
+@pytest.mark.parametrize("sparse", [False, True])
+def test_rowblock_hot_stream_on_the_device_is_the_packed_form(pkg, orc, dev, sparse):
+    """The device reads the hot stream in packed form (12 bytes per lane and round), with rows_advanced in two pieces
+    (a lane-group's first window of a step lies up to a wavefront's run of rows from where the run starts; with mostly
+    empty rows every window does): the product, new values, and the arrays the host builder makes."""
+    rng = np.random.default_rng(77 + sparse)
+    n = 3000
+    if sparse:  # most rows empty
+        rp, ci = random_csr(rng, n, 30, p_empty=0.97, hub_rows=((9, 2500), (2900, 2000)))
+    else:
+        rp, ci = random_csr(rng, n, 60, p_empty=0.05, hub_rows=((9, 2500),))
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    kw = dict(rowblock="force", rowblock_steps=2, rowblock_table_rows=64, rowblock_blocks_per_round=2)
+    plan = pkg.spmm.Plan(csr, 16, **kw)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=2, table_rows=64, blocks_per_round=2)
+    C = pkg._cabi
+    hot = lay.array(C.MPS_PLAN_ARRAY_RB_HOT, np.uint32).reshape(-1, 2)
+    assert (hot[:, 0] >> lay.info.hot_mark_shift).max() > 31  # the high piece of rows_advanced is in use
+    assert plan.array(C.MPS_PLAN_ARRAY_RB_HOT).size == 0
+    assert np.array_equal(plan.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED), lay.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED, np.uint32))
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    val2 = rng.random(ci.size).astype(np.float32)
+    plan.set_values(to_dev(dev, val2)[0])
+    ref2, scale2 = orc.spmm_f64(rp, ci, val2, X, want_abs=True)
+    check_fp32(plan.spmm(d_X).cpu().numpy(), ref2, scale2, rel_elem=False)
+    fresh = pkg.spmm.Plan(make_csr(pkg, dev, rp, ci, val2), 16, **kw)
+    assert torch.equal(plan.spmm(d_X), fresh.spmm(d_X))
+    assert np.array_equal(plan.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED), fresh.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED))
+
+
 def test_rowblock_plan_rejects_other_shapes(pkg, dev):
     rng = np.random.default_rng(2)
     rp, ci = random_csr(rng, 100, 10)

@@ -96,6 +96,7 @@ def walk_layout(pkg, lay, X, n):
 
 CASES = [
     # n, max_deg, hubs, steps, table_rows, block_rows, blocks_per_round
+    (2000, 3, ((5, 1500),), 2, 16, 1000, 2),  # sparse: hot windows more than 31 rows apart
     (300, 40, ((5, 280), (150, 300)), 3, 16, 64, 4),
     (97, 12, (), 2, 8, 0, 2),
     (513, 60, ((0, 500), (512, 400)), 5, 32, 40, 8),
@@ -129,6 +130,22 @@ def test_layout_walk_reproduces_the_product(pkg, case):
         assert ((src >= 0).sum() + 0) <= ci.size
     hot_src = lay.array(C.MPS_PLAN_ARRAY_RB_HOT_SRC, np.int32)
     assert (hot_src >= 0).sum() == lay.info.hot_nnz
+    # the packed form of the hot stream, what the device reads: the same entries, 12 bytes per lane and round
+    # {value A, value B, half A | half B << 16}; a half is the table slot and, above bit 11, a 5-bit piece of the
+    # window's rows_advanced (entry 0: the low piece, entry 1: the high one)
+    hot = lay.array(C.MPS_PLAN_ARRAY_RB_HOT, np.uint32).reshape(-1, 2)
+    packed = lay.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED, np.uint32).reshape(-1, 3)  # one row per (round, lane)
+    bits = lay.info.hot_mark_shift
+    assert bits <= 11 and packed.shape[0] * 2 == hot.shape[0]
+    assert np.array_equal(packed[:, 0], hot[0::2, 1]) and np.array_equal(packed[:, 1], hot[1::2, 1])
+    slot = (hot[:, 0] & ((1 << bits) - 1)).reshape(-1, 64, 2)   # [round][lane][A / B]
+    adv = (hot[:, 0] >> bits).reshape(-1, 16, 4, 2)             # [round][group][entry][A / B]
+    assert adv.max(initial=0) < 1024 and not adv[:, :, 1:, :].any()
+    piece = np.zeros_like(adv)
+    piece[:, :, 0, :] = adv[:, :, 0, :] & 31
+    piece[:, :, 1, :] = adv[:, :, 0, :] >> 5
+    half = slot | (piece.reshape(-1, 64, 2) << 11)
+    assert np.array_equal(packed[:, 2].reshape(-1, 64), half[:, :, 0] | (half[:, :, 1] << 16))
 
 
 def test_hot_columns_are_the_busiest_and_dealt_round_robin(pkg):
