@@ -1291,6 +1291,12 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
             plan_free(pl);
             return MPS_ERR_UNSUPPORTED;
         }
+        // the builder's tables are indexed by column id
+        int vrc = mps_csr_validate(d_row_ptr, d_col_idx, n_rows, n_rows, nnz, stream);
+        if (vrc != MPS_OK) {
+            plan_free(pl);
+            return vrc;
+        }
         mps_rb::BuildParams bp;
         bp.steps = opt.rowblock_steps;
         bp.table_rows = opt.rowblock_table_rows;
