@@ -358,7 +358,7 @@ def main():
         Yc = np.empty((w.n, K), dtype=np.float32)
         orc.spmm_f32_mt(w.rp, w.ci, val32, X32, threads=threads, out=Yc)  # warm
         passes, spent = 0, 0.0
-        while passes < 20 and spent < 10.0:
+        while passes < 1000 and spent < 10.0:  # about 10 s of CPU work
             c0 = time.perf_counter()
             orc.spmm_f32_mt(w.rp, w.ci, val32, X32, threads=threads, out=Yc)
             spent += time.perf_counter() - c0
