@@ -1,0 +1,40 @@
+"""bench.py without a GPU: the lookup of measured HBM traffic by plan signature, and the refusal of more than one GPU."""
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+import bench  # noqa: E402
+
+
+def test_traffic_is_looked_up_by_plan_signature_and_names_its_profile():
+    table = open(bench.TRAFFIC_TABLE).read()
+    rows = [l for l in table.splitlines() if l.startswith("| `")]
+    assert len(rows) >= 10
+    for line in rows:
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        sig = cells[0].replace("`", "").replace(";", "|")
+        traffic, where = bench.measured_traffic(sig)
+        want = int((float(cells[2]) * float(cells[3]) + float(cells[4]) * float(cells[5])) * 1024)
+        assert traffic == want and traffic > 0
+        assert where.startswith("profiles/") and os.path.exists(os.path.join(ROOT, where))
+    # the headline workload with the library's own plan has a row; a plan of another shape has none
+    assert any(l.startswith("| `%s;rowblock;" % bench.HEADLINE) for l in rows)
+    assert bench.measured_traffic(bench.HEADLINE + "|rowblock|steps=99|table_rows=1|blocks=1") == (None, None)
+
+
+def test_workloads_cover_the_benchmark_configurations():
+    assert bench.HEADLINE in bench.WORKLOADS and len(bench.OTHER_CONFIGS) == 8
+    assert all(w in bench.WORKLOADS for w in bench.OTHER_CONFIGS)
+    ks = sorted(bench.WORKLOADS[w][1] for w in bench.OTHER_CONFIGS if w.startswith("rmat_s20"))
+    assert ks == [16, 32, 64, 128, 256]
+    # algorithmic bytes: row_ptr + col_idx + val + X + Y
+    assert bench.algorithmic_bytes(232965, 114604189, 16, 4, 4) == 947584896
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert p.returncode != 0 and "one GPU" in p.stderr
