@@ -137,10 +137,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
     extern __shared__ __align__(16) char smem[];
     float *table = reinterpret_cast<float *>(smem);                         // [H][16]
     float *acc = table + (size_t)H * 16;                                    // [acc_rows][16]
-    float4 *stage = reinterpret_cast<float4 *>(acc + (size_t)acc_rows * 16);  // [16 waves][64]: the tails
-    float *slots = reinterpret_cast<float *>(stage + kWaveSlots * 64);      // [16 waves][16]
+    float *slots = acc + (size_t)acc_rows * 16;                             // [16 waves][16]
     int *slot_row = reinterpret_cast<int *>(slots + kWaveSlots * 16);       // [16]
-    int *crows = slot_row + kWaveSlots;                                     // [16 waves][16 groups]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -164,9 +162,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
         // ---- every wavefront walks its runs
         long long cur_h = wave_base[((size_t)b * kWaveSlots + wave) * 2];
         long long cur_c = wave_base[((size_t)b * kWaveSlots + wave) * 2 + 1];
-        float4 *st4 = stage + wave * 64;
         float4 *my_slot4 = reinterpret_cast<float4 *>(slots + wave * 16) + s;
-        int *my_crows = crows + wave * 16;
         // the masks live in vector registers (the DPP form of v_and takes no scalar operand); the
         // empty asm keeps the compiler from re-creating them from scalars at every use
         hot_bits = kPackedSlotBits;  // the halves of the packed hot stream: table slot below, a piece of rows_advanced above
@@ -338,8 +334,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             // Tails: what every lane-group still holds for the last row of its run.  A group whose
             // neighbours end in other rows adds its sums to the row at once.  Neighbouring groups
             // can also end in the same row (one that is longer than a run): then the first group of
-            // the stretch of equal rows adds the stretch up in group order, through LDS, and adds
-            // the total.
+            // the stretch of equal rows adds the stretch up in group order, reading the others'
+            // sums lane to lane (no LDS behind it: that space holds table rows), and adds the total.
             auto tails = [&](const Walk &w, int len) {
                 const int row = len > 0 ? w.row : -1;
                 const int prev = __shfl_up(row, 4, 64), next = __shfl_down(row, 4, 64);
@@ -347,12 +343,17 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 const bool shared = row >= 0 && ((g > 0 && prev == row) || (g < kGroups - 1 && next == row));
                 float4 sum = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
                 if (__any(shared)) {
-                    st4[lane] = sum;
-                    if (s == 0) my_crows[g] = row;
-                    wave_lds_sync();
-                    if (shared && first)
-                        for (int k = g + 1; k < kGroups && my_crows[k] == row; ++k) add4(sum, st4[k * 4 + s]);
-                    wave_lds_sync();
+                    // `more`: this group leads a stretch whose end it has not reached.  A group that is read here
+                    // is not the first of its row, so its sums are the ones it came with.
+                    bool more = shared && first;
+                    for (int d = 1; d < kGroups; ++d) {
+                        const int there = __shfl_down(row, 4 * d, 64);  // (all lanes take part in every exchange)
+                        more = more && g + d < kGroups && there == row;
+                        if (!__any(more)) break;
+                        const float4 v = make_float4(__shfl_down(sum.x, 4 * d, 64), __shfl_down(sum.y, 4 * d, 64),
+                                                     __shfl_down(sum.z, 4 * d, 64), __shfl_down(sum.w, 4 * d, 64));
+                        if (more) add4(sum, v);
+                    }
                 }
                 if (row >= 0 && first) {
                     float4 *dst = row == first_row ? my_slot4 : acc4 + (size_t)row * 4 + s;
@@ -516,7 +517,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
         dp->device_bytes += bytes;
     }
-    dp->lds_bytes = (size_t)(L.table_rows + L.acc_rows) * 64 + kStageBytes + kSlotBytes;
+    dp->lds_bytes = (size_t)(L.table_rows + L.acc_rows) * 64 + kSlotBytes;
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);

@@ -61,9 +61,8 @@ constexpr int kWin = 4;            // entries of a window: one per lane of a lan
 constexpr int kPair = 2;           // windows of a lane-group per round: a lane loads its entry of both with one 16-byte load
 constexpr int kRoundEntries = kGroups * kWin * kPair;  // 128 entries = 1 KiB per round
 constexpr int kLdsBytes = 160 * 1024;
-constexpr int kStageBytes = kWaveSlots * 64 * 16;  // 64 float4 per wavefront: what its lane-groups hold at the end of their runs
-// shared-row slots [16][16] floats, their rows [16], tail rows [16][16]
-constexpr int kSlotBytes = kWaveSlots * 16 * 4 + kWaveSlots * 4 + kWaveSlots * 16 * 4;
+// shared-row slots [16][16] floats, their rows [16]
+constexpr int kSlotBytes = kWaveSlots * 16 * 4 + kWaveSlots * 4;
 constexpr int kMaxTableRows = 1536;  // six 16-byte pieces per thread when a table is moved
 
 struct Entry {

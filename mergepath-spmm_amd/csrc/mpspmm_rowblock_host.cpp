@@ -159,7 +159,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     L.cold_bits = cold_bits;
 
     // ---- 1. row blocks: about equal nonzero counts, as few rounds of workgroups as the LDS allows
-    const int budget_rows = (kLdsBytes - kStageBytes - kSlotBytes - 256) / 64;  // table rows + accumulator rows
+    const int budget_rows = (kLdsBytes - kSlotBytes - 256) / 64;  // table rows + accumulator rows
     int cap_limit = std::min(1024, 1 << (32 - cold_bits));                      // rows_advanced must fit above the index
     if (bp.table_rows > 0) cap_limit = std::min(cap_limit, budget_rows - bp.table_rows);
     if (cap_limit < 4) return MPS_ERR_INVALID_ARG;
@@ -193,7 +193,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         if (H > need) H = need;
         H = (H + 3) / 4 * 4;
     }
-    if (H < 1 || (long long)(H + L.acc_rows) * 64 + kStageBytes + kSlotBytes > kLdsBytes) return MPS_ERR_INVALID_ARG;
+    if (H < 1 || (long long)(H + L.acc_rows) * 64 + kSlotBytes > kLdsBytes) return MPS_ERR_INVALID_ARG;
     L.table_rows = H;
     L.steps = T;
     L.hot_bits = bits_for(H > 1 ? H - 1 : 1);
