@@ -17,6 +17,8 @@ CASES = [
     (200, 5, (), 4, 4, 16, 256),
     (5000, 200, ((17, 4800), (4999, 3000)), 6, 256, 0, 64),
     (20000, 64, ((0, 15000),), 8, 0, 0, 0),
+    # two rows far longer than a wavefront's run: every lane-group of several wavefronts ends in the same row
+    (4096, 8, ((7, 4000), (2000, 3500)), 2, 512, 0, 1),
 ]
 
 
