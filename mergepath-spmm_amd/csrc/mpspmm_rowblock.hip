@@ -344,8 +344,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             // Tails: what every lane-group still holds for the last row of its run.  A group whose
             // neighbours end in other rows adds its sums to the row at once.  Neighbouring groups
             // can also end in the same row (one that is longer than a run): then the first group of
-            // the stretch of equal rows adds the stretch up in group order, reading the others'
-            // sums lane to lane (no LDS behind it: that space holds table rows), and adds the total.
+            // the stretch of equal rows gets the stretch's total, summed lane to lane in a fixed
+            // tree (no LDS behind it: that space holds table rows), and adds it.
             auto tails = [&](const Walk &w, int len) {
                 const int row = len > 0 ? w.row : -1;
                 const int prev = __shfl_up(row, 4, 64), next = __shfl_down(row, 4, 64);
@@ -353,16 +353,15 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 const bool shared = row >= 0 && ((g > 0 && prev == row) || (g < kGroups - 1 && next == row));
                 float4 sum = make_float4(w.a[0], w.a[1], w.a[2], w.a[3]);
                 if (__any(shared)) {
-                    // `more`: this group leads a stretch whose end it has not reached.  A group that is read here
-                    // is not the first of its row, so its sums are the ones it came with.
-                    bool more = shared && first;
-                    for (int d = 1; d < kGroups; ++d) {
-                        const int there = __shfl_down(row, 4 * d, 64);  // (all lanes take part in every exchange)
-                        more = more && g + d < kGroups && there == row;
-                        if (!__any(more)) break;
+                    // Sums over 2, 4, 8, 16 neighbouring groups as far as they end in the same row (rows do not
+                    // decrease from group to group, so equal rows at distance d mean equal rows in between): after
+                    // the four exchanges the first group of a stretch holds the stretch's total.
+#pragma unroll
+                    for (int d = 1; d < kGroups; d *= 2) {
+                        const int there = __shfl_down(row, 4 * d, 64);
                         const float4 v = make_float4(__shfl_down(sum.x, 4 * d, 64), __shfl_down(sum.y, 4 * d, 64),
                                                      __shfl_down(sum.z, 4 * d, 64), __shfl_down(sum.w, 4 * d, 64));
-                        if (more) add4(sum, v);
+                        if (row >= 0 && g + d < kGroups && there == row) add4(sum, v);
                     }
                 }
                 if (row >= 0 && first) {
