@@ -416,6 +416,8 @@ typedef struct mps_plan_info {
     /* resident columns (resident_cols > 0): SLICE_COLS entries are column | streamed << mark_shift | row_ends << (mark_shift + 1) */
     int resident_cols;             /* columns whose rows of X are gathered without the streaming hint */
     long long resident_nnz;        /* nonzeros in them                            */
+    int rowblock_cold_index_bits;  /* row-block plans: > 0 when the cold stream is held in packed form (RB_COLD_PACKED): bits of a
+                                      16-bit entry that hold the column, counted from the first column of the step's range */
 } mps_plan_info;
 
 /* Optional parameters of mps_plan_create_ex; zero means "the library chooses". */
@@ -446,12 +448,16 @@ enum {
     MPS_PLAN_ARRAY_RB_META = 10,      /* int[blocks * steps * 16 * 4]: {hot entries, cold entries, first local row, 0} per wavefront */
     MPS_PLAN_ARRAY_RB_WAVE_BASE = 11, /* long long[blocks * 16 * 2]: first round of each wavefront's hot / cold stream */
     MPS_PLAN_ARRAY_RB_HOT = 12,       /* 8 bytes x hot slots: {index | rows_advanced << bits, value}; host layouts only (a device plan holds RB_HOT_PACKED) */
-    MPS_PLAN_ARRAY_RB_COLD = 13,      /* 8 bytes x cold slots                       */
+    MPS_PLAN_ARRAY_RB_COLD = 13,      /* 8 bytes x cold slots; a device plan holds it only when the packed form does not fit */
     MPS_PLAN_ARRAY_RB_HOT_SRC = 14,   /* int[hot slots]: original nonzero index, -1 = padding */
     MPS_PLAN_ARRAY_RB_COLD_SRC = 15,  /* int[cold slots]                            */
-    MPS_PLAN_ARRAY_RB_HOT_PACKED = 16 /* 12 bytes x (hot slots / 2), what the device reads: per round and lane {value A, value B,
+    MPS_PLAN_ARRAY_RB_HOT_PACKED = 16, /* 12 bytes x (hot slots / 2), what the device reads: per round and lane {value A, value B,
                                          half A | half B << 16}, half = table slot | piece << 11; the 5-bit pieces of a window's
                                          entries 0 and 1 are the low and the high half of its rows_advanced */
+    MPS_PLAN_ARRAY_RB_COLD_PACKED = 17, /* 12 bytes x (cold slots / 2), if rowblock_cold_index_bits > 0: the same form; half =
+                                         (column - first column of the step's range) | piece << index_bits, entry e of a window
+                                         holds bits [e p, (e + 1) p) of its rows_advanced, p = 16 - index_bits */
+    MPS_PLAN_ARRAY_RB_COLD_BEGIN = 18 /* int[steps + 1]: first column of every step's range of cold columns */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,

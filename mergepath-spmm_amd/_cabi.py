@@ -41,7 +41,7 @@ MPS_PLAN_NO_COLUMN_TILES = 512
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
  MPS_PLAN_ARRAY_RB_HOT, MPS_PLAN_ARRAY_RB_COLD, MPS_PLAN_ARRAY_RB_HOT_SRC, MPS_PLAN_ARRAY_RB_COLD_SRC,
- MPS_PLAN_ARRAY_RB_HOT_PACKED) = range(17)
+ MPS_PLAN_ARRAY_RB_HOT_PACKED, MPS_PLAN_ARRAY_RB_COLD_PACKED, MPS_PLAN_ARRAY_RB_COLD_BEGIN) = range(19)
 
 
 class PlanInfo(ctypes.Structure):
@@ -55,7 +55,8 @@ class PlanInfo(ctypes.Structure):
                 ("rowblock_steps", ctypes.c_int), ("rowblock_table_rows", ctypes.c_int),
                 ("rowblock_blocks", ctypes.c_int), ("rowblock_acc_rows", ctypes.c_int),
                 ("rowblock_hot_slots", ctypes.c_longlong), ("rowblock_cold_slots", ctypes.c_longlong),
-                ("resident_cols", ctypes.c_int), ("resident_nnz", ctypes.c_longlong)]
+                ("resident_cols", ctypes.c_int), ("resident_nnz", ctypes.c_longlong),
+                ("rowblock_cold_index_bits", ctypes.c_int)]
 
 
 class PlanOptions(ctypes.Structure):

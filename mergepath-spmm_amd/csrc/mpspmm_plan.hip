@@ -1363,6 +1363,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->hot_blocks = plan->hot_blocks;
     info->rowblock_steps = info->rowblock_table_rows = info->rowblock_blocks = info->rowblock_acc_rows = 0;
     info->rowblock_hot_slots = info->rowblock_cold_slots = 0;
+    info->rowblock_cold_index_bits = 0;
     if (plan->rb) {
         const mps_rb::Layout &L = mps_rb::layout_of(plan->rb);
         info->num_slabs = 1;
@@ -1376,6 +1377,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
         info->rowblock_acc_rows = L.acc_rows;
         info->rowblock_hot_slots = L.hot_rounds * mps_rb::kRoundEntries;
         info->rowblock_cold_slots = L.cold_rounds * mps_rb::kRoundEntries;
+        info->rowblock_cold_index_bits = L.cold_index_bits;
     }
     return MPS_OK;
 }
@@ -1409,7 +1411,7 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
     default:
         if (!plan->rb) return MPS_ERR_INVALID_ARG;
         src = mps_rb::device_array(plan->rb, which, &have);
-        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_HOT_PACKED)) return MPS_ERR_INVALID_ARG;
+        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_COLD_BEGIN)) return MPS_ERR_INVALID_ARG;
         break;
     }
     if (plan->rb && which < MPS_PLAN_ARRAY_RB_BLOCK_ROW) return MPS_ERR_INVALID_ARG;

@@ -19,10 +19,11 @@ namespace mps_rb {
 struct DevicePlan {
     Layout host;  // the small tables stay filled; the streams are released after the upload
     uint32_t *hot = nullptr;  // the hot stream in packed form (12 bytes per lane and round)
-    Entry *cold = nullptr;
+    Entry *cold = nullptr;           // the cold stream as the layout holds it, or
+    uint32_t *cold_packed = nullptr;  // in packed form (one of the two)
     int *hot_src = nullptr, *cold_src = nullptr;
     long long *wave_base = nullptr;
-    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr;
+    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr, *cold_begin = nullptr;
     float *hot_x = nullptr;  // [T][H][16] rows of X of the hot columns, gathered per product
     size_t lds_bytes = 0;
     size_t device_bytes = 0;
@@ -125,14 +126,19 @@ __device__ __forceinline__ void fma_from_lane(float (&a)[4], float val, const fl
 // rounds (two windows per lane-group each) that a wavefront needs for n windows dealt to its 16 lane-groups
 __device__ __forceinline__ int rounds_of(int n) { return ((n >> 4) + ((n & 15) != 0) + 1) >> 1; }
 
-template <typename TOut>
+// CPACK: the cold stream is read in its packed form (cold_p; 12 bytes per lane and round, columns counted from the
+// first column of the step's range, cold_begin[t]) instead of as 8-byte entries (cold).
+template <typename TOut, bool CPACK>
 __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__restrict__ hot, const Entry *__restrict__ cold,
+                                                            const uint32_t *__restrict__ cold_p,
+                                                            const int *__restrict__ cold_begin,
                                                             const long long *__restrict__ wave_base,
                                                             const int4 *__restrict__ meta,
                                                             const int *__restrict__ block_row,
                                                             const float4 *__restrict__ hot_x4,
                                                             const float4 *__restrict__ X4, TOut *__restrict__ Y, int T,
-                                                            int H, int acc_rows, int hot_bits, int cold_bits, int keep_from)
+                                                            int H, int acc_rows, int hot_bits, int cold_bits, int keep_from,
+                                                            int cold_ib)
 {
     extern __shared__ __align__(16) char smem[];
     float *table = reinterpret_cast<float *>(smem);                         // [H][16]
@@ -166,7 +172,10 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
         // the masks live in vector registers (the DPP form of v_and takes no scalar operand); the
         // empty asm keeps the compiler from re-creating them from scalars at every use
         hot_bits = kPackedSlotBits;  // the halves of the packed hot stream: table slot below, a piece of rows_advanced above
+        if constexpr (CPACK) cold_bits = cold_ib;  // a 16-bit half: column in the range below, a piece of rows_advanced above
         unsigned hmask = (1u << hot_bits) - 1u, cmask = (1u << cold_bits) - 1u, hot_hi = ~hmask, cold_hi = ~cmask;
+        // packed cold windows: entry e holds bits [e p, (e + 1) p) of rows_advanced above the column, p = 16 - cold_ib
+        const int cs1 = cold_ib - (16 - cold_ib), cs2 = cold_ib - 2 * (16 - cold_ib), cs3 = cold_ib - 3 * (16 - cold_ib);
         asm volatile("" : "+v"(hmask), "+v"(cmask), "+v"(hot_hi), "+v"(cold_hi));
         int4 m = meta_b[wave];
         __syncthreads();
@@ -212,19 +221,25 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 x[2] = table4[and_from_lane<2>(word, hmask) * 4 + s];
                 x[3] = table4[and_from_lane<3>(word, hmask) * 4 + s];
             };
+            // (packed cold entries count their columns from the first column of the step's range)
+            const char *xb = reinterpret_cast<const char *>(X4) + (CPACK ? (size_t)cold_begin[t] * 64 : (size_t)0);
             auto cold_gather = [&](unsigned word, float4 (&x)[kWin]) {
-                const char *xb = reinterpret_cast<const char *>(X4);
                 x[0] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<0>(word, cmask) << 6) | (unsigned)(s << 4)));
                 x[1] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<1>(word, cmask) << 6) | (unsigned)(s << 4)));
                 x[2] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<2>(word, cmask) << 6) | (unsigned)(s << 4)));
                 x[3] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<3>(word, cmask) << 6) | (unsigned)(s << 4)));
             };
             // is_hot: a hot window, whose rows_advanced lies in two pieces above the slots of its entries 0 and 1
+            // (a packed cold window: in four pieces, one above the column of every entry)
             auto window = [&](auto is_hot, Walk &w, unsigned word, unsigned valbits, const float4 (&x)[kWin], unsigned himask,
                               int bits) {
                 if constexpr (decltype(is_hot)::value) {
                     const unsigned lo = and_from_lane<0>(word, himask), hi = and_from_lane<1>(word, himask);
                     if ((lo | hi) != 0) row_end(w, (lo >> kPackedSlotBits) | (hi >> (kPackedSlotBits - kPackedPieceBits)));
+                } else if constexpr (CPACK) {
+                    const unsigned p0 = and_from_lane<0>(word, himask), p1 = and_from_lane<1>(word, himask);
+                    const unsigned p2 = and_from_lane<2>(word, himask), p3 = and_from_lane<3>(word, himask);
+                    if ((p0 | p1 | p2 | p3) != 0) row_end(w, (p0 >> bits) | (p1 >> cs1) | (p2 >> cs2) | (p3 >> cs3));
                 } else {
                     const unsigned hi = and_from_lane<0>(word, himask);
                     if (hi != 0) row_end(w, hi >> bits);
@@ -251,11 +266,17 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             const __amdgpu_buffer_rsrc_t hp = stream_rsrc(hot + (size_t)cur_h * kPackedRoundWords);
             const unsigned hoff = (unsigned)lane * 12u;
             auto load_hot = [&](int r) { return load_round_packed(hp, hoff + (unsigned)r * kHotRoundBytes, keep); };
-            const __amdgpu_buffer_rsrc_t cp = stream_rsrc(cold + (size_t)cur_c * kRoundEntries);
-            const unsigned loff = (unsigned)lane * 16u;
+            const __amdgpu_buffer_rsrc_t cp = CPACK ? stream_rsrc(cold_p + (size_t)cur_c * kPackedRoundWords)
+                                                    : stream_rsrc(cold + (size_t)cur_c * kRoundEntries);
+            constexpr unsigned kColdRoundBytes = CPACK ? kHotRoundBytes : 1024u;
+            const unsigned loff = (unsigned)lane * (CPACK ? 12u : 16u);
+            auto load_cold = [&](int r) {
+                if constexpr (CPACK) return load_round_packed(cp, loff + (unsigned)r * kColdRoundBytes, keep);
+                else return load_round(cp, loff + (unsigned)r * kColdRoundBytes, keep);
+            };
             uint4 nx_h = make_uint4(0u, 0u, 0u, 0u), nx_c = nx_h;
             if (rounds_h > 0) nx_h = load_hot(0);
-            if (rounds_c > 0) nx_c = load_round(cp, loff, keep);
+            if (rounds_c > 0) nx_c = load_cold(0);
             int rh = 0, rc = 0;  // rounds done
             // Round rh / rc has been taken: the next one is requested.  (Two rounds ahead instead of one: 1.5 %
             // slower on the 232,965-row power-law matrix; a round's load is not what the walk waits for.)
@@ -265,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             };
             auto advance_c = [&]() {
                 ++rc;
-                if (rc < rounds_c) nx_c = load_round(cp, loff + (unsigned)rc * 1024u, keep);
+                if (rc < rounds_c) nx_c = load_cold(rc);
             };
             // The rounds in which every lane-group holds two windows: the hot and the cold ones are
             // spread evenly over max(full_h, full_c) passes (a cold round in every pass whose
@@ -439,6 +460,8 @@ void destroy(DevicePlan *dp)
     if (!dp) return;
     (void)hipFree(dp->hot);
     (void)hipFree(dp->cold);
+    (void)hipFree(dp->cold_packed);
+    (void)hipFree(dp->cold_begin);
     (void)hipFree(dp->hot_src);
     (void)hipFree(dp->cold_src);
     (void)hipFree(dp->wave_base);
@@ -506,12 +529,18 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         // power-law matrix, 1.07 GB of streams in 16 steps of 67 MB: 0, 2, 3, 4, 5, 16 steps kept: 0.500, 0.482,
         // 0.484, 0.493, 0.503, 0.516 ms per product.
         const size_t hot_bytes = L.hot_packed.size() * sizeof(uint32_t);
-        const size_t per_step = (hot_bytes + dp->cold_slots * sizeof(Entry)) / (size_t)(L.steps > 0 ? L.steps : 1);
+        const size_t cold_bytes = L.cold_packed.empty() ? dp->cold_slots * sizeof(Entry) : L.cold_packed.size() * sizeof(uint32_t);
+        const size_t per_step = (hot_bytes + cold_bytes) / (size_t)(L.steps > 0 ? L.steps : 1);
         const size_t keep = per_step > 0 ? kStreamKeepBytes / per_step : (size_t)L.steps;
         dp->keep_from = keep >= (size_t)L.steps ? 0 : L.steps - (int)keep;
     }
     if ((rc = upload(dp, &dp->hot, L.hot_packed, st)) != MPS_OK) return fail(rc);
-    if ((rc = upload(dp, &dp->cold, L.cold, st)) != MPS_OK) return fail(rc);
+    if (L.cold_packed.empty()) {
+        if ((rc = upload(dp, &dp->cold, L.cold, st)) != MPS_OK) return fail(rc);
+    } else if ((rc = upload(dp, &dp->cold_packed, L.cold_packed, st)) != MPS_OK) {
+        return fail(rc);
+    }
+    if ((rc = upload(dp, &dp->cold_begin, L.cold_begin, st)) != MPS_OK) return fail(rc);
     if (bp_in.keep_src) {
         if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
         if ((rc = upload(dp, &dp->cold_src, L.cold_src, st)) != MPS_OK) return fail(rc);
@@ -528,14 +557,18 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
     }
     dp->lds_bytes = (size_t)(L.table_rows + L.acc_rows) * 64 + kSlotBytes;
     {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float, false>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
     release(L.hot);
     release(L.hot_packed);
     release(L.cold);
+    release(L.cold_packed);
     release(L.hot_src);
     release(L.cold_src);
     *out = dp;
@@ -549,11 +582,16 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
     if (phases & MPS_PHASE_PREPARE)
         hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
                            reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
-    if (phases & MPS_PHASE_MAIN)
-        hipLaunchKernelGGL((rb_spmm_kernel<float>), dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot,
-                           dp->cold, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta), dp->block_row,
-                           reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X), Y, L.steps,
-                           L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from);
+    if (phases & MPS_PHASE_MAIN) {
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot, dp->cold,
+                               dp->cold_packed, dp->cold_begin, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta),
+                               dp->block_row, reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X),
+                               Y, L.steps, L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from, L.cold_index_bits);
+        };
+        if (dp->cold_packed) launch(rb_spmm_kernel<float, true>);
+        else launch(rb_spmm_kernel<float, false>);
+    }
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
 }
@@ -568,7 +606,7 @@ __global__ __launch_bounds__(256) void rb_set_values_kernel(const float *__restr
     if (e >= 0) entries[i].val = val[e];
 }
 
-// The same for the packed hot stream: entry slot i is value (i % 2) of lane (i % 128) / 2 of round i / 128.
+// The same for a packed stream: entry slot i is value (i % 2) of lane (i % 128) / 2 of round i / 128.
 __global__ __launch_bounds__(256) void rb_set_values_packed_kernel(const float *__restrict__ val,
                                                                     const int *__restrict__ src, size_t slots,
                                                                     uint32_t *__restrict__ packed)
@@ -588,7 +626,10 @@ int set_values(DevicePlan *dp, const float *d_val, hipStream_t st)
     if (dp->hot_slots)
         hipLaunchKernelGGL(rb_set_values_packed_kernel, dim3((unsigned)((dp->hot_slots + 255) / 256)), dim3(256), 0, st, d_val,
                            dp->hot_src, dp->hot_slots, dp->hot);
-    if (dp->cold_slots)
+    if (dp->cold_slots && dp->cold_packed)
+        hipLaunchKernelGGL(rb_set_values_packed_kernel, dim3((unsigned)((dp->cold_slots + 255) / 256)), dim3(256), 0, st, d_val,
+                           dp->cold_src, dp->cold_slots, dp->cold_packed);
+    else if (dp->cold_slots)
         hipLaunchKernelGGL(rb_set_values_kernel, dim3((unsigned)((dp->cold_slots + 255) / 256)), dim3(256), 0, st, d_val,
                            dp->cold_src, dp->cold_slots, dp->cold);
     MPS_HIP_TRY(hipGetLastError());
@@ -607,7 +648,9 @@ const void *device_array(const DevicePlan *dp, int which, size_t *bytes)
     case MPS_PLAN_ARRAY_RB_WAVE_BASE: *bytes = L.wave_base.size() * sizeof(long long); return dp->wave_base;
     case MPS_PLAN_ARRAY_RB_HOT: *bytes = 0; return nullptr;  // host layouts only
     case MPS_PLAN_ARRAY_RB_HOT_PACKED: *bytes = dp->hot_slots / kPair * 12; return dp->hot;
-    case MPS_PLAN_ARRAY_RB_COLD: *bytes = dp->cold_slots * sizeof(Entry); return dp->cold;
+    case MPS_PLAN_ARRAY_RB_COLD: *bytes = dp->cold ? dp->cold_slots * sizeof(Entry) : 0; return dp->cold;
+    case MPS_PLAN_ARRAY_RB_COLD_PACKED: *bytes = dp->cold_packed ? dp->cold_slots / kPair * 12 : 0; return dp->cold_packed;
+    case MPS_PLAN_ARRAY_RB_COLD_BEGIN: *bytes = L.cold_begin.size() * sizeof(int); return dp->cold_begin;
     case MPS_PLAN_ARRAY_RB_HOT_SRC: *bytes = dp->hot_src ? dp->hot_slots * sizeof(int) : 0; return dp->hot_src;
     case MPS_PLAN_ARRAY_RB_COLD_SRC: *bytes = dp->cold_src ? dp->cold_slots * sizeof(int) : 0; return dp->cold_src;
     default: *bytes = 0; return nullptr;

@@ -98,6 +98,8 @@ struct Layout {
     std::vector<Entry> hot, cold;       // rounds of 64 entries
     std::vector<int> hot_src, cold_src; // original nonzero index per entry slot, -1 = padding (optional)
     std::vector<uint32_t> hot_packed;   // the hot stream in packed form
+    std::vector<uint32_t> cold_packed;  // the cold stream in packed form; empty if it does not fit (see pack_cold_stream)
+    int cold_index_bits = 0;            // of a packed cold entry's 16 bits, those of the column (counted from cold_begin[t])
 };
 
 struct BuildParams {
@@ -117,6 +119,14 @@ int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n
 
 // Fills out.hot_packed from out.hot; false if the packed form cannot hold it (no layout of build_layout does that).
 bool pack_hot_stream(Layout &out);
+
+// Fills out.cold_packed from out.cold, 12 bytes per lane and round like the hot stream: {value A, value B, half A |
+// half B << 16}.  A half holds the column minus the first column of the step's range in its low cold_index_bits
+// (12 to 15, what the widest range needs) and, above them, a piece of the window's rows_advanced: entry e of a window
+// carries bits [e * p, (e + 1) * p) of it, p = 16 - cold_index_bits.  Returns false and leaves cold_packed empty when
+// a range is wider than 32,768 columns or a window advances more rows than 4 p bits hold: the kernel then reads
+// out.cold as it is.
+bool pack_cold_stream(Layout &out);
 
 // Steps the library picks for a matrix when the caller names none.
 int default_steps(int n, long long nnz, int table_rows);

@@ -368,7 +368,9 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         }
     });
     // what the device reads instead of L.hot (blocks hold at most 1,024 rows and tables at most 2,048: it always fits)
-    return pack_hot_stream(L) ? MPS_OK : MPS_ERR_UNSUPPORTED;
+    if (!pack_hot_stream(L)) return MPS_ERR_UNSUPPORTED;
+    pack_cold_stream(L);  // (or the device reads L.cold)
+    return MPS_OK;
 }
 
 bool pack_hot_stream(Layout &L)
@@ -400,6 +402,63 @@ bool pack_hot_stream(Layout &L)
     });
     if (!fits.load()) L.hot_packed.clear();
     return fits.load();
+}
+
+bool pack_cold_stream(Layout &L)
+{
+    L.cold_packed.clear();
+    L.cold_index_bits = 0;
+    const int T = L.steps, NB = L.num_blocks;
+    int widest = 1;
+    for (int t = 0; t < T; ++t) widest = std::max(widest, L.cold_begin[(size_t)t + 1] - L.cold_begin[(size_t)t]);
+    const int ib = std::max(12, bits_for(widest > 1 ? widest - 1 : 1));
+    if (ib > 15) return false;
+    const int pb = 16 - ib;
+    const uint32_t idx_mask = (1u << L.cold_bits) - 1u, piece_mask = (1u << pb) - 1u;
+    const uint32_t adv_max = pb * kWin >= 32 ? 0xffffffffu : (1u << (pb * kWin)) - 1u;
+    std::atomic<bool> fits{true};
+    L.cold_packed.assign((size_t)L.cold_rounds * kPackedRoundWords, 0u);
+    parallel_for(NB, 1, [&](int64_t b0, int64_t b1) {
+        for (int64_t b = b0; b < b1; ++b)
+            for (int w = 0; w < kWaves; ++w) {
+                long long r = L.wave_base[((size_t)b * kWaveSlots + (size_t)w) * 2 + 1];
+                for (int t = 0; t < T; ++t) {
+                    const int nc = L.meta[(((size_t)b * T + (size_t)t) * kWaveSlots + (size_t)w) * 4 + 1];
+                    const int first = L.cold_begin[(size_t)t];
+                    const int rounds = rounds_for(nc);
+                    for (int q = 0; q < rounds; ++q, ++r)
+                        for (int lane = 0; lane < 64; ++lane) {
+                            const int g = lane / kWin, e = lane % kWin, lane0 = lane - e;
+                            const int len = (nc >> 4) + (g < (nc & 15));  // windows of this lane-group in the run
+                            uint32_t halves[kPair];
+                            uint32_t *dst = &L.cold_packed[((size_t)r * 64 + (size_t)lane) * 3];
+                            for (int which = 0; which < kPair; ++which) {
+                                const Entry &en = L.cold[(size_t)r * kRoundEntries + (size_t)lane * kPair + (size_t)which];
+                                std::memcpy(dst + which, &en.val, 4);
+                                if (q * kPair + which >= len) {  // no window here: the gather still needs a row of X
+                                    halves[which] = 0u;
+                                    continue;
+                                }
+                                const uint32_t adv = L.cold[(size_t)r * kRoundEntries + (size_t)lane0 * kPair + (size_t)which].word >> L.cold_bits;
+                                const int rel = (int)(en.word & idx_mask) - first;
+                                if (adv > adv_max || rel < 0 || rel >= (1 << ib)) {
+                                    fits.store(false, std::memory_order_relaxed);
+                                    halves[which] = 0u;
+                                    continue;
+                                }
+                                halves[which] = (uint32_t)rel | (((adv >> (pb * e)) & piece_mask) << ib);
+                            }
+                            dst[2] = halves[0] | (halves[1] << 16);
+                        }
+                }
+            }
+    });
+    if (!fits.load()) {
+        std::vector<uint32_t>().swap(L.cold_packed);
+        return false;
+    }
+    L.cold_index_bits = ib;
+    return true;
 }
 
 }  // namespace mps_rb
@@ -460,6 +519,7 @@ int mps_rowblock_layout_info(const mps_rowblock_layout *layout, mps_plan_info *i
     info->rowblock_acc_rows = L.acc_rows;
     info->rowblock_hot_slots = L.hot_rounds * mps_rb::kRoundEntries;
     info->rowblock_cold_slots = L.cold_rounds * mps_rb::kRoundEntries;
+    info->rowblock_cold_index_bits = L.cold_index_bits;
     return MPS_OK;
 }
 
@@ -482,6 +542,8 @@ int mps_rowblock_layout_array(const mps_rowblock_layout *layout, int which, cons
     case MPS_PLAN_ARRAY_RB_HOT_SRC: return give(L.hot_src);
     case MPS_PLAN_ARRAY_RB_COLD_SRC: return give(L.cold_src);
     case MPS_PLAN_ARRAY_RB_HOT_PACKED: return give(L.hot_packed);
+    case MPS_PLAN_ARRAY_RB_COLD_PACKED: return give(L.cold_packed);
+    case MPS_PLAN_ARRAY_RB_COLD_BEGIN: return give(L.cold_begin);
     default: return MPS_ERR_INVALID_ARG;
     }
 }

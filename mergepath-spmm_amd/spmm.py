@@ -241,10 +241,12 @@ class Plan:
             _cabi.MPS_PLAN_ARRAY_RB_META: (i.rowblock_blocks * i.rowblock_steps * 64, np.int32),
             _cabi.MPS_PLAN_ARRAY_RB_WAVE_BASE: (i.rowblock_blocks * 32, np.int64),
             _cabi.MPS_PLAN_ARRAY_RB_HOT: (0, np.uint32),  # host layouts only
-            _cabi.MPS_PLAN_ARRAY_RB_COLD: (2 * int(i.rowblock_cold_slots), np.uint32),
+            _cabi.MPS_PLAN_ARRAY_RB_COLD: (0 if i.rowblock_cold_index_bits else 2 * int(i.rowblock_cold_slots), np.uint32),
             _cabi.MPS_PLAN_ARRAY_RB_HOT_SRC: (int(i.rowblock_hot_slots), np.int32),
             _cabi.MPS_PLAN_ARRAY_RB_COLD_SRC: (int(i.rowblock_cold_slots), np.int32),
             _cabi.MPS_PLAN_ARRAY_RB_HOT_PACKED: (3 * int(i.rowblock_hot_slots) // 2, np.uint32),
+            _cabi.MPS_PLAN_ARRAY_RB_COLD_PACKED: (3 * int(i.rowblock_cold_slots) // 2 if i.rowblock_cold_index_bits else 0, np.uint32),
+            _cabi.MPS_PLAN_ARRAY_RB_COLD_BEGIN: (i.rowblock_steps + 1 if i.rowblock_steps else 0, np.int32),
         }
         n, dt = shapes[which]
         out = np.empty(n, dtype=dt)

@@ -94,8 +94,8 @@ def test_rowblock_plan_set_values_and_sources(pkg, orc, dev):
     lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=3, table_rows=48, blocks_per_round=8)
     C = pkg._cabi
     for which, dt in ((C.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32), (C.MPS_PLAN_ARRAY_RB_META, np.int32),
-                      (C.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32), (C.MPS_PLAN_ARRAY_RB_COLD, np.uint32),
-                      (C.MPS_PLAN_ARRAY_RB_HOT_SRC, np.int32)):
+                      (C.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32), (C.MPS_PLAN_ARRAY_RB_COLD_PACKED, np.uint32),
+                      (C.MPS_PLAN_ARRAY_RB_COLD_BEGIN, np.int32), (C.MPS_PLAN_ARRAY_RB_HOT_SRC, np.int32)):
         assert np.array_equal(lean.array(which) if which != C.MPS_PLAN_ARRAY_RB_HOT_SRC else plan.array(which),
                               lay.array(which, dt))
 
@@ -133,6 +133,42 @@ def test_rowblock_hot_stream_on_the_device_is_the_packed_form(pkg, orc, dev, spa
     fresh = pkg.spmm.Plan(make_csr(pkg, dev, rp, ci, val2), 16, **kw)
     assert torch.equal(plan.spmm(d_X), fresh.spmm(d_X))
     assert np.array_equal(plan.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED), fresh.array(C.MPS_PLAN_ARRAY_RB_HOT_PACKED))
+    # the cold stream likewise: packed on the device (ranges of 1,500 columns, windows at most 255 rows apart)
+    assert plan.info.rowblock_cold_index_bits == 12 and plan.array(C.MPS_PLAN_ARRAY_RB_COLD).size == 0
+    assert np.array_equal(plan.array(C.MPS_PLAN_ARRAY_RB_COLD_PACKED), fresh.array(C.MPS_PLAN_ARRAY_RB_COLD_PACKED))
+    assert np.array_equal(fresh.array(C.MPS_PLAN_ARRAY_RB_COLD_PACKED), pkg.spmm.RowBlockLayout(rp, ci, val2, steps=2, table_rows=64, blocks_per_round=2).array(C.MPS_PLAN_ARRAY_RB_COLD_PACKED, np.uint32))
+
+
+def test_rowblock_cold_stream_stays_unpacked_when_it_does_not_fit(pkg, orc, dev):
+    """Ranges wider than 32,768 columns (one step over 40,000 columns) or windows further apart than the pieces hold
+    leave the cold stream as 8-byte entries: the other instantiation of the kernel reads them."""
+    rng = np.random.default_rng(5)
+    n = 40000
+    rp, ci = random_csr(rng, n, 6, p_empty=0.3, hub_rows=((3, 30000),))
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    C = pkg._cabi
+    plan = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=1, rowblock_table_rows=64, rowblock_blocks_per_round=8)
+    assert plan.info.rowblock_cold_index_bits == 0 and plan.array(C.MPS_PLAN_ARRAY_RB_COLD_PACKED).size == 0
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=1, table_rows=64, blocks_per_round=8)
+    assert np.array_equal(plan.array(C.MPS_PLAN_ARRAY_RB_COLD), lay.array(C.MPS_PLAN_ARRAY_RB_COLD, np.uint32))
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(plan.spmm(d_X, out=torch.full_like(d_X, float("nan"))).cpu().numpy(), ref, scale, rel_elem=False)
+    val2 = rng.random(ci.size).astype(np.float32)
+    plan.set_values(to_dev(dev, val2)[0])
+    ref2, scale2 = orc.spmm_f64(rp, ci, val2, X, want_abs=True)
+    check_fp32(plan.spmm(d_X).cpu().numpy(), ref2, scale2, rel_elem=False)
+    # mostly empty rows, 15-bit ranges (one 4-bit piece... a window 20 rows from the last one does not fit 4 bits)
+    rp3, ci3 = random_csr(rng, 30000, 40, p_empty=0.99, hub_rows=((9, 25000), (29000, 20000)))
+    val3 = rng.random(ci3.size).astype(np.float32)
+    X3 = (rng.random((30000, 16)) * 2 - 1).astype(np.float32)
+    plan3 = pkg.spmm.Plan(make_csr(pkg, dev, rp3, ci3, val3), 16, rowblock="force", rowblock_steps=1, rowblock_table_rows=64,
+                          rowblock_blocks_per_round=2)
+    assert plan3.info.rowblock_cold_index_bits == 0
+    ref3, scale3 = orc.spmm_f64(rp3, ci3, val3, X3, want_abs=True)
+    check_fp32(plan3.spmm(to_dev(dev, X3)[0]).cpu().numpy(), ref3, scale3, rel_elem=False)
 
 
 def test_rowblock_plan_rejects_other_shapes(pkg, dev):

@@ -146,6 +146,42 @@ def test_layout_walk_reproduces_the_product(pkg, case):
     piece[:, :, 1, :] = adv[:, :, 0, :] >> 5
     half = slot | (piece.reshape(-1, 64, 2) << 11)
     assert np.array_equal(packed[:, 2].reshape(-1, 64), half[:, :, 0] | (half[:, :, 1] << 16))
+    # the packed form of the cold stream, where it fits: the same 12 bytes; a half is the column counted from the
+    # first column of the step's range and, above index_bits, the piece of rows_advanced that belongs to the entry
+    # (entry e: bits [e p, (e + 1) p), p = 16 - index_bits)
+    ib = lay.info.rowblock_cold_index_bits
+    cpk = lay.array(C.MPS_PLAN_ARRAY_RB_COLD_PACKED, np.uint32).reshape(-1, 3)
+    if ib == 0:
+        assert cpk.size == 0
+        return
+    pb = 16 - ib
+    cold = lay.array(C.MPS_PLAN_ARRAY_RB_COLD, np.uint32).reshape(-1, 2)
+    cold_begin = lay.array(C.MPS_PLAN_ARRAY_RB_COLD_BEGIN, np.int32)
+    cbits = lay.info.mark_shift
+    assert 12 <= ib <= 15 and cpk.shape[0] * 2 == cold.shape[0] and cold_begin.size == lay.info.rowblock_steps + 1
+    assert np.array_equal(cpk[:, 0], cold[0::2, 1]) and np.array_equal(cpk[:, 1], cold[1::2, 1])
+    half = np.stack([cpk[:, 2] & 0xffff, cpk[:, 2] >> 16], axis=1).reshape(-1, 16, 4, 2)  # [round][group][entry][A / B]
+    rel, piece = half & ((1 << ib) - 1), half >> ib
+    adv_packed = sum(piece[:, :, e, :].astype(np.int64) << (pb * e) for e in range(4))       # [round][group][A / B]
+    col = (cold[:, 0] & ((1 << cbits) - 1)).reshape(-1, 16, 4, 2).astype(np.int64)
+    adv = (cold[:, 0] >> cbits).reshape(-1, 16, 4, 2)[:, :, 0, :]
+    # rounds in stream order belong to (block, wavefront, step): walk them the way the builder laid them out
+    meta = lay.array(C.MPS_PLAN_ARRAY_RB_META, np.int32).reshape(lay.info.rowblock_blocks, lay.info.rowblock_steps, WSLOTS, 4)
+    base = lay.array(C.MPS_PLAN_ARRAY_RB_WAVE_BASE, np.int64).reshape(lay.info.rowblock_blocks, WSLOTS, 2)
+    for b in range(lay.info.rowblock_blocks):
+        for w in range(WAVES):
+            r = int(base[b, w, 1])
+            for t in range(lay.info.rowblock_steps):
+                nk = int(meta[b, t, w, 1])
+                for q in range(rounds_for(nk)):
+                    for g in range(G):
+                        for which in range(2):
+                            if 2 * q + which < dealt_len(nk, g):
+                                assert np.array_equal(rel[r, g, :, which] + cold_begin[t], col[r, g, :, which])
+                                assert adv_packed[r, g, which] == adv[r, g, which]
+                            else:
+                                assert not half[r, g, :, which].any()
+                    r += 1
 
 
 def test_hot_columns_are_the_busiest_and_dealt_round_robin(pkg):
