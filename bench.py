@@ -57,8 +57,8 @@ def plan_signature(workload, info):
     if info is None:
         return "%s|csr" % workload
     if info.rowblock_steps > 0:
-        return "%s|rowblock|steps=%d|table_rows=%d|blocks=%d" % (workload, info.rowblock_steps, info.rowblock_table_rows,
-                                                                  info.rowblock_blocks)
+        return "%s|rowblock|steps=%d|table_rows=%d|blocks=%d|cold_index_bits=%d" % (
+            workload, info.rowblock_steps, info.rowblock_table_rows, info.rowblock_blocks, info.rowblock_cold_index_bits)
     return "%s|slabs=%d|cost=%d|tpw=%d|hot_rows=%d|resident_cols=%d" % (workload, info.num_slabs, info.cost,
                                                                         info.threads_per_wave, info.hot_rows, info.resident_cols)
 

@@ -22,7 +22,7 @@ def test_traffic_is_looked_up_by_plan_signature_and_names_its_profile():
         assert where.startswith("profiles/") and os.path.exists(os.path.join(ROOT, where))
     # the headline workload with the library's own plan has a row; a plan of another shape has none
     assert any(l.startswith("| `%s;rowblock;" % bench.HEADLINE) for l in rows)
-    assert bench.measured_traffic(bench.HEADLINE + "|rowblock|steps=99|table_rows=1|blocks=1") == (None, None)
+    assert bench.measured_traffic(bench.HEADLINE + "|rowblock|steps=99|table_rows=1|blocks=1|cold_index_bits=0") == (None, None)
 
 
 def test_workloads_cover_the_benchmark_configurations():
