@@ -78,6 +78,10 @@ def test_power_law_config_full_size(pkg, orc, dev):
     # the library's own choice here: a row-block plan (rows summed in LDS, more than half of the nonzeros
     # gathered from LDS tables), one block per CU
     assert plan.info.rowblock_steps > 0 and plan.info.rowblock_blocks % 256 == 0 and plan.info.hot_nnz > 0.5 * ci.size
+    # both entry streams in packed form (a step's cold columns span fewer than 16,384 ids): without the source
+    # indices that this plan keeps for mps_plan_set_values, it is smaller than the CSR arrays
+    sources = 4 * (plan.info.rowblock_hot_slots + plan.info.rowblock_cold_slots)
+    assert plan.info.rowblock_cold_index_bits == 14 and plan.info.device_bytes - sources < 8 * ci.size + 4 * rp.size
     Yp = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     # without row blocks: 5 slabs of 3 MiB, 1,728 hot columns per slab (over a third of the nonzeros)
     slab_plan = pkg.spmm.Plan(csr, K, rowblock="off")
