@@ -321,11 +321,14 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 if (do_h) {
                     due_h -= passes;
                     const uint4 cu_h = nx_h;
-                    float4 xha[kWin], xhb[kWin];
+                    float4 xh[kWin];
                     advance_h();
-                    hot_gather(cu_h.x, xha);
-                    hot_gather(cu_h.z, xhb);
-                    pair(kHot, wh, cu_h, xha, xhb, hot_hi, 0, true, true);
+                    // one window after the other: table rows arrive within a hundred cycles or two, and four rows
+                    // in registers instead of eight leave the compiler room (0.3 to 0.6 % faster than both gathered first)
+                    hot_gather(cu_h.x, xh);
+                    window(kHot, wh, cu_h.x, cu_h.y, xh, hot_hi, 0);
+                    hot_gather(cu_h.z, xh);
+                    window(kHot, wh, cu_h.z, cu_h.w, xh, hot_hi, 0);
                 }
                 if (do_c) pair(kCold, wc, cu_c, xca, xcb, cold_hi, cold_bits, true, true);
             }
