@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void rb_gather_hot_kernel(const int *__restric
 }
 
 constexpr int kThreads = kWaveSlots * 64;
-constexpr size_t kStreamKeepBytes = 192u << 20;  // of the entry streams, kept in the last-level cache between products
+constexpr size_t kStreamKeepBytes = 160u << 20;  // of the entry streams, kept in the last-level cache between products
 constexpr int kPrefetch = (kMaxTableRows * 4 + kThreads - 1) / kThreads;  // float4 per thread of one table
 
 // The entry streams are read through buffer descriptors: the base of a wavefront's run of rounds in scalar
@@ -530,7 +530,8 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         // it by.  A product reads a plan once, front to back: left to itself the cache would hold the end of the
         // previous pass and lose it again before the next pass gets there.  Measured on MI355X, 232,965-row
         // power-law matrix, 1.07 GB of streams in 16 steps of 67 MB: 0, 2, 3, 4, 5, 16 steps kept: 0.500, 0.482,
-        // 0.484, 0.493, 0.503, 0.516 ms per product.
+        // 0.484, 0.493, 0.503, 0.516 ms per product; with both streams packed, 16 steps of 50 MB: 2, 3, 4, 5 steps
+        // kept: 0.435, 0.4285, 0.432, 0.442 ms.
         const size_t hot_bytes = L.hot_packed.size() * sizeof(uint32_t);
         const size_t cold_bytes = L.cold_packed.empty() ? dp->cold_slots * sizeof(Entry) : L.cold_packed.size() * sizeof(uint32_t);
         const size_t per_step = (hot_bytes + cold_bytes) / (size_t)(L.steps > 0 ? L.steps : 1);
