@@ -1215,21 +1215,34 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
 }
 
 // Row-block plan or not.  Forced: yes.  Otherwise only for what the kernel is built for (fp32,
-// K = 16) and where it was measured to win on MI355X against the slab plans: long rows (the
-// LDS tables are loaded once per block and step, so a block must hold many nonzeros per
-// table), an X of 12 MiB or more (232,965 rows: 0.53 against 0.58 ms, and 0.35 against
-// 0.38 ms at half the nonzeros; 500,000 rows: 0.73 against 0.75 ms; but 100,000 rows, whose X
-// two slabs cover: 0.175 against 0.140 ms) and columns skewed enough for the tables to serve a
-// quarter of the nonzeros (uniform 232,965-row matrix, 10 %: 0.49 against 0.41 ms) - the
-// last is known only once the builder has counted the columns, see kMinHotShare.
-constexpr double kMinHotShare = 0.25;
+// K = 16) and where it was measured to win on MI355X against the slab plans.  What decides is
+// the work of a block per step: every step costs a block two barriers, a table load and some
+// padded windows, about 5 us, which some 4,000 nonzeros pay for (kMinStepNnz).  Whether the
+// columns are skewed matters little: the gathers of a step stay in L2 either way.  Measured
+// (ms per product, row-block against slab plan; nonzeros per block and step in brackets):
+//   power law 232,965 rows x 16 per row .042/.058 (7.3k), x 128 .148/.231 (29k);
+//   100,000 x 16 .028/.031 (3.1k), x 64 .042/.067 (12k); 60,000 x 16 .024/.022 (3.8k),
+//   x 32 .025/.027 (7.5k); 500,000 x 16 .117/.109 (2.2k), x 32 .152/.186 (4.5k);
+//   1,000,000 x 32 .458/.409 (2.4k), x 64 .596/.674 (4.8k); 2,000,000 x 100 2.28/2.13 (3.8k);
+//   uniform 232,965 x 32 .069/.119 (5.8k), 500,000 x 64 .272/.336 (5.7k),
+//   1,000,000 x 100 .92/1.09 (4.4k); R-MAT scale 20, 16 per row .78/.177 (1.2k).
+// The steps are known only once the builder has counted the columns, so the builder decides
+// (kNotWorthwhile); here only what no step count can save is turned away, before the matrix
+// is copied to the host: with the fewest steps a plan could get (5 MiB of X per step).
+// A matrix whose columns stay near the diagonal is the slab plans' (banded, 233,000 rows x 64 within
+// 2,000 columns of the diagonal: .160/.114; 500,000 x 64 within 3,000: .427/.287): the blocks idle
+// through the steps whose column range they do not touch (kMaxLocalShare, measured by the builder).
+constexpr long long kMinStepNnz = 4000;
+constexpr double kMaxLocalShare = 0.25;
 bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, unsigned flags)
 {
     if (flags & MPS_PLAN_FORCE_ROWBLOCK) return true;
     if (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT)) return false;
     if (elem_bytes != 4 || K != 16 || n_rows < 1) return false;
-    if ((uint64_t)n_rows * 64 < (12u << 20) || n_rows > (1 << 22)) return false;
-    return (long long)nnz >= 128LL * n_rows;
+    if (n_rows > (1 << 22)) return false;
+    const long long blocks = (((long long)n_rows + 1023) / 1024 + 255) / 256 * 256;
+    const long long fewest_steps = std::max<long long>(1, ((long long)n_rows * 64 + (5ll << 20) - 1) / (5ll << 20));
+    return (long long)nnz >= kMinStepNnz * blocks * fewest_steps;
 }
 
 }  // namespace
@@ -1303,7 +1316,8 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.block_rows = opt.rowblock_block_rows;
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
-        bp.min_hot_share = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 0.0 : kMinHotShare;
+        bp.min_step_nnz = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 0 : kMinStepNnz;
+        bp.max_local_share = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 1.0 : kMaxLocalShare;
         int rc = mps_rb::create(d_row_ptr, d_col_idx, static_cast<const float *>(d_val), n_rows, nnz, K, bp,
                                 static_cast<hipStream_t>(stream), &pl->rb);
         if (rc == MPS_OK) {
@@ -1316,7 +1330,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
             plan_free(pl);
             return rc;
         }
-        // columns too evenly used for LDS tables to pay: the slab plan below
+        // too little work per block and step, or columns near the diagonal: the slab plan below
     }
     int rc;
     try {

@@ -108,10 +108,11 @@ struct BuildParams {
     int block_rows = 0;  // 0 = choose; otherwise the most rows a block may hold
     int num_cus = 256;
     bool keep_src = true;
-    double min_hot_share = 0.0;  // give up (kNotWorthwhile) when the tables would serve a smaller share of the nonzeros
+    long long min_step_nnz = 0;  // give up (kNotWorthwhile) when a block has fewer nonzeros per step on average
+    double max_local_share = 1.0;  // give up when the blocks find a larger share of the nonzeros in column ranges of their own
 };
 
-constexpr int kNotWorthwhile = -1;  // build_layout: the matrix is not skewed enough for min_hot_share
+constexpr int kNotWorthwhile = -1;  // build_layout: min_step_nnz or max_local_share not met
 
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,
@@ -129,7 +130,7 @@ bool pack_hot_stream(Layout &out);
 bool pack_cold_stream(Layout &out);
 
 // Steps the library picks for a matrix when the caller names none.
-int default_steps(int n, long long nnz, int table_rows);
+int default_steps(int n, long long nnz, int table_rows, int num_blocks, const long long *table_nnz, int tables);
 
 #ifdef MPSPMM_DEVICE_HPP
 // Device side (mpspmm_rowblock.hip), for translation units that include the HIP runtime.

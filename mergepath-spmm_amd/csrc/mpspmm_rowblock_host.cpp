@@ -130,17 +130,41 @@ void count_block(const int *rp, const int *ci, const ColumnMap &cm, int r0, int 
 
 }  // namespace
 
-int default_steps(int n, long long nnz, int table_rows)
+int default_steps(int n, long long nnz, int table_rows, int num_blocks, const long long *table_nnz, int tables)
 {
-    // Measured on MI355X with power-law graphs of 233,000 to 500,000 rows and 260 to 490 nonzeros per
-    // row: 16 to 24 steps run within 2 % of each other (more steps put more nonzeros on the LDS path,
-    // but every step costs two barriers, a table load per workgroup and more padded windows); 16 makes
-    // the smallest plan.  Never more table slots than columns.
+    // table_nnz[k]: nonzeros in the columns that a (k + 1)-th table would serve (ranks k H .. (k + 1) H - 1 by
+    // nonzero count), for k < tables.  Two things ask for steps, and the larger one decides.
+    // (1) The range of X that a step gathers through L2 should stay in the 4 MiB L2 of an XCD: 5 MiB of X per step
+    //     where the columns are skewed (the busy part of a range stays), 3 MiB where they are not.
+    // (2) Tables: every step puts another H columns into LDS, and costs a block two barriers, a table load and some
+    //     padded windows (about 5 us on MI355X).  A block wants about 28,000 nonzeros per step, and a table is
+    //     worth its step while it serves 1 % of the nonzeros.
+    // Measured on MI355X (ms per product at 2 / 3 / 4 / 6 / 8 / 12 / 16 steps; in brackets what this rule picks):
+    //   power law,   232,965 rows x  32 per row: .057 .055 .057 .066 .077 .090  -       (3)
+    //   power law,   232,965 rows x  64:         .095 .083 .081 .086 .098 .117 .142     (3)
+    //   power law,   232,965 rows x 128:         .175 .151 .148 .145 .149 .163 .188     (4)
+    //   power law,   232,965 rows x 200:         .271 .235 .224 .212 .210 .220 .235     (7)
+    //   power law,   232,965 rows x 492:         13 to 18 steps within 1.5 % of each other (16)
+    //   power law,   500,000 rows x  64:         .280 .245 .231 .226 .232 .257 .301     (7)
+    //   power law,   500,000 rows x 200:         .864 .712 .629 .560 .546 .546 .547     (7)
+    //   power law, 1,000,000 rows x  64:         .721 .662 .635 .604 .577 .573 .636     (13)
+    //   power law, 1,000,000 rows x 128:         1.45 1.31 1.21 1.12 1.06 1.04 1.01     (13)
+    //   uniform,     232,965 rows x 100 (2, 3, 4, 6, 10, 13 steps): .220 .164 .151 .148 .159 .167   (5)
+    //   uniform,     232,965 rows x 300:                            .610 .480 .418 .414 .415 .419   (5)
+    //   uniform,     500,000 rows x  64:                            .448 .389 .339 .283 .280 .296   (11)
+    //   uniform,   1,000,000 rows x 100:                            1.64 1.49 1.37 1.19 .946 .921   (21)
+    // Never more table slots than columns.
     if (table_rows < 1) table_rows = 1;
-    long long t = 16;
+    if (num_blocks < 1) num_blocks = 1;
+    const bool skewed = tables > 0 && nnz > 0 && (double)table_nnz[0] >= 0.05 * (double)nnz;
+    const long long per_step = skewed ? (5ll << 20) : (3ll << 20);
+    const long long for_l2 = ((long long)n * 64 + per_step - 1) / per_step;
+    long long for_tables = (nnz / num_blocks + 14000) / 28000;
+    if (for_tables > tables) for_tables = tables;
+    while (for_tables > 0 && (double)table_nnz[for_tables - 1] < 0.01 * (double)nnz) --for_tables;
+    long long t = std::min<long long>(std::max(for_tables, for_l2), 32);
     const long long most = ((long long)n + table_rows - 1) / table_rows;
     if (t > most) t = most;
-    (void)nnz;
     return (int)std::max<long long>(t, 1);
 }
 
@@ -165,18 +189,39 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     if (cap_limit < 4) return MPS_ERR_INVALID_ARG;
     int cap = bp.block_rows > 0 ? std::min(bp.block_rows, cap_limit) : cap_limit;
     if (cap < 1) cap = 1;
-    for (int m = 1;; ++m) {
+    // Workgroups run one to a CU, so num_cus blocks of equal work are best; more rounds cost every block its steps
+    // again (a step is worth about 5,200 nonzeros of a block's time).  Where the row limit leaves the blocks of the
+    // first round that fits unequal (R-MAT, 2^18 rows in 256 blocks of exactly 1,024: the first block has 11 % of
+    // the nonzeros: 0.85 ms a product, 0.106 ms with 512 blocks), further rounds are tried: the blocks then start in
+    // order of their index as CUs come free, and a product takes about the mean work of a CU plus half of the
+    // largest block; a single round takes what its largest block takes.
+    const long long steps_guess = bp.steps > 0 ? bp.steps : std::max<long long>(1, ((long long)n * 64 + (5ll << 20) - 1) / (5ll << 20));
+    const long long block_fixed = steps_guess * 5200;
+    long long longest_row = 0;
+    for (int r = 0; r < n; ++r) longest_row = std::max<long long>(longest_row, (long long)rp[r + 1] - rp[r]);
+    long long best_cost = -1, best_target = 0;
+    for (int m = 1, tried = 0; tried < 6; ++m) {
         const long long most = (long long)num_cus * m;
         if (((long long)n + cap - 1) / cap > most) continue;
         long long lo = std::max<long long>(1, ((long long)nnz + most - 1) / most), hi = std::max<long long>(nnz, 1);
+        const long long even = lo;
         if (greedy_blocks(rp, n, cap, hi, nullptr) > most) continue;  // cannot happen: rows alone fit
         while (lo < hi) {
             const long long mid = lo + (hi - lo) / 2;
             if (greedy_blocks(rp, n, cap, mid, nullptr) <= most) hi = mid; else lo = mid + 1;
         }
-        greedy_blocks(rp, n, cap, lo, &L.block_row);
-        break;
+        const long long largest = std::max(lo, longest_row);  // a single row may be longer than the target
+        const bool equal = largest <= even + even / 16;
+        const long long cost = equal || m == 1 ? m * (largest + block_fixed)
+                                               : ((long long)nnz + most * block_fixed) / num_cus + (largest + block_fixed) / 2;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best_target = lo;
+        }
+        if (equal) break;  // more rounds of equal blocks only cost more
+        ++tried;
     }
+    greedy_blocks(rp, n, cap, best_target, &L.block_row);
     L.num_blocks = (int)L.block_row.size() - 1;
     int most_rows = 1;
     for (int b = 0; b < L.num_blocks; ++b) most_rows = std::max(most_rows, L.block_row[b + 1] - L.block_row[b]);
@@ -185,20 +230,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     // ---- 2. table size, steps
     int H = bp.table_rows > 0 ? bp.table_rows : std::min(kMaxTableRows, budget_rows - L.acc_rows);
     if (H > kMaxTableRows) H = kMaxTableRows;
-    int T = bp.steps > 0 ? bp.steps : default_steps(n, nnz, H);
-    if (T > 4096) T = 4096;
-    if (bp.table_rows <= 0) {
-        // no more slots than columns to put in them
-        const int need = (n + T - 1) / T;
-        if (H > need) H = need;
-        H = (H + 3) / 4 * 4;
-    }
-    if (H < 1 || (long long)(H + L.acc_rows) * 64 + kSlotBytes > kLdsBytes) return MPS_ERR_INVALID_ARG;
-    L.table_rows = H;
-    L.steps = T;
-    L.hot_bits = bits_for(H > 1 ? H - 1 : 1);
-
-    // ---- 3. nonzeros per column; hot columns by rank, cold columns by id range
+    // ---- 3. nonzeros per column; the steps; hot columns by rank, cold columns by id range
     std::vector<std::atomic<int>> deg((size_t)n);
     for (auto &d : deg) d.store(0, std::memory_order_relaxed);
     parallel_for(nnz, 1 << 20, [&](int64_t a, int64_t b) {
@@ -209,11 +241,57 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     cand.reserve((size_t)n);
     for (int c = 0; c < n; ++c)
         if (d_of(c) > 0) cand.push_back(c);
-    const size_t R = std::min<size_t>((size_t)T * H, cand.size());
     auto hotter = [&](int a, int b) {
         const int da = d_of(a), db = d_of(b);
         return da != db ? da > db : a < b;
     };
+    int T = bp.steps;
+    if (T <= 0) {
+        // what every further table would serve, for as many tables as a plan may get
+        constexpr int kMostTables = 32;
+        const size_t top = std::min<size_t>((size_t)kMostTables * H, cand.size());
+        if (top < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)top, cand.end(), hotter);
+        std::sort(cand.begin(), cand.begin() + (long)top, hotter);
+        long long table_nnz[kMostTables] = {0};
+        for (size_t k = 0; k < top; ++k) table_nnz[k / (size_t)H] += d_of(cand[k]);
+        T = default_steps(n, nnz, H, L.num_blocks, table_nnz, (int)((top + (size_t)H - 1) / (size_t)H));
+    }
+    if (T > 4096) T = 4096;
+    if ((long long)nnz < bp.min_step_nnz * L.num_blocks * T) return kNotWorthwhile;
+    if (bp.max_local_share < 1.0 && nnz > 0) {
+        // Columns near the diagonal (banded, block-diagonal): a block finds its nonzeros in one or two column
+        // ranges of its own and idles through the other steps, while a plan without steps finds such an X in L2
+        // anyway.  Share of the nonzeros in each block's busiest of R equal column ranges, beyond what the busiest
+        // range has of the whole matrix (which is skew, not locality).
+        const int R = std::max(T, 4);
+        std::vector<std::atomic<long long>> range_nnz((size_t)R);
+        for (auto &c : range_nnz) c.store(0, std::memory_order_relaxed);
+        std::atomic<long long> own{0};
+        parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
+            std::vector<long long> cnt((size_t)R);
+            for (int64_t b = b0; b < b1; ++b) {
+                std::fill(cnt.begin(), cnt.end(), 0);
+                for (int e = rp[L.block_row[(size_t)b]]; e < rp[L.block_row[(size_t)b + 1]]; ++e)
+                    ++cnt[(size_t)((long long)ci[e] * R / n)];
+                own.fetch_add(*std::max_element(cnt.begin(), cnt.end()), std::memory_order_relaxed);
+                for (int r = 0; r < R; ++r) range_nnz[(size_t)r].fetch_add(cnt[(size_t)r], std::memory_order_relaxed);
+            }
+        });
+        long long busiest = 0;
+        for (auto &c : range_nnz) busiest = std::max(busiest, c.load(std::memory_order_relaxed));
+        if ((double)(own.load() - busiest) > bp.max_local_share * (double)nnz) return kNotWorthwhile;
+    }
+    if (bp.table_rows <= 0) {
+        // no more slots than columns to put in them
+        const int need = (n + T - 1) / T;
+        if (H > need) H = need;
+        H = (H + 3) / 4 * 4;
+    }
+    if (H < 1 || (long long)(H + L.acc_rows) * 64 + kSlotBytes > kLdsBytes) return MPS_ERR_INVALID_ARG;
+    L.table_rows = H;
+    L.steps = T;
+    L.hot_bits = bits_for(H > 1 ? H - 1 : 1);
+    const size_t R = std::min<size_t>((size_t)T * H, cand.size());
     if (R < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)R, cand.end(), hotter);
     std::sort(cand.begin(), cand.begin() + (long)R, hotter);
     ColumnMap cm;
@@ -229,7 +307,6 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         L.hot_cols[(size_t)t * H + slot] = c;
         L.hot_nnz += d_of(c);
     }
-    if ((double)L.hot_nnz < bp.min_hot_share * (double)nnz) return kNotWorthwhile;
     {
         const long long cold_total = (long long)nnz - L.hot_nnz;
         long long cum = 0;

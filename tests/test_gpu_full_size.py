@@ -118,13 +118,15 @@ def test_power_law_config_full_size(pkg, orc, dev):
 @pytest.mark.parametrize("spec,big_slabs", [("chunglu:n=1000000,nnz=60000000,gamma=2.1,dmax=30000", True),
                                             ("er:n=1000000,deg=60", False)])
 def test_slab_size_follows_the_skew_of_the_matrix(pkg, orc, dev, spec, big_slabs):
-    """X of 64 MB: a power-law matrix gets slabs far beyond the L2 (its popular columns stay
-    cached), a uniform one slabs of at most 6 MiB; both plans give the right product."""
+    """X of 64 MB: among the slab plans a power-law matrix gets slabs far beyond the L2 (its popular
+    columns stay cached), a uniform one slabs of at most 6 MiB; both plans give the right product.
+    Left to choose, the library gives the power-law matrix a row-block plan (13 steps: 4,500 nonzeros
+    per block and step), but not the uniform one, whose 21 steps of 3 MiB leave a block 2,800."""
     K = 16
     rp, ci, val, X = workload(pkg, spec, K)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
-    plan = pkg.spmm.Plan(csr, K)
+    plan = pkg.spmm.Plan(csr, K, rowblock="off" if big_slabs else "auto")
     i = plan.info
     slab_bytes = i.slab_cols * K * 4
     assert i.num_slabs > 1 and i.hot_rows == 0
@@ -134,6 +136,11 @@ def test_slab_size_follows_the_skew_of_the_matrix(pkg, orc, dev, spec, big_slabs
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
     plan.close()
+    if big_slabs:
+        auto = pkg.spmm.Plan(csr, K)
+        assert auto.info.rowblock_steps == 13
+        check_fp32(auto.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+        auto.close()
 
 
 @pytest.mark.parametrize("K", [16, 32, 64, 128, 256])

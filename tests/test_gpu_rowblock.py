@@ -203,20 +203,53 @@ def test_rowblock_plan_power_law_graph(pkg, orc, dev):
     assert torch.equal(Y, Y2)
 
 
-def test_uniform_matrix_falls_back_to_slabs(pkg, orc, dev):
-    # long rows and a large X, but columns used evenly: LDS tables would serve a tenth of the nonzeros,
-    # so the library builds the column-slab plan instead (and a forced row-block plan still works)
+def test_uniform_matrix_gets_a_rowblock_plan_too(pkg, orc, dev):
+    # columns used evenly: the LDS tables serve a twentieth of the nonzeros, but a block still has 20,000
+    # nonzeros per step and the gathers of a step stay in L2, so the library builds the row-block plan
     rp, ci, _ = pkg.graphs.generate("er:n=200000,deg=130", seed=5)
     n, nnz = rp.size - 1, ci.size
-    assert nnz >= 128 * n
     val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
     X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
     plan = pkg.spmm.Plan(csr, 16)
-    assert plan.info.rowblock_steps == 0 and plan.info.num_slabs > 1
+    i = plan.info
+    assert i.rowblock_steps == 5 and i.hot_nnz < 0.25 * nnz  # 12.8 MB of X at 3 MiB a step
+    assert nnz >= 4000 * i.rowblock_blocks * i.rowblock_steps
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(plan.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    slabs = pkg.spmm.Plan(csr, 16, rowblock="off")
+    assert slabs.info.rowblock_steps == 0 and slabs.info.num_slabs > 1
+    check_fp32(slabs.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+
+
+@pytest.mark.parametrize("kind", ["short_rows", "banded"])
+def test_matrices_that_stay_with_the_slab_plans(pkg, orc, dev, kind):
+    """No row-block plan unless asked for: where a block would have fewer than 4,000 nonzeros per step
+    (500,000 rows of 16), and where the columns stay near the diagonal (a band of 2,000 columns either
+    side: every block would idle through the steps of the other column ranges)."""
+    rng = np.random.default_rng(3)
+    if kind == "short_rows":
+        rp, ci, _ = pkg.graphs.generate("chunglu:n=500000,nnz=8000000,gamma=2.1,dmax=9000", seed=5)
+    else:
+        n, deg, w = 120000, 48, 2000
+        c = np.arange(n, dtype=np.int64)[:, None] + rng.integers(-w, w + 1, size=(n, deg))
+        c = np.clip(c, 0, n - 1)
+        c.sort(axis=1)
+        keep = np.ones(c.shape, dtype=bool)
+        keep[:, 1:] = c[:, 1:] != c[:, :-1]
+        rp = np.zeros(n + 1, dtype=np.int32)
+        rp[1:] = np.cumsum(keep.sum(axis=1))
+        ci = c[keep].astype(np.int32)
+    n, nnz = rp.size - 1, ci.size
+    val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
+    X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16)
+    assert plan.info.rowblock_steps == 0
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     check_fp32(plan.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
     forced = pkg.spmm.Plan(csr, 16, rowblock="force")
-    assert forced.info.rowblock_steps > 0 and forced.info.hot_nnz < 0.25 * nnz
+    assert forced.info.rowblock_steps > 0
     check_fp32(forced.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
