@@ -212,6 +212,43 @@ def test_blocks_balance_nonzeros(pkg):
     assert per_block.max() <= ci.size / 16 + np.diff(rp).max()
 
 
+def test_more_rounds_of_blocks_where_one_round_is_unequal(pkg):
+    """16 x 1,024 rows at 16 blocks per round: one round means blocks of exactly 1,024 rows, and the first of them
+    would hold seven eighths of the nonzeros.  The builder takes a second round instead."""
+    rng = np.random.default_rng(6)
+    n = 16 * 1024
+    deg = np.where(np.arange(n) < 1024, 200, 2)
+    rp = np.zeros(n + 1, dtype=np.int32)
+    rp[1:] = np.cumsum(deg)
+    ci = np.concatenate([np.sort(rng.choice(n, size=d, replace=False)) for d in deg]).astype(np.int32)
+    val = np.ones(ci.size, dtype=np.float32)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=1, table_rows=64, blocks_per_round=16, keep_sources=False)
+    brow = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
+    per_block = rp[brow[1:]] - rp[brow[:-1]]
+    assert 16 < brow.size - 1 <= 32 and per_block.max() < ci.size / 10
+    assert (np.diff(brow) <= 1024).all()
+    # rows that one round does hold in equal blocks stay in one round
+    deg2 = np.full(n // 2, 20)
+    rp2 = np.zeros(n // 2 + 1, dtype=np.int32)
+    rp2[1:] = np.cumsum(deg2)
+    ci2 = np.concatenate([np.sort(rng.choice(n // 2, size=20, replace=False)) for _ in deg2]).astype(np.int32)
+    lay2 = pkg.spmm.RowBlockLayout(rp2, ci2, np.ones(ci2.size, dtype=np.float32), steps=1, table_rows=64, blocks_per_round=16,
+                                   keep_sources=False)
+    assert lay2.info.rowblock_blocks == 16
+
+
+@pytest.mark.parametrize("spec,steps,why", [
+    ("er:n=120000,deg=20", 3, "7.7 MB of X, columns used evenly: 3 MiB a step"),
+    ("chunglu:n=120000,nnz=2400000,gamma=2.1,dmax=4000", 2, "7.7 MB of X, skewed columns: 5 MiB a step"),
+    ("chunglu:n=30000,nnz=16000000,gamma=2.1,dmax=6000", 2, "X fits one step, but a block has 62,500 nonzeros: a second table"),
+    ("er:n=190000,deg=190", 4, "141,000 nonzeros per block ask for 5 tables, but a table serves 0.9 % of them: 12.2 MB of X at 3 MiB a step"),
+])
+def test_steps_follow_the_size_of_x_the_work_and_the_skew(pkg, spec, steps, why):
+    rp, ci, _ = pkg.graphs.generate(spec, seed=4)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, np.ones(ci.size, dtype=np.float32), keep_sources=False)
+    assert lay.info.rowblock_steps == steps, why
+
+
 def test_rejects_what_it_is_not_built_for(pkg):
     rp = np.array([0, 1, 2], dtype=np.int32)
     ci = np.array([0, 1], dtype=np.int32)
