@@ -1214,35 +1214,36 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     return MPS_OK;
 }
 
-// Row-block plan or not.  Forced: yes.  Otherwise only for what the kernel is built for (fp32,
-// K = 16) and where it was measured to win on MI355X against the slab plans.  What decides is
-// the work of a block per step: every step costs a block two barriers, a table load and some
-// padded windows, about 5 us, which some 4,000 nonzeros pay for (kMinStepNnz).  Whether the
-// columns are skewed matters little: the gathers of a step stay in L2 either way.  Measured
-// (ms per product, row-block against slab plan; nonzeros per block and step in brackets):
-//   power law 232,965 rows x 16 per row .042/.058 (7.3k), x 128 .148/.231 (29k);
-//   100,000 x 16 .028/.031 (3.1k), x 64 .042/.067 (12k); 60,000 x 16 .024/.022 (3.8k),
-//   x 32 .025/.027 (7.5k); 500,000 x 16 .117/.109 (2.2k), x 32 .152/.186 (4.5k);
-//   1,000,000 x 32 .458/.409 (2.4k), x 64 .596/.674 (4.8k); 2,000,000 x 100 2.28/2.13 (3.8k);
-//   uniform 232,965 x 32 .069/.119 (5.8k), 500,000 x 64 .272/.336 (5.7k),
-//   1,000,000 x 100 .92/1.09 (4.4k); R-MAT scale 20, 16 per row .78/.177 (1.2k).
-// The steps are known only once the builder has counted the columns, so the builder decides
-// (kNotWorthwhile); here only what no step count can save is turned away, before the matrix
-// is copied to the host: with the fewest steps a plan could get (5 MiB of X per step).
-// A matrix whose columns stay near the diagonal is the slab plans' (banded, 233,000 rows x 64 within
-// 2,000 columns of the diagonal: .160/.114; 500,000 x 64 within 3,000: .427/.287): the blocks idle
-// through the steps whose column range they do not touch (kMaxLocalShare, measured by the builder).
-constexpr long long kMinStepNnz = 4000;
+// Row-block plan or not.  Forced: yes.  Otherwise for what the kernel is built for (fp32, K = 16,
+// up to 2^22 rows), with two kinds of matrices left to the slab plans, as measured on MI355X (ms
+// per product, row-block with the builder's choice of steps against slab plan):
+//   power law 232,965 rows x 16 per row .041/.058, x 64 .083/.146, x 492 .44/.58;
+//   100,000 x 16 .027/.029; 60,000 x 16 .017/.020; 500,000 x 16 .089/.112, x 64 .226/.303;
+//   1,000,000 x 16 .199/.222, x 32 .330/.410, x 60 .577/.629; 2,000,000 x 100 2.0-2.3/2.08;
+//   uniform 232,965 x 32 .069/.120; 500,000 x 64 .280/.336; 1,000,000 x 60 .648/.834;
+//   R-MAT scale 16 to 21, 16 per row: .018/.029, .046/.059, .184/.200, .424/.492; scale 18 x 55 .105/.157;
+//   uniform x 8 per row: 4,096 rows .012/.014, 20,000 .013/.015, 60,000 .016/.018, 200,000 .034/.034,
+//   1,000,000 .178/.174, 2,000,000 .363/.343; 4,000,000 x 4: .406/.376.
+// (1) Many short rows: a window of the streams holds four nonzeros of one row and step, and the
+//     slab plans' sliced stream does as well on rows of 8: below 12 nonzeros per row on average
+//     and beyond 2^18 rows the slab plan it is.
+// (2) Columns near the diagonal (block-diagonal 416,349 x 5: .029/.026; banded 233,000 x 64 within
+//     2,000 columns: .160/.114; 500,000 x 64 within 3,000: .427/.287): the blocks idle through the
+//     steps whose column range they do not touch, and a slab plan finds such an X in L2 anyway.
+//     The builder measures that once it has the matrix on the host (kMaxLocalShare) and says
+//     kNotWorthwhile.
 constexpr double kMaxLocalShare = 0.25;
-bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, unsigned flags)
+bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, int cost, int tpw, unsigned flags)
 {
     if (flags & MPS_PLAN_FORCE_ROWBLOCK) return true;
     if (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT)) return false;
-    if (elem_bytes != 4 || K != 16 || n_rows < 1) return false;
+    if (elem_bytes != 4 || K != 16 || n_rows < 1 || nnz < 1) return false;
     if (n_rows > (1 << 22)) return false;
-    const long long blocks = (((long long)n_rows + 1023) / 1024 + 255) / 256 * 256;
-    const long long fewest_steps = std::max<long long>(1, ((long long)n_rows * 64 + (5ll << 20) - 1) / (5ll << 20));
-    return (long long)nnz >= kMinStepNnz * blocks * fewest_steps;
+    // a caller that names a cost or partitions per wavefront of its own is tuning a slab plan: row-block plans have neither
+    int default_cost = 0, max_tpw = 0;
+    if (mps_default_cost(n_rows, nnz, K, elem_bytes, &default_cost) != MPS_OK || cost != default_cost) return false;
+    if (mps_max_threads_per_wave(K, elem_bytes, &max_tpw) != MPS_OK || (tpw != 0 && tpw != max_tpw)) return false;
+    return n_rows <= (1 << 18) || (long long)nnz >= 12LL * n_rows;
 }
 
 }  // namespace
@@ -1299,7 +1300,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     pl->cost = cost;
     pl->keep_sources = !(flags & MPS_PLAN_NO_SOURCES);
     pl->weights = opt.degree_weights;
-    if (rowblock_wanted(n_rows, nnz, K, elem_bytes, flags)) {
+    if (rowblock_wanted(n_rows, nnz, K, elem_bytes, cost, tpw, flags)) {
         if (elem_bytes != 4 || K != 16 || n_rows < 1) {
             plan_free(pl);
             return MPS_ERR_UNSUPPORTED;
@@ -1316,7 +1317,6 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.block_rows = opt.rowblock_block_rows;
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
-        bp.min_step_nnz = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 0 : kMinStepNnz;
         bp.max_local_share = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 1.0 : kMaxLocalShare;
         int rc = mps_rb::create(d_row_ptr, d_col_idx, static_cast<const float *>(d_val), n_rows, nnz, K, bp,
                                 static_cast<hipStream_t>(stream), &pl->rb);
@@ -1330,7 +1330,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
             plan_free(pl);
             return rc;
         }
-        // too little work per block and step, or columns near the diagonal: the slab plan below
+        // columns near the diagonal: the slab plan below
     }
     int rc;
     try {

@@ -108,11 +108,10 @@ struct BuildParams {
     int block_rows = 0;  // 0 = choose; otherwise the most rows a block may hold
     int num_cus = 256;
     bool keep_src = true;
-    long long min_step_nnz = 0;  // give up (kNotWorthwhile) when a block has fewer nonzeros per step on average
     double max_local_share = 1.0;  // give up when the blocks find a larger share of the nonzeros in column ranges of their own
 };
 
-constexpr int kNotWorthwhile = -1;  // build_layout: min_step_nnz or max_local_share not met
+constexpr int kNotWorthwhile = -1;  // build_layout: max_local_share not met
 
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,

@@ -133,12 +133,13 @@ void count_block(const int *rp, const int *ci, const ColumnMap &cm, int r0, int 
 int default_steps(int n, long long nnz, int table_rows, int num_blocks, const long long *table_nnz, int tables)
 {
     // table_nnz[k]: nonzeros in the columns that a (k + 1)-th table would serve (ranks k H .. (k + 1) H - 1 by
-    // nonzero count), for k < tables.  Two things ask for steps, and the larger one decides.
+    // nonzero count), for k < tables.  Every step costs a block two barriers, a table load and some padded windows
+    // (about 3 us on MI355X, the time of 3,000 nonzeros).  Two things ask for steps, and the larger one decides.
     // (1) The range of X that a step gathers through L2 should stay in the 4 MiB L2 of an XCD: 5 MiB of X per step
-    //     where the columns are skewed (the busy part of a range stays), 3 MiB where they are not.
-    // (2) Tables: every step puts another H columns into LDS, and costs a block two barriers, a table load and some
-    //     padded windows (about 5 us on MI355X).  A block wants about 28,000 nonzeros per step, and a table is
-    //     worth its step while it serves 1 % of the nonzeros.
+    //     where the columns are skewed (the busy part of a range stays), 3 MiB where they are not - but no more
+    //     steps than leave a block 6,000 nonzeros each: below that the steps cost more than the L2 misses.
+    // (2) Tables: every step puts another H columns into LDS.  A block wants about 28,000 nonzeros per step, and a
+    //     table is worth its step while it serves 1 % of the nonzeros.
     // Measured on MI355X (ms per product at 2 / 3 / 4 / 6 / 8 / 12 / 16 steps; in brackets what this rule picks):
     //   power law,   232,965 rows x  32 per row: .057 .055 .057 .066 .077 .090  -       (3)
     //   power law,   232,965 rows x  64:         .095 .083 .081 .086 .098 .117 .142     (3)
@@ -147,18 +148,25 @@ int default_steps(int n, long long nnz, int table_rows, int num_blocks, const lo
     //   power law,   232,965 rows x 492:         13 to 18 steps within 1.5 % of each other (16)
     //   power law,   500,000 rows x  64:         .280 .245 .231 .226 .232 .257 .301     (7)
     //   power law,   500,000 rows x 200:         .864 .712 .629 .560 .546 .546 .547     (7)
-    //   power law, 1,000,000 rows x  64:         .721 .662 .635 .604 .577 .573 .636     (13)
+    //   power law, 1,000,000 rows x  64:         .721 .662 .635 .604 .577 .573 .636     (10)
     //   power law, 1,000,000 rows x 128:         1.45 1.31 1.21 1.12 1.06 1.04 1.01     (13)
+    //   power law, 1,000,000 rows x  32 (2, 4, 6, 8, 13 steps): .361 .336 .330 .351 .457                    (5)
+    //   power law, 1,000,000 rows x  16 (1, 2, 3, 4, 13 steps): .216 .202 .199 .203 .331                    (2)
+    //   power law,   500,000 rows x  16 (2, 4 steps):           .089 .096                                   (2)
+    //   R-MAT scale 20, 16 per row (1, 2, 3, 4, 6, 8, 13):      .184 .190 .190 .207 .247 .290 .378          (2)
+    //   R-MAT scale 18, 16 per row (1, 2, 4):                   .046 .053 .067                              (1)
     //   uniform,     232,965 rows x 100 (2, 3, 4, 6, 10, 13 steps): .220 .164 .151 .148 .159 .167   (5)
     //   uniform,     232,965 rows x 300:                            .610 .480 .418 .414 .415 .419   (5)
-    //   uniform,     500,000 rows x  64:                            .448 .389 .339 .283 .280 .296   (11)
-    //   uniform,   1,000,000 rows x 100:                            1.64 1.49 1.37 1.19 .946 .921   (21)
+    //   uniform,     500,000 rows x  64:                            .448 .389 .339 .283 .280 .296   (10)
+    //   uniform,   1,000,000 rows x 100:                            1.64 1.49 1.37 1.19 .946 .921   (16)
+    //   uniform,   1,000,000 rows x  60 (6, 10, 14, 21 steps):      .762 .648 .658 .795             (9)
     // Never more table slots than columns.
     if (table_rows < 1) table_rows = 1;
     if (num_blocks < 1) num_blocks = 1;
     const bool skewed = tables > 0 && nnz > 0 && (double)table_nnz[0] >= 0.05 * (double)nnz;
     const long long per_step = skewed ? (5ll << 20) : (3ll << 20);
-    const long long for_l2 = ((long long)n * 64 + per_step - 1) / per_step;
+    long long for_l2 = ((long long)n * 64 + per_step - 1) / per_step;
+    for_l2 = std::min(for_l2, nnz / num_blocks / 6000);
     long long for_tables = (nnz / num_blocks + 14000) / 28000;
     if (for_tables > tables) for_tables = tables;
     while (for_tables > 0 && (double)table_nnz[for_tables - 1] < 0.01 * (double)nnz) --for_tables;
@@ -189,18 +197,16 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     if (cap_limit < 4) return MPS_ERR_INVALID_ARG;
     int cap = bp.block_rows > 0 ? std::min(bp.block_rows, cap_limit) : cap_limit;
     if (cap < 1) cap = 1;
-    // Workgroups run one to a CU, so num_cus blocks of equal work are best; more rounds cost every block its steps
-    // again (a step is worth about 5,200 nonzeros of a block's time).  Where the row limit leaves the blocks of the
-    // first round that fits unequal (R-MAT, 2^18 rows in 256 blocks of exactly 1,024: the first block has 11 % of
-    // the nonzeros: 0.85 ms a product, 0.106 ms with 512 blocks), further rounds are tried: the blocks then start in
-    // order of their index as CUs come free, and a product takes about the mean work of a CU plus half of the
-    // largest block; a single round takes what its largest block takes.
-    const long long steps_guess = bp.steps > 0 ? bp.steps : std::max<long long>(1, ((long long)n * 64 + (5ll << 20) - 1) / (5ll << 20));
-    const long long block_fixed = steps_guess * 5200;
+    // Workgroups run one to a CU and start in order of their index as CUs come free.  As few rounds of num_cus
+    // blocks as the row limit allows are best (every further round costs about 5 us and 3 us per step: power law,
+    // 500,000 rows x 16, 2 steps: .089 / .103 / .111 ms with 512 / 768 / 1,024 blocks), unless the row limit leaves
+    // the blocks of that round far from equal: R-MAT of 2^18 rows in 256 blocks of exactly 1,024 has 11 % of the
+    // nonzeros in the first (0.85 ms a product, 0.105 with 512 blocks; 768: 0.136).  Then rounds are added until no
+    // block is more than half above its share, or the largest block is a single row.
     long long longest_row = 0;
     for (int r = 0; r < n; ++r) longest_row = std::max<long long>(longest_row, (long long)rp[r + 1] - rp[r]);
-    long long best_cost = -1, best_target = 0;
-    for (int m = 1, tried = 0; tried < 6; ++m) {
+    long long best_target = 0;
+    for (int m = 1, tried = 0; tried < 8; ++m) {
         const long long most = (long long)num_cus * m;
         if (((long long)n + cap - 1) / cap > most) continue;
         long long lo = std::max<long long>(1, ((long long)nnz + most - 1) / most), hi = std::max<long long>(nnz, 1);
@@ -210,15 +216,8 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             const long long mid = lo + (hi - lo) / 2;
             if (greedy_blocks(rp, n, cap, mid, nullptr) <= most) hi = mid; else lo = mid + 1;
         }
-        const long long largest = std::max(lo, longest_row);  // a single row may be longer than the target
-        const bool equal = largest <= even + even / 16;
-        const long long cost = equal || m == 1 ? m * (largest + block_fixed)
-                                               : ((long long)nnz + most * block_fixed) / num_cus + (largest + block_fixed) / 2;
-        if (best_cost < 0 || cost < best_cost) {
-            best_cost = cost;
-            best_target = lo;
-        }
-        if (equal) break;  // more rounds of equal blocks only cost more
+        best_target = lo;
+        if (lo <= even + even / 2 || lo <= longest_row) break;
         ++tried;
     }
     greedy_blocks(rp, n, cap, best_target, &L.block_row);
@@ -257,7 +256,6 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         T = default_steps(n, nnz, H, L.num_blocks, table_nnz, (int)((top + (size_t)H - 1) / (size_t)H));
     }
     if (T > 4096) T = 4096;
-    if ((long long)nnz < bp.min_step_nnz * L.num_blocks * T) return kNotWorthwhile;
     if (bp.max_local_share < 1.0 && nnz > 0) {
         // Columns near the diagonal (banded, block-diagonal): a block finds its nonzeros in one or two column
         // ranges of its own and idles through the other steps, while a plan without steps finds such an X in L2

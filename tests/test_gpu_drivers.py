@@ -61,8 +61,15 @@ def test_merge_path_driver(pkg, orc, graph_file, tmp_path):
         assert j["plan"] == ("--no-plan" not in extra) and (slabs > 1) == ("force" in extra)
         hot = extra[-2:] == ("--hot", "force")  # forced slabs are narrower than the LDS table: all columns hot
         assert (j["hot_rows"] > 0) == hot and ("hot columns: " in out) == hot
-        if not hot:  # with hot columns every segment is split on its own
-            assert j["P"] == orc.num_partitions(slabs * (rp.size - 1), ci.size, 32 if cost == "default" else cost)  # small graph: 32
+        # left to the library (the default cost, which is 32 for a graph this small, and a full wavefront), a matrix
+        # of this size gets a row-block plan, which has no partitions; a caller that names another cost, fewer threads
+        # per wave or a plan switch gets the slab plan it tunes
+        rowblock = cost in ("default", 32) and not extra
+        assert (j["rowblock_steps"] > 0) == rowblock and ("row blocks, " in out) == rowblock
+        if rowblock:
+            assert j["P"] == 0
+        elif not hot:  # with hot columns every segment is split on its own
+            assert j["P"] == orc.num_partitions(slabs * (rp.size - 1), ci.size, cost)
         assert abs(j["checksum"] - Y.astype(np.float64).sum()) <= 1e-6 * np.abs(Y).sum() + 1e-6
 
 

@@ -120,13 +120,13 @@ def test_power_law_config_full_size(pkg, orc, dev):
 def test_slab_size_follows_the_skew_of_the_matrix(pkg, orc, dev, spec, big_slabs):
     """X of 64 MB: among the slab plans a power-law matrix gets slabs far beyond the L2 (its popular
     columns stay cached), a uniform one slabs of at most 6 MiB; both plans give the right product.
-    Left to choose, the library gives the power-law matrix a row-block plan (13 steps: 4,500 nonzeros
-    per block and step), but not the uniform one, whose 21 steps of 3 MiB leave a block 2,800."""
+    Left to choose, the library gives both a row-block plan of 9 steps: the L2 asks for 13 and 21, but
+    a block has 58,600 nonzeros and a step wants 6,000."""
     K = 16
     rp, ci, val, X = workload(pkg, spec, K)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
-    plan = pkg.spmm.Plan(csr, K, rowblock="off" if big_slabs else "auto")
+    plan = pkg.spmm.Plan(csr, K, rowblock="off")
     i = plan.info
     slab_bytes = i.slab_cols * K * 4
     assert i.num_slabs > 1 and i.hot_rows == 0
@@ -136,11 +136,10 @@ def test_slab_size_follows_the_skew_of_the_matrix(pkg, orc, dev, spec, big_slabs
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
     plan.close()
-    if big_slabs:
-        auto = pkg.spmm.Plan(csr, K)
-        assert auto.info.rowblock_steps == 13
-        check_fp32(auto.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
-        auto.close()
+    auto = pkg.spmm.Plan(csr, K)
+    assert auto.info.rowblock_steps == 9 and auto.info.rowblock_blocks == 1024
+    check_fp32(auto.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    auto.close()
 
 
 @pytest.mark.parametrize("K", [16, 32, 64, 128, 256])
@@ -154,9 +153,18 @@ def test_rmat_config_full_size(pkg, orc, dev, K):
     plan = pkg.spmm.Plan(csr, K)
     # K = 64, X of 256 MiB (beyond the last-level cache): the 10 MiB of busiest columns stay plain gathers, the rest
     # is gathered with the streaming hint.  K = 128 and 256: 8-lane groups and one pass per 128 bytes of row pitch.
-    assert plan.info.num_slabs == 1 and (plan.info.resident_cols > 0) == (K == 64)
-    assert plan.info.resident_cols == 0 or plan.info.resident_nnz > 0.4 * ci.size
-    assert plan.info.threads_per_wave == (8 if K >= 128 else 64 // (K // 4)) and (K < 128 or plan.info.cost == 64)
+    if K == 16:
+        # a row-block plan: 1,280 blocks (1,024 blocks of 1,024 rows would put 6 % of the nonzeros into the first)
+        # of 12,600 nonzeros on average, which is worth 2 steps
+        assert plan.info.rowblock_steps == 2 and plan.info.rowblock_blocks == 1280
+        slabs = pkg.spmm.Plan(csr, K, rowblock="off")
+        assert slabs.info.rowblock_steps == 0 and slabs.info.num_slabs == 1 and slabs.info.threads_per_wave == 16
+        check_fp32(slabs.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+        slabs.close()
+    else:
+        assert plan.info.num_slabs == 1 and (plan.info.resident_cols > 0) == (K == 64)
+        assert plan.info.resident_cols == 0 or plan.info.resident_nnz > 0.4 * ci.size
+        assert plan.info.threads_per_wave == (8 if K >= 128 else 64 // (K // 4)) and (K < 128 or plan.info.cost == 64)
     Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     torch.cuda.synchronize()
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)

@@ -567,14 +567,15 @@ def test_plan_spmm_in_a_hip_graph(pkg, orc, dev):
                           dict(tiling="force", slab_bytes=4096 * K * 4, hot="force")),
                          # a row-block plan: gather kernel + main kernel
                          ("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", dict(rowblock="force", rowblock_steps=5)),
-                         ("er:n=4096,deg=8", dict())):
+                         # what the library picks by itself for this size: a row-block plan of one step
+                         ("er:n=4096,deg=8", dict()), ("er:n=4096,deg=8", dict(rowblock="off"))):
         rp, ci, _ = g.generate(spec, seed=8)
         n = rp.size - 1
         val = g.fill_uniform_f32(ci.size, 11, 0.0, 1.0)
         csr = make_csr(pkg, dev, rp, ci, val)
         plan = pkg.spmm.Plan(csr, K, **kwargs)
         assert (plan.info.hot_rows > 0) == (kwargs.get("hot") == "force")
-        assert (plan.info.rowblock_steps > 0) == (kwargs.get("rowblock") == "force")
+        assert (plan.info.rowblock_steps > 0) == (kwargs.get("rowblock") == "force" or not kwargs)
         X = torch.from_numpy(g.fill_uniform_f32(n * K, 13, -1.0, 1.0).reshape(n, K)).to(dev)
         Y = torch.full_like(X, float("nan"))
         eager = plan.spmm(X).clone()

@@ -214,7 +214,8 @@ def test_blocks_balance_nonzeros(pkg):
 
 def test_more_rounds_of_blocks_where_one_round_is_unequal(pkg):
     """16 x 1,024 rows at 16 blocks per round: one round means blocks of exactly 1,024 rows, and the first of them
-    would hold seven eighths of the nonzeros.  The builder takes a second round instead."""
+    would hold seven eighths of the nonzeros.  The builder adds rounds until no block is more than half above its
+    share (two rounds: 15 blocks are full of short rows, which leaves 17 for the long ones, 1.6 times the share)."""
     rng = np.random.default_rng(6)
     n = 16 * 1024
     deg = np.where(np.arange(n) < 1024, 200, 2)
@@ -225,7 +226,7 @@ def test_more_rounds_of_blocks_where_one_round_is_unequal(pkg):
     lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=1, table_rows=64, blocks_per_round=16, keep_sources=False)
     brow = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
     per_block = rp[brow[1:]] - rp[brow[:-1]]
-    assert 16 < brow.size - 1 <= 32 and per_block.max() < ci.size / 10
+    assert 32 < brow.size - 1 <= 48 and per_block.max() <= 1.5 * ci.size / 48
     assert (np.diff(brow) <= 1024).all()
     # rows that one round does hold in equal blocks stay in one round
     deg2 = np.full(n // 2, 20)
@@ -238,8 +239,9 @@ def test_more_rounds_of_blocks_where_one_round_is_unequal(pkg):
 
 
 @pytest.mark.parametrize("spec,steps,why", [
-    ("er:n=120000,deg=20", 3, "7.7 MB of X, columns used evenly: 3 MiB a step"),
-    ("chunglu:n=120000,nnz=2400000,gamma=2.1,dmax=4000", 2, "7.7 MB of X, skewed columns: 5 MiB a step"),
+    ("er:n=120000,deg=60", 3, "7.7 MB of X, columns used evenly: 3 MiB a step"),
+    ("chunglu:n=120000,nnz=7200000,gamma=2.1,dmax=4000", 2, "7.7 MB of X, skewed columns: 5 MiB a step"),
+    ("er:n=120000,deg=20", 1, "9,400 nonzeros per block: a second step would leave fewer than 6,000 each"),
     ("chunglu:n=30000,nnz=16000000,gamma=2.1,dmax=6000", 2, "X fits one step, but a block has 62,500 nonzeros: a second table"),
     ("er:n=190000,deg=190", 4, "141,000 nonzeros per block ask for 5 tables, but a table serves 0.9 % of them: 12.2 MB of X at 3 MiB a step"),
 ])
