@@ -326,8 +326,8 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  *
  * Row-block plans (fp32, K = 16: a row of X is 64 bytes, half a cache line, so
  * every gather through L2 costs a full request for half its payload).  For
- * matrices with enough nonzeros per row block (see below) the plan is built
- * differently: rows are cut into contiguous blocks of about equal
+ * most matrices of this shape (see below) the plan is built differently:
+ * rows are cut into contiguous blocks of about equal
  * nonzero count, one per 1,024-thread workgroup, whose output rows are summed
  * in LDS and written to Y once -- no partial rows, no carry-out records, one
  * kernel.  Columns are dealt to `steps` steps: the steps * table_rows columns
@@ -337,11 +337,15 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  * and a wavefront's hot and cold nonzeros are each dealt evenly to its 16
  * lane-groups.  Results are deterministic.  The layout is built on the host
  * (the CSR arrays are copied back once, at creation).  mps_plan_create picks
- * this kind of plan by itself where it was measured to win: up to 2^22 rows,
- * at least 4,000 nonzeros per block and step (with `steps` chosen from the
- * size of X and the column histogram), and columns that do not stay near the
- * diagonal (banded and block-diagonal matrices keep the slab plans);
- * MPS_PLAN_NO_ROWBLOCK / MPS_PLAN_FORCE_ROWBLOCK override that.
+ * this kind of plan by itself where it was measured to win: fp32, K = 16, up
+ * to 2^22 rows, except for matrices with many short rows (fewer than 12
+ * nonzeros per row on average and more than 2^18 rows) and matrices whose
+ * columns stay near the diagonal (banded, block-diagonal), which keep the
+ * slab plans.  `steps` and the number of blocks follow from the size of X,
+ * the nonzeros per block and the column histogram.  A caller that passes a
+ * cost other than mps_default_cost's, a tpw other than 0 or the maximum, or
+ * one of the tiling / hot-column flags is tuning a slab plan and gets one;
+ * MPS_PLAN_NO_ROWBLOCK / MPS_PLAN_FORCE_ROWBLOCK override the choice.
  *
  * mps_tile_shape: the slab count and width mps_plan_create chooses for an X
  *   of n_rows x K elements (slab_bytes = 0: slabs of 3 or 6 MiB, whichever
