@@ -337,11 +337,12 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  * and a wavefront's hot and cold nonzeros are each dealt evenly to its 16
  * lane-groups.  Results are deterministic.  The layout is built on the host
  * (the CSR arrays are copied back once, at creation).  mps_plan_create picks
- * this kind of plan by itself where it was measured to win: fp32, K = 16, up
- * to 2^22 rows, except for matrices with many short rows (fewer than 12
- * nonzeros per row on average and more than 2^18 rows) and matrices whose
- * columns stay near the diagonal (banded, block-diagonal), which keep the
- * slab plans.  `steps` and the number of blocks follow from the size of X,
+ * this kind of plan by itself where it was measured to win: fp32, K = 16, X
+ * below 192 MiB (3.1 M rows), except for matrices with many short rows and no
+ * busy columns (fewer than 12 nonzeros per row on average, more than 2^18
+ * rows), matrices whose columns stay near the diagonal (banded,
+ * block-diagonal) and matrices with one row far longer than a CU's share of
+ * the nonzeros, which keep the slab plans.  `steps` and the number of blocks follow from the size of X,
  * the nonzeros per block and the column histogram.  A caller that passes a
  * cost other than mps_default_cost's, a tpw other than 0 or the maximum, or
  * one of the tiling / hot-column flags is tuning a slab plan and gets one;

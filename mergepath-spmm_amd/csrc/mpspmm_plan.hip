@@ -1214,36 +1214,41 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
     return MPS_OK;
 }
 
-// Row-block plan or not.  Forced: yes.  Otherwise for what the kernel is built for (fp32, K = 16,
-// up to 2^22 rows), with two kinds of matrices left to the slab plans, as measured on MI355X (ms
-// per product, row-block with the builder's choice of steps against slab plan):
+// Row-block plan or not.  Forced: yes.  Otherwise for what the kernel is built for (fp32, K = 16)
+// while X is smaller than what the slab plans treat with resident columns (R-MAT scale 22, X of
+// 268 MB: 1.11 against 0.95 ms), with three kinds of matrices left to the slab plans, which the
+// builder recognises once it has the matrix on the host (it then says kNotWorthwhile).  Measured on
+// MI355X, ms per product, row-block with the builder's choice of steps against slab plan:
 //   power law 232,965 rows x 16 per row .041/.058, x 64 .083/.146, x 492 .44/.58;
 //   100,000 x 16 .027/.029; 60,000 x 16 .017/.020; 500,000 x 16 .089/.112, x 64 .226/.303;
 //   1,000,000 x 16 .199/.222, x 32 .330/.410, x 60 .577/.629; 2,000,000 x 100 2.0-2.3/2.08;
 //   uniform 232,965 x 32 .069/.120; 500,000 x 64 .280/.336; 1,000,000 x 60 .648/.834;
-//   R-MAT scale 16 to 21, 16 per row: .018/.029, .046/.059, .184/.200, .424/.492; scale 18 x 55 .105/.157;
-//   uniform x 8 per row: 4,096 rows .012/.014, 20,000 .013/.015, 60,000 .016/.018, 200,000 .034/.034,
-//   1,000,000 .178/.174, 2,000,000 .363/.343; 4,000,000 x 4: .406/.376.
-// (1) Many short rows: a window of the streams holds four nonzeros of one row and step, and the
-//     slab plans' sliced stream does as well on rows of 8: below 12 nonzeros per row on average
-//     and beyond 2^18 rows the slab plan it is.
-// (2) Columns near the diagonal (block-diagonal 416,349 x 5: .029/.026; banded 233,000 x 64 within
-//     2,000 columns: .160/.114; 500,000 x 64 within 3,000: .427/.287): the blocks idle through the
-//     steps whose column range they do not touch, and a slab plan finds such an X in L2 anyway.
-//     The builder measures that once it has the matrix on the host (kMaxLocalShare) and says
-//     kNotWorthwhile.
+//   R-MAT scale 16 to 21, 16 per row: .018/.029, .046/.059, .184/.200, .424/.492; scale 18 x 55 .105/.157.
+// (1) Many short rows (fewer than 12 per row on average, more than 2^18 rows) without busy columns
+//     (kMinTableShareShortRows): uniform x 8 per row: 4,096 rows .012/.014, 20,000 .013/.015,
+//     60,000 .016/.018, 200,000 .034/.034, but 1,000,000 .178/.174, 2,000,000 .363/.343,
+//     4,000,000 x 4 .406/.376; with busy columns, R-MAT scale 19 x 8: .056/.071.
+// (2) Columns near the diagonal (kMaxLocalShare; block-diagonal 416,349 x 5: .029/.026; banded
+//     233,000 x 64 within 2,000 columns: .160/.114; 500,000 x 64 within 3,000: .427/.287): the blocks
+//     idle through the steps whose column range they do not touch, and a slab plan finds such an X
+//     in L2 anyway.
+// (3) A row far longer than a CU's share of the nonzeros (kMaxLongestRow; power law 262,144 x 4 with
+//     a row of 50,000: .053/.034): rows are not cut across blocks.  R-MAT scale 18 x 16, whose
+//     longest row is that share, is fine (.046/.059).
 constexpr double kMaxLocalShare = 0.25;
+constexpr double kMaxLongestRow = 2.0;
+constexpr double kMinTableShareShortRows = 0.05;
 bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, int cost, int tpw, unsigned flags)
 {
     if (flags & MPS_PLAN_FORCE_ROWBLOCK) return true;
     if (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT)) return false;
     if (elem_bytes != 4 || K != 16 || n_rows < 1 || nnz < 1) return false;
-    if (n_rows > (1 << 22)) return false;
+    if ((uint64_t)n_rows * 64 >= kResidentMinXBytes) return false;
     // a caller that names a cost or partitions per wavefront of its own is tuning a slab plan: row-block plans have neither
     int default_cost = 0, max_tpw = 0;
     if (mps_default_cost(n_rows, nnz, K, elem_bytes, &default_cost) != MPS_OK || cost != default_cost) return false;
     if (mps_max_threads_per_wave(K, elem_bytes, &max_tpw) != MPS_OK || (tpw != 0 && tpw != max_tpw)) return false;
-    return n_rows <= (1 << 18) || (long long)nnz >= 12LL * n_rows;
+    return true;
 }
 
 }  // namespace
@@ -1317,7 +1322,11 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.block_rows = opt.rowblock_block_rows;
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
-        bp.max_local_share = (flags & MPS_PLAN_FORCE_ROWBLOCK) ? 1.0 : kMaxLocalShare;
+        if (!(flags & MPS_PLAN_FORCE_ROWBLOCK)) {
+            bp.max_local_share = kMaxLocalShare;
+            bp.max_longest_row = kMaxLongestRow;
+            bp.min_table_share_short_rows = kMinTableShareShortRows;
+        }
         int rc = mps_rb::create(d_row_ptr, d_col_idx, static_cast<const float *>(d_val), n_rows, nnz, K, bp,
                                 static_cast<hipStream_t>(stream), &pl->rb);
         if (rc == MPS_OK) {
@@ -1330,7 +1339,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
             plan_free(pl);
             return rc;
         }
-        // columns near the diagonal: the slab plan below
+        // short rows, local columns or one very long row: the slab plan below
     }
     int rc;
     try {

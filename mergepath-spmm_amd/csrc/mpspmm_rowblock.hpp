@@ -108,10 +108,13 @@ struct BuildParams {
     int block_rows = 0;  // 0 = choose; otherwise the most rows a block may hold
     int num_cus = 256;
     bool keep_src = true;
-    double max_local_share = 1.0;  // give up when the blocks find a larger share of the nonzeros in column ranges of their own
+    // build_layout gives up (kNotWorthwhile) ...
+    double max_local_share = 1.0;             // when the blocks find a larger share of the nonzeros in column ranges of their own
+    double max_longest_row = 0.0;             // when the longest row has more than this many times nnz / num_cus nonzeros (0: never)
+    double min_table_share_short_rows = 0.0;  // when rows are many and short and the first table serves a smaller share of the nonzeros
 };
 
-constexpr int kNotWorthwhile = -1;  // build_layout: max_local_share not met
+constexpr int kNotWorthwhile = -1;  // build_layout: one of the three limits of BuildParams not met
 
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,

@@ -137,7 +137,8 @@ int default_steps(int n, long long nnz, int table_rows, int num_blocks, const lo
     // (about 3 us on MI355X, the time of 3,000 nonzeros).  Two things ask for steps, and the larger one decides.
     // (1) The range of X that a step gathers through L2 should stay in the 4 MiB L2 of an XCD: 5 MiB of X per step
     //     where the columns are skewed (the busy part of a range stays), 3 MiB where they are not - but no more
-    //     steps than leave a block 6,000 nonzeros each: below that the steps cost more than the L2 misses.
+    //     steps than leave a block 7,000 (skewed) or 5,000 nonzeros each: below that the steps cost more than the
+    //     L2 misses they save.
     // (2) Tables: every step puts another H columns into LDS.  A block wants about 28,000 nonzeros per step, and a
     //     table is worth its step while it serves 1 % of the nonzeros.
     // Measured on MI355X (ms per product at 2 / 3 / 4 / 6 / 8 / 12 / 16 steps; in brackets what this rule picks):
@@ -148,25 +149,25 @@ int default_steps(int n, long long nnz, int table_rows, int num_blocks, const lo
     //   power law,   232,965 rows x 492:         13 to 18 steps within 1.5 % of each other (16)
     //   power law,   500,000 rows x  64:         .280 .245 .231 .226 .232 .257 .301     (7)
     //   power law,   500,000 rows x 200:         .864 .712 .629 .560 .546 .546 .547     (7)
-    //   power law, 1,000,000 rows x  64:         .721 .662 .635 .604 .577 .573 .636     (10)
+    //   power law, 1,000,000 rows x  64:         .721 .662 .635 .604 .577 .573 .636     (8)
     //   power law, 1,000,000 rows x 128:         1.45 1.31 1.21 1.12 1.06 1.04 1.01     (13)
-    //   power law, 1,000,000 rows x  32 (2, 4, 6, 8, 13 steps): .361 .336 .330 .351 .457                    (5)
+    //   power law, 1,000,000 rows x  32 (2, 4, 6, 8, 13 steps): .361 .336 .330 .351 .457                    (4)
     //   power law, 1,000,000 rows x  16 (1, 2, 3, 4, 13 steps): .216 .202 .199 .203 .331                    (2)
     //   power law,   500,000 rows x  16 (2, 4 steps):           .089 .096                                   (2)
-    //   R-MAT scale 20, 16 per row (1, 2, 3, 4, 6, 8, 13):      .184 .190 .190 .207 .247 .290 .378          (2)
+    //   R-MAT scale 20, 16 per row (1, 2, 3, 4, 6, 8, 13):      .184 .190 .190 .207 .247 .290 .378          (1)
     //   R-MAT scale 18, 16 per row (1, 2, 4):                   .046 .053 .067                              (1)
     //   uniform,     232,965 rows x 100 (2, 3, 4, 6, 10, 13 steps): .220 .164 .151 .148 .159 .167   (5)
     //   uniform,     232,965 rows x 300:                            .610 .480 .418 .414 .415 .419   (5)
-    //   uniform,     500,000 rows x  64:                            .448 .389 .339 .283 .280 .296   (10)
-    //   uniform,   1,000,000 rows x 100:                            1.64 1.49 1.37 1.19 .946 .921   (16)
-    //   uniform,   1,000,000 rows x  60 (6, 10, 14, 21 steps):      .762 .648 .658 .795             (9)
+    //   uniform,     500,000 rows x  64:                            .448 .389 .339 .283 .280 .296   (11)
+    //   uniform,   1,000,000 rows x 100:                            1.64 1.49 1.37 1.19 .946 .921   (19)
+    //   uniform,   1,000,000 rows x  60 (6, 10, 14, 21 steps):      .762 .648 .658 .795             (11)
     // Never more table slots than columns.
     if (table_rows < 1) table_rows = 1;
     if (num_blocks < 1) num_blocks = 1;
     const bool skewed = tables > 0 && nnz > 0 && (double)table_nnz[0] >= 0.05 * (double)nnz;
     const long long per_step = skewed ? (5ll << 20) : (3ll << 20);
     long long for_l2 = ((long long)n * 64 + per_step - 1) / per_step;
-    for_l2 = std::min(for_l2, nnz / num_blocks / 6000);
+    for_l2 = std::min(for_l2, nnz / num_blocks / (skewed ? 7000 : 5000));
     long long for_tables = (nnz / num_blocks + 14000) / 28000;
     if (for_tables > tables) for_tables = tables;
     while (for_tables > 0 && (double)table_nnz[for_tables - 1] < 0.01 * (double)nnz) --for_tables;
@@ -205,6 +206,9 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     // block is more than half above its share, or the largest block is a single row.
     long long longest_row = 0;
     for (int r = 0; r < n; ++r) longest_row = std::max<long long>(longest_row, (long long)rp[r + 1] - rp[r]);
+    // A row is never cut across blocks: a matrix whose longest row outweighs the share of a CU several times is for
+    // the merge-path split of the slab plans (power law, 262,144 rows x 4 with a row of 50,000: .053 against .034 ms).
+    if (bp.max_longest_row > 0.0 && (double)longest_row > bp.max_longest_row * (double)nnz / num_cus) return kNotWorthwhile;
     long long best_target = 0;
     for (int m = 1, tried = 0; tried < 8; ++m) {
         const long long most = (long long)num_cus * m;
@@ -244,17 +248,21 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         const int da = d_of(a), db = d_of(b);
         return da != db ? da > db : a < b;
     };
+    // what every further table would serve, for as many tables as a plan may get
+    constexpr int kMostTables = 32;
+    long long table_nnz[kMostTables] = {0};
+    const size_t top = std::min<size_t>((size_t)kMostTables * H, cand.size());
+    if (top < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)top, cand.end(), hotter);
+    std::sort(cand.begin(), cand.begin() + (long)top, hotter);
+    for (size_t k = 0; k < top; ++k) table_nnz[k / (size_t)H] += d_of(cand[k]);
+    // Many short rows (fewer than 12 nonzeros per row, more than 2^18 rows): a window of the streams holds four
+    // nonzeros of one row, step and kind, and the slab plans' sliced stream does as well on such rows - unless the
+    // first table alone serves a good part of the nonzeros.
+    if (bp.min_table_share_short_rows > 0.0 && n > (1 << 18) && (long long)nnz < 12LL * n &&
+        (double)table_nnz[0] < bp.min_table_share_short_rows * (double)nnz)
+        return kNotWorthwhile;
     int T = bp.steps;
-    if (T <= 0) {
-        // what every further table would serve, for as many tables as a plan may get
-        constexpr int kMostTables = 32;
-        const size_t top = std::min<size_t>((size_t)kMostTables * H, cand.size());
-        if (top < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)top, cand.end(), hotter);
-        std::sort(cand.begin(), cand.begin() + (long)top, hotter);
-        long long table_nnz[kMostTables] = {0};
-        for (size_t k = 0; k < top; ++k) table_nnz[k / (size_t)H] += d_of(cand[k]);
-        T = default_steps(n, nnz, H, L.num_blocks, table_nnz, (int)((top + (size_t)H - 1) / (size_t)H));
-    }
+    if (T <= 0) T = default_steps(n, nnz, H, L.num_blocks, table_nnz, (int)((top + (size_t)H - 1) / (size_t)H));
     if (T > 4096) T = 4096;
     if (bp.max_local_share < 1.0 && nnz > 0) {
         // Columns near the diagonal (banded, block-diagonal): a block finds its nonzeros in one or two column

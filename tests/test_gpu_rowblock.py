@@ -222,14 +222,18 @@ def test_uniform_matrix_gets_a_rowblock_plan_too(pkg, orc, dev):
     check_fp32(slabs.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
 
 
-@pytest.mark.parametrize("kind", ["short_rows", "banded"])
+@pytest.mark.parametrize("kind", ["short_rows", "banded", "long_row"])
 def test_matrices_that_stay_with_the_slab_plans(pkg, orc, dev, kind):
-    """No row-block plan unless asked for: many short rows (a million rows of 8), and columns that stay
-    near the diagonal (a band of 2,000 columns either side: every block would idle through the steps
-    of the other column ranges)."""
+    """No row-block plan unless asked for: many short rows without busy columns (a million rows of 8,
+    columns used evenly), columns that stay near the diagonal (a band of 2,000 columns either side:
+    every block would idle through the steps of the other column ranges), and a row that is many times
+    a CU's share of the nonzeros (rows are not cut across blocks)."""
     rng = np.random.default_rng(3)
     if kind == "short_rows":
         rp, ci, _ = pkg.graphs.generate("er:n=1000000,deg=8", seed=5)
+    elif kind == "long_row":
+        rp, ci, _ = pkg.graphs.generate("chunglu:n=262144,nnz=1000000,gamma=2.1,dmax=50000", seed=5)
+        assert np.diff(rp).max() > 2 * ci.size / 256
     else:
         n, deg, w = 120000, 48, 2000
         c = np.arange(n, dtype=np.int64)[:, None] + rng.integers(-w, w + 1, size=(n, deg))

@@ -241,7 +241,7 @@ def test_more_rounds_of_blocks_where_one_round_is_unequal(pkg):
 @pytest.mark.parametrize("spec,steps,why", [
     ("er:n=120000,deg=60", 3, "7.7 MB of X, columns used evenly: 3 MiB a step"),
     ("chunglu:n=120000,nnz=7200000,gamma=2.1,dmax=4000", 2, "7.7 MB of X, skewed columns: 5 MiB a step"),
-    ("er:n=120000,deg=20", 1, "9,400 nonzeros per block: a second step would leave fewer than 6,000 each"),
+    ("er:n=120000,deg=20", 1, "9,400 nonzeros per block: a second step would leave fewer than 5,000 each"),
     ("chunglu:n=30000,nnz=16000000,gamma=2.1,dmax=6000", 2, "X fits one step, but a block has 62,500 nonzeros: a second table"),
     ("er:n=190000,deg=190", 4, "141,000 nonzeros per block ask for 5 tables, but a table serves 0.9 % of them: 12.2 MB of X at 3 MiB a step"),
 ])
