@@ -267,7 +267,7 @@ int mps_spmm_f32_static(const int *d_row_ptr, const int *d_col_idx, const float 
 #define MPS_PHASE_MAIN 1u
 #define MPS_PHASE_FIXUP 2u
 #define MPS_PHASE_REDUCE 4u /* plans with column slabs only */
-#define MPS_PHASE_PREPARE 8u /* row-block plans only: the small kernel that gathers the hot columns' rows of X */
+#define MPS_PHASE_PREPARE 8u /* row-block plans: the small kernel that gathers the hot columns' rows of X (a plan of one step and at most 256 blocks reads them in its main kernel instead) */
 int mps_spmm_f32_phases(const int *d_row_ptr, const int *d_col_idx, const float *d_val,
                         const float *d_X, float *d_Y, int n_rows, int nnz, int K, int P,
                         const int *d_coord_x, const int *d_coord_y, int tpw,

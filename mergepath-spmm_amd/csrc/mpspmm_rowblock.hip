@@ -128,7 +128,7 @@ __device__ __forceinline__ int rounds_of(int n) { return ((n >> 4) + ((n & 15) !
 
 // CPACK: the cold stream is read in its packed form (cold_p; 12 bytes per lane and round, columns counted from the
 // first column of the step's range, cold_begin[t]) instead of as 8-byte entries (cold).
-template <typename TOut, bool CPACK>
+template <typename TOut, bool CPACK, bool TABLE_FROM_X>
 __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__restrict__ hot, const Entry *__restrict__ cold,
                                                             const uint32_t *__restrict__ cold_p,
                                                             const int *__restrict__ cold_begin,
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                                                             const float4 *__restrict__ hot_x4,
                                                             const float4 *__restrict__ X4, TOut *__restrict__ Y, int T,
                                                             int H, int acc_rows, int hot_bits, int cold_bits, int keep_from,
-                                                            int cold_ib)
+                                                            int cold_ib, const int *__restrict__ table_cols)
 {
     extern __shared__ __align__(16) char smem[];
     float *table = reinterpret_cast<float *>(smem);                         // [H][16]
@@ -158,7 +158,15 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
 
     for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4;
     if (tid < kWaveSlots * 16) slots[tid] = 0.f;
-    for (int i = tid; i < H * 4; i += kThreads) table4[i] = hot_x4[i];
+    if constexpr (TABLE_FROM_X) {
+        // a small plan of one step: its only table straight from X, no gather kernel in front
+        for (int i = tid; i < H * 4; i += kThreads) {
+            const int c = table_cols[i >> 2];
+            table4[i] = c >= 0 ? X4[(size_t)c * 4 + (i & 3)] : zero4;
+        }
+    } else {
+        for (int i = tid; i < H * 4; i += kThreads) table4[i] = hot_x4[i];
+    }
 
 #define RB_PRE_LOAD(k) const float4 pre##k = tid + k * kThreads < H * 4 ? pre_src[tid + k * kThreads] : zero4;
 #define RB_PRE_STORE(k) if (tid + k * kThreads < H * 4) table4[tid + k * kThreads] = pre##k;
@@ -561,11 +569,12 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
     }
     dp->lds_bytes = (size_t)(L.table_rows + L.acc_rows) * 64 + kSlotBytes;
     {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float, false>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(rb_spmm_kernel<float, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
+        hipError_t e = hipSuccess;
+        for (const void *kernel : {reinterpret_cast<const void *>(rb_spmm_kernel<float, false, false>),
+                                   reinterpret_cast<const void *>(rb_spmm_kernel<float, true, false>),
+                                   reinterpret_cast<const void *>(rb_spmm_kernel<float, false, true>),
+                                   reinterpret_cast<const void *>(rb_spmm_kernel<float, true, true>)})
+            if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
@@ -583,7 +592,11 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
 {
     const Layout &L = dp->host;
     const int slots = L.steps * L.table_rows;
-    if (phases & MPS_PHASE_PREPARE)
+    // A plan of one step and one round of blocks loads its table from X in the main kernel: a launch less (4,096 rows
+    // x 8 per row: 9.4 against 11.2 us per product).  With more blocks than CUs the gathers of every block cost more
+    // than the launch (R-MAT scale 18 x 16, 512 blocks: 50 against 46 us).
+    const bool table_from_x = L.steps == 1 && L.num_blocks <= 256;
+    if ((phases & MPS_PHASE_PREPARE) && !table_from_x)
         hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
                            reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
     if (phases & MPS_PHASE_MAIN) {
@@ -591,10 +604,17 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
             hipLaunchKernelGGL(kernel, dim3((unsigned)L.num_blocks), dim3(kThreads), dp->lds_bytes, st, dp->hot, dp->cold,
                                dp->cold_packed, dp->cold_begin, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta),
                                dp->block_row, reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X),
-                               Y, L.steps, L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from, L.cold_index_bits);
+                               Y, L.steps, L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from, L.cold_index_bits,
+                               table_from_x ? dp->hot_cols : nullptr);
         };
-        if (dp->cold_packed) launch(rb_spmm_kernel<float, true>);
-        else launch(rb_spmm_kernel<float, false>);
+        if (table_from_x) {
+            if (dp->cold_packed) launch(rb_spmm_kernel<float, true, true>);
+            else launch(rb_spmm_kernel<float, false, true>);
+        } else if (dp->cold_packed) {
+            launch(rb_spmm_kernel<float, true, false>);
+        } else {
+            launch(rb_spmm_kernel<float, false, false>);
+        }
     }
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
