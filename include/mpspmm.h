@@ -504,8 +504,8 @@ void mps_rowblock_layout_free(mps_rowblock_layout *layout);
  * wavefront, the default cost with half the partitions per wavefront, without
  * hot columns, without tiling, with slabs of 3, 6, 12 and 24 MiB where X holds
  * more than two of them and the library's cost model does not put them 50 %
- * behind the untiled plan; one row-block plan for fp32, K = 16 and rows of 32
- * nonzeros and more on average), runs `repeats` timed products Y = A * X after two warm-ups
+ * behind the untiled plan; one row-block plan for fp32, K = 16 and an X below
+ * 192 MiB), runs `repeats` timed products Y = A * X after two warm-ups
  * (HIP events on the stream) and reports the fastest.  d_Y is overwritten.
  * tried_out (optional) receives every candidate with its time;
  * *n_tried_io is its capacity on entry and the number of candidates on

@@ -1490,7 +1490,7 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, slab, 0.f, 0};
     cand[n_cand++] = {dflt, max_tpw, slab | MPS_PLAN_NO_HOT, 0.f, 0};
     cand[n_cand++] = {dflt, max_tpw, slab | MPS_PLAN_NO_TILING, 0.f, 0};
-    if (elem_bytes == 4 && K == 16 && n_rows >= 1 && (long long)nnz >= 32LL * n_rows)
+    if (elem_bytes == 4 && K == 16 && n_rows >= 1 && nnz >= 1 && (uint64_t)n_rows * 64 < kResidentMinXBytes)
         cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_ROWBLOCK, 0.f, 0};
     // slab sizes the model does not pick on its own: larger slabs pay on skewed graphs
     // (not those the model puts 50 % behind the untiled plan: thousands of slabs for a matrix with short rows)

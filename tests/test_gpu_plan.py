@@ -543,7 +543,7 @@ def test_autotune_picks_a_measured_candidate(pkg, orc, dev, spec, n_candidates, 
     c = pkg._cabi
     tiling = "off" if best["flags"] & c.MPS_PLAN_NO_TILING else "force" if best["flags"] & c.MPS_PLAN_FORCE_TILING else "auto"
     hot = "off" if best["flags"] & c.MPS_PLAN_NO_HOT else "auto"
-    # fp32, K = 16, rows of 32 nonzeros and more: one candidate is a row-block plan, all others are slab plans
+    # fp32, K = 16, X below 192 MiB: one candidate is a row-block plan, all others are slab plans
     assert sum(1 for t in tried if t["flags"] & c.MPS_PLAN_FORCE_ROWBLOCK) == 1
     assert all(t["flags"] & (c.MPS_PLAN_FORCE_ROWBLOCK | c.MPS_PLAN_NO_ROWBLOCK) for t in tried)
     rowblock = "force" if best["flags"] & c.MPS_PLAN_FORCE_ROWBLOCK else "off"
