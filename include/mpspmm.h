@@ -391,6 +391,9 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
 #define MPS_PLAN_NO_ROWBLOCK 16u    /* never build a row-block plan (see below)  */
 #define MPS_PLAN_FORCE_ROWBLOCK 32u /* row-block plan whatever the matrix looks like (fp32, K = 16 only) */
+#define MPS_PLAN_LOCAL_TABLES 1024u  /* row-block plans: one step, every block with a table of consecutive columns of its own
+                                        (what the library builds by itself for matrices whose columns stay within a table's
+                                        width of the diagonal); with MPS_PLAN_FORCE_ROWBLOCK or mps_rowblock_layout_build */
 #define MPS_PLAN_NO_COLUMN_TILES 512u /* untiled plans with rows of X of 512 bytes and more: no passes over 128-byte column tiles */
 #define MPS_PLAN_NO_RESIDENT 256u    /* untiled plans: no streaming hint on the gathers of unpopular columns (see below) */
 #define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
@@ -426,6 +429,7 @@ typedef struct mps_plan_info {
     long long resident_nnz;        /* nonzeros in them                            */
     int rowblock_cold_index_bits;  /* row-block plans: > 0 when the cold stream is held in packed form (RB_COLD_PACKED): bits of a
                                       16-bit entry that hold the column, counted from the first column of the step's range */
+    int rowblock_local_tables;     /* row-block plans: 1 when every block has a table of its own (RB_TABLE_BASE) */
 } mps_plan_info;
 
 /* Optional parameters of mps_plan_create_ex; zero means "the library chooses". */
@@ -465,7 +469,9 @@ enum {
     MPS_PLAN_ARRAY_RB_COLD_PACKED = 17, /* 12 bytes x (cold slots / 2), if rowblock_cold_index_bits > 0: the same form; half =
                                          (column - first column of the step's range) | piece << index_bits, entry e of a window
                                          holds bits [e p, (e + 1) p) of its rows_advanced, p = 16 - index_bits */
-    MPS_PLAN_ARRAY_RB_COLD_BEGIN = 18 /* int[steps + 1]: first column of every step's range of cold columns */
+    MPS_PLAN_ARRAY_RB_COLD_BEGIN = 18, /* int[steps + 1]: first column of every step's range of cold columns */
+    MPS_PLAN_ARRAY_RB_TABLE_BASE = 19  /* int[blocks], plans with local tables: block b's table holds the columns base[b] ..
+                                         base[b] + table_rows - 1 (RB_HOT_COLS is all -1 then) */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,

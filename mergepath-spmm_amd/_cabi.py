@@ -37,11 +37,13 @@ MPS_PLAN_NO_SOURCES = 64
 MPS_PLAN_NO_ROW_MARKS = 128
 MPS_PLAN_NO_RESIDENT = 256
 MPS_PLAN_NO_COLUMN_TILES = 512
+MPS_PLAN_LOCAL_TABLES = 1024
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
  MPS_PLAN_ARRAY_RB_HOT, MPS_PLAN_ARRAY_RB_COLD, MPS_PLAN_ARRAY_RB_HOT_SRC, MPS_PLAN_ARRAY_RB_COLD_SRC,
- MPS_PLAN_ARRAY_RB_HOT_PACKED, MPS_PLAN_ARRAY_RB_COLD_PACKED, MPS_PLAN_ARRAY_RB_COLD_BEGIN) = range(19)
+ MPS_PLAN_ARRAY_RB_HOT_PACKED, MPS_PLAN_ARRAY_RB_COLD_PACKED, MPS_PLAN_ARRAY_RB_COLD_BEGIN,
+ MPS_PLAN_ARRAY_RB_TABLE_BASE) = range(20)
 
 
 class PlanInfo(ctypes.Structure):
@@ -56,7 +58,7 @@ class PlanInfo(ctypes.Structure):
                 ("rowblock_blocks", ctypes.c_int), ("rowblock_acc_rows", ctypes.c_int),
                 ("rowblock_hot_slots", ctypes.c_longlong), ("rowblock_cold_slots", ctypes.c_longlong),
                 ("resident_cols", ctypes.c_int), ("resident_nnz", ctypes.c_longlong),
-                ("rowblock_cold_index_bits", ctypes.c_int)]
+                ("rowblock_cold_index_bits", ctypes.c_int), ("rowblock_local_tables", ctypes.c_int)]
 
 
 class PlanOptions(ctypes.Structure):

@@ -1322,6 +1322,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.block_rows = opt.rowblock_block_rows;
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
+        bp.local_tables = (flags & MPS_PLAN_LOCAL_TABLES) != 0;
         if (!(flags & MPS_PLAN_FORCE_ROWBLOCK)) {
             bp.max_local_share = kMaxLocalShare;
             bp.max_longest_row = kMaxLongestRow;
@@ -1339,7 +1340,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
             plan_free(pl);
             return rc;
         }
-        // short rows, local columns or one very long row: the slab plan below
+        // short rows, one very long row, or local columns that no table of a block's own covers: the slab plan below
     }
     int rc;
     try {
@@ -1387,6 +1388,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->rowblock_steps = info->rowblock_table_rows = info->rowblock_blocks = info->rowblock_acc_rows = 0;
     info->rowblock_hot_slots = info->rowblock_cold_slots = 0;
     info->rowblock_cold_index_bits = 0;
+    info->rowblock_local_tables = 0;
     if (plan->rb) {
         const mps_rb::Layout &L = mps_rb::layout_of(plan->rb);
         info->num_slabs = 1;
@@ -1401,6 +1403,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
         info->rowblock_hot_slots = L.hot_rounds * mps_rb::kRoundEntries;
         info->rowblock_cold_slots = L.cold_rounds * mps_rb::kRoundEntries;
         info->rowblock_cold_index_bits = L.cold_index_bits;
+        info->rowblock_local_tables = L.table_base.empty() ? 0 : 1;
     }
     return MPS_OK;
 }
@@ -1434,7 +1437,7 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
     default:
         if (!plan->rb) return MPS_ERR_INVALID_ARG;
         src = mps_rb::device_array(plan->rb, which, &have);
-        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_COLD_BEGIN)) return MPS_ERR_INVALID_ARG;
+        if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_TABLE_BASE)) return MPS_ERR_INVALID_ARG;
         break;
     }
     if (plan->rb && which < MPS_PLAN_ARRAY_RB_BLOCK_ROW) return MPS_ERR_INVALID_ARG;

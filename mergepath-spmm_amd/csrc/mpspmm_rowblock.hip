@@ -23,7 +23,7 @@ struct DevicePlan {
     uint32_t *cold_packed = nullptr;  // in packed form (one of the two)
     int *hot_src = nullptr, *cold_src = nullptr;
     long long *wave_base = nullptr;
-    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr, *cold_begin = nullptr;
+    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr, *cold_begin = nullptr, *table_base = nullptr;
     float *hot_x = nullptr;  // [T][H][16] rows of X of the hot columns, gathered per product
     size_t lds_bytes = 0;
     size_t device_bytes = 0;
@@ -138,7 +138,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                                                             const float4 *__restrict__ hot_x4,
                                                             const float4 *__restrict__ X4, TOut *__restrict__ Y, int T,
                                                             int H, int acc_rows, int hot_bits, int cold_bits, int keep_from,
-                                                            int cold_ib, const int *__restrict__ table_cols)
+                                                            int cold_ib, const int *__restrict__ table_cols,
+                                                            const int *__restrict__ table_base, int n_cols)
 {
     extern __shared__ __align__(16) char smem[];
     float *table = reinterpret_cast<float *>(smem);                         // [H][16]
@@ -159,10 +160,16 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
     for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4;
     if (tid < kWaveSlots * 16) slots[tid] = 0.f;
     if constexpr (TABLE_FROM_X) {
-        // a small plan of one step: its only table straight from X, no gather kernel in front
-        for (int i = tid; i < H * 4; i += kThreads) {
-            const int c = table_cols[i >> 2];
-            table4[i] = c >= 0 ? X4[(size_t)c * 4 + (i & 3)] : zero4;
+        // a plan of one step: its only table straight from X, no gather kernel in front
+        if (table_base) {
+            // local tables: the block's own H consecutive rows of X, one contiguous read
+            const int c0 = table_base[b];
+            for (int i = tid; i < H * 4; i += kThreads) table4[i] = c0 + (i >> 2) < n_cols ? X4[(size_t)c0 * 4 + i] : zero4;
+        } else {
+            for (int i = tid; i < H * 4; i += kThreads) {
+                const int c = table_cols[i >> 2];
+                table4[i] = c >= 0 ? X4[(size_t)c * 4 + (i & 3)] : zero4;
+            }
         }
     } else {
         for (int i = tid; i < H * 4; i += kThreads) table4[i] = hot_x4[i];
@@ -473,6 +480,7 @@ void destroy(DevicePlan *dp)
     (void)hipFree(dp->cold);
     (void)hipFree(dp->cold_packed);
     (void)hipFree(dp->cold_begin);
+    (void)hipFree(dp->table_base);
     (void)hipFree(dp->hot_src);
     (void)hipFree(dp->cold_src);
     (void)hipFree(dp->wave_base);
@@ -553,6 +561,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         return fail(rc);
     }
     if ((rc = upload(dp, &dp->cold_begin, L.cold_begin, st)) != MPS_OK) return fail(rc);
+    if (!L.table_base.empty() && (rc = upload(dp, &dp->table_base, L.table_base, st)) != MPS_OK) return fail(rc);
     if (bp_in.keep_src) {
         if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
         if ((rc = upload(dp, &dp->cold_src, L.cold_src, st)) != MPS_OK) return fail(rc);
@@ -595,7 +604,8 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
     // A plan of one step and one round of blocks loads its table from X in the main kernel: a launch less (4,096 rows
     // x 8 per row: 9.4 against 11.2 us per product).  With more blocks than CUs the gathers of every block cost more
     // than the launch (R-MAT scale 18 x 16, 512 blocks: 50 against 46 us).
-    const bool table_from_x = L.steps == 1 && L.num_blocks <= 256;
+    // Local tables differ from block to block and are contiguous in X: always read there.
+    const bool table_from_x = L.steps == 1 && (L.num_blocks <= 256 || dp->table_base);
     if ((phases & MPS_PHASE_PREPARE) && !table_from_x)
         hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
                            reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
@@ -605,7 +615,7 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
                                dp->cold_packed, dp->cold_begin, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta),
                                dp->block_row, reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X),
                                Y, L.steps, L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from, L.cold_index_bits,
-                               table_from_x ? dp->hot_cols : nullptr);
+                               table_from_x ? dp->hot_cols : nullptr, dp->table_base, L.n);
         };
         if (table_from_x) {
             if (dp->cold_packed) launch(rb_spmm_kernel<float, true, true>);
@@ -675,6 +685,7 @@ const void *device_array(const DevicePlan *dp, int which, size_t *bytes)
     case MPS_PLAN_ARRAY_RB_COLD: *bytes = dp->cold ? dp->cold_slots * sizeof(Entry) : 0; return dp->cold;
     case MPS_PLAN_ARRAY_RB_COLD_PACKED: *bytes = dp->cold_packed ? dp->cold_slots / kPair * 12 : 0; return dp->cold_packed;
     case MPS_PLAN_ARRAY_RB_COLD_BEGIN: *bytes = L.cold_begin.size() * sizeof(int); return dp->cold_begin;
+    case MPS_PLAN_ARRAY_RB_TABLE_BASE: *bytes = L.table_base.size() * sizeof(int); return dp->table_base;
     case MPS_PLAN_ARRAY_RB_HOT_SRC: *bytes = dp->hot_src ? dp->hot_slots * sizeof(int) : 0; return dp->hot_src;
     case MPS_PLAN_ARRAY_RB_COLD_SRC: *bytes = dp->cold_src ? dp->cold_slots * sizeof(int) : 0; return dp->cold_src;
     default: *bytes = 0; return nullptr;

@@ -93,6 +93,7 @@ struct Layout {
     std::vector<int> block_row;         // [NB + 1]
     std::vector<int> hot_cols;          // [T][H] column of every table slot, -1 = unused
     std::vector<int> cold_begin;        // [T + 1] column-id range of every step's cold columns
+    std::vector<int> table_base;        // [NB] local tables (one step): block b's table is X[base[b] .. base[b] + H); else empty
     std::vector<int> meta;              // [NB][T][16][4] {hot entries, cold entries, first local row, 0}; [..][15] unused
     std::vector<long long> wave_base;   // [NB * 16][2] first round of the wavefront's hot / cold stream; [..][15]: where the block's streams end
     std::vector<Entry> hot, cold;       // rounds of 64 entries
@@ -112,6 +113,8 @@ struct BuildParams {
     double max_local_share = 1.0;             // when the blocks find a larger share of the nonzeros in column ranges of their own
     double max_longest_row = 0.0;             // when the longest row has more than this many times nnz / num_cus nonzeros (0: never)
     double min_table_share_short_rows = 0.0;  // when rows are many and short and the first table serves a smaller share of the nonzeros
+    double min_local_cover = 0.6;             // when the columns are local (max_local_share) and local tables would serve a smaller share
+    bool local_tables = false;                // local tables whatever the matrix looks like
 };
 
 constexpr int kNotWorthwhile = -1;  // build_layout: one of the three limits of BuildParams not met

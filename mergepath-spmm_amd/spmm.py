@@ -177,7 +177,8 @@ class Plan:
 
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
-                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None, column_tiles=True):
+                 rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None, column_tiles=True,
+                 local_tables=False):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -194,6 +195,8 @@ class Plan:
             flags |= _cabi.MPS_PLAN_NO_RESIDENT
         if not column_tiles:
             flags |= _cabi.MPS_PLAN_NO_COLUMN_TILES
+        if local_tables:
+            flags |= _cabi.MPS_PLAN_LOCAL_TABLES
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
                                 int(rowblock_block_rows), int(rowblock_blocks_per_round),
                                 {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes))
@@ -247,6 +250,7 @@ class Plan:
             _cabi.MPS_PLAN_ARRAY_RB_HOT_PACKED: (3 * int(i.rowblock_hot_slots) // 2, np.uint32),
             _cabi.MPS_PLAN_ARRAY_RB_COLD_PACKED: (3 * int(i.rowblock_cold_slots) // 2 if i.rowblock_cold_index_bits else 0, np.uint32),
             _cabi.MPS_PLAN_ARRAY_RB_COLD_BEGIN: (i.rowblock_steps + 1 if i.rowblock_steps else 0, np.int32),
+            _cabi.MPS_PLAN_ARRAY_RB_TABLE_BASE: (i.rowblock_blocks if i.rowblock_local_tables else 0, np.int32),
         }
         n, dt = shapes[which]
         out = np.empty(n, dtype=dt)
@@ -319,14 +323,15 @@ class RowBlockLayout:
     """The layout of a row-block plan, built on the host (mps_rowblock_layout_build): no GPU needed."""
 
     def __init__(self, row_ptr, col_idx, val, K=16, steps=0, table_rows=0, block_rows=0, blocks_per_round=0,
-                 keep_sources=True):
+                 keep_sources=True, local_tables=False):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
         rp = np.ascontiguousarray(row_ptr, dtype=np.int32)
         ci = np.ascontiguousarray(col_idx, dtype=np.int32)
         v = np.ascontiguousarray(val, dtype=np.float32)
-        opt = _cabi.PlanOptions(0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES, 0, int(steps), int(table_rows),
+        opt = _cabi.PlanOptions((0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES) | (_cabi.MPS_PLAN_LOCAL_TABLES if local_tables else 0),
+                                0, int(steps), int(table_rows),
                                 int(block_rows), int(blocks_per_round), 0, 0)
         check(_cabi.lib().mps_rowblock_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size,
                                                     int(K), ctypes.byref(opt), ctypes.byref(self._h)),

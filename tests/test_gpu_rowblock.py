@@ -256,3 +256,33 @@ def test_matrices_that_stay_with_the_slab_plans(pkg, orc, dev, kind):
     forced = pkg.spmm.Plan(csr, 16, rowblock="force")
     assert forced.info.rowblock_steps > 0
     check_fp32(forced.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+
+
+@pytest.mark.parametrize("forced", [True, False])
+def test_local_tables_on_a_block_diagonal_matrix(pkg, orc, dev, forced):
+    """Columns that stay near the diagonal: every block gets a table of consecutive columns of its own (one step,
+    the table read straight from X) - asked for with MPS_PLAN_LOCAL_TABLES, or chosen by the library where such
+    tables serve most of the nonzeros."""
+    rp, ci, _ = pkg.graphs.generate("blockdiag:blocks=300,min=100,max=600,deg=5", seed=9)
+    n, nnz = rp.size - 1, ci.size
+    val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
+    X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    kw = dict(rowblock="force", local_tables=True, rowblock_table_rows=256, rowblock_block_rows=300) if forced else {}
+    plan = pkg.spmm.Plan(csr, 16, **kw)
+    i = plan.info
+    assert i.rowblock_local_tables == 1 and i.rowblock_steps == 1
+    assert (i.hot_nnz > 0.9 * nnz) == (not forced)  # tables of 256 rows miss many of a block's columns
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=True)
+    assert torch.equal(Y, plan.spmm(d_X))
+    base = plan.array(pkg._cabi.MPS_PLAN_ARRAY_RB_TABLE_BASE)
+    assert base.size == i.rowblock_blocks and (base >= 0).all() and (base + i.rowblock_table_rows <= n).all()
+    # new values through the source indices
+    val2 = pkg.graphs.fill_uniform_f32(nnz, 21, 0.0, 1.0)
+    plan.set_values(torch.from_numpy(val2).to(dev))
+    ref2, scale2 = orc.spmm_f64(rp, ci, val2, X, want_abs=True)
+    check_fp32(plan.spmm(d_X).cpu().numpy(), ref2, scale2, rel_elem=True)

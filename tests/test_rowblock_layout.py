@@ -29,6 +29,8 @@ def walk_layout(pkg, lay, X, n):
     hot_bits, cold_bits = i.hot_mark_shift, i.mark_shift
     brow = lay.array(C.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
     hot_cols = lay.array(C.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32).reshape(T, H)
+    table_base = lay.array(C.MPS_PLAN_ARRAY_RB_TABLE_BASE, np.int32)
+    assert table_base.size == (NB if i.rowblock_local_tables else 0)
     meta = lay.array(C.MPS_PLAN_ARRAY_RB_META, np.int32).reshape(NB, T, WSLOTS, 4)
     base = lay.array(C.MPS_PLAN_ARRAY_RB_WAVE_BASE, np.int64).reshape(NB, WSLOTS, 2)
     streams = [lay.array(C.MPS_PLAN_ARRAY_RB_HOT, np.uint32).reshape(-1, 2),
@@ -44,7 +46,11 @@ def walk_layout(pkg, lay, X, n):
         acc = np.zeros((i.rowblock_acc_rows, X.shape[1]))
         cur = base[b].copy()
         for t in range(T):
-            table = np.where(hot_cols[t][:, None] >= 0, X[np.maximum(hot_cols[t], 0)], 0.0)
+            if i.rowblock_local_tables:  # the block's own H consecutive rows of X (zeros beyond its end)
+                cols = int(table_base[b]) + np.arange(H)
+                table = np.where((cols < n)[:, None], X[np.minimum(cols, n - 1)], 0.0)
+            else:
+                table = np.where(hot_cols[t][:, None] >= 0, X[np.maximum(hot_cols[t], 0)], 0.0)
             firsts = meta[b, t, :WAVES, 2]
             assert (np.diff(firsts) >= 0).all(), "first rows of the wavefronts' runs must not decrease"
             slots = np.zeros((WAVES, X.shape[1]))
@@ -71,7 +77,7 @@ def walk_layout(pkg, lay, X, n):
                                 assert e == 0 or (word >> bits[k]) == 0, "only a window's first entry advances rows"
                                 x = table[idx] if k == 0 else X[idx]
                                 if k == 0:
-                                    assert hot_cols[t, idx] >= 0
+                                    assert hot_cols[t, idx] >= 0 or (i.rowblock_local_tables and table_base[b] + idx < n)
                                 src = int(srcs[k][slot0 + 2 * e])
                                 if src >= 0:
                                     assert real == e, "a window's nonzeros come first, padding after them"
@@ -249,6 +255,40 @@ def test_steps_follow_the_size_of_x_the_work_and_the_skew(pkg, spec, steps, why)
     rp, ci, _ = pkg.graphs.generate(spec, seed=4)
     lay = pkg.spmm.RowBlockLayout(rp, ci, np.ones(ci.size, dtype=np.float32), keep_sources=False)
     assert lay.info.rowblock_steps == steps, why
+
+
+@pytest.mark.parametrize("spec,table_rows,block_rows,per_round,share", [
+    ("blockdiag:blocks=40,min=50,max=200,deg=5", 0, 0, 4, 0.95),   # a table covers a block's components
+    ("blockdiag:blocks=40,min=50,max=200,deg=5", 64, 100, 4, 0.2),  # tables narrower than a component: many cold entries
+    ("er:n=300,deg=6", 0, 0, 2, 1.0),                               # fewer columns than table rows: everything is hot
+])
+def test_local_tables_walk_reproduces_the_product(pkg, spec, table_rows, block_rows, per_round, share):
+    """MPS_PLAN_LOCAL_TABLES: one step, block b's table holds the columns base[b] .. base[b] + H - 1 (the window
+    with the most of the block's nonzeros), RB_HOT_COLS is unused; the walk over the streams gives the product."""
+    rp, ci, _ = pkg.graphs.generate(spec, seed=3)
+    n = rp.size - 1
+    rng = np.random.default_rng(12)
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float64)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, table_rows=table_rows, block_rows=block_rows, blocks_per_round=per_round,
+                                  local_tables=True)
+    i = lay.info
+    assert i.rowblock_local_tables == 1 and i.rowblock_steps == 1
+    assert (lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32) == -1).all()
+    base = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_TABLE_BASE, np.int32)
+    brow = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
+    assert (base >= 0).all() and (base <= max(0, n - i.rowblock_table_rows)).all()
+    # hot_nnz counts the nonzeros whose column lies in their block's window
+    blk = np.repeat(np.arange(brow.size - 1), rp[brow[1:]] - rp[brow[:-1]])
+    inside = (ci >= base[blk]) & (ci < base[blk] + i.rowblock_table_rows)
+    assert i.hot_nnz == int(inside.sum()) and i.hot_nnz >= share * ci.size - 1e-9
+    Y, seen = walk_layout(pkg, lay, X, n)
+    assert np.array_equal(np.sort(seen), np.arange(ci.size))
+    A = np.zeros((n, n))
+    A[np.repeat(np.arange(n), np.diff(rp)), ci] = val
+    assert np.allclose(Y, A @ X, rtol=1e-12, atol=1e-12)
+    # without the flag the same matrix gets global tables
+    assert pkg.spmm.RowBlockLayout(rp, ci, val, blocks_per_round=per_round).info.rowblock_local_tables == 0
 
 
 def test_rejects_what_it_is_not_built_for(pkg):
