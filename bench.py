@@ -134,9 +134,10 @@ def layout_text(w, plan):
         return "plain CSR, no plan"
     i = plan.info
     if i.rowblock_steps > 0:
-        return ("row-block plan: %d blocks, %d steps x %d table rows, %.1f %% of the nonzeros from LDS, %.0f MB"
-                % (i.rowblock_blocks, i.rowblock_steps, i.rowblock_table_rows, 100.0 * i.hot_nnz / max(w.nnz, 1),
-                   i.device_bytes / 1e6))
+        return ("row-block plan: %d blocks, %d steps x %d table rows%s, %.1f %% of the nonzeros from LDS, %.0f MB"
+                % (i.rowblock_blocks, i.rowblock_steps, i.rowblock_table_rows,
+                   " (a table of consecutive columns per block)" if i.rowblock_local_tables else "",
+                   100.0 * i.hot_nnz / max(w.nnz, 1), i.device_bytes / 1e6))
     text = "plan: %d column slab(s) of %d, sliced, %.0f MB" % (i.num_slabs, i.slab_cols, i.device_bytes / 1e6)
     if i.resident_cols:
         text += ", streaming hint on gathers outside the %d busiest columns (%.1f %% of the nonzeros)" % (

@@ -340,9 +340,11 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  * this kind of plan by itself where it was measured to win: fp32, K = 16, X
  * below 192 MiB (3.1 M rows), except for matrices with many short rows and no
  * busy columns (fewer than 12 nonzeros per row on average, more than 2^18
- * rows), matrices whose columns stay near the diagonal (banded,
- * block-diagonal) and matrices with one row far longer than a CU's share of
- * the nonzeros, which keep the slab plans.  `steps` and the number of blocks follow from the size of X,
+ * rows), matrices whose columns stay near the diagonal but not within a
+ * table's width of it (wide bands) and matrices with one row far longer than a
+ * CU's share of the nonzeros, which keep the slab plans.  Narrow bands and
+ * block-diagonal matrices get local tables (MPS_PLAN_LOCAL_TABLES): one step,
+ * every block with a table of the consecutive columns it uses most.  `steps` and the number of blocks follow from the size of X,
  * the nonzeros per block and the column histogram.  A caller that passes a
  * cost other than mps_default_cost's, a tpw other than 0 or the maximum, or
  * one of the tiling / hot-column flags is tuning a slab plan and gets one;
