@@ -159,11 +159,12 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
 
     for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4;
     if (tid < kWaveSlots * 16) slots[tid] = 0.f;
+    int local_c0 = 0;  // local tables: the first column of the block's tables
     if constexpr (TABLE_FROM_X) {
-        // a plan of one step: its only table straight from X, no gather kernel in front
+        // the first table straight from X, no gather kernel in front
         if (table_base) {
-            // local tables: the block's own H consecutive rows of X, one contiguous read
-            const int c0 = table_base[b];
+            // local tables: step t holds the block's own rows c0 + t H .. c0 + (t + 1) H - 1 of X, one contiguous read
+            const int c0 = local_c0 = table_base[b];
             for (int i = tid; i < H * 4; i += kThreads) table4[i] = c0 + (i >> 2) < n_cols ? X4[(size_t)c0 * 4 + i] : zero4;
         } else {
             for (int i = tid; i < H * 4; i += kThreads) {
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
         for (int i = tid; i < H * 4; i += kThreads) table4[i] = hot_x4[i];
     }
 
-#define RB_PRE_LOAD(k) const float4 pre##k = tid + k * kThreads < H * 4 ? pre_src[tid + k * kThreads] : zero4;
+#define RB_PRE_LOAD(k) const float4 pre##k = tid + k * kThreads < pre_lim ? pre_src[tid + k * kThreads] : zero4;
 #define RB_PRE_STORE(k) if (tid + k * kThreads < H * 4) table4[tid + k * kThreads] = pre##k;
     static_assert(kPrefetch == 6, "one RB_PRE_LOAD / RB_PRE_STORE per float4 of a table that a thread moves");
 
@@ -414,6 +415,13 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             tails(wc, len_c);
             // the next table: on its way while the wavefronts gather at the barrier
             const float4 *pre_src = hot_x4 + (size_t)min(t + 1, T - 1) * H * 4;
+            int pre_lim = H * 4;
+            if constexpr (TABLE_FROM_X) {
+                // local tables: the next H rows of X after this step's, as far as X goes
+                const long long first = (long long)local_c0 + (long long)min(t + 1, T - 1) * H;
+                pre_src = X4 + first * 4;
+                pre_lim = (int)max(0ll, min((long long)H, (long long)n_cols - first)) * 4;
+            }
             RB_PRE_LOAD(0) RB_PRE_LOAD(1) RB_PRE_LOAD(2) RB_PRE_LOAD(3) RB_PRE_LOAD(4) RB_PRE_LOAD(5)
             m = m_next;
 
@@ -605,7 +613,7 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
     // x 8 per row: 9.4 against 11.2 us per product).  With more blocks than CUs the gathers of every block cost more
     // than the launch (R-MAT scale 18 x 16, 512 blocks: 50 against 46 us).
     // Local tables differ from block to block and are contiguous in X: always read there.
-    const bool table_from_x = L.steps == 1 && (L.num_blocks <= 256 || dp->table_base);
+    const bool table_from_x = (L.steps == 1 && L.num_blocks <= 256) || dp->table_base;
     if ((phases & MPS_PHASE_PREPARE) && !table_from_x)
         hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
                            reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);

@@ -67,15 +67,21 @@ inline int windows_of(int entries) { return (entries + kWin - 1) / kWin; }
 struct ColumnMap {
     std::vector<int16_t> step;  // per column
     std::vector<int16_t> slot;  // per column: table slot, -1 = cold
-    // local tables: one step, and block b's table holds the columns base[b] .. base[b] + H - 1
+    // local tables: block b's table of step t holds the columns base[b] + t H .. base[b] + (t + 1) H - 1; the columns
+    // outside base[b] .. base[b] + T H - 1 are cold, in the first step (below) or the last (above)
     const int *base = nullptr;
-    int H = 0;
-    int step_of(int c) const { return base ? 0 : step[(size_t)c]; }
+    int H = 0, T = 1;
+    int step_of(int b, int c) const
+    {
+        if (!base) return step[(size_t)c];
+        const long long d = (long long)c - base[b];
+        return d < 0 ? 0 : (int)std::min<long long>(d / H, T - 1);
+    }
     int slot_of(int b, int c) const
     {
         if (!base) return slot[(size_t)c];
-        const int d = c - base[b];
-        return d >= 0 && d < H ? d : -1;
+        const long long d = (long long)c - base[b];
+        return d >= 0 && d < (long long)T * H ? (int)(d % H) : -1;
     }
 };
 
@@ -134,7 +140,7 @@ void count_block(const int *rp, const int *ci, const ColumnMap &cm, int b, int r
     for (int lr = 0; lr < nr; ++lr)
         for (int e = rp[r0 + lr]; e < rp[r0 + lr + 1]; ++e) {
             const int c = ci[e];
-            ++cnt[((size_t)cm.step_of(c) * nr + lr) * 2 + (cm.slot_of(b, c) < 0)];
+            ++cnt[((size_t)cm.step_of(b, c) * nr + lr) * 2 + (cm.slot_of(b, c) < 0)];
         }
 }
 
@@ -294,12 +300,36 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     }
     if (bp.local_tables) local = true;
     if (local) {
-        // Local tables: one step, and every block's table holds the H consecutive columns in which the block has
-        // the most nonzeros - for a block-diagonal or narrowly banded matrix nearly all of them, gathered from LDS,
-        // and the table is one contiguous read of X.  Worth it where the tables serve most of the nonzeros; a band
-        // wider than a table stays with the slab plans.
+        // Local tables: block b's table of step t holds the H consecutive columns from base[b] + t H - for a
+        // block-diagonal or banded matrix nearly all of the block's nonzeros, gathered from LDS, and a table is one
+        // contiguous read of X.  As many steps as the blocks' column spans need tables (the span that holds all but
+        // the outer 5 % of a block's nonzeros; nine blocks in ten must fit), 8 at most; base[b] is where a window of
+        // T H columns holds the most of the block's nonzeros.  Worth it where the tables serve most of the
+        // nonzeros; a wider band stays with the slab plans.
         if (bp.table_rows <= 0) H = std::min(H, (n + 3) / 4 * 4);
-        T = 1;
+        std::vector<int> span((size_t)L.num_blocks, 1);
+        parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
+            std::vector<int> cols;
+            for (int64_t b = b0; b < b1; ++b) {
+                const int e0 = rp[L.block_row[(size_t)b]], e1 = rp[L.block_row[(size_t)b + 1]];
+                if (e1 == e0) continue;
+                cols.assign(ci + e0, ci + e1);
+                const size_t lo = cols.size() / 40, hi = cols.size() - 1 - cols.size() / 40;
+                std::nth_element(cols.begin(), cols.begin() + (long)lo, cols.end());
+                const int c_lo = cols[lo];
+                std::nth_element(cols.begin(), cols.begin() + (long)hi, cols.end());
+                span[(size_t)b] = cols[hi] - c_lo + 1;
+            }
+        });
+        T = bp.steps;
+        if (T <= 0) {
+            std::vector<int> sorted(span);
+            const size_t at = sorted.size() - 1 - sorted.size() / 10;
+            std::nth_element(sorted.begin(), sorted.begin() + (long)at, sorted.end());
+            T = std::max(1, std::min(8, (sorted[at] + H - 1) / H));
+        }
+        T = std::max(1, std::min(T, (n + H - 1) / H));
+        const long long W = (long long)T * H;
         L.table_base.assign((size_t)L.num_blocks, 0);
         std::atomic<long long> covered{0};
         parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
@@ -310,15 +340,15 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                 std::sort(cols.begin(), cols.end());
                 size_t best = 0, best_at = 0;
                 for (size_t lo = 0, hi = 0; lo < cols.size(); ++lo) {
-                    while (hi < cols.size() && cols[hi] < cols[lo] + H) ++hi;
+                    while (hi < cols.size() && cols[hi] < cols[lo] + W) ++hi;
                     if (hi - lo > best) {
                         best = hi - lo;
                         best_at = lo;
                     }
                 }
-                int base = cols.empty() ? 0 : cols[best_at];
-                base = std::max(0, std::min(base, n - H));  // the whole table inside X where X has H rows
-                L.table_base[(size_t)b] = base;
+                long long base = cols.empty() ? 0 : cols[best_at];
+                base = std::max(0ll, std::min(base, (long long)n - W));  // all tables inside X where X has T H rows
+                L.table_base[(size_t)b] = (int)base;
                 covered.fetch_add((long long)best, std::memory_order_relaxed);
             }
         });
@@ -331,7 +361,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     if (bp.min_table_share_short_rows > 0.0 && n > (1 << 18) && (long long)nnz < 12LL * n &&
         (double)table_nnz[0] < bp.min_table_share_short_rows * (double)nnz)
         return kNotWorthwhile;
-    if (bp.table_rows <= 0) {
+    if (bp.table_rows <= 0 && !local) {
         // no more slots than columns to put in them
         const int need = (n + T - 1) / T;
         if (H > need) H = need;
@@ -352,6 +382,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     if (local) {
         cm.base = L.table_base.data();
         cm.H = H;
+        cm.T = T;
         std::atomic<long long> in_tables{0};
         parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
             long long hits = 0;
@@ -370,8 +401,8 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         L.hot_nnz += d_of(c);
     }
     if (local) {
-        L.cold_begin.assign(2, n);
-        L.cold_begin[0] = 0;
+        L.cold_begin.assign((size_t)T + 1, 0);  // a block's cold columns lie anywhere outside its tables
+        L.cold_begin[(size_t)T] = n;
     } else {
         const long long cold_total = (long long)nnz - L.hot_nnz;
         long long cum = 0;
@@ -452,7 +483,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                     const int c = ci[e];
                     const int slot = cm.slot_of((int)b, c);
                     const int k = slot < 0;
-                    const int pos = off[((size_t)cm.step_of(c) * nr + lr) * 2 + k]++;
+                    const int pos = off[((size_t)cm.step_of((int)b, c) * nr + lr) * 2 + k]++;
                     s_idx[(size_t)pos] = (uint32_t)(k ? c : slot);
                     s_val[(size_t)pos] = val[e];
                     s_src[(size_t)pos] = e;

@@ -225,9 +225,10 @@ def test_uniform_matrix_gets_a_rowblock_plan_too(pkg, orc, dev):
 @pytest.mark.parametrize("kind", ["short_rows", "banded", "long_row"])
 def test_matrices_that_stay_with_the_slab_plans(pkg, orc, dev, kind):
     """No row-block plan unless asked for: many short rows without busy columns (a million rows of 8,
-    columns used evenly), columns that stay near the diagonal (a band of 2,000 columns either side:
-    every block would idle through the steps of the other column ranges), and a row that is many times
-    a CU's share of the nonzeros (rows are not cut across blocks)."""
+    columns used evenly), columns that stay near the diagonal but not near enough for tables of a
+    block's own (a band of 12,000 columns either side: 8 tables would serve half of it, and with global
+    tables every block would idle through the steps of the other column ranges), and a row that is
+    many times a CU's share of the nonzeros (rows are not cut across blocks)."""
     rng = np.random.default_rng(3)
     if kind == "short_rows":
         rp, ci, _ = pkg.graphs.generate("er:n=1000000,deg=8", seed=5)
@@ -235,7 +236,7 @@ def test_matrices_that_stay_with_the_slab_plans(pkg, orc, dev, kind):
         rp, ci, _ = pkg.graphs.generate("chunglu:n=262144,nnz=1000000,gamma=2.1,dmax=50000", seed=5)
         assert np.diff(rp).max() > 2 * ci.size / 256
     else:
-        n, deg, w = 120000, 48, 2000
+        n, deg, w = 120000, 48, 12000
         c = np.arange(n, dtype=np.int64)[:, None] + rng.integers(-w, w + 1, size=(n, deg))
         c = np.clip(c, 0, n - 1)
         c.sort(axis=1)
@@ -269,20 +270,50 @@ def test_local_tables_on_a_block_diagonal_matrix(pkg, orc, dev, forced):
     X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
-    kw = dict(rowblock="force", local_tables=True, rowblock_table_rows=256, rowblock_block_rows=300) if forced else {}
+    kw = dict(rowblock="force", local_tables=True, rowblock_steps=1, rowblock_table_rows=256, rowblock_block_rows=300) if forced else {}
     plan = pkg.spmm.Plan(csr, 16, **kw)
     i = plan.info
     assert i.rowblock_local_tables == 1 and i.rowblock_steps == 1
-    assert (i.hot_nnz > 0.9 * nnz) == (not forced)  # tables of 256 rows miss many of a block's columns
+    assert (i.hot_nnz > 0.9 * nnz) == (not forced)  # one table of 256 rows misses many of a block's columns
     Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
     torch.cuda.synchronize()
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=True)
     assert torch.equal(Y, plan.spmm(d_X))
     base = plan.array(pkg._cabi.MPS_PLAN_ARRAY_RB_TABLE_BASE)
-    assert base.size == i.rowblock_blocks and (base >= 0).all() and (base + i.rowblock_table_rows <= n).all()
+    assert base.size == i.rowblock_blocks and (base >= 0).all() and (base + i.rowblock_steps * i.rowblock_table_rows <= n).all()
     # new values through the source indices
     val2 = pkg.graphs.fill_uniform_f32(nnz, 21, 0.0, 1.0)
     plan.set_values(torch.from_numpy(val2).to(dev))
     ref2, scale2 = orc.spmm_f64(rp, ci, val2, X, want_abs=True)
     check_fp32(plan.spmm(d_X).cpu().numpy(), ref2, scale2, rel_elem=True)
+
+
+def test_local_tables_of_several_steps_on_a_banded_matrix(pkg, orc, dev):
+    """A band of 2,000 columns either side of the diagonal: the library gives every block three tables of
+    consecutive columns, one per step, and nearly every nonzero is gathered from LDS."""
+    rng = np.random.default_rng(4)
+    n, deg, w = 120000, 48, 2000
+    c = np.arange(n, dtype=np.int64)[:, None] + rng.integers(-w, w + 1, size=(n, deg))
+    c = np.clip(c, 0, n - 1)
+    c.sort(axis=1)
+    keep = np.ones(c.shape, dtype=bool)
+    keep[:, 1:] = c[:, 1:] != c[:, :-1]
+    rp = np.zeros(n + 1, dtype=np.int32)
+    rp[1:] = np.cumsum(keep.sum(axis=1))
+    ci = c[keep].astype(np.int32)
+    nnz = ci.size
+    val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
+    X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    plan = pkg.spmm.Plan(csr, 16)
+    i = plan.info
+    assert i.rowblock_local_tables == 1 and i.rowblock_steps == 3 and i.hot_nnz > 0.95 * nnz
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    torch.cuda.synchronize()
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    assert torch.equal(Y, plan.spmm(d_X))
+    slabs = pkg.spmm.Plan(csr, 16, rowblock="off")
+    check_fp32(slabs.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)

@@ -47,7 +47,7 @@ def walk_layout(pkg, lay, X, n):
         cur = base[b].copy()
         for t in range(T):
             if i.rowblock_local_tables:  # the block's own H consecutive rows of X (zeros beyond its end)
-                cols = int(table_base[b]) + np.arange(H)
+                cols = int(table_base[b]) + t * H + np.arange(H)
                 table = np.where((cols < n)[:, None], X[np.minimum(cols, n - 1)], 0.0)
             else:
                 table = np.where(hot_cols[t][:, None] >= 0, X[np.maximum(hot_cols[t], 0)], 0.0)
@@ -77,7 +77,7 @@ def walk_layout(pkg, lay, X, n):
                                 assert e == 0 or (word >> bits[k]) == 0, "only a window's first entry advances rows"
                                 x = table[idx] if k == 0 else X[idx]
                                 if k == 0:
-                                    assert hot_cols[t, idx] >= 0 or (i.rowblock_local_tables and table_base[b] + idx < n)
+                                    assert hot_cols[t, idx] >= 0 or (i.rowblock_local_tables and table_base[b] + t * H + idx < n)
                                 src = int(srcs[k][slot0 + 2 * e])
                                 if src >= 0:
                                     assert real == e, "a window's nonzeros come first, padding after them"
@@ -257,30 +257,35 @@ def test_steps_follow_the_size_of_x_the_work_and_the_skew(pkg, spec, steps, why)
     assert lay.info.rowblock_steps == steps, why
 
 
-@pytest.mark.parametrize("spec,table_rows,block_rows,per_round,share", [
-    ("blockdiag:blocks=40,min=50,max=200,deg=5", 0, 0, 4, 0.95),   # a table covers a block's components
-    ("blockdiag:blocks=40,min=50,max=200,deg=5", 64, 100, 4, 0.2),  # tables narrower than a component: many cold entries
-    ("er:n=300,deg=6", 0, 0, 2, 1.0),                               # fewer columns than table rows: everything is hot
+@pytest.mark.parametrize("spec,steps,table_rows,block_rows,per_round,share,want_steps", [
+    ("blockdiag:blocks=40,min=50,max=200,deg=5", 0, 0, 0, 4, 0.95, 1),    # a table covers a block's components
+    ("blockdiag:blocks=40,min=50,max=200,deg=5", 1, 64, 100, 4, 0.2, 1),  # one table narrower than a component: many cold entries
+    ("blockdiag:blocks=40,min=50,max=200,deg=5", 0, 64, 100, 4, 0.8, 5),  # as many tables of 64 rows as the blocks' column spans need
+    ("blockdiag:blocks=40,min=50,max=200,deg=5", 3, 32, 50, 4, 0.3, 3),   # three tables of 32 rows, cold columns on either side
+    ("er:n=300,deg=6", 0, 0, 0, 2, 1.0, 1),                                # fewer columns than table rows: everything is hot
+    ("er:n=300,deg=6", 0, 20, 16, 2, 0.4, 8),                              # columns all over: 8 tables at most
 ])
-def test_local_tables_walk_reproduces_the_product(pkg, spec, table_rows, block_rows, per_round, share):
-    """MPS_PLAN_LOCAL_TABLES: one step, block b's table holds the columns base[b] .. base[b] + H - 1 (the window
-    with the most of the block's nonzeros), RB_HOT_COLS is unused; the walk over the streams gives the product."""
+def test_local_tables_walk_reproduces_the_product(pkg, spec, steps, table_rows, block_rows, per_round, share, want_steps):
+    """MPS_PLAN_LOCAL_TABLES: block b's table of step t holds the columns base[b] + t H .. base[b] + (t + 1) H - 1
+    (base[b]: the window of T H columns with the most of the block's nonzeros), RB_HOT_COLS is unused; the walk over
+    the streams gives the product."""
     rp, ci, _ = pkg.graphs.generate(spec, seed=3)
     n = rp.size - 1
     rng = np.random.default_rng(12)
     val = rng.random(ci.size).astype(np.float32)
     X = (rng.random((n, 16)) * 2 - 1).astype(np.float64)
-    lay = pkg.spmm.RowBlockLayout(rp, ci, val, table_rows=table_rows, block_rows=block_rows, blocks_per_round=per_round,
-                                  local_tables=True)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, steps=steps, table_rows=table_rows, block_rows=block_rows,
+                                  blocks_per_round=per_round, local_tables=True)
     i = lay.info
-    assert i.rowblock_local_tables == 1 and i.rowblock_steps == 1
+    assert i.rowblock_local_tables == 1 and i.rowblock_steps == want_steps
     assert (lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32) == -1).all()
     base = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_TABLE_BASE, np.int32)
     brow = lay.array(pkg._cabi.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
-    assert (base >= 0).all() and (base <= max(0, n - i.rowblock_table_rows)).all()
+    width = i.rowblock_steps * i.rowblock_table_rows
+    assert (base >= 0).all() and (base <= max(0, n - width)).all()
     # hot_nnz counts the nonzeros whose column lies in their block's window
     blk = np.repeat(np.arange(brow.size - 1), rp[brow[1:]] - rp[brow[:-1]])
-    inside = (ci >= base[blk]) & (ci < base[blk] + i.rowblock_table_rows)
+    inside = (ci >= base[blk]) & (ci < base[blk] + width)
     assert i.hot_nnz == int(inside.sum()) and i.hot_nnz >= share * ci.size - 1e-9
     Y, seen = walk_layout(pkg, lay, X, n)
     assert np.array_equal(np.sort(seen), np.arange(ci.size))
