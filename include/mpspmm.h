@@ -340,11 +340,12 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  * this kind of plan by itself where it was measured to win: fp32, K = 16, X
  * below 192 MiB (3.1 M rows), except for matrices with many short rows and no
  * busy columns (fewer than 12 nonzeros per row on average, more than 2^18
- * rows), matrices whose columns stay near the diagonal but not within a
- * table's width of it (wide bands) and matrices with one row far longer than a
- * CU's share of the nonzeros, which keep the slab plans.  Narrow bands and
- * block-diagonal matrices get local tables (MPS_PLAN_LOCAL_TABLES): one step,
- * every block with a table of the consecutive columns it uses most.  `steps` and the number of blocks follow from the size of X,
+ * rows), matrices whose columns stay near the diagonal but not within 8
+ * tables' width of it (wide bands) and matrices with one row far longer than a
+ * CU's share of the nonzeros, which keep the slab plans.  Bands of up to
+ * 8 tables' width and block-diagonal matrices get local tables
+ * (MPS_PLAN_LOCAL_TABLES): every block with tables of the consecutive
+ * columns it uses most.  `steps` and the number of blocks follow from the size of X,
  * the nonzeros per block and the column histogram.  A caller that passes a
  * cost other than mps_default_cost's, a tpw other than 0 or the maximum, or
  * one of the tiling / hot-column flags is tuning a slab plan and gets one;
@@ -393,9 +394,10 @@ typedef struct mps_plan mps_plan;
 #define MPS_PLAN_FORCE_HOT 8u    /* hot columns even when they hold few nonzeros or rows of X are wider than 64 bytes (fp16: 32) */
 #define MPS_PLAN_NO_ROWBLOCK 16u    /* never build a row-block plan (see below)  */
 #define MPS_PLAN_FORCE_ROWBLOCK 32u /* row-block plan whatever the matrix looks like (fp32, K = 16 only) */
-#define MPS_PLAN_LOCAL_TABLES 1024u  /* row-block plans: one step, every block with a table of consecutive columns of its own
-                                        (what the library builds by itself for matrices whose columns stay within a table's
-                                        width of the diagonal); with MPS_PLAN_FORCE_ROWBLOCK or mps_rowblock_layout_build */
+#define MPS_PLAN_LOCAL_TABLES 1024u  /* row-block plans: every block with tables of consecutive columns of its own, step t the
+                                        table_rows columns from base[b] + t * table_rows (what the library builds by itself for
+                                        matrices whose columns stay within 8 tables' width of the diagonal); with
+                                        MPS_PLAN_FORCE_ROWBLOCK or mps_rowblock_layout_build */
 #define MPS_PLAN_NO_COLUMN_TILES 512u /* untiled plans with rows of X of 512 bytes and more: no passes over 128-byte column tiles */
 #define MPS_PLAN_NO_RESIDENT 256u    /* untiled plans: no streaming hint on the gathers of unpopular columns (see below) */
 #define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
@@ -472,8 +474,9 @@ enum {
                                          (column - first column of the step's range) | piece << index_bits, entry e of a window
                                          holds bits [e p, (e + 1) p) of its rows_advanced, p = 16 - index_bits */
     MPS_PLAN_ARRAY_RB_COLD_BEGIN = 18, /* int[steps + 1]: first column of every step's range of cold columns */
-    MPS_PLAN_ARRAY_RB_TABLE_BASE = 19  /* int[blocks], plans with local tables: block b's table holds the columns base[b] ..
-                                         base[b] + table_rows - 1 (RB_HOT_COLS is all -1 then) */
+    MPS_PLAN_ARRAY_RB_TABLE_BASE = 19  /* int[blocks], plans with local tables: block b's table of step t holds the columns
+                                         base[b] + t * table_rows .. base[b] + (t + 1) * table_rows - 1 (RB_HOT_COLS is all -1
+                                         then, and RB_COLD_BEGIN is 0 for every step: a block's cold columns lie outside its tables) */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,
