@@ -124,6 +124,7 @@ int mps_csr_write(const char *path, int n_rows, const int *row_ptr, const int *c
  *   "blockdiag:blocks=1178,min=100,max=600,deg=5"
  *                                              disjoint random-geometric blocks
  *   "rmat:scale=20,ef=16,a=0.57,b=0.19,c=0.19" R-MAT, duplicates removed
+ *   "band:n=233000,deg=64,width=2000"          banded: Erdos-Renyi inside |row - column| <= width, no self-loops
  * Column ids are sorted and distinct within every row.  The result depends
  * only on (spec, seed), not on the number of host threads.
  * The graph is held by an opaque handle owned by the library. */

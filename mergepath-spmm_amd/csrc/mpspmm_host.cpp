@@ -172,6 +172,53 @@ int gen_er(const Spec &sp, uint64_t seed, mps_graph *g)
 }
 
 // ---------------------------------------------------------------------------
+// Banded: column j of row i present independently with probability
+// deg / (2 width + 1) for 0 < |i - j| <= width (Erdos-Renyi inside the band,
+// no self-loops; rows near the ends are shorter).
+// ---------------------------------------------------------------------------
+template <typename Emit>
+inline void band_row(uint64_t seed, int i, int n, int width, double log1mp, Emit &&emit)
+{
+    Rng r(seed, (uint64_t)i);
+    const int64_t first = std::max<int64_t>(0, (int64_t)i - width), last = std::min<int64_t>(n - 1, (int64_t)i + width);
+    int64_t j = first - 1;
+    for (;;) {
+        double u = r.u01_open0();
+        double skip = std::floor(std::log(u) / log1mp);
+        if (skip > (double)(2 * (int64_t)width + 1)) break;
+        j += 1 + (int64_t)skip;
+        if (j > last) break;
+        if (j != i) emit((int)j);
+    }
+}
+
+int gen_band(const Spec &sp, uint64_t seed, mps_graph *g)
+{
+    int n = (int)sp.get("n", 4096);
+    double deg = sp.get("deg", 8);
+    int width = (int)sp.get("width", 64);
+    if (n < 2 || width < 1 || width >= n || deg <= 0 || deg >= 2.0 * width + 1) return MPS_ERR_FORMAT;
+    double log1mp = std::log1p(-deg / (2.0 * width + 1));
+    std::vector<int> cnt(n);
+    parallel_for(n, 1024, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) {
+            int c = 0;
+            band_row(seed, (int)i, n, width, log1mp, [&](int) { ++c; });
+            cnt[i] = c;
+        }
+    });
+    if (!counts_to_row_ptr(cnt, g->row_ptr)) return MPS_ERR_UNSUPPORTED;
+    g->col_idx.resize(g->row_ptr[n]);
+    parallel_for(n, 1024, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) {
+            int *dst = g->col_idx.data() + g->row_ptr[i];
+            band_row(seed, (int)i, n, width, log1mp, [&](int j) { *dst++ = j; });
+        }
+    });
+    return MPS_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Chung-Lu: edge (u, v), u != v, present independently with probability
 // min(1, w_u w_v / S).  Expected degrees follow a shifted power law over the
 // rank r = 0..n-1:  w_r = dmax * (1 + r / r0)^(-1 / (gamma - 1)); r0 is
@@ -818,6 +865,7 @@ int mps_graph_generate(const char *spec, uint64_t seed, mps_graph **graph_out)
         else if (sp.name == "chunglu") rc = gen_chunglu(sp, seed, g);
         else if (sp.name == "blockdiag") rc = gen_blockdiag(sp, seed, g);
         else if (sp.name == "rmat") rc = gen_rmat(sp, seed, g);
+        else if (sp.name == "band") rc = gen_band(sp, seed, g);
         else rc = MPS_ERR_FORMAT;
     } catch (const std::bad_alloc &) {
         rc = MPS_ERR_UNSUPPORTED;

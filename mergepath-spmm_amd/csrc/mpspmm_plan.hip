@@ -1231,7 +1231,9 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
 // (2) Columns near the diagonal (kMaxLocalShare; block-diagonal 416,349 x 5: .029/.026; banded
 //     233,000 x 64 within 2,000 columns: .160/.114; 500,000 x 64 within 3,000: .427/.287): the blocks
 //     idle through the steps whose column range they do not touch, and a slab plan finds such an X
-//     in L2 anyway.  Bands of 30,000 and 60,000 of 233,000 columns either side have a local share of 0.51 and
+//     in L2 anyway.  Where up to 8 tables of a block's own consecutive columns cover most of its
+//     nonzeros, the builder makes those instead (local tables: .051/.119 and .122/.291 for the two
+//     bands); only wider bands are turned away.  Bands of 30,000 and 60,000 of 233,000 columns either side have a local share of 0.51 and
 //     0.22 (.184/.120, .168/.126), 100,000 columns 0.06 (.133/.123); matrices without locality 0.00.
 // (3) A row far longer than a CU's share of the nonzeros (kMaxLongestRow; power law 262,144 x 4 with
 //     a row of 50,000: .053/.034): rows are not cut across blocks.  R-MAT scale 18 x 16, whose

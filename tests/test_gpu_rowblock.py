@@ -236,15 +236,7 @@ def test_matrices_that_stay_with_the_slab_plans(pkg, orc, dev, kind):
         rp, ci, _ = pkg.graphs.generate("chunglu:n=262144,nnz=1000000,gamma=2.1,dmax=50000", seed=5)
         assert np.diff(rp).max() > 2 * ci.size / 256
     else:
-        n, deg, w = 120000, 48, 12000
-        c = np.arange(n, dtype=np.int64)[:, None] + rng.integers(-w, w + 1, size=(n, deg))
-        c = np.clip(c, 0, n - 1)
-        c.sort(axis=1)
-        keep = np.ones(c.shape, dtype=bool)
-        keep[:, 1:] = c[:, 1:] != c[:, :-1]
-        rp = np.zeros(n + 1, dtype=np.int32)
-        rp[1:] = np.cumsum(keep.sum(axis=1))
-        ci = c[keep].astype(np.int32)
+        rp, ci, _ = pkg.graphs.generate("band:n=120000,deg=48,width=12000", seed=5)
     n, nnz = rp.size - 1, ci.size
     val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
     X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)
@@ -292,16 +284,8 @@ def test_local_tables_on_a_block_diagonal_matrix(pkg, orc, dev, forced):
 def test_local_tables_of_several_steps_on_a_banded_matrix(pkg, orc, dev):
     """A band of 2,000 columns either side of the diagonal: the library gives every block three tables of
     consecutive columns, one per step, and nearly every nonzero is gathered from LDS."""
-    rng = np.random.default_rng(4)
-    n, deg, w = 120000, 48, 2000
-    c = np.arange(n, dtype=np.int64)[:, None] + rng.integers(-w, w + 1, size=(n, deg))
-    c = np.clip(c, 0, n - 1)
-    c.sort(axis=1)
-    keep = np.ones(c.shape, dtype=bool)
-    keep[:, 1:] = c[:, 1:] != c[:, :-1]
-    rp = np.zeros(n + 1, dtype=np.int32)
-    rp[1:] = np.cumsum(keep.sum(axis=1))
-    ci = c[keep].astype(np.int32)
+    rp, ci, _ = pkg.graphs.generate("band:n=120000,deg=48,width=2000", seed=5)
+    n = rp.size - 1
     nnz = ci.size
     val = pkg.graphs.fill_uniform_f32(nnz, 11, 0.0, 1.0)
     X = pkg.graphs.fill_uniform_f32(n * 16, 13, -1.0, 1.0).reshape(n, 16)

@@ -179,7 +179,14 @@ def test_generators_shape_and_determinism(pkg):
     rp, ci, md = g.generate("rmat:scale=12,ef=16,a=0.57,b=0.19,c=0.19", seed=1)
     assert rp.size - 1 == 4096 and 0.5 * 65536 < ci.size <= 65536 and rows_sorted_distinct(rp, ci)
 
-    for bad in ("nosuch:n=3", "er:n=abc", "er:n", "rmat:scale=40"):
+    rp, ci, md = g.generate("band:n=20000,deg=24,width=300", seed=1)
+    n = rp.size - 1
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    assert n == 20000 and rows_sorted_distinct(rp, ci) and not (rows == ci).any() and np.abs(ci - rows).max() == 300
+    inner = np.diff(rp)[300:-300]
+    assert abs(inner.mean() - 24.0 * 600 / 601) < 0.3 and md < 60  # deg / (2 width + 1) per column of the band, none on the diagonal
+
+    for bad in ("nosuch:n=3", "er:n=abc", "er:n", "rmat:scale=40", "band:n=100,deg=8,width=100", "band:n=100,deg=30,width=10"):
         with pytest.raises(pkg.MpsError) as e:
             g.generate(bad, 1)
         assert e.value.status == pkg._cabi.MPS_ERR_FORMAT, bad
@@ -192,7 +199,8 @@ def test_generators_do_not_depend_on_thread_count(pkg):
         "g = e.load_package().graphs\n"
         "h = hashlib.sha256()\n"
         "for s in ('er:n=3000,deg=8', 'chunglu:n=5000,nnz=200000,gamma=2.1,dmax=800',\n"
-        "          'blockdiag:blocks=9,min=100,max=300,deg=5', 'rmat:scale=11,ef=8,a=0.57,b=0.19,c=0.19'):\n"
+        "          'blockdiag:blocks=9,min=100,max=300,deg=5', 'rmat:scale=11,ef=8,a=0.57,b=0.19,c=0.19',\n"
+        "          'band:n=4000,deg=12,width=50'):\n"
         "    rp, ci, _ = g.generate(s, 5); h.update(rp.tobytes()); h.update(ci.tobytes())\n"
         "h.update(g.fill_uniform_f32(100000, 3, -1.0, 1.0).tobytes())\n"
         "print(h.hexdigest())\n" % ROOT)
