@@ -1233,8 +1233,11 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
 //     idle through the steps whose column range they do not touch, and a slab plan finds such an X
 //     in L2 anyway.  Where up to 8 tables of a block's own consecutive columns cover most of its
 //     nonzeros, the builder makes those instead (local tables: .051/.119 and .122/.291 for the two
-//     bands); only wider bands are turned away.  Bands of 30,000 and 60,000 of 233,000 columns either side have a local share of 0.51 and
-//     0.22 (.184/.120, .168/.126), 100,000 columns 0.06 (.133/.123); matrices without locality 0.00.
+//     bands); only wider bands are turned away.  Bands of 30,000 and 60,000 of 233,000 columns
+//     either side have a local share of 0.51 and 0.22 (.184/.120, .168/.126), 100,000 columns 0.06
+//     (.133/.123: not recognised); matrices without locality 0.00.
+//     The uniform rows of 8 under (1) with 4,096 to 60,000 rows are now .009/.014, .010/.015 and
+//     .014/.018: a plan of one step and one round of blocks needs one launch.
 // (3) A row far longer than a CU's share of the nonzeros (kMaxLongestRow; power law 262,144 x 4 with
 //     a row of 50,000: .053/.034): rows are not cut across blocks.  R-MAT scale 18 x 16, whose
 //     longest row is that share, is fine (.046/.059).
