@@ -23,7 +23,7 @@ struct DevicePlan {
     uint32_t *cold_packed = nullptr;  // in packed form (one of the two)
     int *hot_src = nullptr, *cold_src = nullptr;
     long long *wave_base = nullptr;
-    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr, *cold_begin = nullptr, *table_base = nullptr;
+    int *meta = nullptr, *block_row = nullptr, *hot_cols = nullptr, *cold_begin = nullptr, *table_base = nullptr, *table_used = nullptr;
     float *hot_x = nullptr;  // [T][H][16] rows of X of the hot columns, gathered per product
     size_t lds_bytes = 0;
     size_t device_bytes = 0;
@@ -139,7 +139,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                                                             const float4 *__restrict__ X4, TOut *__restrict__ Y, int T,
                                                             int H, int acc_rows, int hot_bits, int cold_bits, int keep_from,
                                                             int cold_ib, const int *__restrict__ table_cols,
-                                                            const int *__restrict__ table_base, int n_cols)
+                                                            const int *__restrict__ table_base,
+                                                            const int *__restrict__ table_used, int n_cols)
 {
     extern __shared__ __align__(16) char smem[];
     float *table = reinterpret_cast<float *>(smem);                         // [H][16]
@@ -159,13 +160,15 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
 
     for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4;
     if (tid < kWaveSlots * 16) slots[tid] = 0.f;
-    int local_c0 = 0;  // local tables: the first column of the block's tables
+    int local_c0 = 0, local_last = H;  // local tables: the first column of the block's tables, the rows of its last table in use
     if constexpr (TABLE_FROM_X) {
         // the first table straight from X, no gather kernel in front
         if (table_base) {
             // local tables: step t holds the block's own rows c0 + t H .. c0 + (t + 1) H - 1 of X, one contiguous read
             const int c0 = local_c0 = table_base[b];
-            for (int i = tid; i < H * 4; i += kThreads) table4[i] = c0 + (i >> 2) < n_cols ? X4[(size_t)c0 * 4 + i] : zero4;
+            local_last = table_used[b];
+            const int rows0 = T == 1 ? local_last : H;
+            for (int i = tid; i < rows0 * 4; i += kThreads) table4[i] = c0 + (i >> 2) < n_cols ? X4[(size_t)c0 * 4 + i] : zero4;
         } else {
             for (int i = tid; i < H * 4; i += kThreads) {
                 const int c = table_cols[i >> 2];
@@ -420,7 +423,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 // local tables: the next H rows of X after this step's, as far as X goes
                 const long long first = (long long)local_c0 + (long long)min(t + 1, T - 1) * H;
                 pre_src = X4 + first * 4;
-                pre_lim = (int)max(0ll, min((long long)H, (long long)n_cols - first)) * 4;
+                pre_lim = (int)max(0ll, min((long long)(t + 2 >= T ? local_last : H), (long long)n_cols - first)) * 4;
             }
             RB_PRE_LOAD(0) RB_PRE_LOAD(1) RB_PRE_LOAD(2) RB_PRE_LOAD(3) RB_PRE_LOAD(4) RB_PRE_LOAD(5)
             m = m_next;
@@ -489,6 +492,7 @@ void destroy(DevicePlan *dp)
     (void)hipFree(dp->cold_packed);
     (void)hipFree(dp->cold_begin);
     (void)hipFree(dp->table_base);
+    (void)hipFree(dp->table_used);
     (void)hipFree(dp->hot_src);
     (void)hipFree(dp->cold_src);
     (void)hipFree(dp->wave_base);
@@ -570,6 +574,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
     }
     if ((rc = upload(dp, &dp->cold_begin, L.cold_begin, st)) != MPS_OK) return fail(rc);
     if (!L.table_base.empty() && (rc = upload(dp, &dp->table_base, L.table_base, st)) != MPS_OK) return fail(rc);
+    if (!L.table_used.empty() && (rc = upload(dp, &dp->table_used, L.table_used, st)) != MPS_OK) return fail(rc);
     if (bp_in.keep_src) {
         if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
         if ((rc = upload(dp, &dp->cold_src, L.cold_src, st)) != MPS_OK) return fail(rc);
@@ -623,7 +628,7 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
                                dp->cold_packed, dp->cold_begin, dp->wave_base, reinterpret_cast<const int4 *>(dp->meta),
                                dp->block_row, reinterpret_cast<const float4 *>(dp->hot_x), reinterpret_cast<const float4 *>(X),
                                Y, L.steps, L.table_rows, L.acc_rows, L.hot_bits, L.cold_bits, dp->keep_from, L.cold_index_bits,
-                               table_from_x ? dp->hot_cols : nullptr, dp->table_base, L.n);
+                               table_from_x ? dp->hot_cols : nullptr, dp->table_base, dp->table_used, L.n);
         };
         if (table_from_x) {
             if (dp->cold_packed) launch(rb_spmm_kernel<float, true, true>);

@@ -93,7 +93,8 @@ struct Layout {
     std::vector<int> block_row;         // [NB + 1]
     std::vector<int> hot_cols;          // [T][H] column of every table slot, -1 = unused
     std::vector<int> cold_begin;        // [T + 1] column-id range of every step's cold columns
-    std::vector<int> table_base;        // [NB] local tables (one step): block b's table is X[base[b] .. base[b] + H); else empty
+    std::vector<int> table_base;        // [NB] local tables: block b's table of step t is X[base[b] + t H .. base[b] + (t + 1) H); else empty
+    std::vector<int> table_used;        // [NB] local tables: rows of the block's last table that its entries refer to (the rest is not loaded)
     std::vector<int> meta;              // [NB][T][16][4] {hot entries, cold entries, first local row, 0}; [..][15] unused
     std::vector<long long> wave_base;   // [NB * 16][2] first round of the wavefront's hot / cold stream; [..][15]: where the block's streams end
     std::vector<Entry> hot, cold;       // rounds of 64 entries

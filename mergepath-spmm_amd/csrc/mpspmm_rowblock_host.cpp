@@ -356,9 +356,10 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     }
     // Many short rows (fewer than 12 nonzeros per row, more than 2^18 rows): a window of the streams holds four
     // nonzeros of one row, step and kind, and the slab plans' sliced stream does as well on such rows - unless the
-    // first table alone serves a good part of the nonzeros.  Local tables do not change that (block-diagonal,
-    // 416,349 rows x 5: .027 against .026 ms).
-    if (bp.min_table_share_short_rows > 0.0 && n > (1 << 18) && (long long)nnz < 12LL * n &&
+    // first table alone serves a good part of the nonzeros, or every block has one table of its own (block-diagonal,
+    // 416,349 rows x 3 / 5 / 10: .023/.023, .025/.025, .029/.039 ms; 2,000,000 rows x 5: .103/.118; banded, 1,000,000
+    // x 4 within 100 columns: .048/.055; but two tables per block, 2,000,000 x 8 within 500: .154/.138).
+    if (!(local && T == 1) && bp.min_table_share_short_rows > 0.0 && n > (1 << 18) && (long long)nnz < 12LL * n &&
         (double)table_nnz[0] < bp.min_table_share_short_rows * (double)nnz)
         return kNotWorthwhile;
     if (bp.table_rows <= 0 && !local) {
@@ -384,10 +385,18 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         cm.H = H;
         cm.T = T;
         std::atomic<long long> in_tables{0};
+        L.table_used.assign((size_t)L.num_blocks, 0);
         parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
             long long hits = 0;
-            for (int64_t b = b0; b < b1; ++b)
-                for (int e = rp[L.block_row[(size_t)b]]; e < rp[L.block_row[(size_t)b + 1]]; ++e) hits += cm.slot_of((int)b, ci[e]) >= 0;
+            for (int64_t b = b0; b < b1; ++b) {
+                int used = 0;
+                for (int e = rp[L.block_row[(size_t)b]]; e < rp[L.block_row[(size_t)b + 1]]; ++e) {
+                    const int slot = cm.slot_of((int)b, ci[e]);
+                    hits += slot >= 0;
+                    if (slot >= 0 && cm.step_of((int)b, ci[e]) == T - 1) used = std::max(used, slot + 1);
+                }
+                L.table_used[(size_t)b] = used;
+            }
             in_tables.fetch_add(hits, std::memory_order_relaxed);
         });
         L.hot_nnz = in_tables.load();
