@@ -1003,10 +1003,15 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
 }
 
 // Raises the dynamic LDS limit of the hot instantiation that launch_spmm<T, TOut, VEC> uses; called once
-// per plan, so that a product launches kernels only (it may run under stream capture).
+// per plan, so that a product launches kernels only (it may run under stream capture).  The limit is one
+// value per kernel: it is set to what a CU holds, whatever this plan needs, so that a plan with a smaller
+// table cannot lower it under an earlier plan that is still in use.
+constexpr size_t kHotLdsLimit = 160 * 1024;
 template <typename T, typename TOut, int VEC>
 int allow_hot_lds_for(size_t bytes)
 {
+    if (bytes > kHotLdsLimit) return MPS_ERR_UNSUPPORTED;
+    bytes = kHotLdsLimit;
     if constexpr (VEC > 1) {
         auto kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, 1, kHotRoundsPerLoad>;
         MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -29,6 +29,7 @@ struct DevicePlan {
     size_t device_bytes = 0;
     size_t hot_slots = 0, cold_slots = 0;
     int keep_from = 0;  // steps from this one on read their streams with plain loads (see kStreamKeepBytes)
+    int num_cus = 256;  // CUs the layout was built for: one round of blocks is at most this many
 };
 
 namespace {
@@ -77,6 +78,10 @@ __device__ __forceinline__ uint4 load_round_packed(__amdgpu_buffer_rsrc_t r, uns
     return make_uint4(t[2] & 0xffffu, t[0], t[2] >> 16, t[1]);
 }
 
+// (a value, not a named constant: a float4 object whose address is taken - by a ?: between two lvalues, by a
+// reference parameter - is given a private-memory slot of its own and reloaded from there)
+__device__ __forceinline__ float4 zero4f() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+
 __device__ __forceinline__ void add4(float4 &a, const float4 &b)
 {
     a.x += b.x;
@@ -93,28 +98,39 @@ struct Walk {
 
 // Lane j of a lane-group (4 lanes) holds entry j of the group's window.  The other lanes read
 // it through a quad permute folded into the instruction that uses it (DPP): no LDS staging, no
-// separate move.  `word`/`val` were written long before (the window's load), so the two wait
-// states that a DPP read needs after a write of its source have passed.
+// separate move.  A DPP read needs two wait states after a vector-ALU write of its source register,
+// and the compiler neither sees a DPP instruction inside an asm statement nor promises where it puts
+// the half-word unpack of a packed entry or a register copy.  So every asm statement below begins
+// with `s_nop 1` (two wait states) and reads its DPP source only after it: the distance holds by
+// construction, whatever wrote the register last.  Outputs are early-clobber: the sources are read
+// again further down the same statement.
 #define RB_QUAD(j) "quad_perm:[" #j "," #j "," #j "," #j "] row_mask:0xf bank_mask:0xf"
-template <int J>
-__device__ __forceinline__ unsigned and_from_lane(unsigned word, unsigned mask)
+// r[j] = word[lane j of the group] & mask, j = 0 .. N - 1
+template <int N>
+__device__ __forceinline__ void and_from_lanes(unsigned word, unsigned mask, unsigned (&r)[N])
 {
-    unsigned r;
-    if constexpr (J == 0) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(0) : "=v"(r) : "v"(word), "v"(mask));
-    if constexpr (J == 1) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(1) : "=v"(r) : "v"(word), "v"(mask));
-    if constexpr (J == 2) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(2) : "=v"(r) : "v"(word), "v"(mask));
-    if constexpr (J == 3) asm("v_and_b32_dpp %0, %1, %2 " RB_QUAD(3) : "=v"(r) : "v"(word), "v"(mask));
-    return r;
+    static_assert(N == 1 || N == 2 || N == 4, "entries of a window that carry a field");
+    if constexpr (N == 1)
+        asm("s_nop 1\n\tv_and_b32_dpp %0, %1, %2 " RB_QUAD(0) : "=&v"(r[0]) : "v"(word), "v"(mask));
+    if constexpr (N == 2)
+        asm("s_nop 1\n\tv_and_b32_dpp %0, %2, %3 " RB_QUAD(0) "\n\tv_and_b32_dpp %1, %2, %3 " RB_QUAD(1)
+            : "=&v"(r[0]), "=&v"(r[1])
+            : "v"(word), "v"(mask));
+    if constexpr (N == 4)
+        asm("s_nop 1\n\tv_and_b32_dpp %0, %4, %5 " RB_QUAD(0) "\n\tv_and_b32_dpp %1, %4, %5 " RB_QUAD(1)
+            "\n\tv_and_b32_dpp %2, %4, %5 " RB_QUAD(2) "\n\tv_and_b32_dpp %3, %4, %5 " RB_QUAD(3)
+            : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3])
+            : "v"(word), "v"(mask));
 }
 // a += val[lane J of the group] * x   (one fused multiply-add per column, as the compiler's fmaf)
 template <int J>
 __device__ __forceinline__ void fma_from_lane(float (&a)[4], float val, const float4 &x)
 {
-#define RB_FMAC(j)                                                                          \
-    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[0]) : "v"(val), "v"(x.x));         \
-    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[1]) : "v"(val), "v"(x.y));         \
-    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[2]) : "v"(val), "v"(x.z));         \
-    asm("v_fmac_f32_dpp %0, %1, %2 " RB_QUAD(j) : "+v"(a[3]) : "v"(val), "v"(x.w));
+#define RB_FMAC(j)                                                                                        \
+    asm("s_nop 1\n\tv_fmac_f32_dpp %0, %4, %5 " RB_QUAD(j) "\n\tv_fmac_f32_dpp %1, %4, %6 " RB_QUAD(j)    \
+        "\n\tv_fmac_f32_dpp %2, %4, %7 " RB_QUAD(j) "\n\tv_fmac_f32_dpp %3, %4, %8 " RB_QUAD(j)           \
+        : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3])                                                  \
+        : "v"(val), "v"(x.x), "v"(x.y), "v"(x.z), "v"(x.w));
     if constexpr (J == 0) { RB_FMAC(0) }
     if constexpr (J == 1) { RB_FMAC(1) }
     if constexpr (J == 2) { RB_FMAC(2) }
@@ -152,13 +168,11 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 2, s = lane & 3;
     const int b = blockIdx.x;
-    const int row0 = block_row[b], nrows = block_row[b + 1] - row0;
-    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
     float4 *table4 = reinterpret_cast<float4 *>(table);
     float4 *acc4 = reinterpret_cast<float4 *>(acc);
     const int4 *meta_b = meta + (size_t)b * T * kWaveSlots;
 
-    for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4;
+    for (int i = tid; i < acc_rows * 4; i += kThreads) acc4[i] = zero4f();
     if (tid < kWaveSlots * 16) slots[tid] = 0.f;
     int local_c0 = 0, local_last = H;  // local tables: the first column of the block's tables, the rows of its last table in use
     if constexpr (TABLE_FROM_X) {
@@ -168,18 +182,18 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             const int c0 = local_c0 = table_base[b];
             local_last = table_used[b];
             const int rows0 = T == 1 ? local_last : H;
-            for (int i = tid; i < rows0 * 4; i += kThreads) table4[i] = c0 + (i >> 2) < n_cols ? X4[(size_t)c0 * 4 + i] : zero4;
+            for (int i = tid; i < rows0 * 4; i += kThreads) table4[i] = c0 + (i >> 2) < n_cols ? X4[(size_t)c0 * 4 + i] : zero4f();
         } else {
             for (int i = tid; i < H * 4; i += kThreads) {
                 const int c = table_cols[i >> 2];
-                table4[i] = c >= 0 ? X4[(size_t)c * 4 + (i & 3)] : zero4;
+                table4[i] = c >= 0 ? X4[(size_t)c * 4 + (i & 3)] : zero4f();
             }
         }
     } else {
         for (int i = tid; i < H * 4; i += kThreads) table4[i] = hot_x4[i];
     }
 
-#define RB_PRE_LOAD(k) const float4 pre##k = tid + k * kThreads < pre_lim ? pre_src[tid + k * kThreads] : zero4;
+#define RB_PRE_LOAD(k) const float4 pre##k = tid + k * kThreads < pre_lim ? pre_src[tid + k * kThreads] : zero4f();
 #define RB_PRE_STORE(k) if (tid + k * kThreads < H * 4) table4[tid + k * kThreads] = pre##k;
     static_assert(kPrefetch == 6, "one RB_PRE_LOAD / RB_PRE_STORE per float4 of a table that a thread moves");
 
@@ -235,33 +249,36 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 w.a[0] = w.a[1] = w.a[2] = w.a[3] = 0.f;
             };
             auto hot_gather = [&](unsigned word, float4 (&x)[kWin]) {
-                x[0] = table4[and_from_lane<0>(word, hmask) * 4 + s];
-                x[1] = table4[and_from_lane<1>(word, hmask) * 4 + s];
-                x[2] = table4[and_from_lane<2>(word, hmask) * 4 + s];
-                x[3] = table4[and_from_lane<3>(word, hmask) * 4 + s];
+                unsigned slot[kWin];
+                and_from_lanes<kWin>(word, hmask, slot);
+#pragma unroll
+                for (int j = 0; j < kWin; ++j) x[j] = table4[slot[j] * 4 + s];
             };
             // (packed cold entries count their columns from the first column of the step's range)
             const char *xb = reinterpret_cast<const char *>(X4) + (CPACK ? (size_t)cold_begin[t] * 64 : (size_t)0);
             auto cold_gather = [&](unsigned word, float4 (&x)[kWin]) {
-                x[0] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<0>(word, cmask) << 6) | (unsigned)(s << 4)));
-                x[1] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<1>(word, cmask) << 6) | (unsigned)(s << 4)));
-                x[2] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<2>(word, cmask) << 6) | (unsigned)(s << 4)));
-                x[3] = *reinterpret_cast<const float4 *>(xb + (size_t)((and_from_lane<3>(word, cmask) << 6) | (unsigned)(s << 4)));
+                unsigned col[kWin];
+                and_from_lanes<kWin>(word, cmask, col);
+#pragma unroll
+                for (int j = 0; j < kWin; ++j)
+                    x[j] = *reinterpret_cast<const float4 *>(xb + (size_t)((col[j] << 6) | (unsigned)(s << 4)));
             };
             // is_hot: a hot window, whose rows_advanced lies in two pieces above the slots of its entries 0 and 1
             // (a packed cold window: in four pieces, one above the column of every entry)
             auto window = [&](auto is_hot, Walk &w, unsigned word, unsigned valbits, const float4 (&x)[kWin], unsigned himask,
                               int bits) {
                 if constexpr (decltype(is_hot)::value) {
-                    const unsigned lo = and_from_lane<0>(word, himask), hi = and_from_lane<1>(word, himask);
-                    if ((lo | hi) != 0) row_end(w, (lo >> kPackedSlotBits) | (hi >> (kPackedSlotBits - kPackedPieceBits)));
+                    unsigned p[2];
+                    and_from_lanes<2>(word, himask, p);
+                    if ((p[0] | p[1]) != 0) row_end(w, (p[0] >> kPackedSlotBits) | (p[1] >> (kPackedSlotBits - kPackedPieceBits)));
                 } else if constexpr (CPACK) {
-                    const unsigned p0 = and_from_lane<0>(word, himask), p1 = and_from_lane<1>(word, himask);
-                    const unsigned p2 = and_from_lane<2>(word, himask), p3 = and_from_lane<3>(word, himask);
-                    if ((p0 | p1 | p2 | p3) != 0) row_end(w, (p0 >> bits) | (p1 >> cs1) | (p2 >> cs2) | (p3 >> cs3));
+                    unsigned p[4];
+                    and_from_lanes<4>(word, himask, p);
+                    if ((p[0] | p[1] | p[2] | p[3]) != 0) row_end(w, (p[0] >> bits) | (p[1] >> cs1) | (p[2] >> cs2) | (p[3] >> cs3));
                 } else {
-                    const unsigned hi = and_from_lane<0>(word, himask);
-                    if (hi != 0) row_end(w, hi >> bits);
+                    unsigned p[1];
+                    and_from_lanes<1>(word, himask, p);
+                    if (p[0] != 0) row_end(w, p[0] >> bits);
                 }
                 const float v = __uint_as_float(valbits);
                 fma_from_lane<0>(w.a, v, x[0]);
@@ -438,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 wave_lds_sync();
                 const bool leader = q < kWaves && (q == 0 || slot_row[q - 1] != slot_first);
                 if (leader) {
-                    float4 sum = zero4;
+                    float4 sum = zero4f();
                     for (int k = q; k < kWaves && slot_row[k] == slot_first; ++k)
                         add4(sum, *reinterpret_cast<const float4 *>(slots + k * 16 + s * 4));
                     float4 *dst = acc4 + (size_t)slot_first * 4 + s;
@@ -447,7 +464,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                     *dst = o;
                 }
                 wave_lds_sync();
-                *reinterpret_cast<float4 *>(slots + lane * 4) = zero4;
+                *reinterpret_cast<float4 *>(slots + lane * 4) = zero4f();
             }
             if (t + 1 < T) {
                 RB_PRE_STORE(0) RB_PRE_STORE(1) RB_PRE_STORE(2) RB_PRE_STORE(3) RB_PRE_STORE(4) RB_PRE_STORE(5)
@@ -458,7 +475,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
 #undef RB_PRE_LOAD
 #undef RB_PRE_STORE
 
-    // the block's rows, once
+    // the block's rows, once (their range is read here, not held in registers across the walk)
+    const int row0 = block_row[b], nrows = block_row[b + 1] - row0;
     for (int i = tid; i < nrows * 4; i += kThreads) {
         const float4 v = acc4[i];
         const float a[4] = {v.x, v.y, v.z, v.w};
@@ -513,6 +531,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
     if (!dp) return MPS_ERR_UNSUPPORTED;
     int rc = MPS_OK;
     auto fail = [&](int code) {
+        (void)hipStreamSynchronize(st);  // uploads from the layout's host arrays may still be in flight
         destroy(dp);
         return code;
     };
@@ -544,6 +563,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
         // (the caller has run mps_csr_validate on the device arrays: the builder indexes by column id)
         if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
+        dp->num_cus = bp.num_cus;
         rc = build_layout(rp, ci, val, n, nnz, K, bp, dp->host);
         if (rc != MPS_OK) return fail(rc);
     } catch (const std::bad_alloc &) {
@@ -591,12 +611,15 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
     }
     dp->lds_bytes = (size_t)(L.table_rows + L.acc_rows) * 64 + kSlotBytes;
     {
+        // The dynamic-LDS limit of a kernel is one value per kernel, not per plan: it is set to the most any plan
+        // can ask for (kLdsBytes), never to this plan's own size, so that a later plan with a smaller table
+        // cannot lower it under an earlier plan that is still in use.
         hipError_t e = hipSuccess;
         for (const void *kernel : {reinterpret_cast<const void *>(rb_spmm_kernel<float, false, false>),
                                    reinterpret_cast<const void *>(rb_spmm_kernel<float, true, false>),
                                    reinterpret_cast<const void *>(rb_spmm_kernel<float, false, true>),
                                    reinterpret_cast<const void *>(rb_spmm_kernel<float, true, true>)})
-            if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dp->lds_bytes);
+            if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
@@ -618,7 +641,7 @@ int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStr
     // x 8 per row: 9.4 against 11.2 us per product).  With more blocks than CUs the gathers of every block cost more
     // than the launch (R-MAT scale 18 x 16, 512 blocks: 50 against 46 us).
     // Local tables differ from block to block and are contiguous in X: always read there.
-    const bool table_from_x = (L.steps == 1 && L.num_blocks <= 256) || dp->table_base;
+    const bool table_from_x = (L.steps == 1 && L.num_blocks <= dp->num_cus) || dp->table_base;
     if ((phases & MPS_PHASE_PREPARE) && !table_from_x)
         hipLaunchKernelGGL(rb_gather_hot_kernel, dim3((unsigned)((slots * 4 + 255) / 256)), dim3(256), 0, st, dp->hot_cols,
                            reinterpret_cast<const float4 *>(X), reinterpret_cast<float4 *>(dp->hot_x), slots);
