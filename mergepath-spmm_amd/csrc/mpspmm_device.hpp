@@ -1007,20 +1007,27 @@ int launch_spmm(const int *row_ptr, const int *col_idx, const T *val, const T *X
 // value per kernel: it is set to what a CU holds, whatever this plan needs, so that a plan with a smaller
 // table cannot lower it under an earlier plan that is still in use.
 constexpr size_t kHotLdsLimit = 160 * 1024;
+inline int raise_dynamic_lds_limit(const void *kernel, size_t bytes)
+{
+    hipFuncAttributes attr;
+    MPS_HIP_TRY(hipFuncGetAttributes(&attr, kernel));
+    if (attr.sharedSizeBytes + bytes > kHotLdsLimit) return MPS_ERR_UNSUPPORTED;
+    // all that a CU holds beside the kernel's own static buffers
+    MPS_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kHotLdsLimit - attr.sharedSizeBytes)));
+    return MPS_OK;
+}
 template <typename T, typename TOut, int VEC>
 int allow_hot_lds_for(size_t bytes)
 {
-    if (bytes > kHotLdsLimit) return MPS_ERR_UNSUPPORTED;
-    bytes = kHotLdsLimit;
     if constexpr (VEC > 1) {
         auto kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, 1, kHotRoundsPerLoad>;
-        MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        (int)bytes));
+        int rc = raise_dynamic_lds_limit(reinterpret_cast<const void *>(kern), bytes);
+        if (rc != MPS_OK) return rc;
         if constexpr (sizeof(T) == 4) {
             // hot columns come with tiled plans, whose partial rows are scaled when they are summed
             auto pattern_kern = mp_spmm_kernel<T, TOut, VEC, true, kGatherBatch, true, true, 1, kHotRoundsPerLoad, 1>;
-            MPS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(pattern_kern),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+            rc = raise_dynamic_lds_limit(reinterpret_cast<const void *>(pattern_kern), bytes);
+            if (rc != MPS_OK) return rc;
         }
         return MPS_OK;
     } else {

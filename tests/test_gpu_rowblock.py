@@ -301,3 +301,28 @@ def test_local_tables_of_several_steps_on_a_banded_matrix(pkg, orc, dev):
     assert torch.equal(Y, plan.spmm(d_X))
     slabs = pkg.spmm.Plan(csr, 16, rowblock="off")
     check_fp32(slabs.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+
+
+def test_rowblock_small_plan_does_not_lower_the_lds_limit_of_a_large_one(pkg, orc, dev):
+    # The dynamic-LDS limit belongs to the kernel, not to a plan: a plan with a full table, then one with a
+    # 16-row table, then the first again - same bits as before the second one existed.
+    rng = np.random.default_rng(77)
+    n = 6000
+    rp, ci = random_csr(rng, n, 90, hub_rows=((11, 5500),))
+    val = rng.random(ci.size).astype(np.float32)
+    X = (rng.random((n, 16)) * 2 - 1).astype(np.float32)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    big = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=2, rowblock_blocks_per_round=8)
+    assert big.info.rowblock_table_rows > 1000  # what fits beside the accumulators: well over 64 KiB of LDS
+    Y0 = big.spmm(d_X).clone()
+    torch.cuda.synchronize()
+    small = pkg.spmm.Plan(csr, 16, rowblock="force", rowblock_steps=2, rowblock_table_rows=16, rowblock_blocks_per_round=8)
+    Ys = small.spmm(d_X)
+    torch.cuda.synchronize()
+    Y1 = big.spmm(d_X, out=torch.full_like(d_X, float("nan")))  # raises if the launch is refused
+    torch.cuda.synchronize()
+    assert torch.equal(Y0, Y1)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    check_fp32(Y1.cpu().numpy(), ref, scale, rel_elem=False)
+    check_fp32(Ys.cpu().numpy(), ref, scale, rel_elem=False)
