@@ -56,6 +56,9 @@ def plan_signature(workload, info):
     """What decides the HBM traffic of a plan's dominant kernel: the workload and the plan's shape."""
     if info is None:
         return "%s|csr" % workload
+    if info.sweep_panels > 0:
+        return "%s|sweep|panels=%d|tiles=%d|acc_rows=%d|piece=%d" % (workload, info.sweep_panels, info.sweep_tiles,
+                                                                     info.sweep_acc_rows, info.sweep_piece)
     if info.rowblock_steps > 0:
         return "%s|rowblock|steps=%d|table_rows=%d|blocks=%d|cold_index_bits=%d" % (
             workload, info.rowblock_steps, info.rowblock_table_rows, info.rowblock_blocks, info.rowblock_cold_index_bits)
@@ -133,6 +136,11 @@ def layout_text(w, plan):
     if plan is None:
         return "plain CSR, no plan"
     i = plan.info
+    if i.sweep_panels > 0:
+        return ("sweep plan: %d panels x %d column tile(s) of %d bytes, %d accumulator rows per panel, pieces of %d, "
+                "%d row(s) cut across panels, %.1f %% padding, %.0f MB"
+                % (i.sweep_panels, i.sweep_tiles, 16 * i.sweep_lanes, i.sweep_acc_rows, i.sweep_piece, i.sweep_split_rows,
+                   100.0 * (i.sweep_slots - w.nnz) / max(w.nnz, 1), i.device_bytes / 1e6))
     if i.rowblock_steps > 0:
         return ("row-block plan: %d blocks, %d steps x %d table rows%s, %.1f %% of the nonzeros from LDS, %.0f MB"
                 % (i.rowblock_blocks, i.rowblock_steps, i.rowblock_table_rows,
@@ -179,6 +187,11 @@ def main():
     ap.add_argument("--rowblock", default="auto", choices=["auto", "off", "force"],
                     help="row-block plan (rows summed in LDS, popular columns' rows of X in LDS tables): where the "
                          "library picks it / never / always")
+    ap.add_argument("--sweep", default="auto", choices=["auto", "off", "force"],
+                    help="sweep plan (rows summed in LDS, nonzeros visited in column order): where the library picks it / "
+                         "never / always")
+    ap.add_argument("--sweep-piece", type=int, default=0, help="sweep plans: most entries of a row per accumulator row (0 = library default)")
+    ap.add_argument("--sweep-acc-rows", type=int, default=0, help="sweep plans: most accumulator rows per panel (0 = what fits in LDS)")
     ap.add_argument("--rb-steps", type=int, default=0, help="steps (LDS tables) of a row-block plan (0 = library default)")
     ap.add_argument("--rb-table-rows", type=int, default=0, help="rows per LDS table of a row-block plan (0 = what fits)")
     ap.add_argument("--resident", default="auto", choices=["auto", "off"],
@@ -241,7 +254,8 @@ def main():
                   slab_bytes=args.slab_bytes, hot=args.hot, rowblock=args.rowblock, rowblock_steps=args.rb_steps,
                   rowblock_table_rows=args.rb_table_rows, keep_sources=False, resident=args.resident,
                   resident_bytes=args.resident_bytes, weights=None if args.weights == "none" else args.weights,
-                  column_tiles=args.column_tiles == "auto")
+                  column_tiles=args.column_tiles == "auto", sweep=args.sweep, sweep_piece=args.sweep_piece,
+                  sweep_acc_rows=args.sweep_acc_rows)
         kw.update(overrides)
         return sp.Plan(wl.csr, wl.K, **kw), cost
 
@@ -256,6 +270,7 @@ def main():
     torch.cuda.synchronize()
     info = plan.info if plan is not None else None
     rowblock = info is not None and info.rowblock_steps > 0
+    sweep = info is not None and info.sweep_panels > 0
     tiled = info is not None and info.num_slabs > 1
 
     def step(phases=None):
@@ -290,7 +305,7 @@ def main():
         row[0].record()
         for k, ph in enumerate(order):
             if (ph == PH.MPS_PHASE_PREPARE and not rowblock) or (ph == PH.MPS_PHASE_REDUCE and not tiled) or \
-               (ph == PH.MPS_PHASE_FIXUP and rowblock):
+               (ph == PH.MPS_PHASE_FIXUP and (rowblock or (sweep and info.sweep_split_rows == 0))):
                 pass
             elif plan is not None or ph in (PH.MPS_PHASE_MAIN, PH.MPS_PHASE_FIXUP):
                 step(ph)
@@ -310,7 +325,7 @@ def main():
 
     gflops = w.flops / (ms_per_step * 1e6)
     achieved = w.b_alg / (main_ms * 1e6)
-    main_name = "rb_spmm_kernel" if rowblock else ("mp_spmm_kernel (hot + cold launch)" if info is not None and info.hot_rows > 0 else "mp_spmm_kernel")
+    main_name = "sw_spmm_kernel" if sweep else "rb_spmm_kernel" if rowblock else ("mp_spmm_kernel (hot + cold launch)" if info is not None and info.hot_rows > 0 else "mp_spmm_kernel")
     signature = plan_signature(name, info)
     traffic, traffic_from = measured_traffic(signature)
     csr_bytes = 4 * (w.n + 1) + (4 + w.eb) * w.nnz

@@ -399,6 +399,8 @@ typedef struct mps_plan mps_plan;
                                         table_rows columns from base[b] + t * table_rows (what the library builds by itself for
                                         matrices whose columns stay within 8 tables' width of the diagonal); with
                                         MPS_PLAN_FORCE_ROWBLOCK or mps_rowblock_layout_build */
+#define MPS_PLAN_NO_SWEEP 2048u     /* never build a sweep plan (see below)       */
+#define MPS_PLAN_FORCE_SWEEP 4096u  /* sweep plan whatever the matrix looks like (rows of X a multiple of 64 bytes) */
 #define MPS_PLAN_NO_COLUMN_TILES 512u /* untiled plans with rows of X of 512 bytes and more: no passes over 128-byte column tiles */
 #define MPS_PLAN_NO_RESIDENT 256u    /* untiled plans: no streaming hint on the gathers of unpopular columns (see below) */
 #define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
@@ -435,6 +437,18 @@ typedef struct mps_plan_info {
     int rowblock_cold_index_bits;  /* row-block plans: > 0 when the cold stream is held in packed form (RB_COLD_PACKED): bits of a
                                       16-bit entry that hold the column, counted from the first column of the step's range */
     int rowblock_local_tables;     /* row-block plans: 1 when every block has a table of its own (RB_TABLE_BASE) */
+    /* sweep plans (sweep_panels > 0); the fields about slabs, partitions, slices and row blocks are then 0 / 1 */
+    int sweep_panels;              /* panels = workgroups per column tile          */
+    int sweep_acc_rows;            /* accumulator rows per panel in LDS            */
+    int sweep_lanes;               /* lanes per lane-group: 4 (64-byte rows of X) or 8 (128-byte column tiles) */
+    int sweep_tiles;               /* column tiles per row of X                    */
+    int sweep_col_bits;            /* an entry word is column | accumulator row << sweep_col_bits */
+    int sweep_piece;               /* most entries of a row that one accumulator row takes */
+    int sweep_split_rows;          /* rows cut into sub-rows that go to different panels */
+    int sweep_partial_rows;        /* sub-rows of those rows                       */
+    int sweep_listed_rows;         /* entries of SW_ROWS: n_rows - split rows + partial rows */
+    long long sweep_rounds;        /* rounds of all wavefronts                     */
+    long long sweep_slots;         /* entry slots incl. padding                    */
 } mps_plan_info;
 
 /* Optional parameters of mps_plan_create_ex; zero means "the library chooses". */
@@ -448,6 +462,9 @@ typedef struct mps_plan_options {
     int degree_weights;      /* 0: values from d_val.  1: the weight of nonzero (r, c) is deg(r) * deg(c), 2: 1 / sqrt(deg(r) * deg(c))
                                 (MPS_WEIGHT_DEGREE_PRODUCT + 1, MPS_WEIGHT_GCN + 1): d_val is not read, see "degree weights" below */
     size_t resident_bytes;   /* rows of X (of the busiest columns) that an untiled plan gathers without the streaming hint; set: whatever the size of X and the skew */
+    int sweep_piece;         /* sweep plans: most entries of a row per accumulator row */
+    int sweep_acc_rows;      /* sweep plans: most accumulator rows per panel (what fits in LDS if 0 or larger) */
+    int sweep_panels_per_round; /* sweep plans: panels are made in multiples of this (0: the number of CUs) */
 } mps_plan_options;
 
 enum {
@@ -475,9 +492,22 @@ enum {
                                          (column - first column of the step's range) | piece << index_bits, entry e of a window
                                          holds bits [e p, (e + 1) p) of its rows_advanced, p = 16 - index_bits */
     MPS_PLAN_ARRAY_RB_COLD_BEGIN = 18, /* int[steps + 1]: first column of every step's range of cold columns */
-    MPS_PLAN_ARRAY_RB_TABLE_BASE = 19  /* int[blocks], plans with local tables: block b's table of step t holds the columns
+    MPS_PLAN_ARRAY_RB_TABLE_BASE = 19, /* int[blocks], plans with local tables: block b's table of step t holds the columns
                                          base[b] + t * table_rows .. base[b] + (t + 1) * table_rows - 1 (RB_HOT_COLS is all -1
                                          then, and RB_COLD_BEGIN is 0 for every step: a block's cold columns lie outside its tables) */
+    /* sweep plans */
+    MPS_PLAN_ARRAY_SW_PANEL_PTR = 20,   /* int[panels + 1]: a panel's listed rows are SW_ROWS[ptr[p] .. ptr[p + 1]) */
+    MPS_PLAN_ARRAY_SW_ROWS = 21,        /* int[listed rows]: the row of Y a listed row is written to; n_rows + s: partial row s */
+    MPS_PLAN_ARRAY_SW_PIECE_PTR = 22,   /* int[listed rows + panels]: per panel (from ptr[p] + p on) listed rows + 1 entries, the
+                                           first accumulator row of every listed row and, last, the panel's count */
+    MPS_PLAN_ARRAY_SW_WAVE_META = 23,   /* int[panels * 16 * 2]: {first round, rounds} of every wavefront */
+    MPS_PLAN_ARRAY_SW_PANEL_ROUNDS = 24, /* int[panels]: most rounds of a wavefront of the panel */
+    MPS_PLAN_ARRAY_SW_STREAM = 25,      /* 8 bytes x slots: per round, lane-group and lane of its quad {word A, value A, word B,
+                                           value B}; word = column | LDS row of the accumulator row << sweep_col_bits, value fp32;
+                                           lane q of a quad holds entry q of windows A and B; padding: value 0 */
+    MPS_PLAN_ARRAY_SW_SRC = 26,         /* int[slots]: original nonzero index, -1 = padding */
+    MPS_PLAN_ARRAY_SW_SPLIT_ROW = 27,   /* int[split rows] */
+    MPS_PLAN_ARRAY_SW_SPLIT_PTR = 28    /* int[split rows + 1]: partial rows of every split row */
 };
 
 int mps_tile_shape(int n_rows, int nnz, int K, int elem_bytes, size_t slab_bytes, int *num_slabs_out,
@@ -508,6 +538,19 @@ int mps_rowblock_layout_info(const mps_rowblock_layout *layout, mps_plan_info *i
 int mps_rowblock_layout_array(const mps_rowblock_layout *layout, int which, const void **data_out,
                               size_t *bytes_out);
 void mps_rowblock_layout_free(mps_rowblock_layout *layout);
+
+/* The layout of a sweep plan, built from host arrays without a GPU: what
+ * mps_plan_create_ex uploads.  val is fp32 whatever elem_bytes (2 or 4: the
+ * type of X and Y, which decides the lane-group width and the accumulator
+ * size).  options: sweep_* fields and MPS_PLAN_NO_SOURCES.
+ * mps_sweep_layout_array hands out a pointer into the layout (valid until it
+ * is freed) for MPS_PLAN_ARRAY_SW_*. */
+typedef struct mps_sweep_layout mps_sweep_layout;
+int mps_sweep_layout_build(const int *row_ptr, const int *col_idx, const float *val, int n_rows, int nnz, int K,
+                           int elem_bytes, const mps_plan_options *options, mps_sweep_layout **layout_out);
+int mps_sweep_layout_info(const mps_sweep_layout *layout, mps_plan_info *info);
+int mps_sweep_layout_array(const mps_sweep_layout *layout, int which, const void **data_out, size_t *bytes_out);
+void mps_sweep_layout_free(mps_sweep_layout *layout);
 
 /* Parameter sweep for one matrix and K — what the reference leaves to the
  * user's hand (cost and partitions per warp are command-line arguments,

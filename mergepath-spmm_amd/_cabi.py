@@ -38,12 +38,16 @@ MPS_PLAN_NO_ROW_MARKS = 128
 MPS_PLAN_NO_RESIDENT = 256
 MPS_PLAN_NO_COLUMN_TILES = 512
 MPS_PLAN_LOCAL_TABLES = 1024
+MPS_PLAN_NO_SWEEP = 2048
+MPS_PLAN_FORCE_SWEEP = 4096
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,
  MPS_PLAN_ARRAY_RB_HOT, MPS_PLAN_ARRAY_RB_COLD, MPS_PLAN_ARRAY_RB_HOT_SRC, MPS_PLAN_ARRAY_RB_COLD_SRC,
  MPS_PLAN_ARRAY_RB_HOT_PACKED, MPS_PLAN_ARRAY_RB_COLD_PACKED, MPS_PLAN_ARRAY_RB_COLD_BEGIN,
- MPS_PLAN_ARRAY_RB_TABLE_BASE) = range(20)
+ MPS_PLAN_ARRAY_RB_TABLE_BASE, MPS_PLAN_ARRAY_SW_PANEL_PTR, MPS_PLAN_ARRAY_SW_ROWS, MPS_PLAN_ARRAY_SW_PIECE_PTR,
+ MPS_PLAN_ARRAY_SW_WAVE_META, MPS_PLAN_ARRAY_SW_PANEL_ROUNDS, MPS_PLAN_ARRAY_SW_STREAM, MPS_PLAN_ARRAY_SW_SRC,
+ MPS_PLAN_ARRAY_SW_SPLIT_ROW, MPS_PLAN_ARRAY_SW_SPLIT_PTR) = range(29)
 
 
 class PlanInfo(ctypes.Structure):
@@ -58,7 +62,10 @@ class PlanInfo(ctypes.Structure):
                 ("rowblock_blocks", ctypes.c_int), ("rowblock_acc_rows", ctypes.c_int),
                 ("rowblock_hot_slots", ctypes.c_longlong), ("rowblock_cold_slots", ctypes.c_longlong),
                 ("resident_cols", ctypes.c_int), ("resident_nnz", ctypes.c_longlong),
-                ("rowblock_cold_index_bits", ctypes.c_int), ("rowblock_local_tables", ctypes.c_int)]
+                ("rowblock_cold_index_bits", ctypes.c_int), ("rowblock_local_tables", ctypes.c_int)] + \
+               [(n, ctypes.c_int) for n in ("sweep_panels", "sweep_acc_rows", "sweep_lanes", "sweep_tiles", "sweep_col_bits",
+                                             "sweep_piece", "sweep_split_rows", "sweep_partial_rows", "sweep_listed_rows")] + \
+               [("sweep_rounds", ctypes.c_longlong), ("sweep_slots", ctypes.c_longlong)]
 
 
 class PlanOptions(ctypes.Structure):
@@ -66,7 +73,8 @@ class PlanOptions(ctypes.Structure):
     _fields_ = [("flags", ctypes.c_uint), ("slab_bytes", ctypes.c_size_t), ("rowblock_steps", ctypes.c_int),
                 ("rowblock_table_rows", ctypes.c_int), ("rowblock_block_rows", ctypes.c_int),
                 ("rowblock_blocks_per_round", ctypes.c_int), ("degree_weights", ctypes.c_int),
-                ("resident_bytes", ctypes.c_size_t)]
+                ("resident_bytes", ctypes.c_size_t), ("sweep_piece", ctypes.c_int), ("sweep_acc_rows", ctypes.c_int),
+                ("sweep_panels_per_round", ctypes.c_int)]
 
 
 class TuneResult(ctypes.Structure):
@@ -122,6 +130,10 @@ PROTOTYPES = {
     "mps_rowblock_layout_info": (_i, [_vp, _vp]),
     "mps_rowblock_layout_array": (_i, [_vp, _i, ctypes.POINTER(_vp), ctypes.POINTER(_sz)]),
     "mps_rowblock_layout_free": (None, [_vp]),
+    "mps_sweep_layout_build": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, ctypes.POINTER(PlanOptions), ctypes.POINTER(_vp)]),
+    "mps_sweep_layout_info": (_i, [_vp, _vp]),
+    "mps_sweep_layout_array": (_i, [_vp, _i, ctypes.POINTER(_vp), ctypes.POINTER(_sz)]),
+    "mps_sweep_layout_free": (None, [_vp]),
     "mps_plan_destroy": (None, [_vp]),
     "mps_plan_get_info": (_i, [_vp, _vp]),
     "mps_plan_set_values": (_i, [_vp, _vp, _vp]),

@@ -16,6 +16,7 @@
 //   4. the workspace of the SpMM (per-slab partial rows, carry-out records).
 #include "mpspmm_device.hpp"
 #include "mpspmm_rowblock.hpp"
+#include "mpspmm_sweep.hpp"
 
 #include <algorithm>
 #include <cmath>
@@ -61,6 +62,7 @@ struct mps_plan {
     float *col_scale = nullptr, *row_scale = nullptr;  // [n_rows] each
     float *xs = nullptr;            // [n_rows * K]
     mps_rb::DevicePlan *rb = nullptr;  // row-block plan: everything above about slabs and slices is unused
+    mps_sw::DevicePlan *sw = nullptr;  // sweep plan: likewise
 };
 
 namespace {
@@ -575,6 +577,7 @@ void plan_free(mps_plan *pl)
 {
     if (!pl) return;
     mps_rb::destroy(pl->rb);
+    mps_sw::destroy(pl->sw);
     (void)hipFree(pl->vrow_ptr);
     (void)hipFree(pl->coord_x);
     (void)hipFree(pl->coord_y);
@@ -1160,6 +1163,7 @@ int plan_spmm(const mps_plan *pl, const T *X, T *Y, unsigned phases, hipStream_t
         if constexpr (sizeof(T) == 4) return mps_rb::spmm(pl->rb, X, Y, phases, st);
         else return MPS_ERR_INVALID_ARG;
     }
+    if (pl->sw) return mps_sw::spmm(pl->sw, X, Y, phases, st);
     const T *vals = static_cast<const T *>(pl->slice_vals);
     void *carry = static_cast<char *>(pl->workspace) + pl->part_bytes;
     PlanLaunch how;
@@ -1257,6 +1261,19 @@ bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, int cost, int t
     return true;
 }
 
+// Sweep plan or not.  Forced: yes.
+bool sweep_wanted(int n_rows, int nnz, int K, int elem_bytes, int cost, int tpw, unsigned flags)
+{
+    if (flags & MPS_PLAN_FORCE_SWEEP) return true;
+    (void)n_rows;
+    (void)nnz;
+    (void)K;
+    (void)elem_bytes;
+    (void)cost;
+    (void)tpw;
+    return false;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1295,13 +1312,14 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     if ((long long)n_rows + 1 + nnz > INT_MAX) return MPS_ERR_UNSUPPORTED;
     if (opt.degree_weights) {
         // built for fp32 and the slab kernels; the source indices serve new values only
-        if (elem_bytes != 4 || (opt.flags & MPS_PLAN_FORCE_ROWBLOCK)) return MPS_ERR_UNSUPPORTED;
-        opt.flags |= MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_NO_SOURCES;
+        if (elem_bytes != 4 || (opt.flags & (MPS_PLAN_FORCE_ROWBLOCK | MPS_PLAN_FORCE_SWEEP))) return MPS_ERR_UNSUPPORTED;
+        opt.flags |= MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_NO_SWEEP | MPS_PLAN_NO_SOURCES;
         opt.flags &= ~MPS_PLAN_NO_ROW_MARKS;
     }
     const unsigned flags = opt.flags;
     const size_t slab_bytes = opt.slab_bytes;
     if ((flags & MPS_PLAN_FORCE_ROWBLOCK) && (flags & (MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_TILING))) return MPS_ERR_INVALID_ARG;
+    if ((flags & MPS_PLAN_FORCE_SWEEP) && (flags & (MPS_PLAN_NO_SWEEP | MPS_PLAN_FORCE_TILING | MPS_PLAN_FORCE_ROWBLOCK))) return MPS_ERR_INVALID_ARG;
     mps_plan *pl = new (std::nothrow) mps_plan;
     if (!pl) return MPS_ERR_UNSUPPORTED;
     pl->n_rows = n_rows;
@@ -1311,6 +1329,36 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     pl->cost = cost;
     pl->keep_sources = !(flags & MPS_PLAN_NO_SOURCES);
     pl->weights = opt.degree_weights;
+    if (sweep_wanted(n_rows, nnz, K, elem_bytes, cost, tpw, flags)) {
+        if (n_rows < 1 || ((long long)K * elem_bytes) % 64 != 0) {
+            plan_free(pl);
+            return MPS_ERR_UNSUPPORTED;
+        }
+        // the builder indexes X and its own tables by column id
+        int vrc = mps_csr_validate(d_row_ptr, d_col_idx, n_rows, n_rows, nnz, stream);
+        if (vrc != MPS_OK) {
+            plan_free(pl);
+            return vrc;
+        }
+        mps_sw::BuildParams bp;
+        bp.piece = opt.sweep_piece;
+        bp.acc_rows = opt.sweep_acc_rows;
+        bp.num_cus = opt.sweep_panels_per_round;  // 0: ask the device
+        bp.elem_bytes = elem_bytes;
+        bp.keep_src = pl->keep_sources;
+        int rc = mps_sw::create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, bp, static_cast<hipStream_t>(stream), &pl->sw);
+        if (rc == MPS_OK) {
+            pl->device_bytes = mps_sw::device_bytes_of(pl->sw);
+            make_spmm_shape(n_rows, K, 1, 0, elem_bytes, pl->shape);
+            *plan_out = pl;
+            return MPS_OK;
+        }
+        if (rc != MPS_ERR_UNSUPPORTED || (flags & MPS_PLAN_FORCE_SWEEP)) {
+            plan_free(pl);
+            return rc;
+        }
+        // (column ids that leave no room for the accumulator row in an entry word: another kind of plan below)
+    }
     if (rowblock_wanted(n_rows, nnz, K, elem_bytes, cost, tpw, flags)) {
         if (elem_bytes != 4 || K != 16 || n_rows < 1) {
             plan_free(pl);
@@ -1395,6 +1443,14 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->rowblock_hot_slots = info->rowblock_cold_slots = 0;
     info->rowblock_cold_index_bits = 0;
     info->rowblock_local_tables = 0;
+    info->sweep_panels = info->sweep_acc_rows = info->sweep_lanes = info->sweep_tiles = info->sweep_col_bits = 0;
+    info->sweep_piece = info->sweep_split_rows = info->sweep_partial_rows = info->sweep_listed_rows = 0;
+    info->sweep_rounds = info->sweep_slots = 0;
+    if (plan->sw) {
+        info->num_slabs = 1;
+        info->slab_cols = plan->n_rows;
+        mps_sw::fill_info(mps_sw::layout_of(plan->sw), info);
+    }
     if (plan->rb) {
         const mps_rb::Layout &L = mps_rb::layout_of(plan->rb);
         info->num_slabs = 1;
@@ -1419,6 +1475,7 @@ int mps_plan_set_values(mps_plan *plan, const void *d_val, void *stream)
     if (!plan || (plan->nnz > 0 && !d_val)) return MPS_ERR_INVALID_ARG;
     if (!plan->keep_sources || plan->weights) return MPS_ERR_UNSUPPORTED;
     if (plan->rb) return mps_rb::set_values(plan->rb, static_cast<const float *>(d_val), static_cast<hipStream_t>(stream));
+    if (plan->sw) return mps_sw::set_values(plan->sw, d_val, static_cast<hipStream_t>(stream));
     return plan_set_values(plan, d_val, static_cast<hipStream_t>(stream));
 }
 
@@ -1441,12 +1498,17 @@ int mps_plan_copy_array(const mps_plan *plan, int which, void *host_dst, size_t 
         have = (size_t)(plan->hot_rows > 0 ? plan->num_slabs : 0) * (size_t)plan->hot_rows * sizeof(int);
         break;
     default:
+        if (which >= MPS_PLAN_ARRAY_SW_PANEL_PTR && which <= MPS_PLAN_ARRAY_SW_SPLIT_PTR) {
+            if (!plan->sw) return MPS_ERR_INVALID_ARG;
+            src = mps_sw::device_array(plan->sw, which, &have);
+            break;
+        }
         if (!plan->rb) return MPS_ERR_INVALID_ARG;
         src = mps_rb::device_array(plan->rb, which, &have);
         if (!src && have == 0 && (which < MPS_PLAN_ARRAY_RB_BLOCK_ROW || which > MPS_PLAN_ARRAY_RB_TABLE_BASE)) return MPS_ERR_INVALID_ARG;
         break;
     }
-    if (plan->rb && which < MPS_PLAN_ARRAY_RB_BLOCK_ROW) return MPS_ERR_INVALID_ARG;
+    if ((plan->rb || plan->sw) && which < MPS_PLAN_ARRAY_RB_BLOCK_ROW) return MPS_ERR_INVALID_ARG;
     if (bytes != have) return MPS_ERR_INVALID_ARG;
     if (have == 0) return MPS_OK;
     MPS_HIP_TRY(hipMemcpy(host_dst, src, have, hipMemcpyDeviceToHost));

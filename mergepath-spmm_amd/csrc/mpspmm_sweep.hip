@@ -1,0 +1,400 @@
+// Sweep plans, device side: the kernel that walks the layout of
+// mpspmm_sweep.hpp, the fix-up of rows that were cut across panels, and the
+// plan object's device arrays.
+//
+// Same arithmetic as the reference kernel (src/MergePathSpMM.cu:426-477: one
+// fp32 accumulator per output column, a product added per nonzero; the fp16
+// variant src/MergePathSpMM_fp16.cu:427-477 with fp32 sums, as the oracle's
+// orc_spmm_f64_f16in prescribes), with explicit values in place of the degree
+// product (:450, :459-460).  What differs is the order of the nonzeros (by
+// column within a wavefront, so that the gathers of the whole chip stay within
+// a narrow range of X) and where a row is summed (an LDS accumulator row that
+// one wavefront owns, instead of atomics on Y, :445, :477).
+#include "mpspmm_device.hpp"
+#include "mpspmm_sweep.hpp"
+
+#include <new>
+
+namespace mps_sw {
+
+struct DevicePlan {
+    Layout host;  // the small tables stay filled; stream and src are released after the upload
+    uint32_t *stream = nullptr;
+    int *src = nullptr;
+    int *panel_ptr = nullptr, *rows = nullptr, *piece_ptr = nullptr, *wave_meta = nullptr, *panel_rounds = nullptr;
+    int *split_row = nullptr, *split_ptr = nullptr;
+    float *partial = nullptr;  // [partial rows][K] fp32 sums of the sub-rows of split rows
+    size_t lds_bytes = 0, device_bytes = 0, slots = 0;
+};
+
+namespace {
+
+typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+
+// Entry j of the lane-group's window sits in lane j of the quad; all lanes of the quad read it.  (A compiler-made
+// DPP move: the compiler keeps the wait states a DPP read needs after a write of its source.)
+template <int J>
+__device__ __forceinline__ unsigned from_lane(unsigned v)
+{
+    return (unsigned)__builtin_amdgcn_mov_dpp((int)v, J | (J << 2) | (J << 4) | (J << 6), 0xf, 0xf, true);
+}
+
+// 16 bytes of a row of X as fp32 values: 4 floats, or 8 halves widened
+template <typename T>
+struct Piece;
+template <>
+struct Piece<float> {
+    static constexpr int kVec = 4, kPlanes = 1;
+    f4_t raw;
+    __device__ __forceinline__ void load(const char *p) { raw = *reinterpret_cast<const f4_t *>(p); }
+    __device__ __forceinline__ f4_t plane(int) const { return raw; }
+};
+template <>
+struct Piece<half_t> {
+    static constexpr int kVec = 8, kPlanes = 2;
+    half8_t raw;
+    __device__ __forceinline__ void load(const char *p) { raw = *reinterpret_cast<const half8_t *>(p); }
+    __device__ __forceinline__ f4_t plane(int q) const
+    {
+        return q == 0 ? f4_t{(float)raw[0], (float)raw[1], (float)raw[2], (float)raw[3]}
+                      : f4_t{(float)raw[4], (float)raw[5], (float)raw[6], (float)raw[7]};
+    }
+};
+
+// T: element type of X and Y.  L: lanes per lane-group (16 L bytes of a row of X per tile).
+// LDS: kPlanes planes of (acc_rows + 1) x L float4: plane q holds elements 4 q .. 4 q + 3 of every lane's 16 bytes, so
+// that one 16-byte LDS access per lane covers a plane's row exactly like an fp32 row.
+template <typename T, int L>
+__global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restrict__ stream, const int2 *__restrict__ wave_meta,
+                                                            const int *__restrict__ panel_rounds,
+                                                            const int *__restrict__ panel_ptr, const int *__restrict__ rows,
+                                                            const int *__restrict__ piece_ptr, const T *__restrict__ X,
+                                                            T *__restrict__ Y, float *__restrict__ partial, int n, int K,
+                                                            int acc_rows, int col_bits, int bank_rows)
+{
+    extern __shared__ __align__(16) char smem[];
+    f4_t *acc4 = reinterpret_cast<f4_t *>(smem);
+    using P = Piece<T>;
+    constexpr int GPW = 64 / L;        // lane-groups of a wavefront
+    constexpr int RQ = GPW * kWin;     // 16-byte units of a round
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int b = blockIdx.x, tile = blockIdx.y;
+    const int g = lane / L, c = lane % L, s = lane & 3;
+    const int plane_stride = (acc_rows + 1) * L;  // float4 units
+    const f4_t zero = {0.f, 0.f, 0.f, 0.f};
+    for (int i = tid; i < plane_stride * P::kPlanes; i += kThreads) acc4[i] = zero;
+
+    const int2 wm = wave_meta[b * kWaves + wave];
+    const int rounds = __builtin_amdgcn_readfirstlane(wm.y);
+    const int most = panel_rounds[b];
+    const uint4 *ws = stream + (size_t)wm.x * RQ + (g * kWin + s);
+    const unsigned cmask = (1u << col_bits) - 1u;
+    // this lane's 16 bytes of a row of X: row pitch K elements, tile `tile`, piece c
+    const size_t row_pitch = (size_t)K * sizeof(T);
+    const char *xb = reinterpret_cast<const char *>(X) + (size_t)tile * (16 * L) + (size_t)c * 16;
+
+    auto stream_load = [&](int r) {
+        const u4_t t = __builtin_nontemporal_load(reinterpret_cast<const u4_t *>(ws + (size_t)r * RQ));
+        return make_uint4(t[0], t[1], t[2], t[3]);
+    };
+    uint4 nx = make_uint4(0u, 0u, 0u, 0u);
+    if (rounds > 0) nx = stream_load(0);
+    for (int r = 0; r < most; ++r) {
+        // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
+        // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
+        // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
+        if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
+        if (r >= rounds) continue;
+        const uint4 cu = nx;
+        P xa[kWin], xw[kWin];
+#define SW_GATHER(dst, WORD, j) dst[j].load(xb + (size_t)(from_lane<j>(WORD) & cmask) * row_pitch);
+        SW_GATHER(xa, cu.x, 0) SW_GATHER(xa, cu.x, 1) SW_GATHER(xa, cu.x, 2) SW_GATHER(xa, cu.x, 3)
+        SW_GATHER(xw, cu.z, 0) SW_GATHER(xw, cu.z, 1) SW_GATHER(xw, cu.z, 2) SW_GATHER(xw, cu.z, 3)
+#undef SW_GATHER
+        if (r + 1 < rounds) nx = stream_load(r + 1);
+        // One entry after the other: read the accumulator row, add, write it back.  The LDS serves a wavefront's
+        // accesses in order, so an entry sees what the entry before it wrote; the lane-groups of one instruction
+        // hold different rows (the builder's rule); no other wavefront touches this one's rows.
+#define SW_ADD(xs, WORD, VAL, j)                                                       \
+    {                                                                                  \
+        const unsigned vr = from_lane<j>(WORD) >> col_bits;                            \
+        const float v = __uint_as_float(from_lane<j>(VAL));                            \
+        _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
+        {                                                                              \
+            f4_t *at = acc4 + q * plane_stride + vr * L + c;                           \
+            const f4_t x = xs[j].plane(q);                                             \
+            f4_t a = *at;                                                              \
+            a[0] = fmaf(v, x[0], a[0]);                                                \
+            a[1] = fmaf(v, x[1], a[1]);                                                \
+            a[2] = fmaf(v, x[2], a[2]);                                                \
+            a[3] = fmaf(v, x[3], a[3]);                                                \
+            *at = a;                                                                   \
+        }                                                                              \
+    }
+        SW_ADD(xa, cu.x, cu.y, 0) SW_ADD(xa, cu.x, cu.y, 1) SW_ADD(xa, cu.x, cu.y, 2) SW_ADD(xa, cu.x, cu.y, 3)
+        SW_ADD(xw, cu.z, cu.w, 0) SW_ADD(xw, cu.z, cu.w, 1) SW_ADD(xw, cu.z, cu.w, 2) SW_ADD(xw, cu.z, cu.w, 3)
+#undef SW_ADD
+    }
+    __syncthreads();
+
+    // the panel's rows, once: a row's pieces added up in order, rows without nonzeros as zeros
+    const int p0 = panel_ptr[b], nrows = panel_ptr[b + 1] - p0;
+    const int *pp = piece_ptr + p0 + b;
+    for (int i = tid; i < nrows * L; i += kThreads) {
+        const int k = i / L, cc = i % L;
+        const int row = rows[p0 + k];
+        const int a0 = pp[k], a1 = pp[k + 1];
+        float sum[P::kVec];
+#pragma unroll
+        for (int e = 0; e < P::kVec; ++e) sum[e] = 0.f;
+        for (int p = a0; p < a1; ++p) {
+            const int vr = p ^ (((p >> 2) ^ (p >> 4) ^ (p >> 6)) & (bank_rows - 1));
+#pragma unroll
+            for (int q = 0; q < P::kPlanes; ++q) {
+                const f4_t a = acc4[q * plane_stride + vr * L + cc];
+                sum[4 * q] += a[0];
+                sum[4 * q + 1] += a[1];
+                sum[4 * q + 2] += a[2];
+                sum[4 * q + 3] += a[3];
+            }
+        }
+        const size_t col0 = (size_t)tile * (L * P::kVec) + (size_t)cc * P::kVec;
+        if (row < n) {
+            store_acc<P::kVec, true>(Y + (size_t)row * K + col0, sum);
+        } else {
+            store_acc<P::kVec, false>(partial + (size_t)(row - n) * K + col0, sum);  // read again by the fix-up kernel
+        }
+    }
+}
+
+// Y[split_row[i]][:] = the sum of its partial rows, in order.
+template <typename T>
+__global__ __launch_bounds__(256) void sw_fixup_kernel(const int *__restrict__ split_row, const int *__restrict__ split_ptr,
+                                                        const float *__restrict__ partial, T *__restrict__ Y, int n_split, int K)
+{
+    const int quads = K / 4;
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long long)n_split * quads) return;
+    const int r = (int)(i / quads), q = (int)(i % quads);
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int p = split_ptr[r]; p < split_ptr[r + 1]; ++p) {
+        const f4_t a = *reinterpret_cast<const f4_t *>(partial + (size_t)p * K + 4 * q);
+        sum[0] += a[0];
+        sum[1] += a[1];
+        sum[2] += a[2];
+        sum[3] += a[3];
+    }
+    store_acc<4, true>(Y + (size_t)split_row[r] * K + 4 * q, sum);
+}
+
+// New values into the stream: entry slot i (stream order) holds nonzero src[i].
+template <typename T>
+__global__ __launch_bounds__(256) void sw_set_values_kernel(const T *__restrict__ val, const int *__restrict__ src, size_t slots,
+                                                             uint32_t *__restrict__ stream)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= slots) return;
+    const int e = src[i];
+    if (e >= 0) stream[2 * i + 1] = __float_as_uint((float)val[e]);
+}
+
+__global__ __launch_bounds__(256) void sw_widen_values_kernel(const half_t *__restrict__ in, float *__restrict__ out, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (float)in[i];
+}
+
+template <typename T>
+int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
+{
+    const size_t bytes = (src.size() ? src.size() : 1) * sizeof(T);
+    MPS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(dst), bytes));
+    dp->device_bytes += bytes;
+    if (!src.empty()) MPS_HIP_TRY(hipMemcpyAsync(*dst, src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice, st));
+    return MPS_OK;
+}
+
+template <typename T, int L>
+int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
+{
+    const Layout &Lo = dp->host;
+    hipLaunchKernelGGL((sw_spmm_kernel<T, L>), dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles), dim3(kThreads), dp->lds_bytes, st,
+                       reinterpret_cast<const uint4 *>(dp->stream), reinterpret_cast<const int2 *>(dp->wave_meta),
+                       dp->panel_rounds, dp->panel_ptr, dp->rows, dp->piece_ptr, X, Y, dp->partial, Lo.n, Lo.K, Lo.acc_rows,
+                       Lo.col_bits, Lo.bank_rows);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+template <typename T>
+int spmm_typed(const DevicePlan *dp, const T *X, T *Y, unsigned phases, hipStream_t st)
+{
+    const Layout &Lo = dp->host;
+    if (phases & MPS_PHASE_MAIN) {
+        const int rc = Lo.lanes == 8 ? launch_main<T, 8>(dp, X, Y, st) : launch_main<T, 4>(dp, X, Y, st);
+        if (rc != MPS_OK) return rc;
+    }
+    if ((phases & MPS_PHASE_FIXUP) && !Lo.split_row.empty()) {
+        const long long threads = (long long)Lo.split_row.size() * (Lo.K / 4);
+        hipLaunchKernelGGL((sw_fixup_kernel<T>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, dp->split_row,
+                           dp->split_ptr, dp->partial, Y, (int)Lo.split_row.size(), Lo.K);
+        MPS_HIP_TRY(hipGetLastError());
+    }
+    return MPS_OK;
+}
+
+}  // namespace
+
+void destroy(DevicePlan *dp)
+{
+    if (!dp) return;
+    (void)hipFree(dp->stream);
+    (void)hipFree(dp->src);
+    (void)hipFree(dp->panel_ptr);
+    (void)hipFree(dp->rows);
+    (void)hipFree(dp->piece_ptr);
+    (void)hipFree(dp->wave_meta);
+    (void)hipFree(dp->panel_rounds);
+    (void)hipFree(dp->split_row);
+    (void)hipFree(dp->split_ptr);
+    (void)hipFree(dp->partial);
+    delete dp;
+}
+
+// Copies the CSR arrays to the host, builds the layout there and uploads it.  The arrays must have passed
+// mps_csr_validate.  d_val: fp32 or fp16 by bp.elem_bytes.
+int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n, int nnz, int K, const BuildParams &bp_in,
+           hipStream_t st, DevicePlan **out)
+{
+    *out = nullptr;
+    DevicePlan *dp = new (std::nothrow) DevicePlan;
+    if (!dp) return MPS_ERR_UNSUPPORTED;
+    int rc = MPS_OK;
+    auto fail = [&](int code) {
+        (void)hipStreamSynchronize(st);  // uploads from the layout's host arrays may still be in flight
+        destroy(dp);
+        return code;
+    };
+    try {
+        BuildParams bp = bp_in;
+        if (bp.num_cus <= 0) {
+            int dev = 0, cus = 256;
+            hipError_t e = hipGetDevice(&dev);
+            if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            bp.num_cus = cus;
+        }
+        // the CSR arrays come back into pinned host memory (a pageable target takes ten times as long) and are
+        // released as soon as the layout is built; half values are widened on the device first (exact)
+        struct Pinned {
+            void *p = nullptr;
+            ~Pinned() { if (p) (void)hipHostFree(p); }
+        } h_rp, h_ci, h_val;
+        struct Dev {
+            void *p = nullptr;
+            ~Dev() { if (p) (void)hipFree(p); }
+        } wide;
+        hipError_t e = hipHostMalloc(&h_rp.p, ((size_t)n + 1) * sizeof(int), hipHostMallocDefault);
+        if (e == hipSuccess) e = hipHostMalloc(&h_ci.p, ((size_t)nnz + 1) * sizeof(int), hipHostMallocDefault);
+        if (e == hipSuccess) e = hipHostMalloc(&h_val.p, ((size_t)nnz + 1) * sizeof(float), hipHostMallocDefault);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+        const float *val_src = static_cast<const float *>(d_val);
+        if (bp.elem_bytes == 2 && nnz > 0) {
+            e = hipMalloc(&wide.p, (size_t)nnz * sizeof(float));
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            hipLaunchKernelGGL(sw_widen_values_kernel, dim3((unsigned)(((size_t)nnz + 255) / 256)), dim3(256), 0, st,
+                               static_cast<const half_t *>(d_val), static_cast<float *>(wide.p), (size_t)nnz);
+            val_src = static_cast<const float *>(wide.p);
+        }
+        int *rp = static_cast<int *>(h_rp.p), *ci = static_cast<int *>(h_ci.p);
+        float *val = static_cast<float *>(h_val.p);
+        e = hipMemcpyAsync(rp, d_row_ptr, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(ci, d_col_idx, (size_t)nnz * sizeof(int), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(val, val_src, (size_t)nnz * sizeof(float), hipMemcpyDeviceToHost, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+        if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
+        rc = build_layout(rp, ci, val, n, nnz, K, bp, dp->host);
+        if (rc != MPS_OK) return fail(rc);
+    } catch (const std::bad_alloc &) {
+        return fail(MPS_ERR_UNSUPPORTED);
+    }
+    Layout &Lo = dp->host;
+    dp->slots = Lo.stream.size() / 2;
+    if ((rc = upload(dp, &dp->stream, Lo.stream, st)) != MPS_OK) return fail(rc);
+    if (bp_in.keep_src && (rc = upload(dp, &dp->src, Lo.src, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->panel_ptr, Lo.panel_ptr, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->rows, Lo.rows, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->piece_ptr, Lo.piece_ptr, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->wave_meta, Lo.wave_meta, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->panel_rounds, Lo.panel_rounds, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->split_row, Lo.split_row, st)) != MPS_OK) return fail(rc);
+    if ((rc = upload(dp, &dp->split_ptr, Lo.split_ptr, st)) != MPS_OK) return fail(rc);
+    {
+        const size_t bytes = ((size_t)Lo.split_ptr.back() * Lo.K + 4) * sizeof(float);
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&dp->partial), bytes);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+        dp->device_bytes += bytes;
+    }
+    dp->lds_bytes = (size_t)(Lo.acc_rows + 1) * Lo.lanes * 16 * (4 / Lo.elem_bytes);
+    {
+        // the limit belongs to the kernel, not to a plan: always what a CU holds
+        hipError_t e = hipSuccess;
+        for (const void *kernel : {reinterpret_cast<const void *>(sw_spmm_kernel<float, 4>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8>)})
+            if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+    }
+    std::vector<uint32_t>().swap(Lo.stream);
+    std::vector<int>().swap(Lo.src);
+    *out = dp;
+    return MPS_OK;
+}
+
+int spmm(const DevicePlan *dp, const void *X, void *Y, unsigned phases, hipStream_t st)
+{
+    if (dp->host.elem_bytes == 4) return spmm_typed<float>(dp, static_cast<const float *>(X), static_cast<float *>(Y), phases, st);
+    return spmm_typed<half_t>(dp, static_cast<const half_t *>(X), static_cast<half_t *>(Y), phases, st);
+}
+
+int set_values(DevicePlan *dp, const void *d_val, hipStream_t st)
+{
+    if (!dp->src) return MPS_ERR_UNSUPPORTED;
+    if (dp->slots == 0) return MPS_OK;
+    const dim3 grid((unsigned)((dp->slots + 255) / 256));
+    if (dp->host.elem_bytes == 4)
+        hipLaunchKernelGGL((sw_set_values_kernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(d_val), dp->src,
+                           dp->slots, dp->stream);
+    else
+        hipLaunchKernelGGL((sw_set_values_kernel<half_t>), grid, dim3(256), 0, st, static_cast<const half_t *>(d_val), dp->src,
+                           dp->slots, dp->stream);
+    MPS_HIP_TRY(hipGetLastError());
+    return MPS_OK;
+}
+
+const Layout &layout_of(const DevicePlan *dp) { return dp->host; }
+size_t device_bytes_of(const DevicePlan *dp) { return dp->device_bytes; }
+
+const void *device_array(const DevicePlan *dp, int which, size_t *bytes)
+{
+    const Layout &Lo = dp->host;
+    switch (which) {
+    case MPS_PLAN_ARRAY_SW_PANEL_PTR: *bytes = Lo.panel_ptr.size() * sizeof(int); return dp->panel_ptr;
+    case MPS_PLAN_ARRAY_SW_ROWS: *bytes = Lo.rows.size() * sizeof(int); return dp->rows;
+    case MPS_PLAN_ARRAY_SW_PIECE_PTR: *bytes = Lo.piece_ptr.size() * sizeof(int); return dp->piece_ptr;
+    case MPS_PLAN_ARRAY_SW_WAVE_META: *bytes = Lo.wave_meta.size() * sizeof(int); return dp->wave_meta;
+    case MPS_PLAN_ARRAY_SW_PANEL_ROUNDS: *bytes = Lo.panel_rounds.size() * sizeof(int); return dp->panel_rounds;
+    case MPS_PLAN_ARRAY_SW_STREAM: *bytes = dp->slots * 8; return dp->stream;
+    case MPS_PLAN_ARRAY_SW_SRC: *bytes = dp->src ? dp->slots * sizeof(int) : 0; return dp->src;
+    case MPS_PLAN_ARRAY_SW_SPLIT_ROW: *bytes = Lo.split_row.size() * sizeof(int); return dp->split_row;
+    case MPS_PLAN_ARRAY_SW_SPLIT_PTR: *bytes = Lo.split_ptr.size() * sizeof(int); return dp->split_ptr;
+    default: *bytes = 0; return nullptr;
+    }
+}
+
+}  // namespace mps_sw

@@ -1,0 +1,461 @@
+// Sweep plans, host side: the layout builder (see mpspmm_sweep.hpp) and its
+// C entry points.  No counterpart in the reference, whose host side builds
+// the merge-path schedule only (src/MergePathSpMM.cu:300-385).
+#include "mpspmm.h"
+#include "mpspmm_hostpar.hpp"
+#include "mpspmm_sweep.hpp"
+
+#include <algorithm>
+#include <cstring>
+#include <new>
+#include <numeric>
+#include <queue>
+
+namespace mps_sw {
+
+namespace {
+
+struct Item {          // what is dealt to panels: a row, a pair of rows, or a sub-row of a split row
+    long long nnz;
+    int pieces;        // accumulator rows it needs
+    int row;           // first row
+    int nrows;         // 1 or 2
+    int sub;           // -1, or the sub-row index of a split row
+};
+
+struct Entry {
+    int col;
+    int vloc;          // accumulator row, panel-local
+    float val;
+    int src;
+};
+
+int bits_for(unsigned v)
+{
+    int b = 0;
+    while (v) {
+        ++b;
+        v >>= 1;
+    }
+    return b < 1 ? 1 : b;
+}
+
+// Largest first, each to the bin with the smallest load so far; a bin takes at most `cap` of `cost`.
+// false if some item finds no bin.
+template <typename Size, typename Cost>
+bool deal_largest_first(const std::vector<int> &order, Size size_of, Cost cost_of, int bins, long long cap,
+                        std::vector<int> &bin_of)
+{
+    typedef std::pair<long long, int> Load;  // (load, bin): the lightest bin first, the lower index among equals
+    std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+    for (int b = 0; b < bins; ++b) heap.push(Load(0, b));
+    std::vector<long long> used((size_t)bins, 0);
+    std::vector<Load> held;
+    for (int i : order) {
+        held.clear();
+        Load top;
+        for (;;) {
+            if (heap.empty()) return false;
+            top = heap.top();
+            heap.pop();
+            if (used[(size_t)top.second] + cost_of(i) <= cap) break;
+            held.push_back(top);
+        }
+        for (const Load &h : held) heap.push(h);
+        bin_of[(size_t)i] = top.second;
+        used[(size_t)top.second] += cost_of(i);
+        heap.push(Load(top.first + size_of(i), top.second));
+    }
+    return true;
+}
+
+}  // namespace
+
+int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp, Layout &out)
+{
+    if (n < 1 || nnz < 0 || K < 1 || !rp || (nnz > 0 && (!ci || !val))) return MPS_ERR_INVALID_ARG;
+    if (bp.elem_bytes != 4 && bp.elem_bytes != 2) return MPS_ERR_INVALID_ARG;
+    const long long row_bytes = (long long)K * bp.elem_bytes;
+    if (row_bytes % 64 != 0) return MPS_ERR_UNSUPPORTED;
+    const int L = row_bytes % 128 == 0 ? 8 : 4;
+    const int tiles = (int)(row_bytes / (16 * L));
+    const int acc_row_bytes = 16 * L * (4 / bp.elem_bytes);  // fp32 sums of a tile: 16 L bytes of floats, 32 L of halves
+    const int col_bits = bits_for((unsigned)(n - 1));
+    if (col_bits > 32 - kMinRowBits) return MPS_ERR_UNSUPPORTED;
+    const int num_cus = bp.num_cus > 0 ? bp.num_cus : 256;
+    long long vcap = (kLdsBytes - 1024) / acc_row_bytes - 1;           // one row for the padding's sums
+    vcap = std::min<long long>(vcap, (1ll << (32 - col_bits)) - 2);
+    if (bp.acc_rows > 0) vcap = std::min<long long>(vcap, bp.acc_rows);
+    vcap &= ~3ll;
+    if (vcap < 4) return MPS_ERR_UNSUPPORTED;
+    const int U = row_bytes < 128 ? 2 : 1;  // rows of Y per 128-byte line
+
+    out = Layout();
+    out.n = n;
+    out.nnz = nnz;
+    out.K = K;
+    out.elem_bytes = bp.elem_bytes;
+    out.lanes = L;
+    out.tiles = tiles;
+    out.col_bits = col_bits;
+    out.bank_rows = std::max(1, 256 / (16 * L));
+    const int G = out.bank_rows;
+    const int gpw = 64 / L;  // lane-groups of a wavefront = entries of an instruction
+
+    auto deg = [&](int r) { return (long long)rp[r + 1] - rp[r]; };
+
+    // ---- panels: how many, how rows are cut, which row goes where
+    std::vector<Item> items;
+    std::vector<int> item_panel;
+    std::vector<int> split_of((size_t)n, 0);  // sub-rows of a row (0: not split)
+    int NP = 0, piece = 0;
+    for (int R = 1;; ++R) {
+        if (R > 8192) return MPS_ERR_UNSUPPORTED;  // (a row that needs more accumulator rows than a panel holds)
+        NP = num_cus * R;
+        const long long share = std::max<long long>(1, (long long)nnz / NP);
+        // An accumulator row takes one entry per instruction at most, and a wavefront's share is share / 16 / gpw
+        // instructions: a piece of half that many entries finds its instructions among them.
+        piece = bp.piece > 0 ? bp.piece : (int)std::min<long long>(1 << 20, std::max<long long>(8, share / kWaves / gpw / 2));
+        // a row of about a panel's share or more is cut into sub-rows of a third of a share
+        const long long split_from = std::max<long long>(share - share / 10, 4ll * piece);
+        const long long sub_target = std::max<long long>(share / 3, piece);
+        items.clear();
+        out.split_row.clear();
+        out.split_ptr.assign(1, 0);
+        long long totv = 0;
+        auto pieces_of = [&](long long d) { return (int)((d + piece - 1) / piece); };
+        for (int r = 0; r < n; ++r) {
+            const long long d = deg(r);
+            split_of[(size_t)r] = d > split_from && NP > 1 ? (int)((d + sub_target - 1) / sub_target) : 0;
+            if (split_of[(size_t)r] == 1) split_of[(size_t)r] = 0;
+        }
+        for (int r = 0; r < n;) {
+            const int S = split_of[(size_t)r];
+            if (S > 0) {
+                const long long d = deg(r);
+                for (int j = 0; j < S; ++j) {
+                    const long long dj = d / S + (j < d % S);  // entries j, j + S, j + 2 S, ...
+                    items.push_back(Item{dj, pieces_of(dj), r, 1, j});
+                    totv += pieces_of(dj);
+                }
+                out.split_row.push_back(r);
+                out.split_ptr.push_back(out.split_ptr.back() + S);
+                ++r;
+                continue;
+            }
+            int take = 1;
+            if (U == 2 && (r & 1) == 0 && r + 1 < n && split_of[(size_t)r + 1] == 0) take = 2;
+            long long d = 0;
+            int p = 0;
+            for (int k = 0; k < take; ++k) {
+                d += deg(r + k);
+                p += pieces_of(deg(r + k));
+            }
+            items.push_back(Item{d, p, r, take, -1});
+            totv += p;
+            r += take;
+        }
+        if (totv > (long long)NP * vcap) continue;
+        std::vector<int> order;
+        order.reserve(items.size());
+        for (int i = 0; i < (int)items.size(); ++i)
+            if (items[(size_t)i].nnz > 0) order.push_back(i);
+        std::stable_sort(order.begin(), order.end(),
+                         [&](int a, int b) { return items[(size_t)a].nnz > items[(size_t)b].nnz; });
+        item_panel.assign(items.size(), 0);
+        if (!deal_largest_first(
+                order, [&](int i) { return items[(size_t)i].nnz; }, [&](int i) { return (long long)items[(size_t)i].pieces; },
+                NP, vcap, item_panel))
+            continue;
+        // rows without nonzeros: zeros to write, dealt evenly
+        int turn = 0;
+        for (int i = 0; i < (int)items.size(); ++i)
+            if (items[(size_t)i].nnz == 0) item_panel[(size_t)i] = turn++ % NP;
+        break;
+    }
+    out.num_panels = NP;
+    out.piece = piece;
+
+    // a panel's items: those with nonzeros largest first, then the empty ones
+    std::vector<int> panel_count((size_t)NP + 1, 0);
+    for (size_t i = 0; i < items.size(); ++i) panel_count[(size_t)item_panel[i] + 1] += 1;
+    for (int p = 0; p < NP; ++p) panel_count[(size_t)p + 1] += panel_count[(size_t)p];
+    std::vector<int> panel_items(items.size());
+    {
+        std::vector<int> order(items.size());
+        std::iota(order.begin(), order.end(), 0);
+        std::stable_sort(order.begin(), order.end(),
+                         [&](int a, int b) { return items[(size_t)a].nnz > items[(size_t)b].nnz; });
+        std::vector<int> fill(panel_count.begin(), panel_count.end() - 1);
+        for (int i : order) panel_items[(size_t)fill[(size_t)item_panel[(size_t)i]]++] = i;
+    }
+    // partial row of sub-row j of split row r
+    std::vector<int> split_index((size_t)n, -1);
+    for (size_t i = 0; i < out.split_row.size(); ++i) split_index[(size_t)out.split_row[i]] = (int)i;
+
+    // listed rows per panel
+    out.panel_ptr.assign((size_t)NP + 1, 0);
+    for (int p = 0; p < NP; ++p) {
+        int rows = 0;
+        for (int k = panel_count[(size_t)p]; k < panel_count[(size_t)p + 1]; ++k) rows += items[(size_t)panel_items[(size_t)k]].nrows;
+        out.panel_ptr[(size_t)p + 1] = out.panel_ptr[(size_t)p] + rows;
+    }
+    const int listed = out.panel_ptr[(size_t)NP];
+    int acc_rows = 4;
+    for (int p = 0; p < NP; ++p) {
+        int v = 0;
+        for (int k = panel_count[(size_t)p]; k < panel_count[(size_t)p + 1]; ++k) v += items[(size_t)panel_items[(size_t)k]].pieces;
+        acc_rows = std::max(acc_rows, (v + 3) & ~3);
+    }
+    out.acc_rows = acc_rows;
+    const uint32_t pad_word = (uint32_t)acc_rows << col_bits;  // padding: column 0, value 0, the spare accumulator row
+    out.rows.assign((size_t)listed, 0);
+    out.piece_ptr.assign((size_t)listed + NP, 0);
+    out.wave_meta.assign((size_t)NP * kWaves * 2, 0);
+    out.panel_rounds.assign((size_t)NP, 0);
+
+    // ---- every panel on its own: accumulator rows, wavefronts, streams
+    struct PanelOut {
+        std::vector<uint32_t> stream;
+        std::vector<int> src;
+        int wave_rounds[kWaves];
+        int vrows;
+    };
+    std::vector<PanelOut> built((size_t)NP);
+    const int words_per_round = gpw * kWin * 4;  // uint32: lane-groups x 4 lanes x {word A, value A, word B, value B}
+    mps_host::parallel_for(NP, 1, [&](int64_t lo, int64_t hi) {
+        std::vector<int> vsize, vwave, vorder, last;
+        std::vector<Entry> entries[kWaves];
+        std::vector<uint8_t> fill;
+        std::vector<long long> slot;
+        for (int p = (int)lo; p < (int)hi; ++p) {
+            PanelOut &po = built[(size_t)p];
+            // listed rows and their accumulator rows
+            const int k0 = panel_count[(size_t)p], k1 = panel_count[(size_t)p + 1];
+            int lr = out.panel_ptr[(size_t)p];
+            int *pp = out.piece_ptr.data() + lr + p;
+            int v = 0;
+            vsize.clear();
+            for (int k = k0; k < k1; ++k) {
+                const Item &it = items[(size_t)panel_items[(size_t)k]];
+                for (int q = 0; q < it.nrows; ++q) {
+                    const int r = it.row + q;
+                    const long long d = it.sub >= 0 ? it.nnz : deg(r);
+                    const int P = (int)((d + piece - 1) / piece);
+                    out.rows[(size_t)lr] = it.sub >= 0 ? n + out.split_ptr[(size_t)split_index[(size_t)r]] + it.sub : r;
+                    *pp++ = v;
+                    ++lr;
+                    for (int j = 0; j < P; ++j) vsize.push_back((int)(d / P + (j < d % P)));
+                    v += P;
+                }
+            }
+            *pp = v;
+            po.vrows = v;
+            // accumulator rows to wavefronts
+            vorder.resize((size_t)v);
+            std::iota(vorder.begin(), vorder.end(), 0);
+            std::stable_sort(vorder.begin(), vorder.end(), [&](int a, int b) { return vsize[(size_t)a] > vsize[(size_t)b]; });
+            vwave.assign((size_t)v, 0);
+            deal_largest_first(
+                vorder, [&](int i) { return (long long)vsize[(size_t)i]; }, [](int) { return 0ll; }, kWaves, 1, vwave);
+            // entries per wavefront
+            for (auto &e : entries) e.clear();
+            v = 0;
+            for (int k = k0; k < k1; ++k) {
+                const Item &it = items[(size_t)panel_items[(size_t)k]];
+                for (int q = 0; q < it.nrows; ++q) {
+                    const int r = it.row + q;
+                    const int S = it.sub >= 0 ? split_of[(size_t)r] : 1, first = it.sub >= 0 ? it.sub : 0;
+                    const long long d = it.sub >= 0 ? it.nnz : deg(r);
+                    const int P = (int)((d + piece - 1) / piece);
+                    const long long base = rp[r];
+                    for (long long e = 0; e < d; ++e) {
+                        const long long at = base + first + e * S;
+                        const int vl = v + (int)(e % P);
+                        entries[vwave[(size_t)vl]].push_back(Entry{ci[at], vl, val[at], (int)at});
+                    }
+                    v += P;
+                }
+            }
+            // streams: a wavefront's entries by column; one entry per lane-group and instruction, never two of one
+            // accumulator row in an instruction (the second waits for the next instruction that has room)
+            for (int w = 0; w < kWaves; ++w) {
+                std::vector<Entry> &E = entries[w];
+                std::stable_sort(E.begin(), E.end(), [](const Entry &a, const Entry &b) { return a.col < b.col; });
+                const long long ne = (long long)E.size();
+                slot.resize((size_t)ne);
+                fill.assign((size_t)(ne / gpw + 2), 0);
+                last.assign((size_t)po.vrows + 1, -1);
+                long long frontier = 0, top = 0;
+                for (long long e = 0; e < ne; ++e) {
+                    const int vl = E[(size_t)e].vloc;
+                    long long t = std::max<long long>(frontier, (long long)last[(size_t)vl] + 1);
+                    for (;;) {
+                        if (t >= (long long)fill.size()) fill.resize((size_t)t + ne / gpw + 2, 0);
+                        if (fill[(size_t)t] < gpw) break;
+                        ++t;
+                    }
+                    slot[(size_t)e] = t * gpw + fill[(size_t)t];
+                    ++fill[(size_t)t];
+                    last[(size_t)vl] = (int)t;
+                    top = std::max(top, t + 1);
+                    while (frontier < (long long)fill.size() && fill[(size_t)frontier] == gpw) ++frontier;
+                }
+                const int rounds = (int)((top + kRoundInstr - 1) / kRoundInstr);
+                po.wave_rounds[w] = rounds;
+                const size_t at0 = po.stream.size();
+                po.stream.resize(at0 + (size_t)rounds * words_per_round);
+                if (bp.keep_src) po.src.resize((at0 + (size_t)rounds * words_per_round) / 2, -1);
+                uint32_t *s = po.stream.data() + at0;
+                for (size_t i = 0; i < (size_t)rounds * words_per_round; i += 2) {
+                    s[i] = pad_word;
+                    s[i + 1] = 0u;
+                }
+                for (long long e = 0; e < ne; ++e) {
+                    const long long t = slot[(size_t)e] / gpw, g = slot[(size_t)e] % gpw;
+                    const long long round = t / kRoundInstr, w2 = (t % kRoundInstr) / kWin, q = t % kWin;
+                    const size_t at = (size_t)((round * gpw * kWin + g * kWin + q) * 4 + w2 * 2);
+                    uint32_t bits;
+                    std::memcpy(&bits, &E[(size_t)e].val, 4);
+                    s[at] = (uint32_t)E[(size_t)e].col | ((uint32_t)swizzle(E[(size_t)e].vloc, G) << col_bits);
+                    s[at + 1] = bits;
+                    if (bp.keep_src) po.src[(at0 + at) / 2] = E[(size_t)e].src;
+                }
+            }
+        }
+    });
+
+    // ---- put the panels' streams one after the other
+    std::vector<long long> panel_first((size_t)NP + 1, 0);
+    for (int p = 0; p < NP; ++p) {
+        long long rounds = 0;
+        int most = 0;
+        for (int w = 0; w < kWaves; ++w) {
+            out.wave_meta[((size_t)p * kWaves + w) * 2] = (int)(panel_first[(size_t)p] + rounds);
+            out.wave_meta[((size_t)p * kWaves + w) * 2 + 1] = built[(size_t)p].wave_rounds[w];
+            rounds += built[(size_t)p].wave_rounds[w];
+            most = std::max(most, built[(size_t)p].wave_rounds[w]);
+        }
+        out.panel_rounds[(size_t)p] = most;
+        panel_first[(size_t)p + 1] = panel_first[(size_t)p] + rounds;
+    }
+    out.rounds = panel_first[(size_t)NP];
+    if (out.rounds * (long long)words_per_round / 4 > 0x7fffffffll) return MPS_ERR_UNSUPPORTED;  // 16-byte units index the stream
+    out.stream.resize((size_t)out.rounds * words_per_round);
+    if (bp.keep_src) out.src.resize(out.stream.size() / 2);
+    mps_host::parallel_for(NP, 1, [&](int64_t lo, int64_t hi) {
+        for (int p = (int)lo; p < (int)hi; ++p) {
+            PanelOut &po = built[(size_t)p];
+            if (!po.stream.empty())
+                std::memcpy(out.stream.data() + (size_t)panel_first[(size_t)p] * words_per_round, po.stream.data(),
+                            po.stream.size() * sizeof(uint32_t));
+            if (bp.keep_src && !po.src.empty())
+                std::memcpy(out.src.data() + (size_t)panel_first[(size_t)p] * words_per_round / 2, po.src.data(),
+                            po.src.size() * sizeof(int));
+            std::vector<uint32_t>().swap(po.stream);
+            std::vector<int>().swap(po.src);
+        }
+    });
+    return MPS_OK;
+}
+
+}  // namespace mps_sw
+
+struct mps_sweep_layout {
+    mps_sw::Layout L;
+};
+
+extern "C" {
+
+int mps_sweep_layout_build(const int *row_ptr, const int *col_idx, const float *val, int n_rows, int nnz, int K,
+                           int elem_bytes, const mps_plan_options *options, mps_sweep_layout **layout_out)
+{
+    if (!layout_out) return MPS_ERR_INVALID_ARG;
+    *layout_out = nullptr;
+    mps_sw::BuildParams bp;
+    bp.elem_bytes = elem_bytes;
+    if (options) {
+        bp.piece = options->sweep_piece;
+        bp.acc_rows = options->sweep_acc_rows;
+        bp.num_cus = options->sweep_panels_per_round;
+        bp.keep_src = !(options->flags & MPS_PLAN_NO_SOURCES);
+    }
+    if (bp.num_cus <= 0) bp.num_cus = 256;
+    mps_sweep_layout *h = new (std::nothrow) mps_sweep_layout;
+    if (!h) return MPS_ERR_UNSUPPORTED;
+    int rc;
+    try {
+        rc = mps_sw::build_layout(row_ptr, col_idx, val, n_rows, nnz, K, bp, h->L);
+    } catch (const std::bad_alloc &) {
+        rc = MPS_ERR_UNSUPPORTED;
+    }
+    if (rc != MPS_OK) {
+        delete h;
+        return rc;
+    }
+    *layout_out = h;
+    return MPS_OK;
+}
+
+}  // extern "C"
+
+namespace mps_sw {
+void fill_info(const Layout &L, mps_plan_info *info)
+{
+    info->sweep_panels = L.num_panels;
+    info->sweep_acc_rows = L.acc_rows;
+    info->sweep_lanes = L.lanes;
+    info->sweep_tiles = L.tiles;
+    info->sweep_col_bits = L.col_bits;
+    info->sweep_piece = L.piece;
+    info->sweep_split_rows = (int)L.split_row.size();
+    info->sweep_partial_rows = L.split_ptr.empty() ? 0 : L.split_ptr.back();
+    info->sweep_listed_rows = (int)L.rows.size();
+    info->sweep_rounds = L.rounds;
+    info->sweep_slots = L.rounds * (long long)(64 / L.lanes) * kRoundInstr;
+}
+}  // namespace mps_sw
+
+extern "C" {
+
+int mps_sweep_layout_info(const mps_sweep_layout *layout, mps_plan_info *info)
+{
+    if (!layout || !info) return MPS_ERR_INVALID_ARG;
+    const mps_sw::Layout &L = layout->L;
+    std::memset(info, 0, sizeof(*info));
+    info->n_rows = L.n;
+    info->nnz = L.nnz;
+    info->K = L.K;
+    info->elem_bytes = L.elem_bytes;
+    info->num_slabs = 1;
+    info->slab_cols = L.n;
+    mps_sw::fill_info(L, info);
+    return MPS_OK;
+}
+
+int mps_sweep_layout_array(const mps_sweep_layout *layout, int which, const void **data_out, size_t *bytes_out)
+{
+    if (!layout || !data_out || !bytes_out) return MPS_ERR_INVALID_ARG;
+    const mps_sw::Layout &L = layout->L;
+    auto give = [&](const auto &v) {
+        *data_out = v.data();
+        *bytes_out = v.size() * sizeof(v[0]);
+        return (int)MPS_OK;
+    };
+    switch (which) {
+    case MPS_PLAN_ARRAY_SW_PANEL_PTR: return give(L.panel_ptr);
+    case MPS_PLAN_ARRAY_SW_ROWS: return give(L.rows);
+    case MPS_PLAN_ARRAY_SW_PIECE_PTR: return give(L.piece_ptr);
+    case MPS_PLAN_ARRAY_SW_WAVE_META: return give(L.wave_meta);
+    case MPS_PLAN_ARRAY_SW_PANEL_ROUNDS: return give(L.panel_rounds);
+    case MPS_PLAN_ARRAY_SW_STREAM: return give(L.stream);
+    case MPS_PLAN_ARRAY_SW_SRC: return give(L.src);
+    case MPS_PLAN_ARRAY_SW_SPLIT_ROW: return give(L.split_row);
+    case MPS_PLAN_ARRAY_SW_SPLIT_PTR: return give(L.split_ptr);
+    default: return MPS_ERR_INVALID_ARG;
+    }
+}
+
+void mps_sweep_layout_free(mps_sweep_layout *layout) { delete layout; }
+
+}  // extern "C"

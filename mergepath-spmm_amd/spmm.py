@@ -178,7 +178,7 @@ class Plan:
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
                  rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None, column_tiles=True,
-                 local_tables=False):
+                 local_tables=False, sweep="auto", sweep_piece=0, sweep_acc_rows=0, sweep_panels_per_round=0):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -187,6 +187,7 @@ class Plan:
         flags = {"auto": 0, "off": _cabi.MPS_PLAN_NO_TILING, "force": _cabi.MPS_PLAN_FORCE_TILING}[tiling]
         flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_HOT, "force": _cabi.MPS_PLAN_FORCE_HOT}[hot]
         flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_ROWBLOCK, "force": _cabi.MPS_PLAN_FORCE_ROWBLOCK}[rowblock]
+        flags |= {"auto": 0, "off": _cabi.MPS_PLAN_NO_SWEEP, "force": _cabi.MPS_PLAN_FORCE_SWEEP}[sweep]
         if not keep_sources:
             flags |= _cabi.MPS_PLAN_NO_SOURCES
         if not row_marks:
@@ -199,7 +200,8 @@ class Plan:
             flags |= _cabi.MPS_PLAN_LOCAL_TABLES
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
                                 int(rowblock_block_rows), int(rowblock_blocks_per_round),
-                                {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes))
+                                {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes), int(sweep_piece),
+                                int(sweep_acc_rows), int(sweep_panels_per_round))
         check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), None if weights else _ptr(csr.val),
                                              csr.n_rows, csr.nnz,
                                              int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
@@ -251,6 +253,15 @@ class Plan:
             _cabi.MPS_PLAN_ARRAY_RB_COLD_PACKED: (3 * int(i.rowblock_cold_slots) // 2 if i.rowblock_cold_index_bits else 0, np.uint32),
             _cabi.MPS_PLAN_ARRAY_RB_COLD_BEGIN: (i.rowblock_steps + 1 if i.rowblock_steps else 0, np.int32),
             _cabi.MPS_PLAN_ARRAY_RB_TABLE_BASE: (i.rowblock_blocks if i.rowblock_local_tables else 0, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_PANEL_PTR: (i.sweep_panels + 1 if i.sweep_panels else 0, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_ROWS: (i.sweep_listed_rows, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_PIECE_PTR: (i.sweep_listed_rows + i.sweep_panels, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_WAVE_META: (i.sweep_panels * 32, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_PANEL_ROUNDS: (i.sweep_panels, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_STREAM: (2 * int(i.sweep_slots), np.uint32),
+            _cabi.MPS_PLAN_ARRAY_SW_SRC: (int(i.sweep_slots), np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_SPLIT_ROW: (i.sweep_split_rows, np.int32),
+            _cabi.MPS_PLAN_ARRAY_SW_SPLIT_PTR: (i.sweep_split_rows + 1 if i.sweep_panels else 0, np.int32),
         }
         n, dt = shapes[which]
         out = np.empty(n, dtype=dt)
@@ -332,7 +343,7 @@ class RowBlockLayout:
         v = np.ascontiguousarray(val, dtype=np.float32)
         opt = _cabi.PlanOptions((0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES) | (_cabi.MPS_PLAN_LOCAL_TABLES if local_tables else 0),
                                 0, int(steps), int(table_rows),
-                                int(block_rows), int(blocks_per_round), 0, 0)
+                                int(block_rows), int(blocks_per_round), 0, 0, 0, 0, 0)
         check(_cabi.lib().mps_rowblock_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size,
                                                     int(K), ctypes.byref(opt), ctypes.byref(self._h)),
               "mps_rowblock_layout_build")
@@ -353,6 +364,47 @@ class RowBlockLayout:
     def close(self):
         if getattr(self, "_h", None) is not None and self._h.value:
             _cabi.lib().mps_rowblock_layout_free(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class SweepLayout:
+    """The layout of a sweep plan, built on the host (mps_sweep_layout_build): no GPU needed."""
+
+    def __init__(self, row_ptr, col_idx, val, K, elem_bytes=4, piece=0, acc_rows=0, panels_per_round=0, keep_sources=True):
+        import numpy as np
+        self._np = np
+        self._h = ctypes.c_void_p()
+        rp = np.ascontiguousarray(row_ptr, dtype=np.int32)
+        ci = np.ascontiguousarray(col_idx, dtype=np.int32)
+        v = np.ascontiguousarray(val, dtype=np.float32)
+        opt = _cabi.PlanOptions(0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES, 0, 0, 0, 0, 0, 0, 0, int(piece), int(acc_rows),
+                                int(panels_per_round))
+        check(_cabi.lib().mps_sweep_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size, int(K),
+                                                 int(elem_bytes), ctypes.byref(opt), ctypes.byref(self._h)),
+              "mps_sweep_layout_build")
+        self.info = _cabi.PlanInfo()
+        check(_cabi.lib().mps_sweep_layout_info(self._h, ctypes.byref(self.info)), "mps_sweep_layout_info")
+
+    def array(self, which, dtype):
+        """Copy of one of the layout's arrays (MPS_PLAN_ARRAY_SW_*) as a numpy array of `dtype`."""
+        np = self._np
+        data, nbytes = ctypes.c_void_p(), ctypes.c_size_t()
+        check(_cabi.lib().mps_sweep_layout_array(self._h, int(which), ctypes.byref(data), ctypes.byref(nbytes)),
+              "mps_sweep_layout_array")
+        if nbytes.value == 0:
+            return np.zeros(0, dtype=dtype)
+        buf = (ctypes.c_char * nbytes.value).from_address(data.value)
+        return np.frombuffer(buf, dtype=dtype).copy()
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            _cabi.lib().mps_sweep_layout_free(self._h)
             self._h = ctypes.c_void_p()
 
     def __del__(self):
