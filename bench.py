@@ -191,6 +191,7 @@ def main():
                     help="sweep plan (rows summed in LDS, nonzeros visited in column order): where the library picks it / "
                          "never / always")
     ap.add_argument("--sweep-piece", type=int, default=0, help="sweep plans: most entries of a row per accumulator row (0 = library default)")
+    ap.add_argument("--sweep-together", type=int, default=0, help="sweep plans: 1 or 2 instructions added up at the same time (0 = library default)")
     ap.add_argument("--sweep-acc-rows", type=int, default=0, help="sweep plans: most accumulator rows per panel (0 = what fits in LDS)")
     ap.add_argument("--rb-steps", type=int, default=0, help="steps (LDS tables) of a row-block plan (0 = library default)")
     ap.add_argument("--rb-table-rows", type=int, default=0, help="rows per LDS table of a row-block plan (0 = what fits)")
@@ -255,7 +256,7 @@ def main():
                   rowblock_table_rows=args.rb_table_rows, keep_sources=False, resident=args.resident,
                   resident_bytes=args.resident_bytes, weights=None if args.weights == "none" else args.weights,
                   column_tiles=args.column_tiles == "auto", sweep=args.sweep, sweep_piece=args.sweep_piece,
-                  sweep_acc_rows=args.sweep_acc_rows)
+                  sweep_acc_rows=args.sweep_acc_rows, sweep_together=args.sweep_together)
         kw.update(overrides)
         return sp.Plan(wl.csr, wl.K, **kw), cost
 

@@ -444,6 +444,8 @@ typedef struct mps_plan_info {
     int sweep_tiles;               /* column tiles per row of X                    */
     int sweep_col_bits;            /* an entry word is column | accumulator row << sweep_col_bits */
     int sweep_piece;               /* most entries of a row that one accumulator row takes */
+    int sweep_together;            /* 1, or 2: entry q of a round's windows A and B are added up at the same time, no two
+                                      entries of such a pair of instructions share an accumulator row */
     int sweep_split_rows;          /* rows cut into sub-rows that go to different panels */
     int sweep_partial_rows;        /* sub-rows of those rows                       */
     int sweep_listed_rows;         /* entries of SW_ROWS: n_rows - split rows + partial rows */
@@ -465,6 +467,7 @@ typedef struct mps_plan_options {
     int sweep_piece;         /* sweep plans: most entries of a row per accumulator row */
     int sweep_acc_rows;      /* sweep plans: most accumulator rows per panel (what fits in LDS if 0 or larger) */
     int sweep_panels_per_round; /* sweep plans: panels are made in multiples of this (0: the number of CUs) */
+    int sweep_together;      /* sweep plans: 1 or 2 instructions added up at the same time (0: 2 for 64-byte rows of X, else 1) */
 } mps_plan_options;
 
 enum {

@@ -64,7 +64,7 @@ class PlanInfo(ctypes.Structure):
                 ("resident_cols", ctypes.c_int), ("resident_nnz", ctypes.c_longlong),
                 ("rowblock_cold_index_bits", ctypes.c_int), ("rowblock_local_tables", ctypes.c_int)] + \
                [(n, ctypes.c_int) for n in ("sweep_panels", "sweep_acc_rows", "sweep_lanes", "sweep_tiles", "sweep_col_bits",
-                                             "sweep_piece", "sweep_split_rows", "sweep_partial_rows", "sweep_listed_rows")] + \
+                                             "sweep_piece", "sweep_together", "sweep_split_rows", "sweep_partial_rows", "sweep_listed_rows")] + \
                [("sweep_rounds", ctypes.c_longlong), ("sweep_slots", ctypes.c_longlong)]
 
 
@@ -74,7 +74,7 @@ class PlanOptions(ctypes.Structure):
                 ("rowblock_table_rows", ctypes.c_int), ("rowblock_block_rows", ctypes.c_int),
                 ("rowblock_blocks_per_round", ctypes.c_int), ("degree_weights", ctypes.c_int),
                 ("resident_bytes", ctypes.c_size_t), ("sweep_piece", ctypes.c_int), ("sweep_acc_rows", ctypes.c_int),
-                ("sweep_panels_per_round", ctypes.c_int)]
+                ("sweep_panels_per_round", ctypes.c_int), ("sweep_together", ctypes.c_int)]
 
 
 class TuneResult(ctypes.Structure):

@@ -97,7 +97,8 @@ int mergepath_main(int argc, char **argv)
                         tried[i].threads_per_wave, tried[i].flags, tried[i].slab_bytes, tried[i].ms * 1e3);
         cost = best.cost;
         threads_per_wave = best.threads_per_wave;
-        opt.tiling = (int)(best.flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_ROWBLOCK));
+        opt.tiling = (int)(best.flags & (MPS_PLAN_NO_TILING | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_FORCE_ROWBLOCK |
+                                         MPS_PLAN_NO_SWEEP | MPS_PLAN_FORCE_SWEEP));
         opt.hot = (int)(best.flags & (MPS_PLAN_NO_HOT | MPS_PLAN_FORCE_HOT));
         opt.slab_bytes = (size_t)best.slab_bytes;
         opt.use_plan = true;
@@ -142,7 +143,12 @@ int mergepath_main(int argc, char **argv)
 
     std::printf("partitions: %d (cost %d), threads_per_wave %d, max row degree %d\n", P, cost, threads_per_wave,
                 gr.max_degree);
-    if (plan && info.rowblock_steps > 0)
+    if (plan && info.sweep_panels > 0)
+        std::printf("plan: %d panels x %d column tile(s) of %d bytes, %d accumulator rows per panel, %lld entry slots for %d nonzeros, "
+                    "%d row(s) cut across panels, %.1f MB of device memory\n",
+                    info.sweep_panels, info.sweep_tiles, 16 * info.sweep_lanes, info.sweep_acc_rows, info.sweep_slots, nnz,
+                    info.sweep_split_rows, info.device_bytes / 1e6);
+    else if (plan && info.rowblock_steps > 0)
         std::printf("plan: %d row blocks, %d steps of %d table rows, %lld of %d nonzeros (%.1f %%) gathered from LDS, %.1f MB of device memory\n",
                     info.rowblock_blocks, info.rowblock_steps, info.rowblock_table_rows, info.hot_nnz, nnz,
                     nnz ? 100.0 * (double)info.hot_nnz / nnz : 0.0, info.device_bytes / 1e6);
@@ -161,9 +167,9 @@ int mergepath_main(int argc, char **argv)
     char extra[256];
     std::snprintf(extra, sizeof extra,
                   ", \"P\": %d, \"cost\": %d, \"threads_per_wave\": %d, \"plan\": %s, \"num_slabs\": %d, \"hot_rows\": %d, "
-                  "\"rowblock_steps\": %d, \"resident_cols\": %d, \"prep_us\": %.3f",
+                  "\"rowblock_steps\": %d, \"sweep_panels\": %d, \"resident_cols\": %d, \"prep_us\": %.3f",
                   P, cost, threads_per_wave, plan ? "true" : "false", plan ? info.num_slabs : 1, plan ? info.hot_rows : 0,
-                  plan ? info.rowblock_steps : 0, plan ? info.resident_cols : 0, prep.avg_us);
+                  plan ? info.rowblock_steps : 0, plan ? info.sweep_panels : 0, plan ? info.resident_cols : 0, prep.avg_us);
     mps_plan_destroy(plan);
     std::string more = extra;
     if (opt.cpu)

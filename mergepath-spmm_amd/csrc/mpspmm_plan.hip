@@ -1261,17 +1261,82 @@ bool rowblock_wanted(int n_rows, int nnz, int K, int elem_bytes, int cost, int t
     return true;
 }
 
-// Sweep plan or not.  Forced: yes.
-bool sweep_wanted(int n_rows, int nnz, int K, int elem_bytes, int cost, int tpw, unsigned flags)
+// Nonzeros within `width` columns of the diagonal: 16 lanes per row, one count per workgroup added to *count.
+__global__ __launch_bounds__(256) void near_diagonal_kernel(const int *__restrict__ row_ptr, const int *__restrict__ col_idx,
+                                                             int n_rows, int width, unsigned long long *__restrict__ count)
 {
-    if (flags & MPS_PLAN_FORCE_SWEEP) return true;
-    (void)n_rows;
-    (void)nnz;
-    (void)K;
-    (void)elem_bytes;
-    (void)cost;
-    (void)tpw;
-    return false;
+    __shared__ unsigned block_count;
+    if (threadIdx.x == 0) block_count = 0;
+    __syncthreads();
+    const int row = blockIdx.x * 16 + (int)(threadIdx.x >> 4), lane = (int)(threadIdx.x & 15);
+    unsigned mine = 0;
+    if (row < n_rows)
+        for (int e = row_ptr[row] + lane; e < row_ptr[row + 1]; e += 16) {
+            const int d = col_idx[e] - row;
+            mine += (d <= width && d >= -width) ? 1u : 0u;
+        }
+    if (mine) atomicAdd(&block_count, mine);
+    __syncthreads();
+    if (threadIdx.x == 0 && block_count) atomicAdd(count, (unsigned long long)block_count);
+}
+
+// Sweep plan or not.  Forced: yes.  Otherwise for rows of X of 64 bytes or a multiple of 128, when the caller is
+// not tuning a slab plan (a cost, partitions per wavefront or tiling / hot-column switches of its own) and the matrix
+// is not local.  Measured on MI355X, ms per product, sweep plan against the library's other choice:
+//   fp32, K = 16 (against row-block plans, slab plans where those are not built):
+//     R-MAT x 16 per row, scale 16 / 18 / 20 / 21: .035/.014, .046/.044, .118-.128/.183-.197, .278/.433; scale 19 x 8 .047/.055;
+//     power law 232,965 rows x 16 / 64 / 492 per row: .038/.039, .099/.085, .56/.43; 1,000,000 x 16 / 60: .146/.201, .399/.519;
+//     uniform 232,965 x 32: .057/.069; 1,000,000 x 8 / 60: .133/.172, .405/.659;
+//     block-diagonal 416,349 x 5: .040/.025 (row-block plan with local tables).
+//   Wider rows and fp16 (against slab plans): R-MAT scale 20 x 16 at K = 32 / 64 / 128 / 256: .163-.187/.231-.272, .349/.49-.55,
+//     .706/.97, 1.43/2.07; scale 18 at K = 64: .092/.119; scale 22 fp16 K = 64: .94-.97/1.11-1.15; scale 20 fp16 K = 32:
+//     .178/.182; power law 232,965 x 492 at K = 32: .83/.91; x 64 at K = 64: .265/.340; uniform 1,000,000 x 8 at K = 64:
+//     .365/.346; block-diagonal 416,349 x 5 at K = 64: .107/.076.
+// So: with 64-byte fp32 rows, where X is 24 MiB or more (393,216 rows) - below that a row-block plan's tables serve more
+// of the gathers than the sweep's locality saves; with other widths always; and never for a matrix whose nonzeros stay
+// near the diagonal (kSweepMaxNearDiagonal of them within kNearDiagonalWidth columns: block-diagonal and banded
+// matrices, whose X a slab plan finds in L2 anyway and which a row-block plan serves from local tables).
+constexpr uint64_t kSweepMinXBytesK16 = 24ull << 20;
+constexpr int kNearDiagonalWidth = 6000;
+constexpr double kSweepMaxNearDiagonal = 0.6;
+int sweep_wanted(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int K, int elem_bytes, int cost, int tpw,
+                 unsigned flags, hipStream_t st, bool *wanted)
+{
+    *wanted = false;
+    if (flags & MPS_PLAN_FORCE_SWEEP) {
+        *wanted = true;
+        return MPS_OK;
+    }
+    if (flags & (MPS_PLAN_NO_SWEEP | MPS_PLAN_FORCE_ROWBLOCK | MPS_PLAN_LOCAL_TABLES | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING |
+                 MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT | MPS_PLAN_NO_ROW_MARKS))
+        return MPS_OK;
+    const long long row_bytes = (long long)K * elem_bytes;
+    if (n_rows < 1 || nnz < 1 || (row_bytes != 64 && row_bytes % 128 != 0)) return MPS_OK;
+    if (n_rows > (1 << 26)) return MPS_OK;  // an entry word keeps 6 bits for the accumulator row
+    int default_cost = 0, max_tpw = 0;
+    if (mps_default_cost(n_rows, nnz, K, elem_bytes, &default_cost) != MPS_OK || cost != default_cost) return MPS_OK;
+    if (mps_max_threads_per_wave(K, elem_bytes, &max_tpw) != MPS_OK || (tpw != 0 && tpw != max_tpw)) return MPS_OK;
+    if (row_bytes == 64 && elem_bytes == 4 && (uint64_t)n_rows * 64 < kSweepMinXBytesK16) return MPS_OK;
+    // the kernel below follows row_ptr into col_idx: only on arrays that have been checked
+    const int vrc = mps_csr_validate(d_row_ptr, d_col_idx, n_rows, n_rows, nnz, st);
+    if (vrc != MPS_OK) return vrc;
+    unsigned long long *d_count = nullptr, near = 0;
+    MPS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&d_count), sizeof(unsigned long long)));
+    hipError_t e = hipMemsetAsync(d_count, 0, sizeof(unsigned long long), st);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(near_diagonal_kernel, dim3((unsigned)((n_rows + 15) / 16)), dim3(256), 0, st, d_row_ptr, d_col_idx,
+                           n_rows, kNearDiagonalWidth, d_count);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(&near, d_count, sizeof(near), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    (void)hipFree(d_count);
+    if (e != hipSuccess) return MPS_ERR_HIP + (int)e;
+    // (a matrix narrower than the window is all "near the diagonal": what counts then is whether X fits an L2,
+    // and that case never gets here with 64-byte rows; wider rows of a small matrix keep the sweep)
+    const bool small = n_rows <= 2 * kNearDiagonalWidth;
+    *wanted = small || (double)near < kSweepMaxNearDiagonal * (double)nnz;
+    return MPS_OK;
 }
 
 }  // namespace
@@ -1329,21 +1394,33 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     pl->cost = cost;
     pl->keep_sources = !(flags & MPS_PLAN_NO_SOURCES);
     pl->weights = opt.degree_weights;
-    if (sweep_wanted(n_rows, nnz, K, elem_bytes, cost, tpw, flags)) {
+    bool want_sweep = false;
+    if (!opt.degree_weights) {
+        const int src = sweep_wanted(d_row_ptr, d_col_idx, n_rows, nnz, K, elem_bytes, cost, tpw, flags,
+                                     static_cast<hipStream_t>(stream), &want_sweep);
+        if (src != MPS_OK) {
+            plan_free(pl);
+            return src;
+        }
+    }
+    if (want_sweep) {
         if (n_rows < 1 || ((long long)K * elem_bytes) % 64 != 0) {
             plan_free(pl);
             return MPS_ERR_UNSUPPORTED;
         }
         // the builder indexes X and its own tables by column id
-        int vrc = mps_csr_validate(d_row_ptr, d_col_idx, n_rows, n_rows, nnz, stream);
-        if (vrc != MPS_OK) {
-            plan_free(pl);
-            return vrc;
+        if (flags & MPS_PLAN_FORCE_SWEEP) {
+            int vrc = mps_csr_validate(d_row_ptr, d_col_idx, n_rows, n_rows, nnz, stream);
+            if (vrc != MPS_OK) {
+                plan_free(pl);
+                return vrc;
+            }
         }
         mps_sw::BuildParams bp;
         bp.piece = opt.sweep_piece;
         bp.acc_rows = opt.sweep_acc_rows;
         bp.num_cus = opt.sweep_panels_per_round;  // 0: ask the device
+        bp.together = opt.sweep_together;
         bp.elem_bytes = elem_bytes;
         bp.keep_src = pl->keep_sources;
         int rc = mps_sw::create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, bp, static_cast<hipStream_t>(stream), &pl->sw);
@@ -1444,7 +1521,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->rowblock_cold_index_bits = 0;
     info->rowblock_local_tables = 0;
     info->sweep_panels = info->sweep_acc_rows = info->sweep_lanes = info->sweep_tiles = info->sweep_col_bits = 0;
-    info->sweep_piece = info->sweep_split_rows = info->sweep_partial_rows = info->sweep_listed_rows = 0;
+    info->sweep_piece = info->sweep_together = info->sweep_split_rows = info->sweep_partial_rows = info->sweep_listed_rows = 0;
     info->sweep_rounds = info->sweep_slots = 0;
     if (plan->sw) {
         info->num_slabs = 1;
@@ -1555,7 +1632,7 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     // (slab plans: a row-block plan has neither a cost nor partitions per wavefront, it is one candidate of its own)
     mps_tune_result cand[20];
     int n_cand = 0;
-    const unsigned slab = MPS_PLAN_NO_ROWBLOCK;
+    const unsigned slab = MPS_PLAN_NO_ROWBLOCK | MPS_PLAN_NO_SWEEP;
     const int costs[] = {16, 24, 32, 48, 64, 96, 128, 256};
     for (int c : costs) cand[n_cand++] = {c, max_tpw, slab, 0.f, 0};
     if (max_tpw >= 2) cand[n_cand++] = {dflt, max_tpw / 2, slab, 0.f, 0};
@@ -1563,6 +1640,8 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
     cand[n_cand++] = {dflt, max_tpw, slab | MPS_PLAN_NO_TILING, 0.f, 0};
     if (elem_bytes == 4 && K == 16 && n_rows >= 1 && nnz >= 1 && (uint64_t)n_rows * 64 < kResidentMinXBytes)
         cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_ROWBLOCK, 0.f, 0};
+    if (((long long)K * elem_bytes) % 64 == 0 && n_rows >= 1 && nnz >= 1 && n_rows <= (1 << 26))
+        cand[n_cand++] = {dflt, max_tpw, MPS_PLAN_FORCE_SWEEP, 0.f, 0};
     // slab sizes the model does not pick on its own: larger slabs pay on skewed graphs
     // (not those the model puts 50 % behind the untiled plan: thousands of slabs for a matrix with short rows)
     const double untiled_ps = modelled_ps(n_rows, nnz, K, elem_bytes, 1, n_rows, -1.0);
@@ -1591,7 +1670,7 @@ int mps_plan_autotune(const int *d_row_ptr, const int *d_col_idx, const void *d_
         mps_plan *pl = nullptr;
         rc = mps_plan_create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, elem_bytes, c.cost, c.threads_per_wave, c.flags,
                              (size_t)c.slab_bytes, stream, &pl);
-        if ((c.flags & (MPS_PLAN_FORCE_TILING | MPS_PLAN_FORCE_ROWBLOCK)) && (rc == MPS_ERR_UNSORTED || rc == MPS_ERR_UNSUPPORTED)) {
+        if ((c.flags & (MPS_PLAN_FORCE_TILING | MPS_PLAN_FORCE_ROWBLOCK | MPS_PLAN_FORCE_SWEEP)) && (rc == MPS_ERR_UNSORTED || rc == MPS_ERR_UNSUPPORTED)) {
             rc = MPS_OK;  // this matrix cannot be tiled or blocked that way: not a candidate
             continue;
         }

@@ -65,7 +65,7 @@ struct Piece<half_t> {
 // T: element type of X and Y.  L: lanes per lane-group (16 L bytes of a row of X per tile).
 // LDS: kPlanes planes of (acc_rows + 1) x L float4: plane q holds elements 4 q .. 4 q + 3 of every lane's 16 bytes, so
 // that one 16-byte LDS access per lane covers a plane's row exactly like an fp32 row.
-template <typename T, int L>
+template <typename T, int L, int TOGETHER>
 __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restrict__ stream, const int2 *__restrict__ wave_meta,
                                                             const int *__restrict__ panel_rounds,
                                                             const int *__restrict__ panel_ptr, const int *__restrict__ rows,
@@ -99,43 +99,90 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
         const u4_t t = __builtin_nontemporal_load(reinterpret_cast<const u4_t *>(ws + (size_t)r * RQ));
         return make_uint4(t[0], t[1], t[2], t[3]);
     };
-    uint4 nx = make_uint4(0u, 0u, 0u, 0u);
-    if (rounds > 0) nx = stream_load(0);
-    for (int r = 0; r < most; ++r) {
-        // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
-        // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
-        // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
-        if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
-        if (r >= rounds) continue;
-        const uint4 cu = nx;
-        P xa[kWin], xw[kWin];
-#define SW_GATHER(dst, WORD, j) dst[j].load(xb + (size_t)(from_lane<j>(WORD) & cmask) * row_pitch);
-        SW_GATHER(xa, cu.x, 0) SW_GATHER(xa, cu.x, 1) SW_GATHER(xa, cu.x, 2) SW_GATHER(xa, cu.x, 3)
-        SW_GATHER(xw, cu.z, 0) SW_GATHER(xw, cu.z, 1) SW_GATHER(xw, cu.z, 2) SW_GATHER(xw, cu.z, 3)
+    // the rows of X of a round's 8 entries per lane-group: requested a round ahead of their use
+    auto gather = [&](const uint4 &cu, P (&x)[kRoundInstr]) {
+#define SW_GATHER(k, WORD, j) x[k].load(xb + (size_t)(from_lane<j>(WORD) & cmask) * row_pitch);
+        SW_GATHER(0, cu.x, 0) SW_GATHER(1, cu.x, 1) SW_GATHER(2, cu.x, 2) SW_GATHER(3, cu.x, 3)
+        SW_GATHER(4, cu.z, 0) SW_GATHER(5, cu.z, 1) SW_GATHER(6, cu.z, 2) SW_GATHER(7, cu.z, 3)
 #undef SW_GATHER
-        if (r + 1 < rounds) nx = stream_load(r + 1);
-        // One entry after the other: read the accumulator row, add, write it back.  The LDS serves a wavefront's
-        // accesses in order, so an entry sees what the entry before it wrote; the lane-groups of one instruction
-        // hold different rows (the builder's rule); no other wavefront touches this one's rows.
-#define SW_ADD(xs, WORD, VAL, j)                                                       \
+    };
+    // One entry after the other: read the accumulator row, add, write it back.  The LDS serves a wavefront's
+    // accesses in order, so an entry sees what the entry before it wrote; the lane-groups of one instruction hold
+    // different rows (the builder's rule); no other wavefront touches this one's rows.  TOGETHER == 2: entry q of
+    // window A and entry q of window B at the same time (the builder keeps their rows apart too), which halves
+    // the chain of LDS round trips.
+    auto add_round = [&](const uint4 &cu, const P (&x)[kRoundInstr]) {
+#define SW_FMA(a, v, xv)            \
+    a[0] = fmaf(v, xv[0], a[0]);    \
+    a[1] = fmaf(v, xv[1], a[1]);    \
+    a[2] = fmaf(v, xv[2], a[2]);    \
+    a[3] = fmaf(v, xv[3], a[3]);
+#define SW_ADD(k, WORD, VAL, j)                                                        \
     {                                                                                  \
         const unsigned vr = from_lane<j>(WORD) >> col_bits;                            \
         const float v = __uint_as_float(from_lane<j>(VAL));                            \
         _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
         {                                                                              \
             f4_t *at = acc4 + q * plane_stride + vr * L + c;                           \
-            const f4_t x = xs[j].plane(q);                                             \
+            const f4_t xv = x[k].plane(q);                                             \
             f4_t a = *at;                                                              \
-            a[0] = fmaf(v, x[0], a[0]);                                                \
-            a[1] = fmaf(v, x[1], a[1]);                                                \
-            a[2] = fmaf(v, x[2], a[2]);                                                \
-            a[3] = fmaf(v, x[3], a[3]);                                                \
+            SW_FMA(a, v, xv)                                                           \
             *at = a;                                                                   \
         }                                                                              \
     }
-        SW_ADD(xa, cu.x, cu.y, 0) SW_ADD(xa, cu.x, cu.y, 1) SW_ADD(xa, cu.x, cu.y, 2) SW_ADD(xa, cu.x, cu.y, 3)
-        SW_ADD(xw, cu.z, cu.w, 0) SW_ADD(xw, cu.z, cu.w, 1) SW_ADD(xw, cu.z, cu.w, 2) SW_ADD(xw, cu.z, cu.w, 3)
+#define SW_ADD2(j)                                                                     \
+    {                                                                                  \
+        const unsigned vra = from_lane<j>(cu.x) >> col_bits, vrb = from_lane<j>(cu.z) >> col_bits; \
+        const float va = __uint_as_float(from_lane<j>(cu.y)), vb = __uint_as_float(from_lane<j>(cu.w)); \
+        f4_t a[P::kPlanes], b[P::kPlanes];                                             \
+        _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
+        {                                                                              \
+            a[q] = acc4[q * plane_stride + vra * L + c];                               \
+            b[q] = acc4[q * plane_stride + vrb * L + c];                               \
+        }                                                                              \
+        _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
+        {                                                                              \
+            const f4_t xa = x[j].plane(q), xw = x[kWin + j].plane(q);                  \
+            SW_FMA(a[q], va, xa)                                                       \
+            SW_FMA(b[q], vb, xw)                                                       \
+            acc4[q * plane_stride + vra * L + c] = a[q];                               \
+            acc4[q * plane_stride + vrb * L + c] = b[q];                               \
+        }                                                                              \
+    }
+        if constexpr (TOGETHER == 2) {
+            SW_ADD2(0) SW_ADD2(1) SW_ADD2(2) SW_ADD2(3)
+        } else {
+            SW_ADD(0, cu.x, cu.y, 0) SW_ADD(1, cu.x, cu.y, 1) SW_ADD(2, cu.x, cu.y, 2) SW_ADD(3, cu.x, cu.y, 3)
+            SW_ADD(4, cu.z, cu.w, 0) SW_ADD(5, cu.z, cu.w, 1) SW_ADD(6, cu.z, cu.w, 2) SW_ADD(7, cu.z, cu.w, 3)
+        }
+#undef SW_ADD2
 #undef SW_ADD
+#undef SW_FMA
+    };
+    // Round r is added up while the rows of X of round r + 1 are on their way and the entries of round r + 2 are
+    // being read: loads return in the order they were issued, so the entries of a round are requested before the
+    // gathers of the round in front of it.
+    uint4 cu_a = make_uint4(0u, 0u, 0u, 0u), cu_b = cu_a, nx = cu_a;
+    P x_a[kRoundInstr], x_b[kRoundInstr];
+    if (rounds > 0) cu_a = stream_load(0);
+    if (rounds > 1) nx = stream_load(1);
+    if (rounds > 0) gather(cu_a, x_a);
+    auto step = [&](const uint4 &cu, const P (&x)[kRoundInstr], uint4 &cu_next, P (&x_next)[kRoundInstr], int r) {
+        // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
+        // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
+        // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
+        if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
+        if (r >= rounds) return;
+        if (r + 1 < rounds) {
+            cu_next = nx;
+            if (r + 2 < rounds) nx = stream_load(r + 2);
+            gather(cu_next, x_next);
+        }
+        add_round(cu, x);
+    };
+    for (int r = 0; r < most; r += 2) {
+        step(cu_a, x_a, cu_b, x_b, r);
+        step(cu_b, x_b, cu_a, x_a, r + 1);  // (beyond `most` only when it is odd: an odd round never has a barrier)
     }
     __syncthreads();
 
@@ -216,14 +263,14 @@ int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
     return MPS_OK;
 }
 
-template <typename T, int L>
+template <typename T, int L, int TOGETHER>
 int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
 {
     const Layout &Lo = dp->host;
-    hipLaunchKernelGGL((sw_spmm_kernel<T, L>), dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles), dim3(kThreads), dp->lds_bytes, st,
-                       reinterpret_cast<const uint4 *>(dp->stream), reinterpret_cast<const int2 *>(dp->wave_meta),
-                       dp->panel_rounds, dp->panel_ptr, dp->rows, dp->piece_ptr, X, Y, dp->partial, Lo.n, Lo.K, Lo.acc_rows,
-                       Lo.col_bits, Lo.bank_rows);
+    hipLaunchKernelGGL((sw_spmm_kernel<T, L, TOGETHER>), dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles), dim3(kThreads),
+                       dp->lds_bytes, st, reinterpret_cast<const uint4 *>(dp->stream),
+                       reinterpret_cast<const int2 *>(dp->wave_meta), dp->panel_rounds, dp->panel_ptr, dp->rows, dp->piece_ptr, X,
+                       Y, dp->partial, Lo.n, Lo.K, Lo.acc_rows, Lo.col_bits, Lo.bank_rows);
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
 }
@@ -233,7 +280,8 @@ int spmm_typed(const DevicePlan *dp, const T *X, T *Y, unsigned phases, hipStrea
 {
     const Layout &Lo = dp->host;
     if (phases & MPS_PHASE_MAIN) {
-        const int rc = Lo.lanes == 8 ? launch_main<T, 8>(dp, X, Y, st) : launch_main<T, 4>(dp, X, Y, st);
+        const int rc = Lo.lanes == 8 ? (Lo.together == 2 ? launch_main<T, 8, 2>(dp, X, Y, st) : launch_main<T, 8, 1>(dp, X, Y, st))
+                                     : (Lo.together == 2 ? launch_main<T, 4, 2>(dp, X, Y, st) : launch_main<T, 4, 1>(dp, X, Y, st));
         if (rc != MPS_OK) return rc;
     }
     if ((phases & MPS_PHASE_FIXUP) && !Lo.split_row.empty()) {
@@ -342,10 +390,14 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
     {
         // the limit belongs to the kernel, not to a plan: always what a CU holds
         hipError_t e = hipSuccess;
-        for (const void *kernel : {reinterpret_cast<const void *>(sw_spmm_kernel<float, 4>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8>)})
+        for (const void *kernel : {reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 1>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 2>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 1>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 2>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 1>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 2>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 1>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 2>)})
             if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);

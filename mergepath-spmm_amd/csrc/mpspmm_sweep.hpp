@@ -69,6 +69,8 @@ struct Layout {
     int col_bits = 0;     // an entry word is column | accumulator row << col_bits
     int piece = 0;        // most entries of a row that one accumulator row takes
     int bank_rows = 1;    // G of swizzle()
+    int together = 1;     // instructions whose entries are added up at the same time: 1, or 2 (entry q of windows A and B:
+                          // no two entries of such a pair of instructions share an accumulator row)
     long long rounds = 0; // of all wavefronts
     std::vector<int> panel_ptr;     // [NP + 1] a panel's listed rows: rows[panel_ptr[p] .. panel_ptr[p + 1])
     std::vector<int> rows;          // row of Y that a listed row is written to; n + s: partial row s (a sub-row of a split row)
@@ -85,6 +87,7 @@ struct BuildParams {
     int num_cus = 256;   // panels are made in multiples of this
     int piece = 0;       // 0 = choose
     int acc_rows = 0;    // 0 = what fits in LDS
+    int together = 0;    // 0 = choose (2 with 8 lane-groups per wavefront, else 1)
     int elem_bytes = 4;  // of X and Y (values are handed to the builder as fp32 either way)
     bool keep_src = true;
 };

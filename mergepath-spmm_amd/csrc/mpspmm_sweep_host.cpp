@@ -101,6 +101,13 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     out.bank_rows = std::max(1, 256 / (16 * L));
     const int G = out.bank_rows;
     const int gpw = 64 / L;  // lane-groups of a wavefront = entries of an instruction
+    // instructions whose entries are added up at the same time (see Layout::together).  Measured on MI355X, R-MAT
+    // scale 20 / 22, ms per product with 1 / 2: 64-byte rows 0.128 / 0.124; 128-byte tiles 0.163 / 0.168; fp16 rows of
+    // 128 bytes 0.934 / 0.959 (what pairs save on LDS round trips, their 4 % more padding costs again).
+    const int together = bp.together > 0 ? bp.together : (L == 4 ? 2 : 1);
+    if (together != 1 && together != 2) return MPS_ERR_INVALID_ARG;
+    const int group_slots = gpw * together;
+    out.together = together;
 
     auto deg = [&](int r) { return (long long)rp[r + 1] - rp[r]; };
 
@@ -113,8 +120,10 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         if (R > 8192) return MPS_ERR_UNSUPPORTED;  // (a row that needs more accumulator rows than a panel holds)
         NP = num_cus * R;
         const long long share = std::max<long long>(1, (long long)nnz / NP);
-        // An accumulator row takes one entry per instruction at most, and a wavefront's share is share / 16 / gpw
-        // instructions: a piece of half that many entries finds its instructions among them.
+        // An accumulator row takes one entry per instruction (or pair of instructions) at most, and a wavefront's
+        // share is share / 16 / gpw instructions: a piece of half that many entries finds its places among them
+        // (R-MAT scale 20, 16 per row: 1 % padding with one instruction at a time, 5 % with pairs; pieces of half
+        // the size need half as many accumulator rows again, and a third more panels).
         piece = bp.piece > 0 ? bp.piece : (int)std::min<long long>(1 << 20, std::max<long long>(8, share / kWaves / gpw / 2));
         // a row of about a panel's share or more is cut into sub-rows of a third of a share
         const long long split_from = std::max<long long>(share - share / 10, 4ll * piece);
@@ -284,24 +293,25 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                 std::stable_sort(E.begin(), E.end(), [](const Entry &a, const Entry &b) { return a.col < b.col; });
                 const long long ne = (long long)E.size();
                 slot.resize((size_t)ne);
-                fill.assign((size_t)(ne / gpw + 2), 0);
+                fill.assign((size_t)(ne / group_slots + 2), 0);
                 last.assign((size_t)po.vrows + 1, -1);
                 long long frontier = 0, top = 0;
                 for (long long e = 0; e < ne; ++e) {
                     const int vl = E[(size_t)e].vloc;
                     long long t = std::max<long long>(frontier, (long long)last[(size_t)vl] + 1);
                     for (;;) {
-                        if (t >= (long long)fill.size()) fill.resize((size_t)t + ne / gpw + 2, 0);
-                        if (fill[(size_t)t] < gpw) break;
+                        if (t >= (long long)fill.size()) fill.resize((size_t)t + ne / group_slots + 2, 0);
+                        if (fill[(size_t)t] < group_slots) break;
                         ++t;
                     }
-                    slot[(size_t)e] = t * gpw + fill[(size_t)t];
+                    slot[(size_t)e] = t * group_slots + fill[(size_t)t];
                     ++fill[(size_t)t];
                     last[(size_t)vl] = (int)t;
                     top = std::max(top, t + 1);
-                    while (frontier < (long long)fill.size() && fill[(size_t)frontier] == gpw) ++frontier;
+                    while (frontier < (long long)fill.size() && fill[(size_t)frontier] == group_slots) ++frontier;
                 }
-                const int rounds = (int)((top + kRoundInstr - 1) / kRoundInstr);
+                const int groups_per_round = kRoundInstr / together;
+                const int rounds = (int)((top + groups_per_round - 1) / groups_per_round);
                 po.wave_rounds[w] = rounds;
                 const size_t at0 = po.stream.size();
                 po.stream.resize(at0 + (size_t)rounds * words_per_round);
@@ -312,8 +322,11 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                     s[i + 1] = 0u;
                 }
                 for (long long e = 0; e < ne; ++e) {
-                    const long long t = slot[(size_t)e] / gpw, g = slot[(size_t)e] % gpw;
-                    const long long round = t / kRoundInstr, w2 = (t % kRoundInstr) / kWin, q = t % kWin;
+                    // group t, place i in it -> round, window (A / B), lane of the quad, lane-group: a group is one
+                    // instruction, or entry q of both windows
+                    const long long t = slot[(size_t)e] / group_slots, i = slot[(size_t)e] % group_slots;
+                    const long long round = t / groups_per_round, g = i % gpw;
+                    const long long w2 = together == 2 ? i / gpw : (t % kRoundInstr) / kWin, q = t % kWin;
                     const size_t at = (size_t)((round * gpw * kWin + g * kWin + q) * 4 + w2 * 2);
                     uint32_t bits;
                     std::memcpy(&bits, &E[(size_t)e].val, 4);
@@ -378,6 +391,7 @@ int mps_sweep_layout_build(const int *row_ptr, const int *col_idx, const float *
         bp.piece = options->sweep_piece;
         bp.acc_rows = options->sweep_acc_rows;
         bp.num_cus = options->sweep_panels_per_round;
+        bp.together = options->sweep_together;
         bp.keep_src = !(options->flags & MPS_PLAN_NO_SOURCES);
     }
     if (bp.num_cus <= 0) bp.num_cus = 256;
@@ -408,6 +422,7 @@ void fill_info(const Layout &L, mps_plan_info *info)
     info->sweep_tiles = L.tiles;
     info->sweep_col_bits = L.col_bits;
     info->sweep_piece = L.piece;
+    info->sweep_together = L.together;
     info->sweep_split_rows = (int)L.split_row.size();
     info->sweep_partial_rows = L.split_ptr.empty() ? 0 : L.split_ptr.back();
     info->sweep_listed_rows = (int)L.rows.size();

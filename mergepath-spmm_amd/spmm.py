@@ -178,7 +178,8 @@ class Plan:
     def __init__(self, csr, K, cost=None, threads_per_wave=0, tiling="auto", slab_bytes=0, hot="auto",
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
                  rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None, column_tiles=True,
-                 local_tables=False, sweep="auto", sweep_piece=0, sweep_acc_rows=0, sweep_panels_per_round=0):
+                 local_tables=False, sweep="auto", sweep_piece=0, sweep_acc_rows=0, sweep_panels_per_round=0,
+                 sweep_together=0):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -201,7 +202,7 @@ class Plan:
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
                                 int(rowblock_block_rows), int(rowblock_blocks_per_round),
                                 {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes), int(sweep_piece),
-                                int(sweep_acc_rows), int(sweep_panels_per_round))
+                                int(sweep_acc_rows), int(sweep_panels_per_round), int(sweep_together))
         check(_cabi.lib().mps_plan_create_ex(_ptr(csr.row_ptr), _ptr(csr.col_idx), None if weights else _ptr(csr.val),
                                              csr.n_rows, csr.nnz,
                                              int(K), eb, int(default_cost(csr.n_rows, csr.nnz, K, eb) if cost is None else cost),
@@ -343,7 +344,7 @@ class RowBlockLayout:
         v = np.ascontiguousarray(val, dtype=np.float32)
         opt = _cabi.PlanOptions((0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES) | (_cabi.MPS_PLAN_LOCAL_TABLES if local_tables else 0),
                                 0, int(steps), int(table_rows),
-                                int(block_rows), int(blocks_per_round), 0, 0, 0, 0, 0)
+                                int(block_rows), int(blocks_per_round), 0, 0, 0, 0, 0, 0)
         check(_cabi.lib().mps_rowblock_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size,
                                                     int(K), ctypes.byref(opt), ctypes.byref(self._h)),
               "mps_rowblock_layout_build")
@@ -376,7 +377,8 @@ class RowBlockLayout:
 class SweepLayout:
     """The layout of a sweep plan, built on the host (mps_sweep_layout_build): no GPU needed."""
 
-    def __init__(self, row_ptr, col_idx, val, K, elem_bytes=4, piece=0, acc_rows=0, panels_per_round=0, keep_sources=True):
+    def __init__(self, row_ptr, col_idx, val, K, elem_bytes=4, piece=0, acc_rows=0, panels_per_round=0, keep_sources=True,
+                 together=0):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -384,7 +386,7 @@ class SweepLayout:
         ci = np.ascontiguousarray(col_idx, dtype=np.int32)
         v = np.ascontiguousarray(val, dtype=np.float32)
         opt = _cabi.PlanOptions(0 if keep_sources else _cabi.MPS_PLAN_NO_SOURCES, 0, 0, 0, 0, 0, 0, 0, int(piece), int(acc_rows),
-                                int(panels_per_round))
+                                int(panels_per_round), int(together))
         check(_cabi.lib().mps_sweep_layout_build(rp.ctypes.data, ci.ctypes.data, v.ctypes.data, rp.size - 1, ci.size, int(K),
                                                  int(elem_bytes), ctypes.byref(opt), ctypes.byref(self._h)),
               "mps_sweep_layout_build")

@@ -137,7 +137,7 @@ def test_merge_path_driver_auto_cost(pkg, orc, graph_file, tmp_path):
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
     dump = tmp_path / "y.bin"
     out = run("MergePathSpMM", graph_file, K, "auto", 0, 2, "--dump", dump)
-    assert out.count("tune: cost") == 12  # 11 slab plans (the graph is too small for the slab-size candidates) and a row-block plan
+    assert out.count("tune: cost") == 13  # 11 slab plans (the graph is too small for the slab-size candidates), a row-block plan, a sweep plan
     j = last_json(out)
     assert j["plan"] and j["cost"] in (16, 24, 32, 48, 64, 96, 128, 256)
     Y = np.fromfile(dump, dtype=np.float32).reshape(-1, K)

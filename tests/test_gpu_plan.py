@@ -521,9 +521,9 @@ def test_power_law_graph_auto_plan(pkg, orc, dev):
 
 
 @pytest.mark.parametrize("spec,n_candidates,slab_sizes",
-                         [("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", 12, set()),
+                         [("chunglu:n=20000,nnz=1500000,gamma=2.1,dmax=3000", 13, set()),
                           # X = 15.4 MB: slabs of 3 and 6 MiB are candidates too (X holds more than two of them)
-                          ("chunglu:n=240000,nnz=12000000,gamma=2.1,dmax=5000", 14, {3 << 20, 6 << 20})])
+                          ("chunglu:n=240000,nnz=12000000,gamma=2.1,dmax=5000", 15, {3 << 20, 6 << 20})])
 def test_autotune_picks_a_measured_candidate(pkg, orc, dev, spec, n_candidates, slab_sizes):
     """mps_plan_autotune: every candidate is timed, the reported best is the
     fastest of them, and a plan built from it gives the right product."""
@@ -543,12 +543,14 @@ def test_autotune_picks_a_measured_candidate(pkg, orc, dev, spec, n_candidates, 
     c = pkg._cabi
     tiling = "off" if best["flags"] & c.MPS_PLAN_NO_TILING else "force" if best["flags"] & c.MPS_PLAN_FORCE_TILING else "auto"
     hot = "off" if best["flags"] & c.MPS_PLAN_NO_HOT else "auto"
-    # fp32, K = 16, X below 192 MiB: one candidate is a row-block plan, all others are slab plans
+    # fp32, K = 16, X below 192 MiB: one candidate is a row-block plan, one a sweep plan, all others are slab plans
     assert sum(1 for t in tried if t["flags"] & c.MPS_PLAN_FORCE_ROWBLOCK) == 1
-    assert all(t["flags"] & (c.MPS_PLAN_FORCE_ROWBLOCK | c.MPS_PLAN_NO_ROWBLOCK) for t in tried)
-    rowblock = "force" if best["flags"] & c.MPS_PLAN_FORCE_ROWBLOCK else "off"
+    assert sum(1 for t in tried if t["flags"] & c.MPS_PLAN_FORCE_SWEEP) == 1
+    assert all(t["flags"] & (c.MPS_PLAN_FORCE_ROWBLOCK | c.MPS_PLAN_NO_ROWBLOCK | c.MPS_PLAN_FORCE_SWEEP) for t in tried)
+    rowblock = "force" if best["flags"] & c.MPS_PLAN_FORCE_ROWBLOCK else "auto" if best["flags"] & c.MPS_PLAN_FORCE_SWEEP else "off"
+    sweep = "force" if best["flags"] & c.MPS_PLAN_FORCE_SWEEP else "off"
     plan = pkg.spmm.Plan(csr, K, cost=best["cost"], threads_per_wave=best["threads_per_wave"], tiling=tiling, hot=hot,
-                         slab_bytes=best["slab_bytes"], rowblock=rowblock)
+                         slab_bytes=best["slab_bytes"], rowblock=rowblock, sweep=sweep)
     Y = plan.spmm(d_X)
     torch.cuda.synchronize()
     ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)

@@ -21,6 +21,9 @@ CASES = [
     (1000, 20, (), 32, "f16", 0, 0, 4),                            # fp16, 64-byte rows
     (700, 25, ((3, 650),), 128, "f16", 16, 0, 4),                  # fp16, two column tiles
     (1, 1, (), 16, "f32", 0, 0, 1),
+    (3000, 40, ((5, 2800),), 16, "f32", 0, 0, 8, 2),               # 64-byte rows with pairs of instructions added up together
+    (3000, 40, ((5, 2800),), 32, "f32", 0, 0, 8, 1),               # 128-byte rows, one instruction at a time
+    (2000, 30, ((11, 1500),), 64, "f16", 0, 0, 8, 1),
 ]
 
 
@@ -34,12 +37,14 @@ def make_inputs(rng, n, max_deg, hubs, K, dt):
 
 @pytest.mark.parametrize("case", CASES)
 def test_sweep_plan_matches_fp64_loop(pkg, orc, dev, case):
-    n, max_deg, hubs, K, dt, piece, acc_rows, per_round = case
+    n, max_deg, hubs, K, dt, piece, acc_rows, per_round = case[:8]
+    together = case[8] if len(case) > 8 else 0
     rng = np.random.default_rng(abs(hash(case)) % (2 ** 32))
     rp, ci, val, X = make_inputs(rng, n, max_deg, hubs, K, dt)
     csr = make_csr(pkg, dev, rp, ci, val)
     (d_X,) = to_dev(dev, X)
-    plan = pkg.spmm.Plan(csr, K, sweep="force", sweep_piece=piece, sweep_acc_rows=acc_rows, sweep_panels_per_round=per_round)
+    plan = pkg.spmm.Plan(csr, K, sweep="force", sweep_piece=piece, sweep_acc_rows=acc_rows, sweep_panels_per_round=per_round,
+                         sweep_together=together)
     i = plan.info
     assert i.sweep_panels > 0 and i.rowblock_steps == 0
     assert i.sweep_tiles * i.sweep_lanes * 16 == K * X.itemsize

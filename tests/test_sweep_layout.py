@@ -18,6 +18,8 @@ def walk(pkg, lay, n, K, X, elem_bytes):
     C = pkg._cabi
     i = lay.info
     L, tiles, cb, acc_rows, NP = i.sweep_lanes, i.sweep_tiles, i.sweep_col_bits, i.sweep_acc_rows, i.sweep_panels
+    together = i.sweep_together
+    assert together in (1, 2)
     gpw = 64 // L
     G = max(1, 256 // (16 * L))
     assert tiles * L * 16 == K * elem_bytes
@@ -48,9 +50,9 @@ def walk(pkg, lay, n, K, X, elem_bytes):
             most = max(most, rounds)
             last_col = -1
             for r in range(first, first + rounds):
+                rows_of = {}  # (window, lane of quad) -> accumulator rows of that instruction
                 for t in range(ROUND_INSTR):
                     win, q = t // 4, t % 4
-                    rows_here = []
                     for g in range(gpw):
                         word, vb = st[r, g * 4 + q, win]
                         e = sr[r, g * 4 + q, win]
@@ -62,11 +64,17 @@ def walk(pkg, lay, n, K, X, elem_bytes):
                             assert vr < acc_rows
                             assert owner[vr] in (-1, w), "an accumulator row belongs to one wavefront"
                             owner[vr] = w
-                            rows_here.append(vr)
+                            rows_of.setdefault((win, q), []).append(vr)
                             seen[e] += 1
                             wave_entries[b * WAVES + w] += 1
                         acc[vr] += v * X[col]
-                    assert len(set(rows_here)) == len(rows_here), "two entries of one instruction share an accumulator row"
+                # what is added up at the same time never shares an accumulator row: the entries of one instruction,
+                # or (together == 2) of entry q of both windows
+                for q in range(4):
+                    groups = [rows_of.get((0, q), []) + rows_of.get((1, q), [])] if together == 2 else \
+                        [rows_of.get((0, q), []), rows_of.get((1, q), [])]
+                    for rows_here in groups:
+                        assert len(set(rows_here)) == len(rows_here), "two entries added up at the same time share an accumulator row"
         assert prounds[b] == most
         p0, p1 = panel_ptr[b], panel_ptr[b + 1]
         pp = piece_ptr[p0 + b:p1 + b + 1]
@@ -86,26 +94,30 @@ def walk(pkg, lay, n, K, X, elem_bytes):
 
 
 CASES = [
-    # n, max_deg, hubs, K, elem_bytes, piece, acc_rows, panels_per_round
-    (300, 12, ((5, 280),), 16, 4, 0, 0, 4),
-    (97, 6, (), 32, 4, 4, 0, 2),
-    (513, 20, ((0, 500), (512, 400)), 64, 4, 8, 64, 3),
-    (200, 5, (), 16, 4, 2, 16, 8),            # few accumulator rows per panel: several rounds of panels
-    (257, 9, ((100, 257),), 64, 2, 0, 0, 4),  # fp16: 128-byte rows, two accumulator planes
-    (64, 3, (), 32, 2, 0, 0, 1),              # fp16, 64-byte rows: rows dealt in pairs
-    (1, 1, (), 16, 4, 0, 0, 2),
+    # n, max_deg, hubs, K, elem_bytes, piece, acc_rows, panels_per_round, together
+    (300, 12, ((5, 280),), 16, 4, 0, 0, 4, 0),
+    (97, 6, (), 32, 4, 4, 0, 2, 0),
+    (513, 20, ((0, 500), (512, 400)), 64, 4, 8, 64, 3, 0),
+    (200, 5, (), 16, 4, 2, 16, 8, 0),            # few accumulator rows per panel: several rounds of panels
+    (257, 9, ((100, 257),), 64, 2, 0, 0, 4, 0),  # fp16: 128-byte rows, two accumulator planes
+    (64, 3, (), 32, 2, 0, 0, 1, 0),              # fp16, 64-byte rows: rows dealt in pairs
+    (1, 1, (), 16, 4, 0, 0, 2, 0),
+    (300, 12, ((5, 280),), 16, 4, 0, 0, 4, 2),   # 64-byte rows with pairs of instructions
+    (400, 9, ((100, 257),), 32, 4, 0, 0, 4, 1),  # 128-byte rows, one instruction at a time
 ]
 
 
 @pytest.mark.parametrize("case", CASES)
 def test_sweep_layout_walk(pkg, case):
-    n, max_deg, hubs, K, eb, piece, acc_rows, per_round = case
+    n, max_deg, hubs, K, eb, piece, acc_rows, per_round, together = case
     rng = np.random.default_rng(abs(hash(case)) % (2 ** 32))
     rp, ci = random_csr(rng, n, max_deg, p_empty=0.3, hub_rows=hubs)
     val = rng.random(ci.size).astype(np.float32)
     X = rng.random((n, K)) * 2 - 1
-    lay = pkg.spmm.SweepLayout(rp, ci, val, K, elem_bytes=eb, piece=piece, acc_rows=acc_rows, panels_per_round=per_round)
+    lay = pkg.spmm.SweepLayout(rp, ci, val, K, elem_bytes=eb, piece=piece, acc_rows=acc_rows, panels_per_round=per_round,
+                               together=together)
     assert lay.info.sweep_panels % per_round == 0
+    assert lay.info.sweep_together == (together or (2 if lay.info.sweep_lanes == 4 else 1))
     Y, wave_entries = walk(pkg, lay, n, K, X, eb)
     ref = sps.csr_matrix((val.astype(np.float64), ci, rp), shape=(n, n)) @ X
     assert np.allclose(Y, ref, rtol=1e-12, atol=1e-12)
