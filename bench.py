@@ -66,24 +66,37 @@ def plan_signature(workload, info):
                                                                         info.threads_per_wave, info.hot_rows, info.resident_cols)
 
 
-def measured_traffic(signature):
-    """HBM bytes per launch of the dominant kernel for this plan shape, from the table of counter runs under
-    profiles/ (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a
-    plain copy of known size).  None when the table has no row for the signature."""
+def measured_counters(signature):
+    """Counter readings for this plan shape from the table of counter runs under profiles/: HBM bytes per launch of the
+    dominant kernel (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a
+    plain copy of known size), the L2 hit rate of that kernel (TCC_HIT / (TCC_HIT + TCC_MISS), all its requests: the
+    gathers of rows of X, the sparse streams and the stores) and the summary they come from.  (None, None, None) when the
+    table has no row for the signature; the hit rate is None for rows measured before it was collected."""
     try:
         text = open(TRAFFIC_TABLE).read()
     except OSError:
-        return None, None
+        return None, None, None
     for line in text.splitlines():
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
-        # | signature (its own '|' written as ';') | kernel | FETCH_SIZE KiB | fetch factor | WRITE_SIZE KiB | write factor | summary |
-        if len(cells) == 7 and cells[0].replace(";", "|").replace("`", "") == signature:
+        # | signature (its own '|' written as ';') | kernel | FETCH_SIZE KiB | fetch factor | WRITE_SIZE KiB | write factor |
+        #   [TCC_HIT | TCC_MISS |] summary |
+        if len(cells) in (7, 9) and cells[0].replace(";", "|").replace("`", "") == signature:
             try:
                 fetch, ff, write, wf = float(cells[2]), float(cells[3]), float(cells[4]), float(cells[5])
+                hit_rate = None
+                if len(cells) == 9:
+                    hits, misses = float(cells[6]), float(cells[7])
+                    hit_rate = round(hits / (hits + misses), 4) if hits + misses > 0 else None
             except ValueError:
                 continue
-            return int((fetch * ff + write * wf) * 1024), "profiles/" + cells[6].replace("`", "")
-    return None, None
+            return int((fetch * ff + write * wf) * 1024), hit_rate, "profiles/" + cells[-1].replace("`", "")
+    return None, None, None
+
+
+def measured_traffic(signature):
+    """(HBM bytes per launch of the dominant kernel, the summary under profiles/ it comes from) for a plan signature."""
+    traffic, _, where = measured_counters(signature)
+    return traffic, where
 
 
 class Workload:
@@ -153,6 +166,74 @@ def layout_text(w, plan):
     if i.hot_rows:
         text += ", %d hot columns per slab in LDS (%.1f %% of the nonzeros)" % (i.hot_rows, 100.0 * i.hot_nnz / max(w.nnz, 1))
     return text
+
+
+def kernels_of(info, cus):
+    """Which kernel each phase of a product launches for this kind of plan (None: the phase launches nothing)."""
+    if info is None:
+        return {"PREPARE": None, "MAIN": "mp_spmm_kernel", "FIXUP": "mp_fixup_kernel", "REDUCE": None}
+    if info.sweep_panels > 0:
+        return {"PREPARE": None, "MAIN": "sw_spmm_kernel", "FIXUP": "sw_fixup_kernel" if info.sweep_split_rows > 0 else None,
+                "REDUCE": None}
+    if info.rowblock_steps > 0:
+        # a plan of one step and one round of blocks, or with local tables, reads its tables from X in the main kernel
+        from_x = info.rowblock_local_tables or (info.rowblock_steps == 1 and info.rowblock_blocks <= cus)
+        return {"PREPARE": None if from_x else "rb_gather_hot_kernel", "MAIN": "rb_spmm_kernel", "FIXUP": None, "REDUCE": None}
+    return {"PREPARE": None, "MAIN": "mp_spmm_kernel (hot + cold launch)" if info.hot_rows > 0 else "mp_spmm_kernel",
+            "FIXUP": "mp_fixup_kernel", "REDUCE": "tile_reduce_kernel" if info.num_slabs > 1 else None}
+
+
+def phase_times(torch, PH, step, kernels, steps):
+    """Average duration of every phase that launches something, from HIP events on the launch stream, over `steps`
+    products phase by phase; None for a phase that launches nothing."""
+    order = [("PREPARE", PH.MPS_PHASE_PREPARE), ("MAIN", PH.MPS_PHASE_MAIN), ("FIXUP", PH.MPS_PHASE_FIXUP),
+             ("REDUCE", PH.MPS_PHASE_REDUCE)]
+    live = [(name, ph) for name, ph in order if kernels[name] is not None]
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(live) + 1)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    for row in evs:
+        row[0].record()
+        for k, (_, ph) in enumerate(live):
+            step(ph)
+            row[k + 1].record()
+    torch.cuda.synchronize()
+    out = {kernels[name]: None for name, _ in order if kernels[name] is not None}
+    for k, (name, _) in enumerate(live):
+        out[kernels[name]] = round(sum(r[k].elapsed_time(r[k + 1]) for r in evs) / steps, 5)
+    return out
+
+
+GATE_F32 = "|err| <= 1e-5 * sum_j |a_ij x_jk| + 1e-6 per element and ||err|| / ||ref|| <= 1e-5 against the fp64 row loop"
+GATE_F16 = "|err| <= 2e-2 * |ref| + 2e-5 * sum_j |a_ij x_jk| + 1e-6 per element and ||err|| / ||ref|| <= 2e-2 against the fp64 row loop"
+
+
+def check_product(np, orc, w, Yg, with_cpu_loop=None):
+    """The product against the oracle's fp64 row loop: the gate the tests pin (relative to sum_j |a_ij x_jk| where rows
+    are long and their terms cancel), and beside it how many elements miss the bar read literally."""
+    ref, scale = (orc.spmm_f64_f16in if w.f16 else orc.spmm_f64)(w.rp, w.ci, w.val, w.X, want_abs=True)
+    Yg = Yg.astype(np.float64)
+    err_g = np.abs(Yg - ref)
+    literal = (2e-2 * np.abs(ref) + 1e-6) if w.f16 else (1e-5 * np.abs(ref) + 1e-6)
+    gate = (2e-2 * np.abs(ref) + 2e-5 * scale + 1e-6) if w.f16 else (1e-5 * scale + 1e-6)
+    rel_fro = float(np.linalg.norm(err_g) / max(np.linalg.norm(ref), 1e-30))
+    ok = bool(np.isfinite(Yg).all() and rel_fro <= (2e-2 if w.f16 else 1e-5) and (err_g <= gate).all())
+    out = {"ok": ok, "gate": GATE_F16 if w.f16 else GATE_F32, "rel_fro": rel_fro, "max_abs_err": float(err_g.max()),
+           "elements": int(ref.size), "outside_literal_bar_gpu": int((err_g > literal).sum()),
+           "literal_bar": "|err| <= 2e-2 |ref| + 1e-6 (fp16)" if w.f16 else "|err| <= 1e-5 |ref| + 1e-6"}
+    if with_cpu_loop is not None:
+        out["outside_literal_bar_cpu_fp32_loop"] = int((np.abs(with_cpu_loop.astype(np.float64) - ref) > literal).sum())
+    return out
+
+
+def describe_plan(name, w, plan, g, tpw_arg, cost):
+    """The config fields that say what ran: cost, partitions and partitions per wavefront only for plans that have them."""
+    info = plan.info if plan is not None else None
+    slab = info is None or (info.sweep_panels == 0 and info.rowblock_steps == 0)
+    return {"layout": layout_text(w, plan), "plan_signature": plan_signature(name, info),
+            "cost": cost if slab else None, "partitions": (info.num_partitions if info is not None else None) if slab else None,
+            "threads_per_wave": (tpw_arg or g.max_threads_per_wave(w.K, w.eb)) if slab else None,
+            "plan_bytes": int(info.device_bytes) if info is not None else 0,
+            "csr_bytes": int(4 * (w.n + 1) + (4 + w.eb) * w.nnz)}
 
 
 def calibrate_copy(torch, dev):
@@ -260,115 +341,79 @@ def main():
         kw.update(overrides)
         return sp.Plan(wl.csr, wl.K, **kw), cost
 
-    cost = args.cost if args.cost > 0 else sp.default_cost(w.n, w.nnz, K, w.eb)
-    plan = None
-    if args.mode != "plain":
-        plan, cost = make_plan(w)
-        P = plan.info.num_partitions
-    else:
-        sched = sp.generate_mp_sched(w.csr.row_ptr, w.nnz, cost=cost)
-        P = sched.P
-    torch.cuda.synchronize()
-    info = plan.info if plan is not None else None
-    rowblock = info is not None and info.rowblock_steps > 0
-    sweep = info is not None and info.sweep_panels > 0
-    tiled = info is not None and info.num_slabs > 1
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    orc = None if args.no_cpu else entry.load_oracle()
 
-    def step(phases=None):
-        if plan is not None:
-            plan.spmm(w.d_X, out=w.d_Y, phases=phases)
+    def run(wl, wname, steps, warmup, plain=False, graph=False, cpu_loop=None, **overrides):
+        """One workload with one kind of plan: exactly `steps` timed products after `warmup`, then the per-kernel
+        durations, the counter readings on file for that plan shape, and the check against the fp64 row loop."""
+        plan, sched = None, None
+        cost = args.cost if args.cost > 0 else sp.default_cost(wl.n, wl.nnz, wl.K, wl.eb)
+        if plain:
+            sched = sp.generate_mp_sched(wl.csr.row_ptr, wl.nnz, cost=cost)
         else:
-            sp.spmm_merge_path(w.csr, w.d_X, sched, threads_per_wave=args.tpw, out=w.d_Y, phases=phases)
-
-    for _ in range(args.warmup):
-        step()
-    timed_step = step
-    if args.graph:
+            plan, cost = make_plan(wl, **overrides)
         torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
+        info = plan.info if plan is not None else None
+
+        def step(phases=None):
+            if plan is not None:
+                plan.spmm(wl.d_X, out=wl.d_Y, phases=phases)
+            else:
+                sp.spmm_merge_path(wl.csr, wl.d_X, sched, threads_per_wave=args.tpw, out=wl.d_Y, phases=phases)
+
+        for _ in range(warmup):
             step()
-        torch.cuda.current_stream().wait_stream(side)
+        timed_step = step
+        if graph:
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            hip_graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(hip_graph):
+                step()
+            timed_step = hip_graph.replay
+        # ---- timed region: exactly `steps` steps, inputs already in HBM ----------
+        ms, wall_ms = time_steps(torch, timed_step, steps, warmup if graph else 0)
+        kernels = kernels_of(info, cus)
+        kernel_ms = phase_times(torch, PH, step, kernels, steps)
+        main_name = kernels["MAIN"]
+        main_ms = kernel_ms[main_name]
+        desc = describe_plan(wname, wl, plan, g, args.tpw, cost)
+        if plan is None:
+            desc["partitions"] = sched.P
+        traffic, l2_hit, where = measured_counters(desc["plan_signature"])
+        res = {"ms_per_step": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5), "gflops": round(wl.flops / (ms * 1e6), 2),
+               "kernel_ms": kernel_ms, "main_kernel": main_name,
+               "phases": {k.lower(): v for k, v in kernels.items()},  # the kernel each phase launches; null: nothing
+               "frac_step": round(wl.b_alg / (ms * 1e6) / PEAK_HBM_GBS, 4),
+               "frac_main_kernel": round(wl.b_alg / (main_ms * 1e6) / PEAK_HBM_GBS, 4),
+               "traffic": traffic, "l2_hit_rate": l2_hit, "counters_from": where, "algorithmic_bytes": int(wl.b_alg)}
+        res.update(desc)
+        if orc is not None:
+            res["check"] = check_product(np, orc, wl, wl.d_Y.float().cpu().numpy(), cpu_loop)
+        # preprocessing time (once per matrix, not part of a step)
         torch.cuda.synchronize()
-        hip_graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(hip_graph):
-            step()
-        timed_step = hip_graph.replay
-    # ---- timed region: exactly `steps` steps, inputs already in HBM ----------
-    ms_per_step, wall_ms = time_steps(torch, timed_step, args.steps, args.warmup if args.graph else 0)
+        t1 = time.perf_counter()
+        if plan is not None:
+            make_plan(wl, **overrides)[0].close()
+        else:
+            sp.generate_mp_sched(wl.csr.row_ptr, wl.nnz, cost=cost)
+        torch.cuda.synchronize()
+        res["preprocessing_ms"] = round((time.perf_counter() - t1) * 1e3, 3)
+        if plan is not None:
+            plan.close()
+        return res
 
-    # ---- per-kernel durations over the same number of steps (events on the launch stream)
-    order = [PH.MPS_PHASE_PREPARE, PH.MPS_PHASE_MAIN, PH.MPS_PHASE_FIXUP, PH.MPS_PHASE_REDUCE]
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    for row in evs:
-        row[0].record()
-        for k, ph in enumerate(order):
-            if (ph == PH.MPS_PHASE_PREPARE and not rowblock) or (ph == PH.MPS_PHASE_REDUCE and not tiled) or \
-               (ph == PH.MPS_PHASE_FIXUP and (rowblock or (sweep and info.sweep_split_rows == 0))):
-                pass
-            elif plan is not None or ph in (PH.MPS_PHASE_MAIN, PH.MPS_PHASE_FIXUP):
-                step(ph)
-            row[k + 1].record()
-    torch.cuda.synchronize()
-    prep_ms, main_ms, fix_ms, red_ms = [sum(r[k].elapsed_time(r[k + 1]) for r in evs) / args.steps for k in range(4)]
-
-    # preprocessing time (once per matrix, not part of a step)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    if plan is not None:
-        make_plan(w)[0].close()
-    else:
-        sp.generate_mp_sched(w.csr.row_ptr, w.nnz, cost=cost)
-    torch.cuda.synchronize()
-    plan_ms = (time.perf_counter() - t1) * 1e3
-
-    gflops = w.flops / (ms_per_step * 1e6)
-    achieved = w.b_alg / (main_ms * 1e6)
-    main_name = "sw_spmm_kernel" if sweep else "rb_spmm_kernel" if rowblock else ("mp_spmm_kernel (hot + cold launch)" if info is not None and info.hot_rows > 0 else "mp_spmm_kernel")
-    signature = plan_signature(name, info)
-    traffic, traffic_from = measured_traffic(signature)
-    csr_bytes = 4 * (w.n + 1) + (4 + w.eb) * w.nnz
-
-    out = {
-        "metric": "SpMM GFLOP/s (2*nnz*K/t), merge-path CSR x row-major dense",
-        "value": round(gflops, 2),
-        "unit": "GFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "scaling_note": "one GPU only: nothing is scaled",
-        "vs_baseline": None,
-        "dtype": dt,
-        "data": "synthetic (seeded generator, values U[0,1), features U[-1,1))",
-        "launch": "one HIP graph replay per step" if args.graph else "kernel launches per step",
-        "config": {"workload": name, "spec": spec, "n_rows": int(w.n), "nnz": int(w.nnz), "K": K,
-                   "max_row_degree": int(w.max_deg), "cost": cost, "partitions": P,
-                   "threads_per_wave": args.tpw or g.max_threads_per_wave(K, w.eb), "seed": args.seed,
-                   "values": args.values, "weights": "value array" if args.weights == "none" else "one factor per node (no value array)",
-                   "layout": layout_text(w, plan), "plan_signature": signature,
-                   "plan_bytes": int(info.device_bytes) if info is not None else 0, "csr_bytes": int(csr_bytes)},
-        "gbs_algorithmic_per_step": round(w.b_alg / (ms_per_step * 1e6), 2),
-        "hbm_fraction_per_step": round(w.b_alg / (ms_per_step * 1e6) / PEAK_HBM_GBS, 4),
-        "kernel_ms": {main_name: round(main_ms, 5), "rb_gather_hot_kernel": round(prep_ms, 5),
-                      "mp_fixup_kernel": round(fix_ms, 5), "tile_reduce_kernel": round(red_ms, 5),
-                      "preprocessing, host wall time (once per matrix)": round(plan_ms, 3)},
-        "wall_ms_per_step": round(wall_ms, 5),
-        "roofline": {"bound": "hbm", "kernel": main_name, "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": traffic,
-                     "traffic_from": traffic_from, "algorithmic_bytes": int(w.b_alg)},
-        "host_generate_s": round(w.gen_s, 2),
-    }
-
-    ok = True
-    if not args.no_cpu:
+    cpu = None
+    Yc = None
+    if orc is not None:
         # CPU baseline leg: the oracle's multithreaded fp32 CSR x dense loop on this box's host cores,
         # bounded to a few passes over the same workload.
-        orc = entry.load_oracle()
         present = os.cpu_count() or 1
         threads = max(1, min(present, orc.max_threads()))
         val32 = w.val.astype(np.float32) if w.f16 else w.val
@@ -382,49 +427,77 @@ def main():
             spent += time.perf_counter() - c0
             passes += 1
         cpu_s = spent / passes
-        out["cpu_baseline"] = {"value": round(w.flops / cpu_s / 1e9, 3), "unit": "GFLOP/s", "cores": threads,
-                               "cores_present": present, "kind": "port",
-                               "sample": "%d full passes over the same workload, %.3f s each" % (passes, cpu_s)}
-        # the product against the fp64 row loop, beside what the CPU's own sequential fp32 loop achieves
-        ref, scale = (orc.spmm_f64_f16in if w.f16 else orc.spmm_f64)(w.rp, w.ci, w.val, w.X, want_abs=True)
-        Yg = w.d_Y.float().cpu().numpy().astype(np.float64)
-        err_g, err_c = np.abs(Yg - ref), np.abs(Yc.astype(np.float64) - ref)
-        bar = (2e-2 * np.abs(ref) + 2e-5 * scale + 1e-6) if w.f16 else (1e-5 * np.abs(ref) + 1e-6)
-        rel_fro = float(np.linalg.norm(err_g) / max(np.linalg.norm(ref), 1e-30))
-        ok = bool(np.isfinite(Yg).all() and rel_fro <= (2e-2 if w.f16 else 1e-5) and
-                  (err_g <= (2e-2 * np.abs(ref) + 2e-5 * scale + 1e-6 if w.f16 else 1e-5 * scale + 1e-6)).all())
-        out["check_vs_cpu_fp32"] = {"ok": ok, "rel_fro": rel_fro, "max_abs_err": float(err_g.max()),
-                                "elements": int(ref.size),
-                                "outside_literal_bar_gpu": int((err_g > bar).sum()),
-                                "outside_literal_bar_cpu_fp32_loop": int((err_c > bar).sum()),
-                                "literal_bar": "|err| <= 2e-2 |ref| (fp16)" if w.f16 else "|err| <= 1e-5 |ref| + 1e-6"}
-    if plan is not None:
-        plan.close()
+        cpu = {"value": round(w.flops / cpu_s / 1e9, 3), "unit": "GFLOP/s", "cores": threads, "cores_present": present,
+               "kind": "port", "sample": "%d full passes over the same workload, %.3f s each" % (passes, cpu_s)}
+
+    head = run(w, name, args.steps, args.warmup, plain=args.mode == "plain", graph=args.graph, cpu_loop=Yc)
+    achieved = w.b_alg / (head["kernel_ms"][head["main_kernel"]] * 1e6)
+    out = {
+        "metric": "SpMM GFLOP/s (2*nnz*K/t), merge-path CSR x row-major dense",
+        "value": head["gflops"],
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "scaling_note": "one GPU only: nothing is scaled",
+        "vs_baseline": None,
+        "dtype": dt,
+        "data": "synthetic (seeded generator, values U[0,1), features U[-1,1))",
+        "launch": "one HIP graph replay per step" if args.graph else "kernel launches per step",
+        "config": {"workload": name, "spec": spec, "n_rows": int(w.n), "nnz": int(w.nnz), "K": K,
+                   "max_row_degree": int(w.max_deg), "cost": head["cost"], "partitions": head["partitions"],
+                   "threads_per_wave": head["threads_per_wave"], "seed": args.seed,
+                   "values": args.values, "weights": "value array" if args.weights == "none" else "one factor per node (no value array)",
+                   "layout": head["layout"], "plan_signature": head["plan_signature"],
+                   "plan_bytes": head["plan_bytes"], "csr_bytes": head["csr_bytes"]},
+        "gbs_algorithmic_per_step": round(w.b_alg / (head["ms_per_step"] * 1e6), 2),
+        "hbm_fraction_per_step": head["frac_step"],
+        "kernel_ms": dict(head["kernel_ms"], **{"preprocessing, host wall time (once per matrix)": head["preprocessing_ms"]}),
+        "phases": head["phases"],
+        "wall_ms_per_step": head["wall_ms_per_step"],
+        "roofline": {"bound": "hbm", "kernel": head["main_kernel"], "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": head["traffic"],
+                     "l2_hit_rate": head["l2_hit_rate"], "traffic_from": head["counters_from"],
+                     "algorithmic_bytes": int(w.b_alg)},
+        "host_generate_s": round(w.gen_s, 2),
+    }
+    ok = True
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+        out["check_vs_cpu_fp32"] = head["check"]
+        ok = head["check"]["ok"]
 
     if not args.no_configs and not custom and args.workload == HEADLINE:
-        # the other configurations of the benchmark, each with the library's own plan, the same timed loop
-        del w
-        torch.cuda.empty_cache()
+        # the other configurations of the benchmark, each with the library's own plan and the same timed loop; first
+        # the headline graph once more with the merge-path slab plan (partitioner, LDS-staged windows, carry-out fix-up)
         rows = []
         steps_c, warm_c = min(args.steps, 30), min(args.warmup, 10)
-        cache = {}
+        r = run(w, name, steps_c, warm_c, rowblock="off", sweep="off")
+        rows.append(dict({"workload": name + "|slab", "n_rows": int(w.n), "nnz": int(w.nnz), "K": K, "dtype": dt}, **r))
+        del w
+        torch.cuda.empty_cache()
         for cname in OTHER_CONFIGS:
             cspec, cK, cdt = WORKLOADS[cname]
             wl = Workload(pkg, cname, cspec, cK, cdt, args.seed, torch, dev)
-            pl, ccost = make_plan(wl)
-            ms, _ = time_steps(torch, lambda: pl.spmm(wl.d_X, out=wl.d_Y), steps_c, warm_c)
-            rows.append({"workload": cname, "n_rows": int(wl.n), "nnz": int(wl.nnz), "K": cK, "dtype": cdt,
-                         "ms_per_step": round(ms, 5), "gflops": round(wl.flops / (ms * 1e6), 2),
-                         "frac": round(wl.b_alg / (ms * 1e6) / PEAK_HBM_GBS, 4), "layout": layout_text(wl, pl)})
-            pl.close()
-            del wl, pl
+            r = run(wl, cname, steps_c, warm_c)
+            rows.append(dict({"workload": cname, "n_rows": int(wl.n), "nnz": int(wl.nnz), "K": cK, "dtype": cdt}, **r))
+            del wl
             torch.cuda.empty_cache()
+        for r in rows:
+            r["frac"] = r["frac_step"]
+            if "check" in r:
+                ok = ok and r["check"]["ok"]
         out["configs"] = rows
-        out["configs_note"] = "frac = algorithmic bytes / whole-step time / 8 TB/s; %d steps after %d warm-ups each" % (steps_c, warm_c)
+        out["configs_note"] = ("frac = algorithmic bytes / whole-step time / 8 TB/s, frac_main_kernel the same over the main "
+                               "kernel's time; %d steps after %d warm-ups each; kernel_ms: a phase that launches nothing has "
+                               "no entry; traffic and l2_hit_rate from the counter runs under profiles/" % (steps_c, warm_c))
 
     print(json.dumps(out))
     if not ok:
-        sys.exit("bench.py: the product is outside the tolerance of the fp64 row loop")
+        sys.exit("bench.py: a product is outside the tolerance of the fp64 row loop")
 
 
 if __name__ == "__main__":

@@ -40,6 +40,35 @@ int bits_for(unsigned v)
     return b < 1 ? 1 : b;
 }
 
+// Indices 0 .. n - 1 with size_of(i) > 0, largest first, equal sizes in index order (a counting sort: sizes are
+// mostly small; the few above the table are sorted by comparison).
+template <typename Size>
+std::vector<int> largest_first(int n, Size size_of)
+{
+    constexpr long long kTable = 1 << 16;
+    std::vector<int> count((size_t)kTable + 1, 0), big, order;
+    for (int i = 0; i < n; ++i) {
+        const long long s = size_of(i);
+        if (s >= kTable) big.push_back(i);
+        else if (s > 0) ++count[(size_t)s];
+    }
+    std::stable_sort(big.begin(), big.end(), [&](int a, int b) { return size_of(a) > size_of(b); });
+    // first place of every size among the small ones, largest size first
+    long long at = (long long)big.size();
+    for (long long s = kTable - 1; s >= 1; --s) {
+        const int c = count[(size_t)s];
+        count[(size_t)s] = (int)at;
+        at += c;
+    }
+    order.resize((size_t)at);
+    std::copy(big.begin(), big.end(), order.begin());
+    for (int i = 0; i < n; ++i) {
+        const long long s = size_of(i);
+        if (s > 0 && s < kTable) order[(size_t)count[(size_t)s]++] = i;
+    }
+    return order;
+}
+
 // Largest first, each to the bin with the smallest load so far; a bin takes at most `cap` of `cost`.
 // false if some item finds no bin.
 template <typename Size, typename Cost>
@@ -113,7 +142,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
 
     // ---- panels: how many, how rows are cut, which row goes where
     std::vector<Item> items;
-    std::vector<int> item_panel;
+    std::vector<int> item_panel, order;  // order: the items that hold nonzeros, largest first
     std::vector<int> split_of((size_t)n, 0);  // sub-rows of a row (0: not split)
     int NP = 0, piece = 0;
     for (int R = 1;; ++R) {
@@ -165,12 +194,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             r += take;
         }
         if (totv > (long long)NP * vcap) continue;
-        std::vector<int> order;
-        order.reserve(items.size());
-        for (int i = 0; i < (int)items.size(); ++i)
-            if (items[(size_t)i].nnz > 0) order.push_back(i);
-        std::stable_sort(order.begin(), order.end(),
-                         [&](int a, int b) { return items[(size_t)a].nnz > items[(size_t)b].nnz; });
+        order = largest_first((int)items.size(), [&](int i) { return items[(size_t)i].nnz; });
         item_panel.assign(items.size(), 0);
         if (!deal_largest_first(
                 order, [&](int i) { return items[(size_t)i].nnz; }, [&](int i) { return (long long)items[(size_t)i].pieces; },
@@ -191,12 +215,10 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     for (int p = 0; p < NP; ++p) panel_count[(size_t)p + 1] += panel_count[(size_t)p];
     std::vector<int> panel_items(items.size());
     {
-        std::vector<int> order(items.size());
-        std::iota(order.begin(), order.end(), 0);
-        std::stable_sort(order.begin(), order.end(),
-                         [&](int a, int b) { return items[(size_t)a].nnz > items[(size_t)b].nnz; });
         std::vector<int> fill(panel_count.begin(), panel_count.end() - 1);
         for (int i : order) panel_items[(size_t)fill[(size_t)item_panel[(size_t)i]]++] = i;
+        for (int i = 0; i < (int)items.size(); ++i)
+            if (items[(size_t)i].nnz == 0) panel_items[(size_t)fill[(size_t)item_panel[(size_t)i]]++] = i;
     }
     // partial row of sub-row j of split row r
     std::vector<int> split_index((size_t)n, -1);
@@ -261,9 +283,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             *pp = v;
             po.vrows = v;
             // accumulator rows to wavefronts
-            vorder.resize((size_t)v);
-            std::iota(vorder.begin(), vorder.end(), 0);
-            std::stable_sort(vorder.begin(), vorder.end(), [&](int a, int b) { return vsize[(size_t)a] > vsize[(size_t)b]; });
+            vorder = largest_first(v, [&](int i) { return (long long)vsize[(size_t)i]; });
             vwave.assign((size_t)v, 0);
             deal_largest_first(
                 vorder, [&](int i) { return (long long)vsize[(size_t)i]; }, [](int) { return 0ll; }, kWaves, 1, vwave);

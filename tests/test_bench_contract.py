@@ -25,6 +25,49 @@ def test_traffic_is_looked_up_by_plan_signature_and_names_its_profile():
     assert bench.measured_traffic(bench.HEADLINE + "|rowblock|steps=99|table_rows=1|blocks=1|cold_index_bits=0") == (None, None)
 
 
+def test_hit_rate_comes_from_the_same_row_and_old_rows_have_none():
+    table = open(bench.TRAFFIC_TABLE).read()
+    seen_rate = False
+    for line in table.splitlines():
+        if not line.startswith("| `"):
+            continue
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        sig = cells[0].replace("`", "").replace(";", "|")
+        traffic, rate, where = bench.measured_counters(sig)
+        assert traffic and where
+        if len(cells) == 9:
+            assert rate == round(float(cells[6]) / (float(cells[6]) + float(cells[7])), 4) and 0.0 < rate < 1.0
+            seen_rate = True
+        else:
+            assert len(cells) == 7 and rate is None
+    assert seen_rate
+    assert bench.measured_counters("no such plan") == (None, None, None)
+
+
+class FakeInfo:
+    def __init__(self, **kw):
+        self.sweep_panels = self.sweep_split_rows = self.rowblock_steps = self.rowblock_blocks = 0
+        self.rowblock_local_tables = self.hot_rows = 0
+        self.num_slabs = 1
+        self.__dict__.update(kw)
+
+
+def test_phases_that_launch_nothing_have_no_kernel():
+    k = bench.kernels_of(FakeInfo(sweep_panels=256), 256)
+    assert k == {"PREPARE": None, "MAIN": "sw_spmm_kernel", "FIXUP": None, "REDUCE": None}
+    assert bench.kernels_of(FakeInfo(sweep_panels=512, sweep_split_rows=1), 256)["FIXUP"] == "sw_fixup_kernel"
+    k = bench.kernels_of(FakeInfo(rowblock_steps=16, rowblock_blocks=256), 256)
+    assert k == {"PREPARE": "rb_gather_hot_kernel", "MAIN": "rb_spmm_kernel", "FIXUP": None, "REDUCE": None}
+    # one step, one round of blocks, or tables of a block's own: the table comes from X inside the main kernel
+    assert bench.kernels_of(FakeInfo(rowblock_steps=1, rowblock_blocks=256), 256)["PREPARE"] is None
+    assert bench.kernels_of(FakeInfo(rowblock_steps=1, rowblock_blocks=512, rowblock_local_tables=1), 256)["PREPARE"] is None
+    assert bench.kernels_of(FakeInfo(rowblock_steps=1, rowblock_blocks=512), 256)["PREPARE"] == "rb_gather_hot_kernel"
+    k = bench.kernels_of(FakeInfo(num_slabs=5, hot_rows=1728), 256)
+    assert k["REDUCE"] == "tile_reduce_kernel" and k["FIXUP"] == "mp_fixup_kernel" and "hot + cold" in k["MAIN"]
+    assert bench.kernels_of(FakeInfo(), 256)["REDUCE"] is None
+    assert bench.kernels_of(None, 256)["MAIN"] == "mp_spmm_kernel"
+
+
 def test_workloads_cover_the_benchmark_configurations():
     assert bench.HEADLINE in bench.WORKLOADS and len(bench.OTHER_CONFIGS) == 8
     assert all(w in bench.WORKLOADS for w in bench.OTHER_CONFIGS)
