@@ -66,16 +66,27 @@ def plan_signature(workload, info):
                                                                         info.threads_per_wave, info.hot_rows, info.resident_cols)
 
 
-def measured_counters(signature):
+def lines_read_once(w, info):
+    """128-byte lines that a product of a row-block or sweep plan touches exactly once - the plan's entry streams and
+    the rows of Y - and that therefore miss L2 by nature; None for the other kinds of plan, whose partial rows are
+    written and read again."""
+    if info is None or (info.sweep_panels == 0 and info.rowblock_steps == 0):
+        return None
+    streams = 8 * int(info.sweep_slots) * info.sweep_tiles if info.sweep_panels > 0 else int(info.device_bytes)
+    return (streams + w.n * w.K * w.eb) // 128
+
+
+def measured_counters(signature, with_requests=False, other_lines=None):
     """Counter readings for this plan shape from the table of counter runs under profiles/: HBM bytes per launch of the
     dominant kernel (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a
     plain copy of known size), the L2 hit rate of that kernel (TCC_HIT / (TCC_HIT + TCC_MISS), all its requests: the
     gathers of rows of X, the sparse streams and the stores) and the summary they come from.  (None, None, None) when the
     table has no row for the signature; the hit rate is None for rows measured before it was collected."""
+    none = (None, None, None, None) if with_requests else (None, None, None)
     try:
         text = open(TRAFFIC_TABLE).read()
     except OSError:
-        return None, None, None
+        return none
     for line in text.splitlines():
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
         # | signature (its own '|' written as ';') | kernel | FETCH_SIZE KiB | fetch factor | WRITE_SIZE KiB | write factor |
@@ -83,14 +94,18 @@ def measured_counters(signature):
         if len(cells) in (7, 9) and cells[0].replace(";", "|").replace("`", "") == signature:
             try:
                 fetch, ff, write, wf = float(cells[2]), float(cells[3]), float(cells[4]), float(cells[5])
-                hit_rate = None
+                hit_rate = gather_rate = None
                 if len(cells) == 9:
                     hits, misses = float(cells[6]), float(cells[7])
                     hit_rate = round(hits / (hits + misses), 4) if hits + misses > 0 else None
+                    # the gathers of rows of X alone: all requests less the lines that are touched once (they miss)
+                    if other_lines is not None and hits + misses > other_lines and misses >= other_lines:
+                        gather_rate = round(hits / (hits + misses - other_lines), 4)
             except ValueError:
                 continue
-            return int((fetch * ff + write * wf) * 1024), hit_rate, "profiles/" + cells[-1].replace("`", "")
-    return None, None, None
+            found = (int((fetch * ff + write * wf) * 1024), hit_rate, "profiles/" + cells[-1].replace("`", ""))
+            return found + (gather_rate,) if with_requests else found
+    return none
 
 
 def measured_traffic(signature):
@@ -386,13 +401,15 @@ def main():
         desc = describe_plan(wname, wl, plan, g, args.tpw, cost)
         if plan is None:
             desc["partitions"] = sched.P
-        traffic, l2_hit, where = measured_counters(desc["plan_signature"])
+        traffic, l2_hit, where, gather_hit = measured_counters(desc["plan_signature"], with_requests=True,
+                                                               other_lines=lines_read_once(wl, info))
         res = {"ms_per_step": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5), "gflops": round(wl.flops / (ms * 1e6), 2),
                "kernel_ms": kernel_ms, "main_kernel": main_name,
                "phases": {k.lower(): v for k, v in kernels.items()},  # the kernel each phase launches; null: nothing
                "frac_step": round(wl.b_alg / (ms * 1e6) / PEAK_HBM_GBS, 4),
                "frac_main_kernel": round(wl.b_alg / (main_ms * 1e6) / PEAK_HBM_GBS, 4),
-               "traffic": traffic, "l2_hit_rate": l2_hit, "counters_from": where, "algorithmic_bytes": int(wl.b_alg)}
+               "traffic": traffic, "l2_hit_rate": l2_hit, "l2_hit_rate_gathers_est": gather_hit, "counters_from": where,
+               "algorithmic_bytes": int(wl.b_alg)}
         res.update(desc)
         if orc is not None:
             res["check"] = check_product(np, orc, wl, wl.d_Y.float().cpu().numpy(), cpu_loop)
@@ -460,7 +477,8 @@ def main():
         "wall_ms_per_step": head["wall_ms_per_step"],
         "roofline": {"bound": "hbm", "kernel": head["main_kernel"], "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": head["traffic"],
-                     "l2_hit_rate": head["l2_hit_rate"], "traffic_from": head["counters_from"],
+                     "l2_hit_rate": head["l2_hit_rate"], "l2_hit_rate_gathers_est": head["l2_hit_rate_gathers_est"],
+                     "traffic_from": head["counters_from"],
                      "algorithmic_bytes": int(w.b_alg)},
         "host_generate_s": round(w.gen_s, 2),
     }

@@ -42,6 +42,22 @@ def test_hit_rate_comes_from_the_same_row_and_old_rows_have_none():
             assert len(cells) == 7 and rate is None
     assert seen_rate
     assert bench.measured_counters("no such plan") == (None, None, None)
+    assert bench.measured_counters("no such plan", with_requests=True, other_lines=5) == (None, None, None, None)
+
+
+def test_gather_hit_rate_leaves_out_the_lines_that_are_read_once():
+    info = FakeInfo(sweep_panels=256, sweep_slots=16932864, sweep_tiles=1, device_bytes=0)
+
+    class W:
+        n, K, eb = 1 << 20, 16, 4
+
+    once = bench.lines_read_once(W, info)
+    assert once == (8 * 16932864 + (1 << 20) * 64) // 128
+    sig = "rmat_s20_f32_k16|sweep|panels=256|tiles=1|acc_rows=2444|piece=122"
+    traffic, rate, where, gathers = bench.measured_counters(sig, with_requests=True, other_lines=once)
+    assert traffic and where and rate < gathers < 1.0
+    # slab plans write partial rows and read them again: no such estimate
+    assert bench.lines_read_once(W, FakeInfo()) is None and bench.lines_read_once(W, None) is None
 
 
 class FakeInfo:
