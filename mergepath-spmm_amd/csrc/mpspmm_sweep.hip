@@ -48,6 +48,10 @@ struct Piece<float> {
     static constexpr int kVec = 4, kPlanes = 1;
     f4_t raw;
     __device__ __forceinline__ void load(const char *p) { raw = *reinterpret_cast<const f4_t *>(p); }
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned base)
+    {
+        raw = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, (int)base, 0));
+    }
     __device__ __forceinline__ f4_t plane(int) const { return raw; }
 };
 template <>
@@ -55,6 +59,10 @@ struct Piece<half_t> {
     static constexpr int kVec = 8, kPlanes = 2;
     half8_t raw;
     __device__ __forceinline__ void load(const char *p) { raw = *reinterpret_cast<const half8_t *>(p); }
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned base)
+    {
+        raw = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, (int)base, 0));
+    }
     __device__ __forceinline__ f4_t plane(int q) const
     {
         return q == 0 ? f4_t{(float)raw[0], (float)raw[1], (float)raw[2], (float)raw[3]}
@@ -62,10 +70,12 @@ struct Piece<half_t> {
     }
 };
 
-// T: element type of X and Y.  L: lanes per lane-group (16 L bytes of a row of X per tile).
+// T: element type of X and Y.  L: lanes per lane-group (16 L bytes of a row of X per tile).  FAR: X is addressed with
+// 64-bit pointers; otherwise (X below 4 GiB, fewer than 2^24 rows) with a 32-bit offset that one 24-bit
+// multiply-add forms.
 // LDS: kPlanes planes of (acc_rows + 1) x L float4: plane q holds elements 4 q .. 4 q + 3 of every lane's 16 bytes, so
 // that one 16-byte LDS access per lane covers a plane's row exactly like an fp32 row.
-template <typename T, int L, int TOGETHER>
+template <typename T, int L, int TOGETHER, bool FAR>
 __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restrict__ stream, const int2 *__restrict__ wave_meta,
                                                             const int *__restrict__ panel_rounds,
                                                             const int *__restrict__ panel_ptr, const int *__restrict__ rows,
@@ -92,98 +102,112 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     const uint4 *ws = stream + (size_t)wm.x * RQ + (g * kWin + s);
     const unsigned cmask = (1u << col_bits) - 1u;
     // this lane's 16 bytes of a row of X: row pitch K elements, tile `tile`, piece c
-    const size_t row_pitch = (size_t)K * sizeof(T);
-    const char *xb = reinterpret_cast<const char *>(X) + (size_t)tile * (16 * L) + (size_t)c * 16;
+    const unsigned row_pitch = (unsigned)K * (unsigned)sizeof(T);
+    const unsigned lane_off = (unsigned)c * 16u, tile_off = (unsigned)tile * (16u * L);
+    [[maybe_unused]] const char *xb = reinterpret_cast<const char *>(X) + tile_off + lane_off;
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(X), 0, 0xffffffff, 0x00020000);
+    const unsigned plane_bytes = (unsigned)plane_stride * 16u;
 
     auto stream_load = [&](int r) {
         const u4_t t = __builtin_nontemporal_load(reinterpret_cast<const u4_t *>(ws + (size_t)r * RQ));
         return make_uint4(t[0], t[1], t[2], t[3]);
     };
-    // the rows of X of a round's 8 entries per lane-group: requested a round ahead of their use
-    auto gather = [&](const uint4 &cu, P (&x)[kRoundInstr]) {
-#define SW_GATHER(k, WORD, j) x[k].load(xb + (size_t)(from_lane<j>(WORD) & cmask) * row_pitch);
-        SW_GATHER(0, cu.x, 0) SW_GATHER(1, cu.x, 1) SW_GATHER(2, cu.x, 2) SW_GATHER(3, cu.x, 3)
-        SW_GATHER(4, cu.z, 0) SW_GATHER(5, cu.z, 1) SW_GATHER(6, cu.z, 2) SW_GATHER(7, cu.z, 3)
-#undef SW_GATHER
-    };
+    // The row of X of entry k of a round (of 8 entries per lane-group), and where in the LDS (plane 0) this lane adds it.
+    P x[kRoundInstr];
+    unsigned at[kRoundInstr];
+#define SW_GATHER(k, WORD, j)                                                                \
+    {                                                                                        \
+        const unsigned w = from_lane<j>(WORD);                                               \
+        at[k] = (w >> col_bits) * (16u * L) + lane_off;                                      \
+        if constexpr (FAR) {                                                                 \
+            x[k].load(xb + (size_t)(w & cmask) * row_pitch);                                 \
+        } else {                                                                             \
+            x[k].load(x_rsrc, __umul24(w & cmask, row_pitch) + lane_off, tile_off);          \
+        }                                                                                    \
+    }
     // One entry after the other: read the accumulator row, add, write it back.  The LDS serves a wavefront's
     // accesses in order, so an entry sees what the entry before it wrote; the lane-groups of one instruction hold
     // different rows (the builder's rule); no other wavefront touches this one's rows.  TOGETHER == 2: entry q of
     // window A and entry q of window B at the same time (the builder keeps their rows apart too), which halves
     // the chain of LDS round trips.
-    auto add_round = [&](const uint4 &cu, const P (&x)[kRoundInstr]) {
 #define SW_FMA(a, v, xv)            \
     a[0] = fmaf(v, xv[0], a[0]);    \
     a[1] = fmaf(v, xv[1], a[1]);    \
     a[2] = fmaf(v, xv[2], a[2]);    \
     a[3] = fmaf(v, xv[3], a[3]);
-#define SW_ADD(k, WORD, VAL, j)                                                        \
+#define SW_AT(k, q) reinterpret_cast<f4_t *>(smem + at[k] + (q) * plane_bytes)
+#define SW_ADD(k, VAL, j)                                                              \
     {                                                                                  \
-        const unsigned vr = from_lane<j>(WORD) >> col_bits;                            \
         const float v = __uint_as_float(from_lane<j>(VAL));                            \
         _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
         {                                                                              \
-            f4_t *at = acc4 + q * plane_stride + vr * L + c;                           \
             const f4_t xv = x[k].plane(q);                                             \
-            f4_t a = *at;                                                              \
+            f4_t a = *SW_AT(k, q);                                                     \
             SW_FMA(a, v, xv)                                                           \
-            *at = a;                                                                   \
+            *SW_AT(k, q) = a;                                                          \
         }                                                                              \
     }
 #define SW_ADD2(j)                                                                     \
     {                                                                                  \
-        const unsigned vra = from_lane<j>(cu.x) >> col_bits, vrb = from_lane<j>(cu.z) >> col_bits; \
         const float va = __uint_as_float(from_lane<j>(cu.y)), vb = __uint_as_float(from_lane<j>(cu.w)); \
         f4_t a[P::kPlanes], b[P::kPlanes];                                             \
         _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
         {                                                                              \
-            a[q] = acc4[q * plane_stride + vra * L + c];                               \
-            b[q] = acc4[q * plane_stride + vrb * L + c];                               \
+            a[q] = *SW_AT(j, q);                                                       \
+            b[q] = *SW_AT(kWin + j, q);                                                \
         }                                                                              \
         _Pragma("unroll") for (int q = 0; q < P::kPlanes; ++q)                         \
         {                                                                              \
             const f4_t xa = x[j].plane(q), xw = x[kWin + j].plane(q);                  \
             SW_FMA(a[q], va, xa)                                                       \
             SW_FMA(b[q], vb, xw)                                                       \
-            acc4[q * plane_stride + vra * L + c] = a[q];                               \
-            acc4[q * plane_stride + vrb * L + c] = b[q];                               \
+            *SW_AT(j, q) = a[q];                                                       \
+            *SW_AT(kWin + j, q) = b[q];                                                \
         }                                                                              \
     }
-        if constexpr (TOGETHER == 2) {
-            SW_ADD2(0) SW_ADD2(1) SW_ADD2(2) SW_ADD2(3)
-        } else {
-            SW_ADD(0, cu.x, cu.y, 0) SW_ADD(1, cu.x, cu.y, 1) SW_ADD(2, cu.x, cu.y, 2) SW_ADD(3, cu.x, cu.y, 3)
-            SW_ADD(4, cu.z, cu.w, 0) SW_ADD(5, cu.z, cu.w, 1) SW_ADD(6, cu.z, cu.w, 2) SW_ADD(7, cu.z, cu.w, 3)
+    // Entry k of round r is added up, and the registers that held its row of X at once take the request for entry k
+    // of round r + 1: every row of X is asked for a round ahead of its use, in one set of registers, and the entries
+    // of round r + 2 are read meanwhile.  No branch goes around a load (where two paths with different loads in
+    // flight meet, the compiler waits for all of them): past the wavefront's last round the loop asks for that
+    // round's entries and rows a second time and drops them.
+    if (rounds > 0) {
+        const int last = rounds - 1;
+        uint4 cu = stream_load(0), nx = stream_load(min(1, last));
+        SW_GATHER(0, cu.x, 0) SW_GATHER(1, cu.x, 1) SW_GATHER(2, cu.x, 2) SW_GATHER(3, cu.x, 3)
+        SW_GATHER(4, cu.z, 0) SW_GATHER(5, cu.z, 1) SW_GATHER(6, cu.z, 2) SW_GATHER(7, cu.z, 3)
+        for (int r = 0; r < rounds; ++r) {
+            // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
+            // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
+            // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
+            if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
+            const uint4 cn = nx;
+            nx = stream_load(min(r + 2, last));
+            if constexpr (TOGETHER == 2) {
+                SW_ADD2(0) SW_GATHER(0, cn.x, 0) SW_GATHER(4, cn.z, 0)
+                SW_ADD2(1) SW_GATHER(1, cn.x, 1) SW_GATHER(5, cn.z, 1)
+                SW_ADD2(2) SW_GATHER(2, cn.x, 2) SW_GATHER(6, cn.z, 2)
+                SW_ADD2(3) SW_GATHER(3, cn.x, 3) SW_GATHER(7, cn.z, 3)
+            } else {
+                SW_ADD(0, cu.y, 0) SW_GATHER(0, cn.x, 0)
+                SW_ADD(1, cu.y, 1) SW_GATHER(1, cn.x, 1)
+                SW_ADD(2, cu.y, 2) SW_GATHER(2, cn.x, 2)
+                SW_ADD(3, cu.y, 3) SW_GATHER(3, cn.x, 3)
+                SW_ADD(4, cu.w, 0) SW_GATHER(4, cn.z, 0)
+                SW_ADD(5, cu.w, 1) SW_GATHER(5, cn.z, 1)
+                SW_ADD(6, cu.w, 2) SW_GATHER(6, cn.z, 2)
+                SW_ADD(7, cu.w, 3) SW_GATHER(7, cn.z, 3)
+            }
+            cu = cn;
         }
+    }
 #undef SW_ADD2
 #undef SW_ADD
+#undef SW_AT
 #undef SW_FMA
-    };
-    // Round r is added up while the rows of X of round r + 1 are on their way and the entries of round r + 2 are
-    // being read: loads return in the order they were issued, so the entries of a round are requested before the
-    // gathers of the round in front of it.
-    uint4 cu_a = make_uint4(0u, 0u, 0u, 0u), cu_b = cu_a, nx = cu_a;
-    P x_a[kRoundInstr], x_b[kRoundInstr];
-    if (rounds > 0) cu_a = stream_load(0);
-    if (rounds > 1) nx = stream_load(1);
-    if (rounds > 0) gather(cu_a, x_a);
-    auto step = [&](const uint4 &cu, const P (&x)[kRoundInstr], uint4 &cu_next, P (&x_next)[kRoundInstr], int r) {
-        // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
-        // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
-        // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
-        if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
-        if (r >= rounds) return;
-        if (r + 1 < rounds) {
-            cu_next = nx;
-            if (r + 2 < rounds) nx = stream_load(r + 2);
-            gather(cu_next, x_next);
-        }
-        add_round(cu, x);
-    };
-    for (int r = 0; r < most; r += 2) {
-        step(cu_a, x_a, cu_b, x_b, r);
-        step(cu_b, x_b, cu_a, x_a, r + 1);  // (beyond `most` only when it is odd: an odd round never has a barrier)
-    }
+#undef SW_GATHER
+    // the barriers of the rounds that other wavefronts of the panel still have, and the one before the sums are read
+    for (int r = (rounds + kSyncRounds - 1) & ~(kSyncRounds - 1); r < most; r += kSyncRounds) __syncthreads();
     __syncthreads();
 
     // the panel's rows, once: a row's pieces added up in order, rows without nonzeros as zeros
@@ -263,16 +287,26 @@ int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
     return MPS_OK;
 }
 
-template <typename T, int L, int TOGETHER>
+template <typename T, int L, int TOGETHER, bool FAR>
 int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
 {
     const Layout &Lo = dp->host;
-    hipLaunchKernelGGL((sw_spmm_kernel<T, L, TOGETHER>), dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles), dim3(kThreads),
+    hipLaunchKernelGGL((sw_spmm_kernel<T, L, TOGETHER, FAR>), dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles), dim3(kThreads),
                        dp->lds_bytes, st, reinterpret_cast<const uint4 *>(dp->stream),
                        reinterpret_cast<const int2 *>(dp->wave_meta), dp->panel_rounds, dp->panel_ptr, dp->rows, dp->piece_ptr, X,
                        Y, dp->partial, Lo.n, Lo.K, Lo.acc_rows, Lo.col_bits, Lo.bank_rows);
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
+}
+
+template <typename T, int L, int TOGETHER>
+int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
+{
+    // 32-bit offsets into X where every row starts below 4 GiB and a column index fits the 24-bit multiply
+    const Layout &Lo = dp->host;
+    const bool far = Lo.col_bits > 24 || (unsigned long long)Lo.n * (unsigned long long)Lo.K * sizeof(T) > 0xffffff00ull ||
+                     (unsigned long long)Lo.K * sizeof(T) >= (1ull << 24);
+    return far ? launch_main<T, L, TOGETHER, true>(dp, X, Y, st) : launch_main<T, L, TOGETHER, false>(dp, X, Y, st);
 }
 
 template <typename T>
@@ -390,14 +424,22 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
     {
         // the limit belongs to the kernel, not to a plan: always what a CU holds
         hipError_t e = hipSuccess;
-        for (const void *kernel : {reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 1>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 2>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 1>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 2>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 1>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 2>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 1>),
-                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 2>)})
+        for (const void *kernel : {reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 1, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 1, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 2, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 4, 2, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 1, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 1, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 2, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<float, 8, 2, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 1, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 1, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 2, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 4, 2, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 1, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 1, true>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 2, false>),
+                                   reinterpret_cast<const void *>(sw_spmm_kernel<half_t, 8, 2, true>)})
             if (e == hipSuccess) e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
