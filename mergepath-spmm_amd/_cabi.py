@@ -40,6 +40,7 @@ MPS_PLAN_NO_COLUMN_TILES = 512
 MPS_PLAN_LOCAL_TABLES = 1024
 MPS_PLAN_NO_SWEEP = 2048
 MPS_PLAN_FORCE_SWEEP = 4096
+MPS_PLAN_HOST_BUILD = 8192
 (MPS_PLAN_ARRAY_VROW_PTR, MPS_PLAN_ARRAY_COORD_X, MPS_PLAN_ARRAY_COORD_Y, MPS_PLAN_ARRAY_WAVE_OFF,
  MPS_PLAN_ARRAY_SLICE_COLS, MPS_PLAN_ARRAY_SLICE_SRC, MPS_PLAN_ARRAY_SLICE_VALS, MPS_PLAN_ARRAY_HOT_COLS,
  MPS_PLAN_ARRAY_RB_BLOCK_ROW, MPS_PLAN_ARRAY_RB_HOT_COLS, MPS_PLAN_ARRAY_RB_META, MPS_PLAN_ARRAY_RB_WAVE_BASE,

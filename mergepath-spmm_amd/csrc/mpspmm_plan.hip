@@ -1454,6 +1454,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
         bp.local_tables = (flags & MPS_PLAN_LOCAL_TABLES) != 0;
+        bp.host_build = (flags & MPS_PLAN_HOST_BUILD) != 0;
         if (!(flags & MPS_PLAN_FORCE_ROWBLOCK)) {
             bp.max_local_share = kMaxLocalShare;
             bp.max_longest_row = kMaxLongestRow;

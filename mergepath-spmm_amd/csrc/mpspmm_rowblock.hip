@@ -500,6 +500,448 @@ void release(std::vector<T> &v)
     std::vector<T>().swap(v);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The builder's passes over the nonzeros, on the device.  The layout is the one that build_layout makes on the host,
+// entry for entry: what needs only row_ptr or the nonzero counts of the columns is decided by the same host code
+// (plan_blocks, plan_columns), and the kernels below count, cut and place the way passes 1 and 2 of build_layout and
+// pack_hot_stream / pack_cold_stream do.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kBuildMaxSteps = 64;  // a wavefront ranks the nonzeros of a row in an LDS table of 2 counters per step
+
+__global__ __launch_bounds__(256) void rbb_degree_kernel(const int *__restrict__ ci, int nnz, int *__restrict__ deg)
+{
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < (size_t)nnz; e += (size_t)gridDim.x * blockDim.x)
+        atomicAdd(&deg[ci[e]], 1);
+}
+
+// One workgroup per row block: range_nnz[r] += the block's nonzeros in column range r of R equal ones; *own += the
+// count of its busiest range.
+__global__ __launch_bounds__(256) void rbb_ranges_kernel(const int *__restrict__ rp, const int *__restrict__ ci,
+                                                          const int *__restrict__ block_row, int n, int R,
+                                                          unsigned long long *__restrict__ range_nnz,
+                                                          unsigned long long *__restrict__ own)
+{
+    extern __shared__ int hist[];  // [R], then the block's maximum
+    const int b = blockIdx.x, tid = threadIdx.x;
+    for (int i = tid; i <= R; i += 256) hist[i] = 0;
+    __syncthreads();
+    const int e1 = rp[block_row[b + 1]];
+    for (int e = rp[block_row[b]] + tid; e < e1; e += 256) atomicAdd(&hist[(int)((long long)ci[e] * R / n)], 1);
+    __syncthreads();
+    int most = 0;
+    for (int i = tid; i < R; i += 256) {
+        const int c = hist[i];
+        most = max(most, c);
+        if (c) atomicAdd(&range_nnz[i], (unsigned long long)c);
+    }
+    atomicMax(&hist[R], most);
+    __syncthreads();
+    if (tid == 0) atomicAdd(own, (unsigned long long)hist[R]);
+}
+
+// One wavefront per row.  Every nonzero gets its key (step, kind: 0 hot, 1 cold) and its rank among the nonzeros of
+// the row with that key, in CSR order.  PLACE false: cnt[((t n) + row) 2 + kind] = nonzeros of the key.  PLACE true:
+// the nonzero is written to its place in the packed hot or cold stream (pass 2 of build_layout).
+struct PlaceArgs {
+    const float *val;
+    const int *pre, *prevrow, *block_row, *meta, *run_start, *step_windows, *cold_begin;
+    const long long *round_off;
+    uint32_t *hot, *cold;
+    int *hot_src, *cold_src, *overflow;
+    int num_blocks, cold_ib;
+};
+
+__device__ __forceinline__ void put_entry(uint32_t *stream, int *src, long long round, int g, int e, int which, bool real,
+                                          uint32_t value, uint32_t half, int nonzero)
+{
+    const size_t at = ((size_t)round * 64 + (size_t)(g * kWin + e)) * 3;
+    if (real) stream[at + which] = value;
+    reinterpret_cast<uint16_t *>(stream + at + 2)[which] = (uint16_t)half;
+    if (real && src) src[(size_t)round * kRoundEntries + (size_t)(g * kWin + e) * kPair + which] = nonzero;
+}
+
+template <bool PLACE>
+__global__ __launch_bounds__(256) void rbb_rows_kernel(const int *__restrict__ rp, const int *__restrict__ ci,
+                                                        const int16_t *__restrict__ col_step,
+                                                        const int16_t *__restrict__ col_slot, int n, int T, int *cnt,
+                                                        PlaceArgs pa)
+{
+    __shared__ int counters[4][2 * kBuildMaxSteps];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + wave;
+    if (r >= n) return;  // (no barrier below: a wavefront works on its own)
+    volatile int *base = counters[wave];
+    base[lane] = 0;
+    base[lane + 64] = 0;
+    const int e0 = rp[r], e1 = rp[r + 1];
+    int b = 0, lr = 0;
+    if constexpr (PLACE) {
+        int lo = 0, hi = pa.num_blocks;  // the block of the row: block_row[b] <= r < block_row[b + 1]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (pa.block_row[mid] <= r) lo = mid; else hi = mid;
+        }
+        b = lo;
+        lr = r - pa.block_row[b];
+    }
+    for (int at = e0; at < e1; at += 64) {
+        const int e = at + lane;
+        const bool valid = e < e1;
+        int c = 0, slot = -1, key = -1;
+        if (valid) {
+            c = ci[e];
+            slot = col_slot[c];
+            key = col_step[c] * 2 + (slot < 0);
+        }
+        int rank = 0;
+        unsigned long long todo = __ballot(valid);
+        while (todo) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const int lkey = __shfl(key, leader);
+            const bool mine = valid && key == lkey;
+            const unsigned long long same = __ballot(mine);
+            const int before = base[lkey];
+            if (mine) rank = before + __popcll(same & ((1ull << lane) - 1ull));
+            if (lane == leader) base[lkey] = before + __popcll(same);
+            todo &= ~same;
+        }
+        if constexpr (PLACE) {
+            if (!valid) continue;
+            const int t = key >> 1, k = key & 1;
+            const size_t gi = ((size_t)t * n + r) * 2;
+            const int group = cnt[gi + k];
+            const int wi = rank >> 2, en = rank & 3;
+            const int pre_h = pa.pre[gi], pre_c = pa.pre[gi + 1];
+            const int pk = (k ? pre_c : pre_h) + wi;  // windows of this kind before this one in the step
+            const long long q = (long long)pre_h + pre_c + (k ? (cnt[gi] + kWin - 1) / kWin : 0) + wi;  // windows before it
+            const size_t bt = (size_t)b * T + t;
+            const long long E = pa.step_windows[bt];
+            int w = (int)min(q * kWaves / E, (long long)(kWaves - 1));  // the run of window q: runs start at w E / 16
+            while (w > 0 && q < (long long)w * E / kWaves) --w;
+            while (q >= (long long)(w + 1) * E / kWaves) ++w;
+            const size_t run = bt * kWaveSlots + w;
+            int g, j;
+            deal(pa.meta[run * 4 + k], pk - pa.run_start[run * 2 + k], &g, &j);
+            const int prev = j == 0 ? pa.meta[run * 4 + 2] : (wi > 0 ? lr : pa.prevrow[gi + k]);
+            const uint32_t adv = (uint32_t)(lr - prev);
+            const long long round = pa.round_off[run * 2 + k] + j / kPair;
+            const int which = j % kPair;
+            const int pads = rank == group - 1 ? kWin - 1 - en : 0;  // the window's last nonzero repeated with value 0
+            const uint32_t value = __float_as_uint(pa.val[e]);
+            if (k == 0) {
+                if (adv > kPackedAdvMax) *pa.overflow = 1;
+                const uint32_t piece_mask = (1u << kPackedPieceBits) - 1u;
+                for (int ee = en; ee <= en + pads; ++ee) {
+                    const uint32_t piece = ee == 0 ? (adv & piece_mask) : ee == 1 ? ((adv >> kPackedPieceBits) & piece_mask) : 0u;
+                    put_entry(pa.hot, pa.hot_src, round, g, ee, which, ee == en, value, (uint32_t)slot | (piece << kPackedSlotBits), e);
+                }
+            } else {
+                const int ib = pa.cold_ib, pb = 16 - ib;
+                const uint32_t piece_mask = (1u << pb) - 1u;
+                const uint32_t adv_max = pb * kWin >= 32 ? 0xffffffffu : (1u << (pb * kWin)) - 1u;
+                const int rel = c - pa.cold_begin[t];
+                if (adv > adv_max || rel < 0 || rel >= (1 << ib)) {
+                    *pa.overflow = 1;
+                    continue;
+                }
+                for (int ee = en; ee <= en + pads; ++ee)
+                    put_entry(pa.cold, pa.cold_src, round, g, ee, which, ee == en, value,
+                              (uint32_t)rel | (((adv >> (pb * ee)) & piece_mask) << ib), e);
+            }
+        }
+    }
+    if constexpr (!PLACE)
+        for (int key = lane; key < 2 * T; key += 64) cnt[((size_t)(key >> 1) * n + r) * 2 + (key & 1)] = base[key];
+}
+
+// Exclusive sums and exclusive maxima over the 1,024 threads of a workgroup (scratch: 17 ints of LDS).
+__device__ __forceinline__ int block_sum_before(int v, int *total, int *scratch)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(inc, d);
+        if (lane >= d) inc += o;
+    }
+    if (lane == 63) scratch[wave] = inc;
+    __syncthreads();
+    if (wave == 0) {
+        const int s = lane < 16 ? scratch[lane] : 0;
+        int si = s;
+        for (int d = 1; d < 16; d <<= 1) {
+            const int o = __shfl_up(si, d);
+            if (lane >= d) si += o;
+        }
+        if (lane < 16) scratch[lane] = si - s;
+        if (lane == 15) scratch[16] = si;
+    }
+    __syncthreads();
+    const int before = inc - v + scratch[wave];
+    *total = scratch[16];
+    __syncthreads();
+    return before;
+}
+
+__device__ __forceinline__ int block_max_before(int v, int *scratch)  // -1 where nothing comes before
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(inc, d);
+        if (lane >= d) inc = max(inc, o);
+    }
+    if (lane == 63) scratch[wave] = inc;
+    __syncthreads();
+    if (wave == 0) {
+        int si = lane < 16 ? scratch[lane] : -1;
+        for (int d = 1; d < 16; d <<= 1) {
+            const int o = __shfl_up(si, d);
+            if (lane >= d) si = max(si, o);
+        }
+        const int ex = __shfl_up(si, 1);
+        if (lane < 16) scratch[lane] = lane == 0 ? -1 : ex;
+    }
+    __syncthreads();
+    const int up = __shfl_up(inc, 1);
+    const int before = max(lane == 0 ? -1 : up, scratch[wave]);
+    __syncthreads();
+    return before;
+}
+
+// One workgroup per (block, step), one thread per row of the block (pass 1 of build_layout, split_step): the windows
+// of kind k before every row (pre), the last row before it that has any (prevrow), the 16 equal runs (meta:
+// {hot windows, cold windows, first row, 0}; run_start: hot and cold windows of the step before the run), the step's
+// windows in all.
+__global__ __launch_bounds__(1024) void rbb_split_kernel(const int *__restrict__ cnt, const int *__restrict__ block_row, int n,
+                                                          int T, int *__restrict__ pre, int *__restrict__ prevrow,
+                                                          int *__restrict__ meta, int *__restrict__ run_start,
+                                                          int *__restrict__ step_windows)
+{
+    __shared__ int scratch[17], first_row[kWaves], hstart[kWaves + 1], cstart[kWaves + 1];
+    const int b = blockIdx.x / T, t = blockIdx.x % T, lr = threadIdx.x;
+    const int r0 = block_row[b], nr = block_row[b + 1] - r0;
+    const size_t gi = ((size_t)t * n + (size_t)(r0 + lr)) * 2;
+    int h = 0, c = 0;
+    if (lr < nr) {
+        h = (cnt[gi] + kWin - 1) / kWin;
+        c = (cnt[gi + 1] + kWin - 1) / kWin;
+    }
+    int hot_total, cold_total;
+    const int hq = block_sum_before(h, &hot_total, scratch), cq = block_sum_before(c, &cold_total, scratch);
+    const int ph = block_max_before(h > 0 ? lr : -1, scratch), pc = block_max_before(c > 0 ? lr : -1, scratch);
+    if (lr < nr) {
+        pre[gi] = hq;
+        pre[gi + 1] = cq;
+        prevrow[gi] = ph;
+        prevrow[gi + 1] = pc;
+    }
+    if (lr < kWaves) {  // runs that find nothing left (a step without windows)
+        first_row[lr] = 0;
+        hstart[lr] = hot_total;
+        cstart[lr] = cold_total;
+    }
+    if (lr == 0) {
+        hstart[kWaves] = hot_total;
+        cstart[kWaves] = cold_total;
+    }
+    __syncthreads();
+    const long long E = (long long)hot_total + cold_total, q = (long long)hq + cq;
+    if (h + c > 0)
+        for (int w = 0; w < kWaves; ++w) {
+            const long long S = (long long)w * E / kWaves;
+            if (S < q || S >= q + h + c) continue;
+            const long long d = S - q;
+            first_row[w] = lr;
+            hstart[w] = d < h ? hq + (int)d : hq + h;
+            cstart[w] = d < h ? cq : cq + (int)(d - h);
+        }
+    __syncthreads();
+    const size_t bt = (size_t)b * T + t;
+    if (lr < kWaves) {
+        int *m = meta + (bt * kWaveSlots + lr) * 4;
+        m[0] = hstart[lr + 1] - hstart[lr];
+        m[1] = cstart[lr + 1] - cstart[lr];
+        m[2] = first_row[lr];
+        m[3] = 0;
+        run_start[(bt * kWaveSlots + lr) * 2] = hstart[lr];
+        run_start[(bt * kWaveSlots + lr) * 2 + 1] = cstart[lr];
+    }
+    if (lr == 0) step_windows[bt] = (int)E;
+}
+
+// Device memory that lives for the length of a build
+struct Scratch {
+    void *p = nullptr;
+    ~Scratch()
+    {
+        if (p) (void)hipFree(p);
+    }
+    hipError_t get(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 4); }
+    template <typename T>
+    T *as() const
+    {
+        return static_cast<T *>(p);
+    }
+};
+
+#define RBB_TRY(expr)                                           \
+    do {                                                        \
+        const hipError_t e_ = (expr);                           \
+        if (e_ != hipSuccess) return MPS_ERR_HIP + (int)e_;     \
+    } while (0)
+
+// Builds the layout with the passes over the nonzeros on the device.  The streams end up in dp's device arrays, the
+// small tables in dp->host as after build_layout.  kNeedHost: this matrix is for the host builder (local tables,
+// more than kBuildMaxSteps steps, a cold stream that cannot be packed); nothing of dp is to be kept then.
+int build_on_device(const int *d_rp, const int *d_ci, const float *d_val, int n, int nnz, const BuildParams &bp, hipStream_t st,
+                    DevicePlan *dp)
+{
+    Layout &L = dp->host;
+    std::vector<int> rp((size_t)n + 1);
+    RBB_TRY(hipMemcpyAsync(rp.data(), d_rp, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToHost, st));
+    RBB_TRY(hipStreamSynchronize(st));
+    if (rp[0] != 0 || rp[(size_t)n] != nnz) return MPS_ERR_INVALID_CSR;
+    int H = 0;
+    int rc = plan_blocks(rp.data(), n, nnz, bp, L, &H);
+    if (rc != MPS_OK) return rc;
+    const int NB = L.num_blocks;
+    if ((rc = upload(dp, &dp->block_row, L.block_row, st)) != MPS_OK) return rc;
+
+    // nonzeros per column
+    Scratch d_deg;
+    RBB_TRY(d_deg.get((size_t)n * sizeof(int)));
+    RBB_TRY(hipMemsetAsync(d_deg.p, 0, (size_t)n * sizeof(int), st));
+    if (nnz > 0)
+        hipLaunchKernelGGL(rbb_degree_kernel, dim3((unsigned)std::min<long long>(((long long)nnz + 255) / 256, 8192)), dim3(256), 0,
+                           st, d_ci, nnz, d_deg.as<int>());
+    std::vector<int> deg((size_t)n);
+    RBB_TRY(hipMemcpyAsync(deg.data(), d_deg.p, (size_t)n * sizeof(int), hipMemcpyDeviceToHost, st));
+    RBB_TRY(hipStreamSynchronize(st));
+    int failed = MPS_OK;
+    auto block_ranges = [&](int R, long long *own, long long *busiest) {
+        *own = *busiest = 0;
+        Scratch d_ranges;
+        std::vector<unsigned long long> ranges((size_t)R + 1, 0ull);
+        hipError_t e = d_ranges.get(ranges.size() * sizeof(unsigned long long));
+        if (e == hipSuccess) e = hipMemsetAsync(d_ranges.p, 0, ranges.size() * sizeof(unsigned long long), st);
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(rbb_ranges_kernel, dim3((unsigned)NB), dim3(256), ((size_t)R + 1) * sizeof(int), st, d_rp, d_ci,
+                               dp->block_row, n, R, d_ranges.as<unsigned long long>(), d_ranges.as<unsigned long long>() + R);
+            e = hipMemcpyAsync(ranges.data(), d_ranges.p, ranges.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost, st);
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        if (e != hipSuccess) {
+            failed = MPS_ERR_HIP + (int)e;
+            return;
+        }
+        *own = (long long)ranges[(size_t)R];
+        for (int r = 0; r < R; ++r) *busiest = std::max(*busiest, (long long)ranges[(size_t)r]);
+    };
+    ColumnMap cm;
+    rc = plan_columns(rp.data(), nullptr, n, nnz, bp, L, H, deg.data(), block_ranges, cm);
+    if (failed != MPS_OK) return failed;
+    if (rc != MPS_OK) return rc;
+    const int T = L.steps;
+    if (T > kBuildMaxSteps || (size_t)T * (size_t)n * 2 * sizeof(int) > ((size_t)512 << 20)) return kNeedHost;
+    if (L.hot_bits > kPackedSlotBits) return MPS_ERR_UNSUPPORTED;
+    int widest = 1;
+    for (int t = 0; t < T; ++t) widest = std::max(widest, L.cold_begin[(size_t)t + 1] - L.cold_begin[(size_t)t]);
+    const int ib = std::max(12, bits_for(widest > 1 ? widest - 1 : 1));
+    if (ib > 15) return kNeedHost;
+
+    // passes 1 and 2
+    Scratch d_step, d_slot, d_cnt, d_pre, d_prev, d_run_start, d_windows, d_round_off, d_flag;
+    const size_t groups = (size_t)T * (size_t)n * 2, runs = (size_t)NB * T * kWaveSlots;
+    RBB_TRY(d_step.get((size_t)n * sizeof(int16_t)));
+    RBB_TRY(d_slot.get((size_t)n * sizeof(int16_t)));
+    RBB_TRY(d_cnt.get(groups * sizeof(int)));
+    RBB_TRY(d_pre.get(groups * sizeof(int)));
+    RBB_TRY(d_prev.get(groups * sizeof(int)));
+    RBB_TRY(d_run_start.get(runs * 2 * sizeof(int)));
+    RBB_TRY(d_windows.get((size_t)NB * T * sizeof(int)));
+    RBB_TRY(d_round_off.get(runs * 2 * sizeof(long long)));
+    RBB_TRY(d_flag.get(sizeof(int)));
+    RBB_TRY(hipMemcpyAsync(d_step.p, cm.step.data(), (size_t)n * sizeof(int16_t), hipMemcpyHostToDevice, st));
+    RBB_TRY(hipMemcpyAsync(d_slot.p, cm.slot.data(), (size_t)n * sizeof(int16_t), hipMemcpyHostToDevice, st));
+    RBB_TRY(hipMemsetAsync(d_flag.p, 0, sizeof(int), st));
+    if ((rc = upload(dp, &dp->cold_begin, L.cold_begin, st)) != MPS_OK) return rc;
+    RBB_TRY(hipMalloc(reinterpret_cast<void **>(&dp->meta), runs * 4 * sizeof(int)));
+    dp->device_bytes += runs * 4 * sizeof(int);
+    const dim3 row_grid((unsigned)((n + 3) / 4));
+    PlaceArgs pa{};
+    hipLaunchKernelGGL(rbb_rows_kernel<false>, row_grid, dim3(256), 0, st, d_rp, d_ci, d_step.as<int16_t>(), d_slot.as<int16_t>(), n,
+                       T, d_cnt.as<int>(), pa);
+    hipLaunchKernelGGL(rbb_split_kernel, dim3((unsigned)(NB * T)), dim3(1024), 0, st, d_cnt.as<int>(), dp->block_row, n, T,
+                       d_pre.as<int>(), d_prev.as<int>(), dp->meta, d_run_start.as<int>(), d_windows.as<int>());
+    L.meta.resize(runs * 4);
+    RBB_TRY(hipMemcpyAsync(L.meta.data(), dp->meta, runs * 4 * sizeof(int), hipMemcpyDeviceToHost, st));
+    RBB_TRY(hipStreamSynchronize(st));
+    // where every wavefront's streams start, and where it stands at the start of every step
+    std::vector<long long> round_off(runs * 2);
+    L.wave_base.assign((size_t)NB * kWaveSlots * 2, 0);
+    long long hr = 0, cr = 0;
+    for (int b = 0; b < NB; ++b)
+        for (int w = 0; w < kWaveSlots; ++w) {
+            L.wave_base[((size_t)b * kWaveSlots + w) * 2] = hr;
+            L.wave_base[((size_t)b * kWaveSlots + w) * 2 + 1] = cr;
+            for (int t = 0; t < T; ++t) {
+                const size_t run = ((size_t)b * T + t) * kWaveSlots + w;
+                round_off[run * 2] = hr;
+                round_off[run * 2 + 1] = cr;
+                hr += rounds_for(L.meta[run * 4]);
+                cr += rounds_for(L.meta[run * 4 + 1]);
+            }
+        }
+    L.hot_rounds = hr;
+    L.cold_rounds = cr;
+    L.cold_index_bits = ib;
+    RBB_TRY(hipMemcpyAsync(d_round_off.p, round_off.data(), round_off.size() * sizeof(long long), hipMemcpyHostToDevice, st));
+    if ((rc = upload(dp, &dp->wave_base, L.wave_base, st)) != MPS_OK) return rc;
+    const size_t hot_bytes = (size_t)hr * kPackedRoundWords * sizeof(uint32_t), cold_bytes = (size_t)cr * kPackedRoundWords * sizeof(uint32_t);
+    RBB_TRY(hipMalloc(reinterpret_cast<void **>(&dp->hot), hot_bytes ? hot_bytes : 4));
+    if (cold_bytes) {
+        RBB_TRY(hipMalloc(reinterpret_cast<void **>(&dp->cold_packed), cold_bytes));
+        RBB_TRY(hipMemsetAsync(dp->cold_packed, 0, cold_bytes, st));
+    } else {  // (no cold entries: like the host builder's plan, which then holds an empty unpacked stream)
+        RBB_TRY(hipMalloc(reinterpret_cast<void **>(&dp->cold), sizeof(Entry)));
+    }
+    dp->device_bytes += (hot_bytes ? hot_bytes : 4) + (cold_bytes ? cold_bytes : sizeof(Entry));
+    RBB_TRY(hipMemsetAsync(dp->hot, 0, hot_bytes, st));
+    if (bp.keep_src) {
+        const size_t hs = (size_t)hr * kRoundEntries * sizeof(int), cs = (size_t)cr * kRoundEntries * sizeof(int);
+        RBB_TRY(hipMalloc(reinterpret_cast<void **>(&dp->hot_src), hs ? hs : 4));
+        RBB_TRY(hipMalloc(reinterpret_cast<void **>(&dp->cold_src), cs ? cs : 4));
+        dp->device_bytes += (hs ? hs : 4) + (cs ? cs : 4);
+        RBB_TRY(hipMemsetAsync(dp->hot_src, 0xff, hs, st));
+        RBB_TRY(hipMemsetAsync(dp->cold_src, 0xff, cs, st));
+    }
+    pa.val = d_val;
+    pa.pre = d_pre.as<int>();
+    pa.prevrow = d_prev.as<int>();
+    pa.block_row = dp->block_row;
+    pa.meta = dp->meta;
+    pa.run_start = d_run_start.as<int>();
+    pa.step_windows = d_windows.as<int>();
+    pa.cold_begin = dp->cold_begin;
+    pa.round_off = d_round_off.as<long long>();
+    pa.hot = dp->hot;
+    pa.cold = dp->cold_packed;
+    pa.hot_src = dp->hot_src;
+    pa.cold_src = dp->cold_src;
+    pa.overflow = d_flag.as<int>();
+    pa.num_blocks = NB;
+    pa.cold_ib = ib;
+    hipLaunchKernelGGL(rbb_rows_kernel<true>, row_grid, dim3(256), 0, st, d_rp, d_ci, d_step.as<int16_t>(), d_slot.as<int16_t>(), n,
+                       T, d_cnt.as<int>(), pa);
+    RBB_TRY(hipGetLastError());
+    int overflow = 0;
+    RBB_TRY(hipMemcpyAsync(&overflow, d_flag.p, sizeof(int), hipMemcpyDeviceToHost, st));
+    RBB_TRY(hipStreamSynchronize(st));
+    if (overflow) return kNeedHost;  // a window advances more rows than the packed forms hold
+    return MPS_OK;
+}
+#undef RBB_TRY
+
 }  // namespace
 
 void destroy(DevicePlan *dp)
@@ -521,7 +963,8 @@ void destroy(DevicePlan *dp)
     delete dp;
 }
 
-// Copies the CSR arrays to the host, builds the layout there and uploads it.  The arrays must have passed
+// Builds the layout - with the passes over the nonzeros on the device where build_on_device takes the matrix, else
+// from a copy of the CSR arrays on the host - and uploads what is not on the device yet.  The arrays must have passed
 // mps_csr_validate.
 int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n, int nnz, int K, const BuildParams &bp_in,
            hipStream_t st, DevicePlan **out)
@@ -535,6 +978,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         destroy(dp);
         return code;
     };
+    bool on_device = false;
     try {
         BuildParams bp = bp_in;
         if (bp.num_cus <= 0) {
@@ -544,34 +988,53 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
             if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
             bp.num_cus = cus;
         }
-        // The CSR arrays come back into pinned host memory (a pageable target takes ten times as long: 0.27 s
-        // against 0.02 s per GiB on MI355X hosts) and are released as soon as the layout is built.
-        struct Pinned {
-            void *p = nullptr;
-            ~Pinned() { if (p) (void)hipHostFree(p); }
-        } h_rp, h_ci, h_val;
-        hipError_t e = hipHostMalloc(&h_rp.p, ((size_t)n + 1) * sizeof(int), hipHostMallocDefault);
-        if (e == hipSuccess) e = hipHostMalloc(&h_ci.p, ((size_t)nnz + 1) * sizeof(int), hipHostMallocDefault);
-        if (e == hipSuccess) e = hipHostMalloc(&h_val.p, ((size_t)nnz + 1) * sizeof(float), hipHostMallocDefault);
-        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
-        int *rp = static_cast<int *>(h_rp.p), *ci = static_cast<int *>(h_ci.p);
-        float *val = static_cast<float *>(h_val.p);
-        e = hipMemcpyAsync(rp, d_row_ptr, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToHost, st);
-        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(ci, d_col_idx, (size_t)nnz * sizeof(int), hipMemcpyDeviceToHost, st);
-        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(val, d_val, (size_t)nnz * sizeof(float), hipMemcpyDeviceToHost, st);
-        if (e == hipSuccess) e = hipStreamSynchronize(st);
-        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
-        // (the caller has run mps_csr_validate on the device arrays: the builder indexes by column id)
-        if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
+        if (K != 16) return fail(MPS_ERR_UNSUPPORTED);
         dp->num_cus = bp.num_cus;
-        rc = build_layout(rp, ci, val, n, nnz, K, bp, dp->host);
-        if (rc != MPS_OK) return fail(rc);
+        if (!bp.host_build) {
+            rc = build_on_device(d_row_ptr, d_col_idx, d_val, n, nnz, bp, st, dp);
+            if (rc == MPS_OK) {
+                on_device = true;
+            } else {
+                // start again from an empty plan: for another error than kNeedHost, to give it back
+                (void)hipStreamSynchronize(st);
+                destroy(dp);
+                dp = nullptr;
+                if (rc != kNeedHost) return rc;
+                dp = new (std::nothrow) DevicePlan;
+                if (!dp) return MPS_ERR_UNSUPPORTED;
+                dp->num_cus = bp.num_cus;
+            }
+        }
+        if (!on_device) {
+            // The CSR arrays come back into pinned host memory (a pageable target takes ten times as long: 0.27 s
+            // against 0.02 s per GiB on MI355X hosts) and are released as soon as the layout is built.
+            struct Pinned {
+                void *p = nullptr;
+                ~Pinned() { if (p) (void)hipHostFree(p); }
+            } h_rp, h_ci, h_val;
+            hipError_t e = hipHostMalloc(&h_rp.p, ((size_t)n + 1) * sizeof(int), hipHostMallocDefault);
+            if (e == hipSuccess) e = hipHostMalloc(&h_ci.p, ((size_t)nnz + 1) * sizeof(int), hipHostMallocDefault);
+            if (e == hipSuccess) e = hipHostMalloc(&h_val.p, ((size_t)nnz + 1) * sizeof(float), hipHostMallocDefault);
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            int *rp = static_cast<int *>(h_rp.p), *ci = static_cast<int *>(h_ci.p);
+            float *val = static_cast<float *>(h_val.p);
+            e = hipMemcpyAsync(rp, d_row_ptr, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToHost, st);
+            if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(ci, d_col_idx, (size_t)nnz * sizeof(int), hipMemcpyDeviceToHost, st);
+            if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(val, d_val, (size_t)nnz * sizeof(float), hipMemcpyDeviceToHost, st);
+            if (e == hipSuccess) e = hipStreamSynchronize(st);
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            // (the caller has run mps_csr_validate on the device arrays: the builder indexes by column id)
+            if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
+            rc = build_layout(rp, ci, val, n, nnz, K, bp, dp->host);
+            if (rc != MPS_OK) return fail(rc);
+        }
     } catch (const std::bad_alloc &) {
         return fail(MPS_ERR_UNSUPPORTED);
     }
     Layout &L = dp->host;
-    dp->hot_slots = L.hot.size();
-    dp->cold_slots = L.cold.size();
+    dp->hot_slots = (size_t)L.hot_rounds * kRoundEntries;
+    dp->cold_slots = (size_t)L.cold_rounds * kRoundEntries;
+    const bool cold_is_packed = on_device ? dp->cold_packed != nullptr : !L.cold_packed.empty();
     {
         // The streams of the last steps, as many as fit kStreamKeepBytes, are read with plain loads and so stay in
         // the 256 MiB last-level cache from one product to the next; all others carry the streaming hint and pass
@@ -580,28 +1043,30 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         // power-law matrix, 1.07 GB of streams in 16 steps of 67 MB: 0, 2, 3, 4, 5, 16 steps kept: 0.500, 0.482,
         // 0.484, 0.493, 0.503, 0.516 ms per product; with both streams packed, 16 steps of 50 MB: 2, 3, 4, 5 steps
         // kept: 0.435, 0.4285, 0.432, 0.442 ms.
-        const size_t hot_bytes = L.hot_packed.size() * sizeof(uint32_t);
-        const size_t cold_bytes = L.cold_packed.empty() ? dp->cold_slots * sizeof(Entry) : L.cold_packed.size() * sizeof(uint32_t);
+        const size_t hot_bytes = (size_t)L.hot_rounds * kPackedRoundWords * sizeof(uint32_t);
+        const size_t cold_bytes = cold_is_packed ? (size_t)L.cold_rounds * kPackedRoundWords * sizeof(uint32_t) : dp->cold_slots * sizeof(Entry);
         const size_t per_step = (hot_bytes + cold_bytes) / (size_t)(L.steps > 0 ? L.steps : 1);
         const size_t keep = per_step > 0 ? kStreamKeepBytes / per_step : (size_t)L.steps;
         dp->keep_from = keep >= (size_t)L.steps ? 0 : L.steps - (int)keep;
     }
-    if ((rc = upload(dp, &dp->hot, L.hot_packed, st)) != MPS_OK) return fail(rc);
-    if (L.cold_packed.empty()) {
-        if ((rc = upload(dp, &dp->cold, L.cold, st)) != MPS_OK) return fail(rc);
-    } else if ((rc = upload(dp, &dp->cold_packed, L.cold_packed, st)) != MPS_OK) {
-        return fail(rc);
+    if (!on_device) {
+        if ((rc = upload(dp, &dp->hot, L.hot_packed, st)) != MPS_OK) return fail(rc);
+        if (L.cold_packed.empty()) {
+            if ((rc = upload(dp, &dp->cold, L.cold, st)) != MPS_OK) return fail(rc);
+        } else if ((rc = upload(dp, &dp->cold_packed, L.cold_packed, st)) != MPS_OK) {
+            return fail(rc);
+        }
+        if ((rc = upload(dp, &dp->cold_begin, L.cold_begin, st)) != MPS_OK) return fail(rc);
+        if (!L.table_base.empty() && (rc = upload(dp, &dp->table_base, L.table_base, st)) != MPS_OK) return fail(rc);
+        if (!L.table_used.empty() && (rc = upload(dp, &dp->table_used, L.table_used, st)) != MPS_OK) return fail(rc);
+        if (bp_in.keep_src) {
+            if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
+            if ((rc = upload(dp, &dp->cold_src, L.cold_src, st)) != MPS_OK) return fail(rc);
+        }
+        if ((rc = upload(dp, &dp->wave_base, L.wave_base, st)) != MPS_OK) return fail(rc);
+        if ((rc = upload(dp, &dp->meta, L.meta, st)) != MPS_OK) return fail(rc);
+        if ((rc = upload(dp, &dp->block_row, L.block_row, st)) != MPS_OK) return fail(rc);
     }
-    if ((rc = upload(dp, &dp->cold_begin, L.cold_begin, st)) != MPS_OK) return fail(rc);
-    if (!L.table_base.empty() && (rc = upload(dp, &dp->table_base, L.table_base, st)) != MPS_OK) return fail(rc);
-    if (!L.table_used.empty() && (rc = upload(dp, &dp->table_used, L.table_used, st)) != MPS_OK) return fail(rc);
-    if (bp_in.keep_src) {
-        if ((rc = upload(dp, &dp->hot_src, L.hot_src, st)) != MPS_OK) return fail(rc);
-        if ((rc = upload(dp, &dp->cold_src, L.cold_src, st)) != MPS_OK) return fail(rc);
-    }
-    if ((rc = upload(dp, &dp->wave_base, L.wave_base, st)) != MPS_OK) return fail(rc);
-    if ((rc = upload(dp, &dp->meta, L.meta, st)) != MPS_OK) return fail(rc);
-    if ((rc = upload(dp, &dp->block_row, L.block_row, st)) != MPS_OK) return fail(rc);
     if ((rc = upload(dp, &dp->hot_cols, L.hot_cols, st)) != MPS_OK) return fail(rc);
     {
         const size_t bytes = (size_t)L.steps * L.table_rows * 16 * sizeof(float);

@@ -49,7 +49,9 @@
 #ifndef MPSPMM_ROWBLOCK_HPP
 #define MPSPMM_ROWBLOCK_HPP
 
+#include <algorithm>
 #include <cstdint>
+#include <functional>
 #include <vector>
 
 namespace mps_rb {
@@ -116,9 +118,71 @@ struct BuildParams {
     double min_table_share_short_rows = 0.0;  // when rows are many and short and the first table serves a smaller share of the nonzeros
     double min_local_cover = 0.6;             // when the columns are local (max_local_share) and local tables would serve a smaller share
     bool local_tables = false;                // local tables whatever the matrix looks like
+    bool host_build = false;                  // create(): every pass over the nonzeros on the host (the device passes build the same layout)
 };
 
 constexpr int kNotWorthwhile = -1;  // build_layout: one of the three limits of BuildParams not met
+constexpr int kNeedHost = -2;       // plan_columns: the layout asks for the column indices on the host (local tables)
+
+// Where a column's nonzeros go: the step, and the slot of the step's LDS table (-1: cold, gathered through L2).
+struct ColumnMap {
+    std::vector<int16_t> step;  // per column
+    std::vector<int16_t> slot;  // per column: table slot, -1 = cold
+    // local tables: block b's table of step t holds the columns base[b] + t H .. base[b] + (t + 1) H - 1; the columns
+    // outside base[b] .. base[b] + T H - 1 are cold, in the first step (below) or the last (above)
+    const int *base = nullptr;
+    int H = 0, T = 1;
+    int step_of(int b, int c) const
+    {
+        if (!base) return step[(size_t)c];
+        const long long d = (long long)c - base[b];
+        return d < 0 ? 0 : (int)std::min<long long>(d / H, T - 1);
+    }
+    int slot_of(int b, int c) const
+    {
+        if (!base) return slot[(size_t)c];
+        const long long d = (long long)c - base[b];
+        return d >= 0 && d < (long long)T * H ? (int)(d % H) : -1;
+    }
+};
+
+// The builder in its parts, so that the passes over the nonzeros can run where the nonzeros are.
+// plan_blocks: the row blocks, the accumulator rows and the most table rows that fit beside them (from row_ptr alone).
+int plan_blocks(const int *row_ptr, int n, int nnz, const BuildParams &bp, Layout &out, int *table_rows);
+// plan_columns: steps, tables, hot and cold columns.  deg[c]: nonzeros of column c.  block_ranges(R, own, busiest):
+// *own = over all blocks, the nonzeros in the block's busiest of R equal column ranges; *busiest = the nonzeros of the
+// busiest range of the whole matrix.  col_idx may be null: then kNeedHost comes back where the layout needs it
+// (local tables).  Other returns: an mps_status, or kNotWorthwhile.
+int plan_columns(const int *row_ptr, const int *col_idx, int n, int nnz, const BuildParams &bp, Layout &out, int table_rows,
+                 const int *deg, const std::function<void(int, long long *, long long *)> &block_ranges, ColumnMap &cm);
+#if defined(__HIP__) || defined(__HIPCC__)
+#define MPS_RB_HD __host__ __device__
+#else
+#define MPS_RB_HD
+#endif
+// i-th element of a list of len entries dealt evenly and in order to 16 lane-groups (the first len % 16 groups hold one
+// entry more): its lane-group g and its place j there.
+MPS_RB_HD inline void deal(int len, int i, int *g, int *j)
+{
+    const int base = len / kGroups, rem = len % kGroups, big = base + 1;
+    if (i < rem * big) {
+        *g = i / big;
+        *j = i - *g * big;
+    } else {
+        const int i2 = i - rem * big;
+        *g = rem + i2 / base;
+        *j = i2 % base;
+    }
+}
+// bits that hold the values 0..v
+inline int bits_for(long long v)
+{
+    int b = 1;
+    while ((v >> b) != 0) ++b;
+    return b;
+}
+// rounds (two windows per lane-group each) that a wavefront needs for `windows` windows dealt to its 16 lane-groups
+inline int rounds_for(int windows) { return (windows / kGroups + (windows % kGroups != 0) + kPair - 1) / kPair; }
 
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,

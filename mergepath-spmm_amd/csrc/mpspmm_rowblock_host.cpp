@@ -16,13 +16,6 @@ namespace {
 
 using mps_host::parallel_for;
 
-int bits_for(long long v)  // bits that hold the values 0..v
-{
-    int b = 1;
-    while ((v >> b) != 0) ++b;
-    return b;
-}
-
 // Contiguous row blocks of at most `cap` rows and (except for a single row
 // that is longer) at most `target` nonzeros each, taken greedily.
 int greedy_blocks(const int *rp, int n, int cap, long long target, std::vector<int> *out)
@@ -44,46 +37,7 @@ int greedy_blocks(const int *rp, int n, int cap, long long target, std::vector<i
     return count;
 }
 
-// i-th element of a list of len entries dealt evenly and in order to 16
-// lane-groups: the first len % 16 groups hold one entry more.
-inline void deal(int len, int i, int *g, int *j)
-{
-    const int base = len / kGroups, rem = len % kGroups, big = base + 1;
-    if (i < rem * big) {
-        *g = i / big;
-        *j = i - *g * big;
-    } else {
-        const int i2 = i - rem * big;
-        *g = rem + i2 / base;
-        *j = i2 % base;
-    }
-}
-
-// rounds (two windows per lane-group each) that a wavefront needs for n windows dealt to its 16 lane-groups
-inline int rounds_for(int n) { return (n / kGroups + (n % kGroups != 0) + kPair - 1) / kPair; }
-
 inline int windows_of(int entries) { return (entries + kWin - 1) / kWin; }
-
-struct ColumnMap {
-    std::vector<int16_t> step;  // per column
-    std::vector<int16_t> slot;  // per column: table slot, -1 = cold
-    // local tables: block b's table of step t holds the columns base[b] + t H .. base[b] + (t + 1) H - 1; the columns
-    // outside base[b] .. base[b] + T H - 1 are cold, in the first step (below) or the last (above)
-    const int *base = nullptr;
-    int H = 0, T = 1;
-    int step_of(int b, int c) const
-    {
-        if (!base) return step[(size_t)c];
-        const long long d = (long long)c - base[b];
-        return d < 0 ? 0 : (int)std::min<long long>(d / H, T - 1);
-    }
-    int slot_of(int b, int c) const
-    {
-        if (!base) return slot[(size_t)c];
-        const long long d = (long long)c - base[b];
-        return d >= 0 && d < (long long)T * H ? (int)(d % H) : -1;
-    }
-};
 
 // Everything about one (block, step): where each wavefront's run starts.
 struct StepSplit {
@@ -193,18 +147,16 @@ int default_steps(int n, long long nnz, int table_rows, int num_blocks, const lo
     return (int)std::max<long long>(t, 1);
 }
 
-int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp,
-                 Layout &L)
+int plan_blocks(const int *rp, int n, int nnz, const BuildParams &bp, Layout &L, int *table_rows)
 {
-    if (!rp || n < 1 || nnz < 0 || (nnz > 0 && (!ci || !val))) return MPS_ERR_INVALID_ARG;
-    if (K != 16) return MPS_ERR_UNSUPPORTED;
+    if (!rp || n < 1 || nnz < 0) return MPS_ERR_INVALID_ARG;
     const int cold_bits = bits_for(n > 1 ? n - 1 : 1);
     if (cold_bits > 22) return MPS_ERR_UNSUPPORTED;
     const int num_cus = bp.num_cus > 0 ? bp.num_cus : 256;
     L = Layout();
     L.n = n;
     L.nnz = nnz;
-    L.K = K;
+    L.K = 16;
     L.cold_bits = cold_bits;
 
     // ---- 1. row blocks: about equal nonzero counts, as few rounds of workgroups as the LDS allows
@@ -249,13 +201,15 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     // ---- 2. table size, steps
     int H = bp.table_rows > 0 ? bp.table_rows : std::min(kMaxTableRows, budget_rows - L.acc_rows);
     if (H > kMaxTableRows) H = kMaxTableRows;
+    *table_rows = H;
+    return MPS_OK;
+}
+
+int plan_columns(const int *rp, const int *ci, int n, int nnz, const BuildParams &bp, Layout &L, int H, const int *deg,
+                 const std::function<void(int, long long *, long long *)> &block_ranges, ColumnMap &cm)
+{
     // ---- 3. nonzeros per column; the steps; hot columns by rank, cold columns by id range
-    std::vector<std::atomic<int>> deg((size_t)n);
-    for (auto &d : deg) d.store(0, std::memory_order_relaxed);
-    parallel_for(nnz, 1 << 20, [&](int64_t a, int64_t b) {
-        for (int64_t e = a; e < b; ++e) deg[(size_t)ci[e]].fetch_add(1, std::memory_order_relaxed);
-    });
-    auto d_of = [&](int c) { return deg[(size_t)c].load(std::memory_order_relaxed); };
+    auto d_of = [&](int c) { return deg[(size_t)c]; };
     std::vector<int> cand;
     cand.reserve((size_t)n);
     for (int c = 0; c < n; ++c)
@@ -280,25 +234,12 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         // ranges of its own and idles through the other steps, while a plan without steps finds such an X in L2
         // anyway.  Share of the nonzeros in each block's busiest of R equal column ranges, beyond what the busiest
         // range has of the whole matrix (which is skew, not locality).
-        const int R = std::max(T, 4);
-        std::vector<std::atomic<long long>> range_nnz((size_t)R);
-        for (auto &c : range_nnz) c.store(0, std::memory_order_relaxed);
-        std::atomic<long long> own{0};
-        parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
-            std::vector<long long> cnt((size_t)R);
-            for (int64_t b = b0; b < b1; ++b) {
-                std::fill(cnt.begin(), cnt.end(), 0);
-                for (int e = rp[L.block_row[(size_t)b]]; e < rp[L.block_row[(size_t)b + 1]]; ++e)
-                    ++cnt[(size_t)((long long)ci[e] * R / n)];
-                own.fetch_add(*std::max_element(cnt.begin(), cnt.end()), std::memory_order_relaxed);
-                for (int r = 0; r < R; ++r) range_nnz[(size_t)r].fetch_add(cnt[(size_t)r], std::memory_order_relaxed);
-            }
-        });
-        long long busiest = 0;
-        for (auto &c : range_nnz) busiest = std::max(busiest, c.load(std::memory_order_relaxed));
-        if ((double)(own.load() - busiest) > bp.max_local_share * (double)nnz) local = true;
+        long long own = 0, busiest = 0;
+        block_ranges(std::max(T, 4), &own, &busiest);
+        if ((double)(own - busiest) > bp.max_local_share * (double)nnz) local = true;
     }
     if (bp.local_tables) local = true;
+    if (local && !ci) return kNeedHost;  // local tables are laid out from the column indices themselves
     if (local) {
         // Local tables: block b's table of step t holds the H consecutive columns from base[b] + t H - for a
         // block-diagonal or banded matrix nearly all of the block's nonzeros, gathered from LDS, and a table is one
@@ -375,7 +316,6 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     const size_t R = std::min<size_t>((size_t)T * H, cand.size());
     if (R < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)R, cand.end(), hotter);
     std::sort(cand.begin(), cand.begin() + (long)R, hotter);
-    ColumnMap cm;
     cm.step.assign((size_t)n, 0);
     cm.slot.assign((size_t)n, -1);
     L.hot_cols.assign((size_t)T * H, -1);
@@ -426,6 +366,57 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             cum += d_of(c);
         }
     }
+
+    return MPS_OK;
+}
+
+// nonzeros per column
+static void count_columns(const int *ci, int n, int nnz, std::vector<int> &deg)
+{
+    std::vector<std::atomic<int>> cnt((size_t)n);
+    for (auto &d : cnt) d.store(0, std::memory_order_relaxed);
+    parallel_for(nnz, 1 << 20, [&](int64_t a, int64_t b) {
+        for (int64_t e = a; e < b; ++e) cnt[(size_t)ci[e]].fetch_add(1, std::memory_order_relaxed);
+    });
+    deg.resize((size_t)n);
+    for (int c = 0; c < n; ++c) deg[(size_t)c] = cnt[(size_t)c].load(std::memory_order_relaxed);
+}
+
+int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp,
+                 Layout &L)
+{
+    if (!rp || n < 1 || nnz < 0 || (nnz > 0 && (!ci || !val))) return MPS_ERR_INVALID_ARG;
+    if (K != 16) return MPS_ERR_UNSUPPORTED;
+    int H = 0;
+    int rc = plan_blocks(rp, n, nnz, bp, L, &H);
+    if (rc != MPS_OK) return rc;
+    std::vector<int> deg;
+    count_columns(ci, n, nnz, deg);
+    // Share of the nonzeros in each block's busiest of R equal column ranges (own), and what the busiest range has
+    // of the whole matrix.
+    auto block_ranges = [&](int R, long long *own_out, long long *busiest_out) {
+        std::vector<std::atomic<long long>> range_nnz((size_t)R);
+        for (auto &c : range_nnz) c.store(0, std::memory_order_relaxed);
+        std::atomic<long long> own{0};
+        parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
+            std::vector<long long> cnt((size_t)R);
+            for (int64_t b = b0; b < b1; ++b) {
+                std::fill(cnt.begin(), cnt.end(), 0);
+                for (int e = rp[L.block_row[(size_t)b]]; e < rp[L.block_row[(size_t)b + 1]]; ++e)
+                    ++cnt[(size_t)((long long)ci[e] * R / n)];
+                own.fetch_add(*std::max_element(cnt.begin(), cnt.end()), std::memory_order_relaxed);
+                for (int r = 0; r < R; ++r) range_nnz[(size_t)r].fetch_add(cnt[(size_t)r], std::memory_order_relaxed);
+            }
+        });
+        long long busiest = 0;
+        for (auto &c : range_nnz) busiest = std::max(busiest, c.load(std::memory_order_relaxed));
+        *own_out = own.load();
+        *busiest_out = busiest;
+    };
+    ColumnMap cm;
+    rc = plan_columns(rp, ci, n, nnz, bp, L, H, deg.data(), block_ranges, cm);
+    if (rc != MPS_OK) return rc;
+    const int T = L.steps;
 
     // ---- 4. pass 1: windows and first rows of every wavefront's runs
     const int NB = L.num_blocks;

@@ -179,7 +179,7 @@ class Plan:
                  rowblock="auto", rowblock_steps=0, rowblock_table_rows=0, rowblock_block_rows=0,
                  rowblock_blocks_per_round=0, keep_sources=True, row_marks=True, resident="auto", resident_bytes=0, weights=None, column_tiles=True,
                  local_tables=False, sweep="auto", sweep_piece=0, sweep_acc_rows=0, sweep_panels_per_round=0,
-                 sweep_together=0):
+                 sweep_together=0, host_build=False):
         import numpy as np
         self._np = np
         self._h = ctypes.c_void_p()
@@ -199,6 +199,8 @@ class Plan:
             flags |= _cabi.MPS_PLAN_NO_COLUMN_TILES
         if local_tables:
             flags |= _cabi.MPS_PLAN_LOCAL_TABLES
+        if host_build:
+            flags |= _cabi.MPS_PLAN_HOST_BUILD
         opt = _cabi.PlanOptions(flags, int(slab_bytes), int(rowblock_steps), int(rowblock_table_rows),
                                 int(rowblock_block_rows), int(rowblock_blocks_per_round),
                                 {None: 0, "degree": 1, "gcn": 2}[weights], int(resident_bytes), int(sweep_piece),
