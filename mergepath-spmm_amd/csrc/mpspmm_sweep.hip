@@ -277,8 +277,8 @@ __global__ __launch_bounds__(256) void sw_widen_values_kernel(const half_t *__re
     if (i < n) out[i] = (float)in[i];
 }
 
-template <typename T>
-int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
+template <typename T, typename A>
+int upload(DevicePlan *dp, T **dst, const std::vector<T, A> &src, hipStream_t st)
 {
     const size_t bytes = (src.size() ? src.size() : 1) * sizeof(T);
     MPS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(dst), bytes));
@@ -444,8 +444,8 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
-    std::vector<uint32_t>().swap(Lo.stream);
-    std::vector<int>().swap(Lo.src);
+    Bulk<uint32_t>().swap(Lo.stream);
+    Bulk<int>().swap(Lo.src);
     *out = dp;
     return MPS_OK;
 }

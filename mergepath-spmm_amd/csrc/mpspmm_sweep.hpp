@@ -43,6 +43,8 @@
 #define MPSPMM_SWEEP_HPP
 
 #include <cstdint>
+#include <memory>
+#include <new>
 #include <vector>
 
 namespace mps_sw {
@@ -59,6 +61,24 @@ constexpr int kMinRowBits = 6;      // an entry word keeps at least this many bi
 // LDS row of accumulator row v: rows that are a multiple of 16 apart (the pieces of one long row that a wavefront
 // holds) would otherwise share their banks.  G = accumulator rows per 256 bytes (a power of two).
 inline int swizzle(int v, int G) { return v ^ (((v >> 2) ^ (v >> 4) ^ (v >> 6)) & (G - 1)); }
+
+// A vector whose resize() leaves new elements as they are: the stream of a large matrix is hundreds of MB that the
+// builder overwrites anyway, and zeroing them first is a serial pass over fresh pages.
+template <typename T>
+struct LeaveAlone : std::allocator<T> {
+    template <typename U>
+    struct rebind {
+        using other = LeaveAlone<U>;
+    };
+    template <typename U, typename... Args>
+    void construct(U *p, Args &&...args)
+    {
+        if constexpr (sizeof...(Args) == 0) ::new (static_cast<void *>(p)) U;
+        else ::new (static_cast<void *>(p)) U(static_cast<Args &&>(args)...);
+    }
+};
+template <typename T>
+using Bulk = std::vector<T, LeaveAlone<T>>;
 
 struct Layout {
     int n = 0, nnz = 0, K = 0, elem_bytes = 4;
@@ -77,8 +97,8 @@ struct Layout {
     std::vector<int> piece_ptr;     // [rows + NP] per panel, listed rows + 1 entries: first accumulator row of every listed row
     std::vector<int> wave_meta;     // [NP * 16][2] {first round, rounds} of every wavefront
     std::vector<int> panel_rounds;  // [NP] most rounds of a wavefront of the panel
-    std::vector<uint32_t> stream;   // rounds x (64 / L lane-groups) x 4 lanes x {word A, value A, word B, value B}
-    std::vector<int> src;           // original nonzero index of every entry slot (stream order, 2 per 16 bytes), -1 = padding (optional)
+    Bulk<uint32_t> stream;          // rounds x (64 / L lane-groups) x 4 lanes x {word A, value A, word B, value B}
+    Bulk<int> src;                  // original nonzero index of every entry slot (stream order, 2 per 16 bytes), -1 = padding (optional)
     std::vector<int> split_row;     // rows that are cut into sub-rows
     std::vector<int> split_ptr;     // [split rows + 1] their partial rows: split_ptr[i] .. split_ptr[i + 1]
 };

@@ -6,6 +6,7 @@
 #include "mpspmm_sweep.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <new>
 #include <numeric>
@@ -145,6 +146,25 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     std::vector<int> item_panel, order;  // order: the items that hold nonzeros, largest first
     std::vector<int> split_of((size_t)n, 0);  // sub-rows of a row (0: not split)
     int NP = 0, piece = 0;
+    // rows per degree: what a number of panels needs in accumulator rows is summed over these, not over the rows
+    std::vector<std::pair<long long, long long>> by_degree;  // (degree, rows), degrees in ascending order
+    {
+        constexpr long long kSmall = 1 << 16;
+        std::vector<long long> small((size_t)kSmall, 0), large;
+        for (int r = 0; r < n; ++r) {
+            const long long d = deg(r);
+            if (d < kSmall) ++small[(size_t)d]; else large.push_back(d);
+        }
+        for (long long d = 0; d < kSmall; ++d)
+            if (small[(size_t)d]) by_degree.emplace_back(d, small[(size_t)d]);
+        std::sort(large.begin(), large.end());
+        for (size_t i = 0; i < large.size();) {
+            size_t j = i;
+            while (j < large.size() && large[j] == large[i]) ++j;
+            by_degree.emplace_back(large[i], (long long)(j - i));
+            i = j;
+        }
+    }
     for (int R = 1;; ++R) {
         if (R > 8192) return MPS_ERR_UNSUPPORTED;  // (a row that needs more accumulator rows than a panel holds)
         NP = num_cus * R;
@@ -157,16 +177,31 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         // a row of about a panel's share or more is cut into sub-rows of a third of a share
         const long long split_from = std::max<long long>(share - share / 10, 4ll * piece);
         const long long sub_target = std::max<long long>(share / 3, piece);
+        auto pieces_of = [&](long long d) { return (int)((d + piece - 1) / piece); };
+        auto sub_rows_of = [&](long long d) {
+            const int S = d > split_from && NP > 1 ? (int)((d + sub_target - 1) / sub_target) : 0;
+            return S == 1 ? 0 : S;
+        };
+        {
+            long long need = 0;  // accumulator rows in all
+            for (const auto &dc : by_degree) {
+                const long long d = dc.first;
+                const int S = sub_rows_of(d);
+                long long p = 0;
+                if (S > 0) {
+                    for (int j = 0; j < S; ++j) p += pieces_of(d / S + (j < d % S));
+                } else {
+                    p = pieces_of(d);
+                }
+                need += p * dc.second;
+            }
+            if (need > (long long)NP * vcap) continue;
+        }
         items.clear();
         out.split_row.clear();
         out.split_ptr.assign(1, 0);
         long long totv = 0;
-        auto pieces_of = [&](long long d) { return (int)((d + piece - 1) / piece); };
-        for (int r = 0; r < n; ++r) {
-            const long long d = deg(r);
-            split_of[(size_t)r] = d > split_from && NP > 1 ? (int)((d + sub_target - 1) / sub_target) : 0;
-            if (split_of[(size_t)r] == 1) split_of[(size_t)r] = 0;
-        }
+        for (int r = 0; r < n; ++r) split_of[(size_t)r] = sub_rows_of(deg(r));
         for (int r = 0; r < n;) {
             const int S = split_of[(size_t)r];
             if (S > 0) {
@@ -196,10 +231,29 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         if (totv > (long long)NP * vcap) continue;
         order = largest_first((int)items.size(), [&](int i) { return items[(size_t)i].nnz; });
         item_panel.assign(items.size(), 0);
-        if (!deal_largest_first(
-                order, [&](int i) { return items[(size_t)i].nnz; }, [&](int i) { return (long long)items[(size_t)i].pieces; },
-                NP, vcap, item_panel))
+        auto nnz_of = [&](int i) { return items[(size_t)i].nnz; };
+        auto pieces_needed = [&](int i) { return (long long)items[(size_t)i].pieces; };
+        // Many items and many panels: the panels in up to 16 sets of at least 16, the items (largest first) dealt to
+        // the sets in turn, and every set dealt on a thread of its own.  The sets get the same mix of sizes, so the
+        // panels end up as even as from one deal (a set's total differs from another's by less than its largest item).
+        const int sets = items.size() >= (size_t)100000 ? std::min(16, NP / 16) : 1;
+        if (sets > 1) {
+            std::vector<std::vector<int>> set_order((size_t)sets);
+            for (auto &o : set_order) o.reserve(order.size() / (size_t)sets + 1);
+            for (size_t k = 0; k < order.size(); ++k) set_order[k % (size_t)sets].push_back(order[k]);
+            std::atomic<bool> dealt{true};
+            mps_host::parallel_for(sets, 1, [&](int64_t lo, int64_t hi) {
+                for (int64_t q = lo; q < hi; ++q) {
+                    const int first = (int)(q * NP / sets), bins = (int)((q + 1) * NP / sets) - first;
+                    if (!deal_largest_first(set_order[(size_t)q], nnz_of, pieces_needed, bins, vcap, item_panel))
+                        dealt.store(false, std::memory_order_relaxed);
+                    for (int i : set_order[(size_t)q]) item_panel[(size_t)i] += first;
+                }
+            });
+            if (!dealt.load()) continue;
+        } else if (!deal_largest_first(order, nnz_of, pieces_needed, NP, vcap, item_panel)) {
             continue;
+        }
         // rows without nonzeros: zeros to write, dealt evenly
         int turn = 0;
         for (int i = 0; i < (int)items.size(); ++i)
@@ -247,7 +301,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
 
     // ---- every panel on its own: accumulator rows, wavefronts, streams
     struct PanelOut {
-        std::vector<uint32_t> stream;
+        Bulk<uint32_t> stream;
         std::vector<int> src;
         int wave_rounds[kWaves];
         int vrows;
@@ -385,7 +439,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             if (bp.keep_src && !po.src.empty())
                 std::memcpy(out.src.data() + (size_t)panel_first[(size_t)p] * words_per_round / 2, po.src.data(),
                             po.src.size() * sizeof(int));
-            std::vector<uint32_t>().swap(po.stream);
+            Bulk<uint32_t>().swap(po.stream);
             std::vector<int>().swap(po.src);
         }
     });
