@@ -71,17 +71,19 @@ std::vector<int> largest_first(int n, Size size_of)
 }
 
 // Largest first, each to the bin with the smallest load so far; a bin takes at most `cap` of `cost`.
-// false if some item finds no bin.
+// load, used: per bin, what it holds before (may be null: nothing) and after.  false if some item finds no bin.
 template <typename Size, typename Cost>
-bool deal_largest_first(const std::vector<int> &order, Size size_of, Cost cost_of, int bins, long long cap,
-                        std::vector<int> &bin_of)
+bool deal_largest_first(const int *order, size_t count, Size size_of, Cost cost_of, int bins, long long cap, std::vector<int> &bin_of,
+                        long long *load = nullptr, long long *used_io = nullptr)
 {
     typedef std::pair<long long, int> Load;  // (load, bin): the lightest bin first, the lower index among equals
     std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
-    for (int b = 0; b < bins; ++b) heap.push(Load(0, b));
+    for (int b = 0; b < bins; ++b) heap.push(Load(load ? load[b] : 0, b));
     std::vector<long long> used((size_t)bins, 0);
+    if (used_io) used.assign(used_io, used_io + bins);
     std::vector<Load> held;
-    for (int i : order) {
+    for (size_t k = 0; k < count; ++k) {
+        const int i = order[k];
         held.clear();
         Load top;
         for (;;) {
@@ -96,7 +98,16 @@ bool deal_largest_first(const std::vector<int> &order, Size size_of, Cost cost_o
         used[(size_t)top.second] += cost_of(i);
         heap.push(Load(top.first + size_of(i), top.second));
     }
+    if (load)
+        for (; !heap.empty(); heap.pop()) load[heap.top().second] = heap.top().first;
+    if (used_io) std::copy(used.begin(), used.end(), used_io);
     return true;
+}
+
+template <typename Size, typename Cost>
+bool deal_largest_first(const std::vector<int> &order, Size size_of, Cost cost_of, int bins, long long cap, std::vector<int> &bin_of)
+{
+    return deal_largest_first(order.data(), order.size(), size_of, cost_of, bins, cap, bin_of);
 }
 
 }  // namespace
@@ -233,26 +244,30 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         item_panel.assign(items.size(), 0);
         auto nnz_of = [&](int i) { return items[(size_t)i].nnz; };
         auto pieces_needed = [&](int i) { return (long long)items[(size_t)i].pieces; };
-        // Many items and many panels: the panels in up to 16 sets of at least 16, the items (largest first) dealt to
-        // the sets in turn, and every set dealt on a thread of its own.  The sets get the same mix of sizes, so the
-        // panels end up as even as from one deal (a set's total differs from another's by less than its largest item).
+        // Many items and many panels: the first 32 items per panel (the long rows) from one deal; then the panels in up
+        // to 16 sets of at least 16, the other items (largest first) dealt to the sets in turn, and every set dealt on
+        // a thread of its own from where the first deal left its panels.  The sets get the same mix of sizes, so the
+        // panels end up as even as from one deal.
         const int sets = items.size() >= (size_t)100000 ? std::min(16, NP / 16) : 1;
-        if (sets > 1) {
+        const size_t head = sets > 1 ? std::min(order.size(), (size_t)32 * (size_t)NP) : order.size();
+        std::vector<long long> load((size_t)NP, 0), used((size_t)NP, 0);
+        if (!deal_largest_first(order.data(), head, nnz_of, pieces_needed, NP, vcap, item_panel, load.data(), used.data())) continue;
+        if (head < order.size()) {
             std::vector<std::vector<int>> set_order((size_t)sets);
-            for (auto &o : set_order) o.reserve(order.size() / (size_t)sets + 1);
-            for (size_t k = 0; k < order.size(); ++k) set_order[k % (size_t)sets].push_back(order[k]);
+            for (auto &o : set_order) o.reserve((order.size() - head) / (size_t)sets + 1);
+            for (size_t k = head; k < order.size(); ++k) set_order[k % (size_t)sets].push_back(order[k]);
             std::atomic<bool> dealt{true};
             mps_host::parallel_for(sets, 1, [&](int64_t lo, int64_t hi) {
                 for (int64_t q = lo; q < hi; ++q) {
                     const int first = (int)(q * NP / sets), bins = (int)((q + 1) * NP / sets) - first;
-                    if (!deal_largest_first(set_order[(size_t)q], nnz_of, pieces_needed, bins, vcap, item_panel))
+                    const std::vector<int> &mine = set_order[(size_t)q];
+                    if (!deal_largest_first(mine.data(), mine.size(), nnz_of, pieces_needed, bins, vcap, item_panel,
+                                            load.data() + first, used.data() + first))
                         dealt.store(false, std::memory_order_relaxed);
-                    for (int i : set_order[(size_t)q]) item_panel[(size_t)i] += first;
+                    for (int i : mine) item_panel[(size_t)i] += first;
                 }
             });
             if (!dealt.load()) continue;
-        } else if (!deal_largest_first(order, nnz_of, pieces_needed, NP, vcap, item_panel)) {
-            continue;
         }
         // rows without nonzeros: zeros to write, dealt evenly
         int turn = 0;
