@@ -116,14 +116,14 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     // The row of X of entry k of a round (of 8 entries per lane-group), and where in the LDS (plane 0) this lane adds it.
     P x[kRoundInstr];
     unsigned at[kRoundInstr];
-#define SW_GATHER(k, WORD, j)                                                                \
+#define SW_GATHER(k, WORD, j, CM)                                                             \
     {                                                                                        \
         const unsigned w = from_lane<j>(WORD);                                               \
         at[k] = (w >> col_bits) * (16u * L) + lane_off;                                      \
         if constexpr (FAR) {                                                                 \
-            x[k].load(xb + (size_t)(w & cmask) * row_pitch);                                 \
+            x[k].load(xb + (size_t)(w & (CM)) * row_pitch);                                  \
         } else {                                                                             \
-            x[k].load(x_rsrc, __umul24(w & cmask, row_pitch) + lane_off, tile_off);          \
+            x[k].load(x_rsrc, __umul24(w & (CM), row_pitch) + lane_off, tile_off);           \
         }                                                                                    \
     }
     // One entry after the other: read the accumulator row, add, write it back.  The LDS serves a wavefront's
@@ -169,13 +169,13 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     // Entry k of round r is added up, and the registers that held its row of X at once take the request for entry k
     // of round r + 1: every row of X is asked for a round ahead of its use, in one set of registers, and the entries
     // of round r + 2 are read meanwhile.  No branch goes around a load (where two paths with different loads in
-    // flight meet, the compiler waits for all of them): past the wavefront's last round the loop asks for that
-    // round's entries and rows a second time and drops them.
+    // flight meet, the compiler waits for all of them): past the wavefront's last round the loop reads that round's
+    // entries a second time, asks for row 0 of X in place of their rows, and drops both.
     if (rounds > 0) {
         const int last = rounds - 1;
         uint4 cu = stream_load(0), nx = stream_load(min(1, last));
-        SW_GATHER(0, cu.x, 0) SW_GATHER(1, cu.x, 1) SW_GATHER(2, cu.x, 2) SW_GATHER(3, cu.x, 3)
-        SW_GATHER(4, cu.z, 0) SW_GATHER(5, cu.z, 1) SW_GATHER(6, cu.z, 2) SW_GATHER(7, cu.z, 3)
+        SW_GATHER(0, cu.x, 0, cmask) SW_GATHER(1, cu.x, 1, cmask) SW_GATHER(2, cu.x, 2, cmask) SW_GATHER(3, cu.x, 3, cmask)
+        SW_GATHER(4, cu.z, 0, cmask) SW_GATHER(5, cu.z, 1, cmask) SW_GATHER(6, cu.z, 2, cmask) SW_GATHER(7, cu.z, 3, cmask)
         for (int r = 0; r < rounds; ++r) {
             // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
             // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
@@ -183,20 +183,21 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
             if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
             const uint4 cn = nx;
             nx = stream_load(min(r + 2, last));
+            const unsigned cm = r < last ? cmask : 0u;  // (past the last round: row 0 of X, eight times)
             if constexpr (TOGETHER == 2) {
-                SW_ADD2(0) SW_GATHER(0, cn.x, 0) SW_GATHER(4, cn.z, 0)
-                SW_ADD2(1) SW_GATHER(1, cn.x, 1) SW_GATHER(5, cn.z, 1)
-                SW_ADD2(2) SW_GATHER(2, cn.x, 2) SW_GATHER(6, cn.z, 2)
-                SW_ADD2(3) SW_GATHER(3, cn.x, 3) SW_GATHER(7, cn.z, 3)
+                SW_ADD2(0) SW_GATHER(0, cn.x, 0, cm) SW_GATHER(4, cn.z, 0, cm)
+                SW_ADD2(1) SW_GATHER(1, cn.x, 1, cm) SW_GATHER(5, cn.z, 1, cm)
+                SW_ADD2(2) SW_GATHER(2, cn.x, 2, cm) SW_GATHER(6, cn.z, 2, cm)
+                SW_ADD2(3) SW_GATHER(3, cn.x, 3, cm) SW_GATHER(7, cn.z, 3, cm)
             } else {
-                SW_ADD(0, cu.y, 0) SW_GATHER(0, cn.x, 0)
-                SW_ADD(1, cu.y, 1) SW_GATHER(1, cn.x, 1)
-                SW_ADD(2, cu.y, 2) SW_GATHER(2, cn.x, 2)
-                SW_ADD(3, cu.y, 3) SW_GATHER(3, cn.x, 3)
-                SW_ADD(4, cu.w, 0) SW_GATHER(4, cn.z, 0)
-                SW_ADD(5, cu.w, 1) SW_GATHER(5, cn.z, 1)
-                SW_ADD(6, cu.w, 2) SW_GATHER(6, cn.z, 2)
-                SW_ADD(7, cu.w, 3) SW_GATHER(7, cn.z, 3)
+                SW_ADD(0, cu.y, 0) SW_GATHER(0, cn.x, 0, cm)
+                SW_ADD(1, cu.y, 1) SW_GATHER(1, cn.x, 1, cm)
+                SW_ADD(2, cu.y, 2) SW_GATHER(2, cn.x, 2, cm)
+                SW_ADD(3, cu.y, 3) SW_GATHER(3, cn.x, 3, cm)
+                SW_ADD(4, cu.w, 0) SW_GATHER(4, cn.z, 0, cm)
+                SW_ADD(5, cu.w, 1) SW_GATHER(5, cn.z, 1, cm)
+                SW_ADD(6, cu.w, 2) SW_GATHER(6, cn.z, 2, cm)
+                SW_ADD(7, cu.w, 3) SW_GATHER(7, cn.z, 3, cm)
             }
             cu = cn;
         }
