@@ -336,8 +336,12 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  * the others through L2, a contiguous range of column ids per step.  Inside a
  * (block, step) the nonzeros are cut into 16 equal runs (one per wavefront)
  * and a wavefront's hot and cold nonzeros are each dealt evenly to its 16
- * lane-groups.  Results are deterministic.  The layout is built on the host
- * (the CSR arrays are copied back once, at creation).  mps_plan_create picks
+ * lane-groups.  Results are deterministic.  The layout is built with the passes
+ * over the nonzeros on the device (row_ptr and the nonzero counts of the
+ * columns go to the host for the decisions); with local tables, more than 64
+ * steps, a cold stream that its packed form cannot hold, or
+ * MPS_PLAN_HOST_BUILD, on the host from a copy of the CSR arrays.  Both ways
+ * give the same plan.  mps_plan_create picks
  * this kind of plan by itself where it was measured to win: fp32, K = 16, X
  * below 192 MiB (3.1 M rows), except for matrices with many short rows and no
  * busy columns (fewer than 12 nonzeros per row on average, more than 2^18
