@@ -41,6 +41,29 @@ int bits_for(unsigned v)
     return b < 1 ? 1 : b;
 }
 
+// Entries by column, equal columns in the order they came (a radix sort from the low digits up: a wavefront's entries
+// are a few thousand 16-byte records, and a comparison sort of them was half of the builder's time).
+void sort_by_column(std::vector<Entry> &E, std::vector<Entry> &tmp, std::vector<int> &count, int col_bits)
+{
+    if (E.size() < 64) {
+        std::stable_sort(E.begin(), E.end(), [](const Entry &a, const Entry &b) { return a.col < b.col; });
+        return;
+    }
+    const int passes = (col_bits + 10) / 11, digit_bits = (col_bits + passes - 1) / passes;
+    const uint32_t mask = (1u << digit_bits) - 1u;
+    tmp.resize(E.size());
+    Entry *from = E.data(), *to = tmp.data();
+    for (int p = 0; p < passes; ++p) {
+        const int shift = p * digit_bits;
+        count.assign((size_t)mask + 2, 0);
+        for (size_t i = 0; i < E.size(); ++i) ++count[(((uint32_t)from[i].col >> shift) & mask) + 1];
+        for (size_t d = 0; d <= mask; ++d) count[d + 1] += count[d];
+        for (size_t i = 0; i < E.size(); ++i) to[count[((uint32_t)from[i].col >> shift) & mask]++] = from[i];
+        std::swap(from, to);
+    }
+    if (from != E.data()) E.swap(tmp);
+}
+
 // Indices 0 .. n - 1 with size_of(i) > 0, largest first, equal sizes in index order (a counting sort: sizes are
 // mostly small; the few above the table are sorted by comparison).
 template <typename Size>
@@ -325,7 +348,8 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     const int words_per_round = gpw * kWin * 4;  // uint32: lane-groups x 4 lanes x {word A, value A, word B, value B}
     mps_host::parallel_for(NP, 1, [&](int64_t lo, int64_t hi) {
         std::vector<int> vsize, vwave, vorder, last;
-        std::vector<Entry> entries[kWaves];
+        std::vector<Entry> entries[kWaves], sort_tmp;
+        std::vector<int> sort_count;
         std::vector<uint8_t> fill;
         std::vector<long long> slot;
         for (int p = (int)lo; p < (int)hi; ++p) {
@@ -379,7 +403,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             // accumulator row in an instruction (the second waits for the next instruction that has room)
             for (int w = 0; w < kWaves; ++w) {
                 std::vector<Entry> &E = entries[w];
-                std::stable_sort(E.begin(), E.end(), [](const Entry &a, const Entry &b) { return a.col < b.col; });
+                sort_by_column(E, sort_tmp, sort_count, col_bits);
                 const long long ne = (long long)E.size();
                 slot.resize((size_t)ne);
                 fill.assign((size_t)(ne / group_slots + 2), 0);
