@@ -93,3 +93,35 @@ def test_plans_that_the_host_passes_build(pkg, orc, dev):
     csr, plan, host = both_plans(pkg, dev, rp3, ci3, val3, rowblock_steps=1, rowblock_table_rows=64, rowblock_blocks_per_round=2)
     assert plan.info.rowblock_cold_index_bits == 0
     same_plan(pkg, plan, host)
+
+
+def test_device_passes_on_random_shapes(pkg, dev):
+    """Forty matrices and parameter sets drawn at random (sizes, row lengths, empty rows, long rows, steps, table and
+    block sizes): the device passes and the host passes agree on every one, or turn it away with the same status."""
+    rng = np.random.default_rng(2024)
+    built = 0
+    for trial in range(40):
+        n = int(rng.choice([7, 60, 333, 1500, 6000, 25000]))
+        max_deg = int(rng.choice([1, 3, 9, 40, 150]))
+        hubs = tuple((int(rng.integers(0, n)), int(rng.integers(1, n + 1))) for _ in range(int(rng.integers(0, 3))))
+        hubs = tuple(dict(hubs).items())  # (one entry per row)
+        rp, ci = random_csr(rng, n, max_deg, p_empty=float(rng.choice([0.0, 0.3, 0.9])), hub_rows=hubs)
+        val = rng.random(ci.size).astype(np.float32)
+        kw = dict(rowblock_steps=int(rng.choice([0, 1, 2, 5, 17, 40])), rowblock_table_rows=int(rng.choice([0, 4, 24, 200, 1024])),
+                  rowblock_block_rows=int(rng.choice([0, 0, 8, 100])), rowblock_blocks_per_round=int(rng.choice([0, 1, 3, 16, 256])))
+        csr = make_csr(pkg, dev, rp, ci, val)
+        status = []
+        plans = []
+        for host in (False, True):
+            try:
+                plans.append(pkg.spmm.Plan(csr, 16, rowblock="force", host_build=host, **kw))
+                status.append(0)
+            except pkg._cabi.MpsError as e:
+                status.append(e.status)
+        assert status[0] == status[1], (trial, n, max_deg, hubs, kw, status)
+        if status[0] == 0:
+            same_plan(pkg, plans[0], plans[1])
+            X = torch.rand((n, 16), dtype=torch.float32, device=dev)
+            assert torch.equal(plans[0].spmm(X), plans[1].spmm(X)), (trial, n, kw)
+            built += 1
+    assert built >= 25
