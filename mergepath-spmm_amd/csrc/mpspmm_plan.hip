@@ -1300,9 +1300,10 @@ constexpr uint64_t kSweepMinXBytesK16 = 24ull << 20;
 constexpr int kNearDiagonalWidth = 6000;
 constexpr double kSweepMaxNearDiagonal = 0.6;
 int sweep_wanted(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz, int K, int elem_bytes, int cost, int tpw,
-                 unsigned flags, hipStream_t st, bool *wanted)
+                 unsigned flags, hipStream_t st, bool *wanted, bool *near_diagonal)
 {
     *wanted = false;
+    *near_diagonal = false;  // set where it was looked for and found
     if (flags & MPS_PLAN_FORCE_SWEEP) {
         *wanted = true;
         return MPS_OK;
@@ -1336,6 +1337,7 @@ int sweep_wanted(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz
     // and that case never gets here with 64-byte rows; wider rows of a small matrix keep the sweep)
     const bool small = n_rows <= 2 * kNearDiagonalWidth;
     *wanted = small || (double)near < kSweepMaxNearDiagonal * (double)nnz;
+    *near_diagonal = !*wanted;
     return MPS_OK;
 }
 
@@ -1394,10 +1396,10 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
     pl->cost = cost;
     pl->keep_sources = !(flags & MPS_PLAN_NO_SOURCES);
     pl->weights = opt.degree_weights;
-    bool want_sweep = false;
+    bool want_sweep = false, near_diagonal = false;
     if (!opt.degree_weights) {
         const int src = sweep_wanted(d_row_ptr, d_col_idx, n_rows, nnz, K, elem_bytes, cost, tpw, flags,
-                                     static_cast<hipStream_t>(stream), &want_sweep);
+                                     static_cast<hipStream_t>(stream), &want_sweep, &near_diagonal);
         if (src != MPS_OK) {
             plan_free(pl);
             return src;
@@ -1454,7 +1456,8 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.num_cus = opt.rowblock_blocks_per_round;  // 0: ask the device
         bp.keep_src = pl->keep_sources;
         bp.local_tables = (flags & MPS_PLAN_LOCAL_TABLES) != 0;
-        bp.host_build = (flags & MPS_PLAN_HOST_BUILD) != 0;
+        // (a matrix that keeps to its diagonal gets local tables, which the host passes lay out: straight there)
+        bp.host_build = (flags & MPS_PLAN_HOST_BUILD) != 0 || near_diagonal;
         if (!(flags & MPS_PLAN_FORCE_ROWBLOCK)) {
             bp.max_local_share = kMaxLocalShare;
             bp.max_longest_row = kMaxLongestRow;
