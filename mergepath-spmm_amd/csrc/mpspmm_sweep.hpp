@@ -112,6 +112,20 @@ struct BuildParams {
     bool keep_src = true;
 };
 
+// A row as a panel lists it: entries first, first + stride, ... of row `row` of the matrix (a whole row: 0 and 1; sub-row
+// j of a row cut into S: j and S), dealt to `pieces` accumulator rows from first_piece on (entry e to piece e mod pieces).
+struct ListedRow {
+    int row, first, stride, entries, pieces, first_piece;
+    long long entries_before;  // of the panel's entries, in listing order
+};
+
+// The builder in two parts.  plan_panels: everything that needs row_ptr alone (panels, rows cut across panels, listed
+// rows, accumulator rows); it fills the small tables of `out` except wave_meta and panel_rounds.  build_streams: the
+// passes over the nonzeros (accumulator rows to wavefronts, entries by column, list scheduling, the stream).
+int plan_panels(const int *row_ptr, int n, int nnz, int K, const BuildParams &bp, Layout &out, std::vector<ListedRow> &listed_rows);
+int build_streams(const int *row_ptr, const int *col_idx, const float *val, const BuildParams &bp, Layout &out,
+                  const std::vector<ListedRow> &listed_rows);
+
 // Host arrays in, layout out.  Returns an mps_status (MPS_ERR_UNSUPPORTED for a row of X that is not a multiple of
 // 64 bytes or a matrix whose column ids leave no room for the accumulator row in an entry word).
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K, const BuildParams &bp,

@@ -135,9 +135,9 @@ bool deal_largest_first(const std::vector<int> &order, Size size_of, Cost cost_o
 
 }  // namespace
 
-int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp, Layout &out)
+int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Layout &out, std::vector<ListedRow> &listed_rows)
 {
-    if (n < 1 || nnz < 0 || K < 1 || !rp || (nnz > 0 && (!ci || !val))) return MPS_ERR_INVALID_ARG;
+    if (n < 1 || nnz < 0 || K < 1 || !rp) return MPS_ERR_INVALID_ARG;
     if (bp.elem_bytes != 4 && bp.elem_bytes != 2) return MPS_ERR_INVALID_ARG;
     const long long row_bytes = (long long)K * bp.elem_bytes;
     if (row_bytes % 64 != 0) return MPS_ERR_UNSUPPORTED;
@@ -163,14 +163,12 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     out.tiles = tiles;
     out.col_bits = col_bits;
     out.bank_rows = std::max(1, 256 / (16 * L));
-    const int G = out.bank_rows;
     const int gpw = 64 / L;  // lane-groups of a wavefront = entries of an instruction
     // instructions whose entries are added up at the same time (see Layout::together).  Measured on MI355X, R-MAT
     // scale 20 / 22, ms per product with 1 / 2: 64-byte rows 0.128 / 0.124; 128-byte tiles 0.163 / 0.168; fp16 rows of
     // 128 bytes 0.934 / 0.959 (what pairs save on LDS round trips, their 4 % more padding costs again).
     const int together = bp.together > 0 ? bp.together : (L == 4 ? 2 : 1);
     if (together != 1 && together != 2) return MPS_ERR_INVALID_ARG;
-    const int group_slots = gpw * together;
     out.together = together;
 
     auto deg = [&](int r) { return (long long)rp[r + 1] - rp[r]; };
@@ -331,13 +329,55 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         acc_rows = std::max(acc_rows, (v + 3) & ~3);
     }
     out.acc_rows = acc_rows;
-    const uint32_t pad_word = (uint32_t)acc_rows << col_bits;  // padding: column 0, value 0, the spare accumulator row
     out.rows.assign((size_t)listed, 0);
     out.piece_ptr.assign((size_t)listed + NP, 0);
     out.wave_meta.assign((size_t)NP * kWaves * 2, 0);
     out.panel_rounds.assign((size_t)NP, 0);
 
-    // ---- every panel on its own: accumulator rows, wavefronts, streams
+    // the listed rows of every panel: which entries of the matrix they hold and where their accumulator rows start
+    listed_rows.resize((size_t)listed);
+    mps_host::parallel_for(NP, 64, [&](int64_t lo, int64_t hi) {
+        for (int p = (int)lo; p < (int)hi; ++p) {
+            int lr = out.panel_ptr[(size_t)p];
+            int *pp = out.piece_ptr.data() + lr + p;
+            int v = 0;
+            long long before = 0;
+            for (int k = panel_count[(size_t)p]; k < panel_count[(size_t)p + 1]; ++k) {
+                const Item &it = items[(size_t)panel_items[(size_t)k]];
+                for (int q = 0; q < it.nrows; ++q) {
+                    const int r = it.row + q;
+                    const long long d = it.sub >= 0 ? it.nnz : deg(r);
+                    const int P = (int)((d + piece - 1) / piece);
+                    out.rows[(size_t)lr] = it.sub >= 0 ? n + out.split_ptr[(size_t)split_index[(size_t)r]] + it.sub : r;
+                    ListedRow &L = listed_rows[(size_t)lr];
+                    L.row = r;
+                    L.first = it.sub >= 0 ? it.sub : 0;
+                    L.stride = it.sub >= 0 ? split_of[(size_t)r] : 1;
+                    L.entries = (int)d;
+                    L.pieces = P;
+                    L.first_piece = v;
+                    L.entries_before = before;
+                    *pp++ = v;
+                    ++lr;
+                    v += P;
+                    before += d;
+                }
+            }
+            *pp = v;
+        }
+    });
+    return MPS_OK;
+}
+
+int build_streams(const int *rp, const int *ci, const float *val, const BuildParams &bp, Layout &out,
+                  const std::vector<ListedRow> &listed_rows)
+{
+    if (out.nnz > 0 && (!ci || !val)) return MPS_ERR_INVALID_ARG;
+    const int NP = out.num_panels, L = out.lanes, G = out.bank_rows, gpw = 64 / L, together = out.together, piece = out.piece;
+    const int group_slots = gpw * together, col_bits = out.col_bits;
+    const uint32_t pad_word = (uint32_t)out.acc_rows << col_bits;  // padding: column 0, value 0, the spare accumulator row
+    (void)piece;
+        // ---- every panel on its own: accumulator rows, wavefronts, streams
     struct PanelOut {
         Bulk<uint32_t> stream;
         std::vector<int> src;
@@ -354,26 +394,15 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         std::vector<long long> slot;
         for (int p = (int)lo; p < (int)hi; ++p) {
             PanelOut &po = built[(size_t)p];
-            // listed rows and their accumulator rows
-            const int k0 = panel_count[(size_t)p], k1 = panel_count[(size_t)p + 1];
-            int lr = out.panel_ptr[(size_t)p];
-            int *pp = out.piece_ptr.data() + lr + p;
+            // the sizes of the accumulator rows
+            const int l0 = out.panel_ptr[(size_t)p], l1 = out.panel_ptr[(size_t)p + 1];
             int v = 0;
             vsize.clear();
-            for (int k = k0; k < k1; ++k) {
-                const Item &it = items[(size_t)panel_items[(size_t)k]];
-                for (int q = 0; q < it.nrows; ++q) {
-                    const int r = it.row + q;
-                    const long long d = it.sub >= 0 ? it.nnz : deg(r);
-                    const int P = (int)((d + piece - 1) / piece);
-                    out.rows[(size_t)lr] = it.sub >= 0 ? n + out.split_ptr[(size_t)split_index[(size_t)r]] + it.sub : r;
-                    *pp++ = v;
-                    ++lr;
-                    for (int j = 0; j < P; ++j) vsize.push_back((int)(d / P + (j < d % P)));
-                    v += P;
-                }
+            for (int l = l0; l < l1; ++l) {
+                const ListedRow &R = listed_rows[(size_t)l];
+                for (int j = 0; j < R.pieces; ++j) vsize.push_back(R.entries / R.pieces + (j < R.entries % R.pieces));
+                v += R.pieces;
             }
-            *pp = v;
             po.vrows = v;
             // accumulator rows to wavefronts
             vorder = largest_first(v, [&](int i) { return (long long)vsize[(size_t)i]; });
@@ -382,21 +411,13 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                 vorder, [&](int i) { return (long long)vsize[(size_t)i]; }, [](int) { return 0ll; }, kWaves, 1, vwave);
             // entries per wavefront
             for (auto &e : entries) e.clear();
-            v = 0;
-            for (int k = k0; k < k1; ++k) {
-                const Item &it = items[(size_t)panel_items[(size_t)k]];
-                for (int q = 0; q < it.nrows; ++q) {
-                    const int r = it.row + q;
-                    const int S = it.sub >= 0 ? split_of[(size_t)r] : 1, first = it.sub >= 0 ? it.sub : 0;
-                    const long long d = it.sub >= 0 ? it.nnz : deg(r);
-                    const int P = (int)((d + piece - 1) / piece);
-                    const long long base = rp[r];
-                    for (long long e = 0; e < d; ++e) {
-                        const long long at = base + first + e * S;
-                        const int vl = v + (int)(e % P);
-                        entries[vwave[(size_t)vl]].push_back(Entry{ci[at], vl, val[at], (int)at});
-                    }
-                    v += P;
+            for (int l = l0; l < l1; ++l) {
+                const ListedRow &R = listed_rows[(size_t)l];
+                const long long base = rp[R.row];
+                for (long long e = 0; e < R.entries; ++e) {
+                    const long long at = base + R.first + e * R.stride;
+                    const int vl = R.first_piece + (int)(e % R.pieces);
+                    entries[vwave[(size_t)vl]].push_back(Entry{ci[at], vl, val[at], (int)at});
                 }
             }
             // streams: a wavefront's entries by column; one entry per lane-group and instruction, never two of one
@@ -483,6 +504,14 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
         }
     });
     return MPS_OK;
+}
+
+int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp, Layout &out)
+{
+    if (nnz > 0 && (!ci || !val)) return MPS_ERR_INVALID_ARG;
+    std::vector<ListedRow> listed_rows;
+    const int rc = plan_panels(rp, n, nnz, K, bp, out, listed_rows);
+    return rc != MPS_OK ? rc : build_streams(rp, ci, val, bp, out, listed_rows);
 }
 
 }  // namespace mps_sw
