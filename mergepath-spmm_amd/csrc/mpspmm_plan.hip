@@ -1425,6 +1425,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         bp.together = opt.sweep_together;
         bp.elem_bytes = elem_bytes;
         bp.keep_src = pl->keep_sources;
+        bp.host_build = (flags & MPS_PLAN_HOST_BUILD) != 0;
         int rc = mps_sw::create(d_row_ptr, d_col_idx, d_val, n_rows, nnz, K, bp, static_cast<hipStream_t>(stream), &pl->sw);
         if (rc == MPS_OK) {
             pl->device_bytes = mps_sw::device_bytes_of(pl->sw);

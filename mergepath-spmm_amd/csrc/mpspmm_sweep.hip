@@ -355,6 +355,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
     DevicePlan *dp = new (std::nothrow) DevicePlan;
     if (!dp) return MPS_ERR_UNSUPPORTED;
     int rc = MPS_OK;
+    bool on_device = false;
     auto fail = [&](int code) {
         (void)hipStreamSynchronize(st);  // uploads from the layout's host arrays may still be in flight
         destroy(dp);
@@ -369,20 +370,12 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
             if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
             bp.num_cus = cus;
         }
-        // the CSR arrays come back into pinned host memory (a pageable target takes ten times as long) and are
-        // released as soon as the layout is built; half values are widened on the device first (exact)
-        struct Pinned {
-            void *p = nullptr;
-            ~Pinned() { if (p) (void)hipHostFree(p); }
-        } h_rp, h_ci, h_val;
+        // half values are widened on the device first (exact): both builders take fp32 values
         struct Dev {
             void *p = nullptr;
             ~Dev() { if (p) (void)hipFree(p); }
         } wide;
-        hipError_t e = hipHostMalloc(&h_rp.p, ((size_t)n + 1) * sizeof(int), hipHostMallocDefault);
-        if (e == hipSuccess) e = hipHostMalloc(&h_ci.p, ((size_t)nnz + 1) * sizeof(int), hipHostMallocDefault);
-        if (e == hipSuccess) e = hipHostMalloc(&h_val.p, ((size_t)nnz + 1) * sizeof(float), hipHostMallocDefault);
-        if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+        hipError_t e = hipSuccess;
         const float *val_src = static_cast<const float *>(d_val);
         if (bp.elem_bytes == 2 && nnz > 0) {
             e = hipMalloc(&wide.p, (size_t)nnz * sizeof(float));
@@ -391,23 +384,60 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
                                static_cast<const half_t *>(d_val), static_cast<float *>(wide.p), (size_t)nnz);
             val_src = static_cast<const float *>(wide.p);
         }
-        int *rp = static_cast<int *>(h_rp.p), *ci = static_cast<int *>(h_ci.p);
-        float *val = static_cast<float *>(h_val.p);
-        e = hipMemcpyAsync(rp, d_row_ptr, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToHost, st);
-        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(ci, d_col_idx, (size_t)nnz * sizeof(int), hipMemcpyDeviceToHost, st);
-        if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(val, val_src, (size_t)nnz * sizeof(float), hipMemcpyDeviceToHost, st);
+        // panels, listed rows and accumulator rows need row_ptr alone
+        std::vector<int> rp((size_t)n + 1);
+        e = hipMemcpyAsync(rp.data(), d_row_ptr, ((size_t)n + 1) * sizeof(int), hipMemcpyDeviceToHost, st);
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
         if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
-        rc = build_layout(rp, ci, val, n, nnz, K, bp, dp->host);
+        std::vector<ListedRow> listed_rows;
+        rc = plan_panels(rp.data(), n, nnz, K, bp, dp->host, listed_rows);
         if (rc != MPS_OK) return fail(rc);
+        if (!bp.host_build) {
+            // the passes over the nonzeros where the nonzeros are
+            DeviceStreams ds;
+            rc = build_streams_on_device(d_row_ptr, d_col_idx, val_src, bp, dp->host, listed_rows, st, &ds);
+            if (rc == MPS_OK) {
+                dp->stream = ds.stream;
+                dp->src = ds.src;
+                dp->slots = ds.slots;
+                dp->device_bytes += ds.bytes;
+                on_device = true;
+            } else {
+                (void)hipStreamSynchronize(st);
+                (void)hipFree(ds.stream);
+                (void)hipFree(ds.src);
+                if (rc != kNeedHost) return fail(rc);
+            }
+        }
+        if (!on_device) {
+            // the CSR arrays come back into pinned host memory (a pageable target takes ten times as long) and are
+            // released as soon as the layout is built
+            struct Pinned {
+                void *p = nullptr;
+                ~Pinned() { if (p) (void)hipHostFree(p); }
+            } h_ci, h_val;
+            e = hipHostMalloc(&h_ci.p, ((size_t)nnz + 1) * sizeof(int), hipHostMallocDefault);
+            if (e == hipSuccess) e = hipHostMalloc(&h_val.p, ((size_t)nnz + 1) * sizeof(float), hipHostMallocDefault);
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            int *ci = static_cast<int *>(h_ci.p);
+            float *val = static_cast<float *>(h_val.p);
+            if (nnz > 0) e = hipMemcpyAsync(ci, d_col_idx, (size_t)nnz * sizeof(int), hipMemcpyDeviceToHost, st);
+            if (e == hipSuccess && nnz > 0) e = hipMemcpyAsync(val, val_src, (size_t)nnz * sizeof(float), hipMemcpyDeviceToHost, st);
+            if (e == hipSuccess) e = hipStreamSynchronize(st);
+            if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
+            rc = build_streams(rp.data(), ci, val, bp, dp->host, listed_rows);
+            if (rc != MPS_OK) return fail(rc);
+        }
     } catch (const std::bad_alloc &) {
         return fail(MPS_ERR_UNSUPPORTED);
     }
     Layout &Lo = dp->host;
-    dp->slots = Lo.stream.size() / 2;
-    if ((rc = upload(dp, &dp->stream, Lo.stream, st)) != MPS_OK) return fail(rc);
-    if (bp_in.keep_src && (rc = upload(dp, &dp->src, Lo.src, st)) != MPS_OK) return fail(rc);
+    if (!on_device) {
+        dp->slots = Lo.stream.size() / 2;
+        if ((rc = upload(dp, &dp->stream, Lo.stream, st)) != MPS_OK) return fail(rc);
+        if (bp_in.keep_src && (rc = upload(dp, &dp->src, Lo.src, st)) != MPS_OK) return fail(rc);
+    }
     if ((rc = upload(dp, &dp->panel_ptr, Lo.panel_ptr, st)) != MPS_OK) return fail(rc);
     if ((rc = upload(dp, &dp->rows, Lo.rows, st)) != MPS_OK) return fail(rc);
     if ((rc = upload(dp, &dp->piece_ptr, Lo.piece_ptr, st)) != MPS_OK) return fail(rc);

@@ -110,7 +110,10 @@ struct BuildParams {
     int together = 0;    // 0 = choose (2 with 8 lane-groups per wavefront, else 1)
     int elem_bytes = 4;  // of X and Y (values are handed to the builder as fp32 either way)
     bool keep_src = true;
+    bool host_build = false;  // create(): the passes over the nonzeros on the host (the device passes build the same layout)
 };
+
+constexpr int kNeedHost = -2;  // build_streams_on_device: this layout is for the host passes
 
 // A row as a panel lists it: entries first, first + stride, ... of row `row` of the matrix (a whole row: 0 and 1; sub-row
 // j of a row cut into S: j and S), dealt to `pieces` accumulator rows from first_piece on (entry e to piece e mod pieces).
@@ -139,6 +142,16 @@ void fill_info(const Layout &L, mps_plan_info *info);
 
 #ifdef MPSPMM_DEVICE_HPP
 struct DevicePlan;
+// build_streams on the device (mpspmm_sweep_build.hip): row_ptr, col_idx and fp32 values on the device in, the stream
+// (and the source index of every slot, if bp.keep_src) in device memory out; fills out.wave_meta, out.panel_rounds and
+// out.rounds.  Returns an mps_status or kNeedHost; whatever *ds holds afterwards is the caller's to free.
+struct DeviceStreams {
+    uint32_t *stream = nullptr;
+    int *src = nullptr;
+    size_t slots = 0, bytes = 0;
+};
+int build_streams_on_device(const int *d_row_ptr, const int *d_col_idx, const float *d_val, const BuildParams &bp, Layout &out,
+                            const std::vector<ListedRow> &listed_rows, hipStream_t st, DeviceStreams *ds);
 int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n, int nnz, int K, const BuildParams &bp,
            hipStream_t st, DevicePlan **out);
 void destroy(DevicePlan *dp);

@@ -229,36 +229,63 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
             }
             if (need > (long long)NP * vcap) continue;
         }
+        // the items, in row order: the rows in chunks that start at even rows (so that pairs never span two chunks),
+        // every chunk on its own, then one after the other
+        mps_host::parallel_for(n, 1 << 16, [&](int64_t lo, int64_t hi) {
+            for (int64_t r = lo; r < hi; ++r) split_of[(size_t)r] = sub_rows_of(deg((int)r));
+        });
+        constexpr int kChunkRows = 1 << 16;
+        const int chunks = (n + kChunkRows - 1) / kChunkRows;
+        std::vector<std::vector<Item>> chunk_items((size_t)chunks);
+        std::vector<std::vector<int>> chunk_split((size_t)chunks);
+        mps_host::parallel_for(chunks, 1, [&](int64_t c0, int64_t c1) {
+            for (int64_t c = c0; c < c1; ++c) {
+                std::vector<Item> &mine = chunk_items[(size_t)c];
+                const int r_end = (int)std::min<long long>(n, (c + 1) * (long long)kChunkRows);
+                mine.reserve((size_t)kChunkRows / (size_t)U + 16);
+                for (int r = (int)(c * kChunkRows); r < r_end;) {
+                    const int S = split_of[(size_t)r];
+                    if (S > 0) {
+                        const long long d = deg(r);
+                        for (int j = 0; j < S; ++j) {
+                            const long long dj = d / S + (j < d % S);  // entries j, j + S, j + 2 S, ...
+                            mine.push_back(Item{dj, pieces_of(dj), r, 1, j});
+                        }
+                        chunk_split[(size_t)c].push_back(r);
+                        ++r;
+                        continue;
+                    }
+                    int take = 1;
+                    if (U == 2 && (r & 1) == 0 && r + 1 < n && split_of[(size_t)r + 1] == 0) take = 2;
+                    long long d = 0;
+                    int p = 0;
+                    for (int k = 0; k < take; ++k) {
+                        d += deg(r + k);
+                        p += pieces_of(deg(r + k));
+                    }
+                    mine.push_back(Item{d, p, r, take, -1});
+                    r += take;
+                }
+            }
+        });
         items.clear();
         out.split_row.clear();
         out.split_ptr.assign(1, 0);
         long long totv = 0;
-        for (int r = 0; r < n; ++r) split_of[(size_t)r] = sub_rows_of(deg(r));
-        for (int r = 0; r < n;) {
-            const int S = split_of[(size_t)r];
-            if (S > 0) {
-                const long long d = deg(r);
-                for (int j = 0; j < S; ++j) {
-                    const long long dj = d / S + (j < d % S);  // entries j, j + S, j + 2 S, ...
-                    items.push_back(Item{dj, pieces_of(dj), r, 1, j});
-                    totv += pieces_of(dj);
+        {
+            std::vector<size_t> first((size_t)chunks + 1, 0);
+            for (int c = 0; c < chunks; ++c) first[(size_t)c + 1] = first[(size_t)c] + chunk_items[(size_t)c].size();
+            items.resize(first[(size_t)chunks]);
+            mps_host::parallel_for(chunks, 1, [&](int64_t c0, int64_t c1) {
+                for (int64_t c = c0; c < c1; ++c)
+                    std::copy(chunk_items[(size_t)c].begin(), chunk_items[(size_t)c].end(), items.begin() + (long)first[(size_t)c]);
+            });
+            for (int c = 0; c < chunks; ++c)
+                for (int r : chunk_split[(size_t)c]) {
+                    out.split_row.push_back(r);
+                    out.split_ptr.push_back(out.split_ptr.back() + split_of[(size_t)r]);
                 }
-                out.split_row.push_back(r);
-                out.split_ptr.push_back(out.split_ptr.back() + S);
-                ++r;
-                continue;
-            }
-            int take = 1;
-            if (U == 2 && (r & 1) == 0 && r + 1 < n && split_of[(size_t)r + 1] == 0) take = 2;
-            long long d = 0;
-            int p = 0;
-            for (int k = 0; k < take; ++k) {
-                d += deg(r + k);
-                p += pieces_of(deg(r + k));
-            }
-            items.push_back(Item{d, p, r, take, -1});
-            totv += p;
-            r += take;
+            for (const Item &it : items) totv += it.pieces;
         }
         if (totv > (long long)NP * vcap) continue;
         order = largest_first((int)items.size(), [&](int i) { return items[(size_t)i].nnz; });
@@ -314,20 +341,24 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
     std::vector<int> split_index((size_t)n, -1);
     for (size_t i = 0; i < out.split_row.size(); ++i) split_index[(size_t)out.split_row[i]] = (int)i;
 
-    // listed rows per panel
+    // listed rows and accumulator rows per panel
     out.panel_ptr.assign((size_t)NP + 1, 0);
-    for (int p = 0; p < NP; ++p) {
-        int rows = 0;
-        for (int k = panel_count[(size_t)p]; k < panel_count[(size_t)p + 1]; ++k) rows += items[(size_t)panel_items[(size_t)k]].nrows;
-        out.panel_ptr[(size_t)p + 1] = out.panel_ptr[(size_t)p] + rows;
-    }
+    std::vector<int> panel_pieces((size_t)NP, 0);
+    mps_host::parallel_for(NP, 16, [&](int64_t lo, int64_t hi) {
+        for (int64_t p = lo; p < hi; ++p) {
+            int rows = 0, v = 0;
+            for (int k = panel_count[(size_t)p]; k < panel_count[(size_t)p + 1]; ++k) {
+                rows += items[(size_t)panel_items[(size_t)k]].nrows;
+                v += items[(size_t)panel_items[(size_t)k]].pieces;
+            }
+            out.panel_ptr[(size_t)p + 1] = rows;
+            panel_pieces[(size_t)p] = v;
+        }
+    });
+    for (int p = 0; p < NP; ++p) out.panel_ptr[(size_t)p + 1] += out.panel_ptr[(size_t)p];
     const int listed = out.panel_ptr[(size_t)NP];
     int acc_rows = 4;
-    for (int p = 0; p < NP; ++p) {
-        int v = 0;
-        for (int k = panel_count[(size_t)p]; k < panel_count[(size_t)p + 1]; ++k) v += items[(size_t)panel_items[(size_t)k]].pieces;
-        acc_rows = std::max(acc_rows, (v + 3) & ~3);
-    }
+    for (int p = 0; p < NP; ++p) acc_rows = std::max(acc_rows, (panel_pieces[(size_t)p] + 3) & ~3);
     out.acc_rows = acc_rows;
     out.rows.assign((size_t)listed, 0);
     out.piece_ptr.assign((size_t)listed + NP, 0);
