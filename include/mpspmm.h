@@ -405,8 +405,8 @@ typedef struct mps_plan mps_plan;
                                         MPS_PLAN_FORCE_ROWBLOCK or mps_rowblock_layout_build */
 #define MPS_PLAN_NO_SWEEP 2048u     /* never build a sweep plan (see below)       */
 #define MPS_PLAN_FORCE_SWEEP 4096u  /* sweep plan whatever the matrix looks like (rows of X a multiple of 64 bytes) */
-#define MPS_PLAN_HOST_BUILD 8192u   /* row-block plans: every pass over the nonzeros on the host, from a copy of the CSR arrays (the
-                                       library makes these passes on the device where it can; both give the same plan) */
+#define MPS_PLAN_HOST_BUILD 8192u   /* row-block and sweep plans: every pass over the nonzeros on the host, from a copy of the CSR
+                                       arrays (the library makes these passes on the device where it can; both give the same plan) */
 #define MPS_PLAN_NO_COLUMN_TILES 512u /* untiled plans with rows of X of 512 bytes and more: no passes over 128-byte column tiles */
 #define MPS_PLAN_NO_RESIDENT 256u    /* untiled plans: no streaming hint on the gathers of unpopular columns (see below) */
 #define MPS_PLAN_NO_ROW_MARKS 128u  /* plain column ids in the sliced array; the kernel follows row_ptr as on the caller's
