@@ -999,6 +999,11 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
                 (void)hipStreamSynchronize(st);
                 destroy(dp);
                 dp = nullptr;
+                // (the device passes need room beside the matrix for their counts and ranks: without it, the host's)
+                if (rc == MPS_ERR_HIP + (int)hipErrorOutOfMemory) {
+                    (void)hipGetLastError();
+                    rc = kNeedHost;
+                }
                 if (rc != kNeedHost) return rc;
                 dp = new (std::nothrow) DevicePlan;
                 if (!dp) return MPS_ERR_UNSUPPORTED;

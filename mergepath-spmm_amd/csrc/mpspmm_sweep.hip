@@ -407,6 +407,11 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
                 (void)hipStreamSynchronize(st);
                 (void)hipFree(ds.stream);
                 (void)hipFree(ds.src);
+                // (the device passes sort two copies of the entries: without room for them, the host's)
+                if (rc == MPS_ERR_HIP + (int)hipErrorOutOfMemory) {
+                    (void)hipGetLastError();
+                    rc = kNeedHost;
+                }
                 if (rc != kNeedHost) return fail(rc);
             }
         }
