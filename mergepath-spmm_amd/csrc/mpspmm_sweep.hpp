@@ -1,5 +1,6 @@
-// Sweep plans: layout shared by the host-side builder (mpspmm_sweep_host.cpp)
-// and the device side (mpspmm_sweep.hip).  Not installed.
+// Sweep plans: layout shared by the builder (mpspmm_sweep_host.cpp; its passes
+// over the nonzeros also on the device, mpspmm_sweep_build.hip) and the kernel
+// (mpspmm_sweep.hip).  Not installed.
 //
 // The reference walks a partition's nonzeros in row order and gathers the
 // dense row of every nonzero from memory (src/MergePathSpMM.cu:426-477); rows
