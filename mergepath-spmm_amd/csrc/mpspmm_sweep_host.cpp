@@ -165,8 +165,9 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
     out.bank_rows = std::max(1, 256 / (16 * L));
     const int gpw = 64 / L;  // lane-groups of a wavefront = entries of an instruction
     // instructions whose entries are added up at the same time (see Layout::together).  Measured on MI355X, R-MAT
-    // scale 20 / 22, ms per product with 1 / 2: 64-byte rows 0.128 / 0.124; 128-byte tiles 0.163 / 0.168; fp16 rows of
-    // 128 bytes 0.934 / 0.959 (what pairs save on LDS round trips, their 4 % more padding costs again).
+    // scale 20 / 22, ms per product with 1 / 2: 64-byte rows 0.1285 / 0.1278; 128-byte tiles 0.167 / 0.168 (K = 256:
+    // 1.358 / 1.384); fp16 rows of 128 bytes 0.934 / 0.960 (what pairs save on LDS round trips, their 4 % more padding
+    // costs again).
     const int together = bp.together > 0 ? bp.together : (L == 4 ? 2 : 1);
     if (together != 1 && together != 2) return MPS_ERR_INVALID_ARG;
     out.together = together;
