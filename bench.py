@@ -248,6 +248,7 @@ def describe_plan(name, w, plan, g, tpw_arg, cost):
             "cost": cost if slab else None, "partitions": (info.num_partitions if info is not None else None) if slab else None,
             "threads_per_wave": (tpw_arg or g.max_threads_per_wave(w.K, w.eb)) if slab else None,
             "plan_bytes": int(info.device_bytes) if info is not None else 0,
+            "plan_built_on": None if info is None else ("device" if info.built_on_device else "host"),
             "csr_bytes": int(4 * (w.n + 1) + (4 + w.eb) * w.nnz)}
 
 
@@ -469,7 +470,7 @@ def main():
                    "threads_per_wave": head["threads_per_wave"], "seed": args.seed,
                    "values": args.values, "weights": "value array" if args.weights == "none" else "one factor per node (no value array)",
                    "layout": head["layout"], "plan_signature": head["plan_signature"],
-                   "plan_bytes": head["plan_bytes"], "csr_bytes": head["csr_bytes"]},
+                   "plan_bytes": head["plan_bytes"], "plan_built_on": head["plan_built_on"], "csr_bytes": head["csr_bytes"]},
         "gbs_algorithmic_per_step": round(w.b_alg / (head["ms_per_step"] * 1e6), 2),
         "hbm_fraction_per_step": head["frac_step"],
         "kernel_ms": dict(head["kernel_ms"], **{"preprocessing, host wall time (once per matrix)": head["preprocessing_ms"]}),

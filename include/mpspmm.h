@@ -457,6 +457,8 @@ typedef struct mps_plan_info {
     int sweep_listed_rows;         /* entries of SW_ROWS: n_rows - split rows + partial rows */
     long long sweep_rounds;        /* rounds of all wavefronts                     */
     long long sweep_slots;         /* entry slots incl. padding                    */
+    int built_on_device;           /* row-block and sweep plans: 1 if the passes over the nonzeros ran on the device, 0 if
+                                      on the host (the plan is the same either way); slab plans: always 1 */
 } mps_plan_info;
 
 /* Optional parameters of mps_plan_create_ex; zero means "the library chooses". */

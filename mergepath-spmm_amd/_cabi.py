@@ -66,7 +66,7 @@ class PlanInfo(ctypes.Structure):
                 ("rowblock_cold_index_bits", ctypes.c_int), ("rowblock_local_tables", ctypes.c_int)] + \
                [(n, ctypes.c_int) for n in ("sweep_panels", "sweep_acc_rows", "sweep_lanes", "sweep_tiles", "sweep_col_bits",
                                              "sweep_piece", "sweep_together", "sweep_split_rows", "sweep_partial_rows", "sweep_listed_rows")] + \
-               [("sweep_rounds", ctypes.c_longlong), ("sweep_slots", ctypes.c_longlong)]
+               [("sweep_rounds", ctypes.c_longlong), ("sweep_slots", ctypes.c_longlong), ("built_on_device", ctypes.c_int)]
 
 
 class PlanOptions(ctypes.Structure):

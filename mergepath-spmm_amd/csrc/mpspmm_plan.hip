@@ -1528,10 +1528,12 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
     info->sweep_panels = info->sweep_acc_rows = info->sweep_lanes = info->sweep_tiles = info->sweep_col_bits = 0;
     info->sweep_piece = info->sweep_together = info->sweep_split_rows = info->sweep_partial_rows = info->sweep_listed_rows = 0;
     info->sweep_rounds = info->sweep_slots = 0;
+    info->built_on_device = 1;
     if (plan->sw) {
         info->num_slabs = 1;
         info->slab_cols = plan->n_rows;
         mps_sw::fill_info(mps_sw::layout_of(plan->sw), info);
+        info->built_on_device = mps_sw::built_on_device(plan->sw) ? 1 : 0;
     }
     if (plan->rb) {
         const mps_rb::Layout &L = mps_rb::layout_of(plan->rb);
@@ -1548,6 +1550,7 @@ int mps_plan_get_info(const mps_plan *plan, mps_plan_info *info)
         info->rowblock_cold_slots = L.cold_rounds * mps_rb::kRoundEntries;
         info->rowblock_cold_index_bits = L.cold_index_bits;
         info->rowblock_local_tables = L.table_base.empty() ? 0 : 1;
+        info->built_on_device = mps_rb::built_on_device(plan->rb) ? 1 : 0;
     }
     return MPS_OK;
 }

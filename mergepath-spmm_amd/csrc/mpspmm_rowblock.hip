@@ -30,6 +30,7 @@ struct DevicePlan {
     size_t hot_slots = 0, cold_slots = 0;
     int keep_from = 0;  // steps from this one on read their streams with plain loads (see kStreamKeepBytes)
     int num_cus = 256;  // CUs the layout was built for: one round of blocks is at most this many
+    bool built_on_device = false;
 };
 
 namespace {
@@ -1093,6 +1094,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
+    dp->built_on_device = on_device;
     release(L.hot);
     release(L.hot_packed);
     release(L.cold);
@@ -1177,6 +1179,7 @@ int set_values(DevicePlan *dp, const float *d_val, hipStream_t st)
 }
 
 const Layout &layout_of(const DevicePlan *dp) { return dp->host; }
+bool built_on_device(const DevicePlan *dp) { return dp->built_on_device; }
 
 const void *device_array(const DevicePlan *dp, int which, size_t *bytes)
 {

@@ -211,6 +211,7 @@ void destroy(DevicePlan *dp);
 int spmm(const DevicePlan *dp, const float *X, float *Y, unsigned phases, hipStream_t st);
 int set_values(DevicePlan *dp, const float *d_val, hipStream_t st);
 const Layout &layout_of(const DevicePlan *dp);
+bool built_on_device(const DevicePlan *dp);  // the passes over the nonzeros ran on the device
 size_t device_bytes_of(const DevicePlan *dp);
 // Device array `which` (MPS_PLAN_ARRAY_RB_*) and its size in bytes; nullptr if the plan does not hold it.
 const void *device_array(const DevicePlan *dp, int which, size_t *bytes);

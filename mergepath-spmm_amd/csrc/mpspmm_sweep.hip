@@ -25,6 +25,7 @@ struct DevicePlan {
     int *split_row = nullptr, *split_ptr = nullptr;
     float *partial = nullptr;  // [partial rows][K] fp32 sums of the sub-rows of split rows
     size_t lds_bytes = 0, device_bytes = 0, slots = 0;
+    bool built_on_device = false;
 };
 
 namespace {
@@ -480,6 +481,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
     }
+    dp->built_on_device = on_device;
     Bulk<uint32_t>().swap(Lo.stream);
     Bulk<int>().swap(Lo.src);
     *out = dp;
@@ -508,6 +510,7 @@ int set_values(DevicePlan *dp, const void *d_val, hipStream_t st)
 }
 
 const Layout &layout_of(const DevicePlan *dp) { return dp->host; }
+bool built_on_device(const DevicePlan *dp) { return dp->built_on_device; }
 size_t device_bytes_of(const DevicePlan *dp) { return dp->device_bytes; }
 
 const void *device_array(const DevicePlan *dp, int which, size_t *bytes)

@@ -159,6 +159,7 @@ void destroy(DevicePlan *dp);
 int spmm(const DevicePlan *dp, const void *X, void *Y, unsigned phases, hipStream_t st);
 int set_values(DevicePlan *dp, const void *d_val, hipStream_t st);
 const Layout &layout_of(const DevicePlan *dp);
+bool built_on_device(const DevicePlan *dp);  // the passes over the nonzeros ran on the device
 size_t device_bytes_of(const DevicePlan *dp);
 const void *device_array(const DevicePlan *dp, int which, size_t *bytes);
 #endif
