@@ -412,9 +412,10 @@ def main():
                "traffic": traffic, "l2_hit_rate": l2_hit, "l2_hit_rate_gathers_est": gather_hit, "counters_from": where,
                "algorithmic_bytes": int(wl.b_alg)}
         res.update(desc)
-        if orc is not None:
-            res["check"] = check_product(np, orc, wl, wl.d_Y.float().cpu().numpy(), cpu_loop)
-        # preprocessing time (once per matrix, not part of a step)
+        # preprocessing time (once per matrix, not part of a step): a second plan of the same kind, timed before the
+        # check below, whose OpenMP threads keep spinning for a while after their loop and would share the cores with
+        # the builder's
+        Y_step = wl.d_Y.float().cpu().numpy() if orc is not None else None
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         if plan is not None:
@@ -423,6 +424,8 @@ def main():
             sp.generate_mp_sched(wl.csr.row_ptr, wl.nnz, cost=cost)
         torch.cuda.synchronize()
         res["preprocessing_ms"] = round((time.perf_counter() - t1) * 1e3, 3)
+        if orc is not None:
+            res["check"] = check_product(np, orc, wl, Y_step, cpu_loop)
         if plan is not None:
             plan.close()
         return res
