@@ -70,14 +70,18 @@ __device__ __forceinline__ uint4 load_round(__amdgpu_buffer_rsrc_t r, unsigned o
     return make_uint4(t[0], t[1], t[2], t[3]);
 }
 
-// The same from the packed hot stream: 12 bytes {value A, value B, half A | half B << 16}.
+// The same from a packed stream: 12 bytes {value A, value B, half A | half B << 16}, as loaded.  The halves are taken
+// apart where the round is used (unpack_round), not here: a round is requested one round ahead, behind the gathers of
+// the round before it, and loads return in order - an instruction that touches the loaded words straight away would
+// wait for those gathers as well.
 __device__ __forceinline__ uint4 load_round_packed(__amdgpu_buffer_rsrc_t r, unsigned off, bool keep)
 {
     typedef unsigned u3_t __attribute__((ext_vector_type(3)));
     const u3_t t = keep ? __builtin_amdgcn_raw_buffer_load_b96(r, (int)off, 0, 0)
                         : __builtin_amdgcn_raw_buffer_load_b96(r, (int)off, 0, 2);
-    return make_uint4(t[2] & 0xffffu, t[0], t[2] >> 16, t[1]);
+    return make_uint4(t[0], t[1], t[2], 0u);
 }
+__device__ __forceinline__ uint4 unpack_round(const uint4 &t) { return make_uint4(t.z & 0xffffu, t.x, t.z >> 16, t.y); }
 
 // (a value, not a named constant: a float4 object whose address is taken - by a ?: between two lvalues, by a
 // reference parameter - is given a private-memory slot of its own and reloaded from there)
@@ -311,7 +315,12 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 if constexpr (CPACK) return load_round_packed(cp, loff + (unsigned)r * kColdRoundBytes, keep);
                 else return load_round(cp, loff + (unsigned)r * kColdRoundBytes, keep);
             };
-            uint4 nx_h = make_uint4(0u, 0u, 0u, 0u), nx_c = nx_h;
+            uint4 nx_h = make_uint4(0u, 0u, 0u, 0u), nx_c = nx_h;  // as loaded
+            auto take_h = [&]() { return unpack_round(nx_h); };
+            auto take_c = [&]() {
+                if constexpr (CPACK) return unpack_round(nx_c);
+                else return nx_c;
+            };
             if (rounds_h > 0) nx_h = load_hot(0);
             if (rounds_c > 0) nx_c = load_cold(0);
             int rh = 0, rc = 0;  // rounds done
@@ -346,7 +355,13 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 due_h += full_h;
                 due_c += full_c;
                 const bool do_h = due_h >= passes && rh < full_h, do_c = due_c >= passes && rc < full_c;
-                const uint4 cu_c = nx_c;
+                // Both rounds have arrived before anything else is requested.  (Left to the compiler, the wait for the
+                // hot round stands where the round is taken apart, behind the cold gathers of this pass: loads return
+                // in order, and with a pass that has no cold round in the same code it must assume that nothing was
+                // requested after the round - it waits for everything, the gathers included, and the hot round then
+                // runs with no gather in flight.)
+                asm volatile("" : "+v"(nx_h.z), "+v"(nx_c.z));
+                const uint4 cu_c = take_c();
                 float4 xca[kWin], xcb[kWin];
                 if (do_c) {
                     due_c -= passes;
@@ -357,7 +372,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 }
                 if (do_h) {
                     due_h -= passes;
-                    const uint4 cu_h = nx_h;
+                    const uint4 cu_h = take_h();
                     float4 xh[kWin];
                     advance_h();
                     // one window after the other: table rows arrive within a hundred cycles or two, and four rows
@@ -371,7 +386,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             }
             // what the rounding of the shares left over
             while (rh < full_h) {
-                const uint4 cu_h = nx_h;
+                const uint4 cu_h = take_h();
                 float4 xha[kWin], xhb[kWin];
                 advance_h();
                 hot_gather(cu_h.x, xha);
@@ -379,7 +394,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 pair(kHot, wh, cu_h, xha, xhb, hot_hi, 0, true, true);
             }
             while (rc < full_c) {
-                const uint4 cu_c = nx_c;
+                const uint4 cu_c = take_c();
                 float4 xca[kWin], xcb[kWin];
                 cold_gather(cu_c.x, xca);
                 cold_gather(cu_c.z, xcb);
@@ -388,16 +403,18 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             }
             // the last round of a run: lane-groups hold two, one or none of its windows (the rest is padding)
             if (rc < rounds_c) {
+                const uint4 cu_c = take_c();
                 float4 xca[kWin], xcb[kWin];
-                cold_gather(nx_c.x, xca);
-                cold_gather(nx_c.z, xcb);
-                pair(kCold, wc, nx_c, xca, xcb, cold_hi, cold_bits, 2 * rc < len_c, 2 * rc + 1 < len_c);
+                cold_gather(cu_c.x, xca);
+                cold_gather(cu_c.z, xcb);
+                pair(kCold, wc, cu_c, xca, xcb, cold_hi, cold_bits, 2 * rc < len_c, 2 * rc + 1 < len_c);
             }
             if (rh < rounds_h) {
+                const uint4 cu_h = take_h();
                 float4 xha[kWin], xhb[kWin];
-                hot_gather(nx_h.x, xha);
-                hot_gather(nx_h.z, xhb);
-                pair(kHot, wh, nx_h, xha, xhb, hot_hi, 0, 2 * rh < len_h, 2 * rh + 1 < len_h);
+                hot_gather(cu_h.x, xha);
+                hot_gather(cu_h.z, xhb);
+                pair(kHot, wh, cu_h, xha, xhb, hot_hi, 0, 2 * rh < len_h, 2 * rh + 1 < len_h);
             }
             cur_h += rounds_h;
             cur_c += rounds_c;
