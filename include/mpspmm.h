@@ -404,7 +404,8 @@ typedef struct mps_plan mps_plan;
                                         matrices whose columns stay within 8 tables' width of the diagonal); with
                                         MPS_PLAN_FORCE_ROWBLOCK or mps_rowblock_layout_build */
 #define MPS_PLAN_NO_SWEEP 2048u     /* never build a sweep plan (see below)       */
-#define MPS_PLAN_FORCE_SWEEP 4096u  /* sweep plan whatever the matrix looks like (rows of X a multiple of 64 bytes) */
+#define MPS_PLAN_FORCE_SWEEP 4096u  /* sweep plan whatever the matrix looks like (rows of X of whole dwords: any K in fp32, an even K in fp16;
+                                       an X of 4 GiB or more: rows of whole 16 bytes) */
 #define MPS_PLAN_HOST_BUILD 8192u   /* row-block and sweep plans: every pass over the nonzeros on the host, from a copy of the CSR
                                        arrays (the library makes these passes on the device where it can; both give the same plan) */
 #define MPS_PLAN_NO_COLUMN_TILES 512u /* untiled plans with rows of X of 512 bytes and more: no passes over 128-byte column tiles */
@@ -446,7 +447,7 @@ typedef struct mps_plan_info {
     /* sweep plans (sweep_panels > 0); the fields about slabs, partitions, slices and row blocks are then 0 / 1 */
     int sweep_panels;              /* panels = workgroups per column tile          */
     int sweep_acc_rows;            /* accumulator rows per panel in LDS            */
-    int sweep_lanes;               /* lanes per lane-group: 4 (64-byte rows of X) or 8 (128-byte column tiles) */
+    int sweep_lanes;               /* lanes per lane-group: 4 (rows of X of up to 64 bytes) or 8 (128-byte column tiles; the last one may be narrower) */
     int sweep_tiles;               /* column tiles per row of X                    */
     int sweep_col_bits;            /* an entry word is column | accumulator row << sweep_col_bits */
     int sweep_piece;               /* most entries of a row that one accumulator row takes */

@@ -1280,7 +1280,8 @@ __global__ __launch_bounds__(256) void near_diagonal_kernel(const int *__restric
     if (threadIdx.x == 0 && block_count) atomicAdd(count, (unsigned long long)block_count);
 }
 
-// Sweep plan or not.  Forced: yes.  Otherwise for rows of X of 64 bytes or a multiple of 128, when the caller is
+// Sweep plan or not.  Forced: yes.  Otherwise for rows of X of 64 bytes or a multiple of 128 (and the widths that
+// the comment inside sweep_wanted() adds to these), when the caller is
 // not tuning a slab plan (a cost, partitions per wavefront or tiling / hot-column switches of its own) and the matrix
 // is not local.  Measured on MI355X, ms per product, sweep plan against the library's other choice:
 //   fp32, K = 16 (against row-block plans, slab plans where those are not built):
@@ -1311,8 +1312,18 @@ int sweep_wanted(const int *d_row_ptr, const int *d_col_idx, int n_rows, int nnz
     if (flags & (MPS_PLAN_NO_SWEEP | MPS_PLAN_FORCE_ROWBLOCK | MPS_PLAN_LOCAL_TABLES | MPS_PLAN_FORCE_TILING | MPS_PLAN_NO_TILING |
                  MPS_PLAN_FORCE_HOT | MPS_PLAN_NO_HOT | MPS_PLAN_NO_ROW_MARKS))
         return MPS_OK;
+    // Rows of X that a sweep plan is chosen for: whole 128-byte tiles or one 64-byte tile, and, of the rows that leave
+    // lanes of their last tile idle, those that fit one tile or are whole 64 bytes, as long as every lane's 16 bytes are
+    // aligned.  Measured on MI355X, sweep plan against slab plan, ms per product: R-MAT scale 20 fp32 K = 8, 12, 20, 24,
+    // 48: 0.122 / 0.164, 0.151 / 0.219, 0.205 / 0.240, 0.206 / 0.244, 0.347 / 0.394; the 232,965-row power-law matrix
+    // K = 8, 12, 24, 48: 0.506 / 0.683, 0.563 / 0.924, 0.842 / 1.035, 1.56 / 1.72; R-MAT scale 22 fp16 K = 24, 40:
+    // 0.826 / 0.860, 1.03 / 1.17.  Left to the slab plans: rows of several tiles that start anywhere in a 128-byte
+    // line (fp32 K = 100: 0.925 / 0.894 and 3.59 / 3.51) and rows whose pitch is no multiple of 16 bytes, where a
+    // lane's 16 bytes lie across two aligned ones (fp32 K = 41: 0.494 / 0.526; fp16 K = 100: 2.81 / 2.31).
     const long long row_bytes = (long long)K * elem_bytes;
-    if (n_rows < 1 || nnz < 1 || (row_bytes != 64 && row_bytes % 128 != 0)) return MPS_OK;
+    const bool whole_tiles = row_bytes == 64 || row_bytes % 128 == 0;
+    const bool idle_lanes_pay = row_bytes % 16 == 0 && (row_bytes < 128 || row_bytes % 64 == 0);
+    if (n_rows < 1 || nnz < 1 || !(whole_tiles || idle_lanes_pay)) return MPS_OK;
     if (n_rows > (1 << 26)) return MPS_OK;  // an entry word keeps 6 bits for the accumulator row
     int default_cost = 0, max_tpw = 0;
     if (mps_default_cost(n_rows, nnz, K, elem_bytes, &default_cost) != MPS_OK || cost != default_cost) return MPS_OK;
@@ -1406,7 +1417,7 @@ int mps_plan_create_ex(const int *d_row_ptr, const int *d_col_idx, const void *d
         }
     }
     if (want_sweep) {
-        if (n_rows < 1 || ((long long)K * elem_bytes) % 64 != 0) {
+        if (n_rows < 1 || ((long long)K * elem_bytes) % 4 != 0) {
             plan_free(pl);
             return MPS_ERR_UNSUPPORTED;
         }

@@ -49,9 +49,9 @@ struct Piece<float> {
     static constexpr int kVec = 4, kPlanes = 1;
     f4_t raw;
     __device__ __forceinline__ void load(const char *p) { raw = *reinterpret_cast<const f4_t *>(p); }
-    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned base)
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off)
     {
-        raw = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, (int)base, 0));
+        raw = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
     }
     __device__ __forceinline__ f4_t plane(int) const { return raw; }
 };
@@ -60,9 +60,9 @@ struct Piece<half_t> {
     static constexpr int kVec = 8, kPlanes = 2;
     half8_t raw;
     __device__ __forceinline__ void load(const char *p) { raw = *reinterpret_cast<const half8_t *>(p); }
-    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off, unsigned base)
+    __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t r, unsigned off)
     {
-        raw = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, (int)base, 0));
+        raw = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0));
     }
     __device__ __forceinline__ f4_t plane(int q) const
     {
@@ -71,9 +71,30 @@ struct Piece<half_t> {
     }
 };
 
+// A lane's 16 bytes of a row of Y (or of a partial row): `valid` of the kVec sums, the others lie past the row's end.
+// Rows whose pitch is no multiple of 16 bytes start anywhere on a dword boundary.
+template <typename TOut, int VEC>
+__device__ __forceinline__ void store_piece(TOut *p, const float (&sum)[VEC], int valid)
+{
+    if (valid >= VEC) {
+        store_acc<VEC, true>(p, sum);
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            if (e < valid) __builtin_nontemporal_store((TOut)sum[e], p + e);
+    }
+}
+
 // T: element type of X and Y.  L: lanes per lane-group (16 L bytes of a row of X per tile).  FAR: X is addressed with
 // 64-bit pointers; otherwise (X below 4 GiB, fewer than 2^24 rows) with a 32-bit offset that one 24-bit
-// multiply-add forms.
+// multiply-add forms, through a buffer descriptor that knows the size of X.
+// K is any number of elements that fills whole dwords: a row of X is ceil(16 L-byte tiles), and in the last tile
+//   * a lane whose 16 bytes begin past the row's end reads the tile's first 16 bytes instead (the line that lane 0
+//     of its lane-group asks for anyway) and adds them to a part of the accumulator row that is never written out;
+//   * a lane whose 16 bytes begin inside the row and end past it reads the first elements of the next row with its
+//     own last ones and never writes those sums out either.  Past the last row of X there is no next row: the buffer
+//     descriptor's range check, which works dword by dword on such loads, returns zeros there and requests nothing.
+//     (With 64-bit pointers nothing checks the range: FAR plans are built for rows of whole 16 bytes only.)
 // LDS: kPlanes planes of (acc_rows + 1) x L float4: plane q holds elements 4 q .. 4 q + 3 of every lane's 16 bytes, so
 // that one 16-byte LDS access per lane covers a plane's row exactly like an fp32 row.
 template <typename T, int L, int TOGETHER, bool FAR>
@@ -105,9 +126,10 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     // this lane's 16 bytes of a row of X: row pitch K elements, tile `tile`, piece c
     const unsigned row_pitch = (unsigned)K * (unsigned)sizeof(T);
     const unsigned lane_off = (unsigned)c * 16u, tile_off = (unsigned)tile * (16u * L);
-    [[maybe_unused]] const char *xb = reinterpret_cast<const char *>(X) + tile_off + lane_off;
+    const unsigned x_off = tile_off + lane_off < row_pitch ? tile_off + lane_off : tile_off;
+    [[maybe_unused]] const char *xb = reinterpret_cast<const char *>(X) + x_off;
     [[maybe_unused]] const __amdgpu_buffer_rsrc_t x_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(X), 0, 0xffffffff, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(X), 0, FAR ? 0xffffffffu : (unsigned)n * row_pitch, 0x00020000);
     const unsigned plane_bytes = (unsigned)plane_stride * 16u;
 
     auto stream_load = [&](int r) {
@@ -124,7 +146,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
         if constexpr (FAR) {                                                                 \
             x[k].load(xb + (size_t)(w & (CM)) * row_pitch);                                  \
         } else {                                                                             \
-            x[k].load(x_rsrc, __umul24(w & (CM), row_pitch) + lane_off, tile_off);           \
+            x[k].load(x_rsrc, __umul24(w & (CM), row_pitch) + x_off);                        \
         }                                                                                    \
     }
     // One entry after the other: read the accumulator row, add, write it back.  The LDS serves a wavefront's
@@ -233,33 +255,28 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
                 sum[4 * q + 3] += a[3];
             }
         }
-        const size_t col0 = (size_t)tile * (L * P::kVec) + (size_t)cc * P::kVec;
+        const int col0 = tile * (L * P::kVec) + cc * P::kVec;
         if (row < n) {
-            store_acc<P::kVec, true>(Y + (size_t)row * K + col0, sum);
+            if (col0 < K) store_piece<T, P::kVec>(Y + (size_t)row * K + col0, sum, K - col0);
         } else {
-            store_acc<P::kVec, false>(partial + (size_t)(row - n) * K + col0, sum);  // read again by the fix-up kernel
+            // read again by the fix-up kernel; a partial row has whole tiles
+            store_acc<P::kVec, false>(partial + (size_t)(row - n) * ((size_t)gridDim.y * (L * P::kVec)) + col0, sum);
         }
     }
 }
 
-// Y[split_row[i]][:] = the sum of its partial rows, in order.
+// Y[split_row[i]][:] = the sum of its partial rows (pitch Kp floats: whole tiles), in order.
 template <typename T>
 __global__ __launch_bounds__(256) void sw_fixup_kernel(const int *__restrict__ split_row, const int *__restrict__ split_ptr,
-                                                        const float *__restrict__ partial, T *__restrict__ Y, int n_split, int K)
+                                                        const float *__restrict__ partial, T *__restrict__ Y, int n_split, int K,
+                                                        int Kp)
 {
-    const int quads = K / 4;
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= (long long)n_split * quads) return;
-    const int r = (int)(i / quads), q = (int)(i % quads);
-    float sum[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int p = split_ptr[r]; p < split_ptr[r + 1]; ++p) {
-        const f4_t a = *reinterpret_cast<const f4_t *>(partial + (size_t)p * K + 4 * q);
-        sum[0] += a[0];
-        sum[1] += a[1];
-        sum[2] += a[2];
-        sum[3] += a[3];
-    }
-    store_acc<4, true>(Y + (size_t)split_row[r] * K + 4 * q, sum);
+    if (i >= (long long)n_split * K) return;
+    const int r = (int)(i / K), e = (int)(i % K);
+    float sum = 0.f;
+    for (int p = split_ptr[r]; p < split_ptr[r + 1]; ++p) sum += partial[(size_t)p * Kp + e];
+    Y[(size_t)split_row[r] * K + e] = (T)sum;
 }
 
 // New values into the stream: entry slot i (stream order) holds nonzero src[i].
@@ -289,6 +306,17 @@ int upload(DevicePlan *dp, T **dst, const std::vector<T, A> &src, hipStream_t st
     return MPS_OK;
 }
 
+// 32-bit offsets into X where every row starts below 4 GiB and a column index fits the 24-bit multiply; 64-bit pointers
+// otherwise
+bool needs_far(const Layout &Lo)
+{
+    const unsigned long long pitch = (unsigned long long)Lo.K * (unsigned long long)Lo.elem_bytes;
+    return Lo.col_bits > 24 || (unsigned long long)Lo.n * pitch > 0xffffff00ull || pitch >= (1ull << 24);
+}
+
+// elements of a row in whole tiles: the pitch of the partial rows
+int padded_width(const Layout &Lo) { return Lo.tiles * Lo.lanes * (16 / Lo.elem_bytes); }
+
 template <typename T, int L, int TOGETHER, bool FAR>
 int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
 {
@@ -304,11 +332,7 @@ int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
 template <typename T, int L, int TOGETHER>
 int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
 {
-    // 32-bit offsets into X where every row starts below 4 GiB and a column index fits the 24-bit multiply
-    const Layout &Lo = dp->host;
-    const bool far = Lo.col_bits > 24 || (unsigned long long)Lo.n * (unsigned long long)Lo.K * sizeof(T) > 0xffffff00ull ||
-                     (unsigned long long)Lo.K * sizeof(T) >= (1ull << 24);
-    return far ? launch_main<T, L, TOGETHER, true>(dp, X, Y, st) : launch_main<T, L, TOGETHER, false>(dp, X, Y, st);
+    return needs_far(dp->host) ? launch_main<T, L, TOGETHER, true>(dp, X, Y, st) : launch_main<T, L, TOGETHER, false>(dp, X, Y, st);
 }
 
 template <typename T>
@@ -321,9 +345,9 @@ int spmm_typed(const DevicePlan *dp, const T *X, T *Y, unsigned phases, hipStrea
         if (rc != MPS_OK) return rc;
     }
     if ((phases & MPS_PHASE_FIXUP) && !Lo.split_row.empty()) {
-        const long long threads = (long long)Lo.split_row.size() * (Lo.K / 4);
+        const long long threads = (long long)Lo.split_row.size() * Lo.K;
         hipLaunchKernelGGL((sw_fixup_kernel<T>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, dp->split_row,
-                           dp->split_ptr, dp->partial, Y, (int)Lo.split_row.size(), Lo.K);
+                           dp->split_ptr, dp->partial, Y, (int)Lo.split_row.size(), Lo.K, padded_width(Lo));
         MPS_HIP_TRY(hipGetLastError());
     }
     return MPS_OK;
@@ -394,6 +418,9 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
         std::vector<ListedRow> listed_rows;
         rc = plan_panels(rp.data(), n, nnz, K, bp, dp->host, listed_rows);
         if (rc != MPS_OK) return fail(rc);
+        // (an X of 4 GiB or more is read through pointers, with nothing to catch the lane that reads past the end of
+        // its last row: rows of whole 16 bytes only)
+        if (needs_far(dp->host) && ((long long)K * bp.elem_bytes) % 16 != 0) return fail(MPS_ERR_UNSUPPORTED);
         if (!bp.host_build) {
             // the passes over the nonzeros where the nonzeros are
             DeviceStreams ds;
@@ -452,7 +479,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
     if ((rc = upload(dp, &dp->split_row, Lo.split_row, st)) != MPS_OK) return fail(rc);
     if ((rc = upload(dp, &dp->split_ptr, Lo.split_ptr, st)) != MPS_OK) return fail(rc);
     {
-        const size_t bytes = ((size_t)Lo.split_ptr.back() * Lo.K + 4) * sizeof(float);
+        const size_t bytes = ((size_t)Lo.split_ptr.back() * padded_width(Lo) + 4) * sizeof(float);
         hipError_t e = hipMalloc(reinterpret_cast<void **>(&dp->partial), bytes);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
         dp->device_bytes += bytes;

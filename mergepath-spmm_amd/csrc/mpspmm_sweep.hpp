@@ -39,7 +39,8 @@
 //     its entry of two windows of 4 with one 16-byte load, and the 4 lanes of
 //     a quad pass their entries round with quad permutes.
 //   * Rows of X wider than 128 bytes are handled in column tiles of 128 bytes
-//     (blockIdx.y): the same stream once per tile.
+//     (blockIdx.y): the same stream once per tile.  A row need not fill its last
+//     tile (or, below 64 bytes, its only one): lanes past the row's end stay idle.
 #ifndef MPSPMM_SWEEP_HPP
 #define MPSPMM_SWEEP_HPP
 

@@ -140,9 +140,11 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
     if (n < 1 || nnz < 0 || K < 1 || !rp) return MPS_ERR_INVALID_ARG;
     if (bp.elem_bytes != 4 && bp.elem_bytes != 2) return MPS_ERR_INVALID_ARG;
     const long long row_bytes = (long long)K * bp.elem_bytes;
-    if (row_bytes % 64 != 0) return MPS_ERR_UNSUPPORTED;
-    const int L = row_bytes % 128 == 0 ? 8 : 4;
-    const int tiles = (int)(row_bytes / (16 * L));
+    if (row_bytes % 4 != 0) return MPS_ERR_UNSUPPORTED;  // (an odd number of halves: rows of X that start between two dwords)
+    // Rows of up to 64 bytes: one tile of 4 lanes; wider ones: tiles of 8 lanes (128 bytes), the last of them as wide as
+    // what is left of the row - lanes past the row's end add up bytes that nobody reads.
+    const int L = row_bytes <= 64 ? 4 : 8;
+    const int tiles = (int)((row_bytes + 16 * L - 1) / (16 * L));
     const int acc_row_bytes = 16 * L * (4 / bp.elem_bytes);  // fp32 sums of a tile: 16 L bytes of floats, 32 L of halves
     const int col_bits = bits_for((unsigned)(n - 1));
     if (col_bits > 32 - kMinRowBits) return MPS_ERR_UNSUPPORTED;
@@ -152,7 +154,7 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
     if (bp.acc_rows > 0) vcap = std::min<long long>(vcap, bp.acc_rows);
     vcap &= ~3ll;
     if (vcap < 4) return MPS_ERR_UNSUPPORTED;
-    const int U = row_bytes < 128 ? 2 : 1;  // rows of Y per 128-byte line
+    const int U = row_bytes <= 64 ? 2 : 1;  // rows of Y per 128-byte line
 
     out = Layout();
     out.n = n;

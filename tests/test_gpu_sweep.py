@@ -24,6 +24,26 @@ CASES = [
     (3000, 40, ((5, 2800),), 16, "f32", 0, 0, 8, 2),               # 64-byte rows with pairs of instructions added up together
     (3000, 40, ((5, 2800),), 32, "f32", 0, 0, 8, 1),               # 128-byte rows, one instruction at a time
     (2000, 30, ((11, 1500),), 64, "f16", 0, 0, 8, 1),
+    # rows of X that do not fill whole tiles: lanes past the row's end, lanes that straddle it, rows that start
+    # between two 16-byte boundaries
+    (300, 40, ((5, 280),), 8, "f32", 0, 0, 4),                     # 32-byte rows: half of the 4 lanes idle
+    (500, 30, ((7, 450),), 12, "f32", 0, 0, 4),
+    (400, 25, ((3, 390), (399, 380)), 20, "f32", 0, 0, 4),         # 80 bytes of a 128-byte tile
+    (1000, 30, ((999, 900),), 24, "f32", 4, 0, 8),
+    (600, 35, ((0, 550), (599, 500)), 41, "f32", 0, 0, 8),         # 164-byte rows: two tiles, the last lane straddles the end
+    (800, 20, ((5, 700),), 48, "f32", 0, 0, 4, 2),
+    (3000, 60, ((17, 2800), (2999, 2000)), 100, "f32", 0, 0, 64),  # four tiles, the last of them 16 bytes; rows cut across panels
+    (200, 15, ((199, 190),), 7, "f32", 0, 0, 2),
+    (150, 10, ((149, 140),), 1, "f32", 0, 0, 2),                   # one float per row
+    (350, 22, ((349, 300),), 33, "f32", 0, 0, 4),
+    (5000, 100, ((4999, 4500),), 200, "f32", 0, 0, 64),
+    (400, 30, ((399, 350),), 8, "f16", 0, 0, 4),                   # 16-byte rows of halves
+    (500, 30, ((499, 450),), 24, "f16", 0, 0, 4),
+    (600, 30, ((599, 500),), 40, "f16", 0, 0, 8),                  # 80-byte rows: a 128-byte tile, two planes
+    (700, 30, ((699, 600), (0, 650)), 72, "f16", 0, 0, 8),         # 144 bytes: two tiles
+    (300, 20, ((299, 250),), 2, "f16", 0, 0, 2),                   # one dword per row
+    (450, 25, ((449, 400),), 6, "f16", 0, 0, 4),
+    (2500, 50, ((2499, 2300),), 100, "f16", 0, 0, 32),
 ]
 
 
@@ -42,15 +62,23 @@ def test_sweep_plan_matches_fp64_loop(pkg, orc, dev, case):
     rng = np.random.default_rng(abs(hash(case)) % (2 ** 32))
     rp, ci, val, X = make_inputs(rng, n, max_deg, hubs, K, dt)
     csr = make_csr(pkg, dev, rp, ci, val)
-    (d_X,) = to_dev(dev, X)
+    # X between NaNs: what a lane reads past the end of a row must not reach a sum that is written out
+    guard = 64
+    xbuf = torch.full((n * K + 2 * guard,), float("nan"), dtype=torch.float32 if dt == "f32" else torch.float16, device=dev)
+    d_X = xbuf[guard:guard + n * K].view(n, K)
+    d_X.copy_(torch.from_numpy(X))
     plan = pkg.spmm.Plan(csr, K, sweep="force", sweep_piece=piece, sweep_acc_rows=acc_rows, sweep_panels_per_round=per_round,
                          sweep_together=together)
     i = plan.info
     assert i.sweep_panels > 0 and i.rowblock_steps == 0
-    assert i.sweep_tiles * i.sweep_lanes * 16 == K * X.itemsize
-    Y = torch.full_like(d_X, float("nan"))
+    tile_bytes = i.sweep_lanes * 16
+    assert (i.sweep_tiles - 1) * tile_bytes < K * X.itemsize <= i.sweep_tiles * tile_bytes
+    # Y in the middle of a buffer of NaNs: nothing is written before its first or after its last element
+    buf = torch.full((n * K + 2 * guard,), float("nan"), dtype=d_X.dtype, device=dev)
+    Y = buf[guard:guard + n * K].view(n, K)
     plan.spmm(d_X, out=Y)
     torch.cuda.synchronize()
+    assert torch.isnan(buf[:guard]).all() and torch.isnan(buf[guard + n * K:]).all()
     if dt == "f32":
         ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
         check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
@@ -132,13 +160,39 @@ def test_sweep_plan_set_values_and_sources(pkg, orc, dev):
         assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
 
 
-def test_sweep_plan_refuses_rows_it_has_no_lane_group_for(pkg, dev):
+def test_sweep_plan_refuses_rows_that_start_between_dwords(pkg, dev):
     rng = np.random.default_rng(2)
-    rp, ci, val, X = make_inputs(rng, 100, 5, (), 24, "f32")  # 96-byte rows
+    rp, ci, val, X = make_inputs(rng, 100, 5, (), 25, "f16")  # 50-byte rows
     csr = make_csr(pkg, dev, rp, ci, val)
     with pytest.raises(pkg._cabi.MpsError) as e:
-        pkg.spmm.Plan(csr, 24, sweep="force")
+        pkg.spmm.Plan(csr, 25, sweep="force")
     assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
+
+
+def test_sweep_plan_is_chosen_for_rows_that_leave_lanes_idle(pkg, orc, dev):
+    # the library's own choice: one tile that the row does not fill, or whole 64 bytes; not rows of several tiles that
+    # start anywhere in a line, not rows whose pitch is no multiple of 16 bytes
+    rng = np.random.default_rng(12)
+    n = 6000
+    rp, ci = random_csr(rng, n, 30, p_empty=0.1, hub_rows=((3, 5000),))
+    for dt, K, sweep in (("f32", 8, True), ("f32", 12, True), ("f32", 24, True), ("f32", 48, True), ("f32", 32, True),
+                         ("f32", 41, False), ("f32", 36, False), ("f32", 100, False), ("f32", 18, False),
+                         ("f16", 24, True), ("f16", 40, True), ("f16", 96, True), ("f16", 100, False), ("f16", 20, False)):
+        npdt = np.float32 if dt == "f32" else np.float16
+        val = rng.random(ci.size).astype(npdt)
+        X = (rng.random((n, K)) * 2 - 1).astype(npdt)
+        csr = make_csr(pkg, dev, rp, ci, val)
+        (d_X,) = to_dev(dev, X)
+        plan = pkg.spmm.Plan(csr, K)
+        assert (plan.info.sweep_panels > 0) == sweep, (dt, K)
+        Y = plan.spmm(d_X)
+        torch.cuda.synchronize()
+        if dt == "f32":
+            ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+            check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+        else:
+            ref, scale = orc.spmm_f64_f16in(rp, ci, val, X, want_abs=True)
+            check_fp16(Y.cpu().numpy(), ref, scale)
 
 
 def test_sweep_plan_under_graph_capture(pkg, orc, dev):

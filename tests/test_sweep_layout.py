@@ -22,7 +22,7 @@ def walk(pkg, lay, n, K, X, elem_bytes):
     assert together in (1, 2)
     gpw = 64 // L
     G = max(1, 256 // (16 * L))
-    assert tiles * L * 16 == K * elem_bytes
+    assert (tiles - 1) * L * 16 < K * elem_bytes <= tiles * L * 16 and L == (4 if K * elem_bytes <= 64 else 8)
     panel_ptr = lay.array(C.MPS_PLAN_ARRAY_SW_PANEL_PTR, np.int32)
     rows = lay.array(C.MPS_PLAN_ARRAY_SW_ROWS, np.int32)
     piece_ptr = lay.array(C.MPS_PLAN_ARRAY_SW_PIECE_PTR, np.int32)
@@ -104,6 +104,9 @@ CASES = [
     (1, 1, (), 16, 4, 0, 0, 2, 0),
     (300, 12, ((5, 280),), 16, 4, 0, 0, 4, 2),   # 64-byte rows with pairs of instructions
     (400, 9, ((100, 257),), 32, 4, 0, 0, 4, 1),  # 128-byte rows, one instruction at a time
+    (150, 8, ((7, 140),), 12, 4, 0, 0, 2, 0),    # 48-byte rows: one tile of 4 lanes, one of them idle
+    (220, 8, ((9, 200),), 41, 4, 0, 0, 2, 0),    # 164-byte rows: two tiles of 8 lanes
+    (180, 8, ((3, 170),), 40, 2, 0, 0, 2, 0),    # fp16, 80-byte rows
 ]
 
 
@@ -147,5 +150,5 @@ def test_sweep_layout_rejects_what_it_cannot_hold(pkg):
     ci = np.array([0, 1], dtype=np.int32)
     val = np.ones(2, dtype=np.float32)
     with pytest.raises(pkg._cabi.MpsError) as e:
-        pkg.spmm.SweepLayout(rp, ci, val, 12)  # rows of X of 48 bytes
+        pkg.spmm.SweepLayout(rp, ci, val, 13, elem_bytes=2)  # rows of X of 26 bytes: they start between two dwords
     assert e.value.status == pkg._cabi.MPS_ERR_UNSUPPORTED
