@@ -195,6 +195,30 @@ def test_rmat_config_full_size(pkg, orc, dev, K):
             check_against_cpu_fp32_loops(loops, ref, Yg.cpu().numpy())
 
 
+@pytest.mark.parametrize("K", [24, 48])
+def test_rmat_full_size_widths_that_leave_lanes_idle(pkg, orc, dev, K):
+    # R-MAT scale 20 at widths between the benchmark's: 96-byte rows (one tile of 8 lanes, two of them idle) and
+    # 192-byte rows (two tiles, half of the second idle); the library's choice is a sweep plan for both
+    rp, ci, val, X = workload(pkg, pkg.graphs.CONFIG_SPECS["rmat_s20"], K)
+    csr = make_csr(pkg, dev, rp, ci, val)
+    (d_X,) = to_dev(dev, X)
+    ref, scale = orc.spmm_f64(rp, ci, val, X, want_abs=True)
+    plan = pkg.spmm.Plan(csr, K)
+    i = plan.info
+    assert i.sweep_panels == 512 and i.sweep_lanes == 8 and i.sweep_tiles == (K * 4 + 127) // 128
+    Y = plan.spmm(d_X, out=torch.full_like(d_X, float("nan")))
+    torch.cuda.synchronize()
+    check_fp32(Y.cpu().numpy(), ref, scale, rel_elem=False)
+    other = pkg.spmm.Plan(csr, K, sweep="off")
+    assert other.info.sweep_panels == 0
+    check_fp32(other.spmm(d_X).cpu().numpy(), ref, scale, rel_elem=False)
+    # the same bits from the plan built with the passes over the nonzeros on the host
+    host = pkg.spmm.Plan(csr, K, host_build=True)
+    assert torch.equal(host.spmm(d_X), Y)
+    for pl in (plan, other, host):
+        pl.close()
+
+
 def test_block_diagonal_config_full_size(pkg, orc, dev):
     # config 3: 1,178 disjoint random-geometric blocks, fp32, K = 16; rows are short, so the
     # per-element bar (1e-5 relative, 1e-6 absolute) applies literally
