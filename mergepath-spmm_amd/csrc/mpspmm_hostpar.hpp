@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <condition_variable>
 #include <cstdint>
 #include <cstdlib>
 #include <exception>
@@ -32,6 +33,101 @@ inline int host_threads()
     }();
     return n;
 }
+
+// The workers: started at the first parallel_for that wants them and kept until the process ends (a builder makes
+// ten to twenty parallel_for calls per plan, and starting 15 threads costs 0.3-0.6 ms each time).  One job at a
+// time: a call that finds the pool busy - another thread's call, or a call from inside a chunk - runs its chunks on
+// the calling thread alone.
+class Pool {
+public:
+    static Pool &get()
+    {
+        static Pool pool;
+        return pool;
+    }
+    // job() on up to `helpers` workers and on the calling thread; returns when all of them have returned
+    template <typename Job>
+    void run(int helpers, Job &job)
+    {
+        if (inside() || helpers < 1 || !busy_.try_lock()) {
+            job();
+            return;
+        }
+        std::lock_guard<std::mutex> release(busy_, std::adopt_lock);
+        inside() = true;
+        struct Leave {
+            ~Leave() { inside() = false; }
+        } leave;
+        {
+            std::lock_guard<std::mutex> hold(lock_);
+            grow(helpers);
+            call_ = [](void *j) { (*static_cast<Job *>(j))(); };
+            job_ = &job;
+            wanted_ = std::min<int>(helpers, (int)threads_.size());
+            started_ = 0;
+            ++generation_;
+        }
+        wake_.notify_all();
+        job();
+        std::unique_lock<std::mutex> hold(lock_);
+        wanted_ = started_;  // workers that have not woken up yet find nothing to do
+        done_.wait(hold, [&] { return running_ == 0; });
+        job_ = nullptr;
+    }
+
+private:
+    Pool() = default;
+    ~Pool()
+    {
+        {
+            std::lock_guard<std::mutex> hold(lock_);
+            stop_ = true;
+        }
+        wake_.notify_all();
+        for (auto &t : threads_) t.join();
+    }
+    static bool &inside()
+    {
+        static thread_local bool in = false;
+        return in;
+    }
+    void grow(int helpers)  // lock_ held
+    {
+        try {
+            while ((int)threads_.size() < helpers) threads_.emplace_back([this] { work(); });
+        } catch (const std::system_error &) {
+            // fewer threads than asked for: the ones that started and the caller share the chunks
+        }
+    }
+    void work()
+    {
+        inside() = true;  // a parallel_for inside a chunk runs on the worker alone
+        unsigned long long seen = 0;
+        std::unique_lock<std::mutex> hold(lock_);
+        for (;;) {
+            wake_.wait(hold, [&] { return stop_ || generation_ != seen; });
+            if (stop_) return;
+            seen = generation_;
+            if (started_ >= wanted_) continue;
+            ++started_;
+            ++running_;
+            void (*call)(void *) = call_;
+            void *job = job_;
+            hold.unlock();
+            call(job);  // (the job catches what its chunks throw)
+            hold.lock();
+            if (--running_ == 0) done_.notify_all();
+        }
+    }
+    std::mutex busy_, lock_;
+    std::condition_variable wake_, done_;
+    std::vector<std::thread> threads_;
+    void (*call_)(void *) = nullptr;
+    void *job_ = nullptr;
+    unsigned long long generation_ = 0;
+    int wanted_ = 0, started_ = 0, running_ = 0;
+    bool stop_ = false;
+};
 
 template <typename F>
 void parallel_for(int64_t n, int64_t grain, F &&fn)
@@ -63,15 +159,7 @@ void parallel_for(int64_t n, int64_t grain, F &&fn)
             if (!failure) failure = std::current_exception();
         }
     };
-    std::vector<std::thread> th;
-    th.reserve(nt - 1);
-    try {
-        for (int t = 1; t < nt; ++t) th.emplace_back(worker);
-    } catch (const std::system_error &) {
-        // fewer threads than asked for: the ones that started and this one share the chunks
-    }
-    worker();
-    for (auto &t : th) t.join();
+    Pool::get().run(nt - 1, worker);
     if (failure) std::rethrow_exception(failure);
 }
 

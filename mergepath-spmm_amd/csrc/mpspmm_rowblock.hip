@@ -502,8 +502,8 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
     }
 }
 
-template <typename T>
-int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
+template <typename T, typename A>
+int upload(DevicePlan *dp, T **dst, const std::vector<T, A> &src, hipStream_t st)
 {
     const size_t bytes = (src.size() ? src.size() : 1) * sizeof(T);
     MPS_HIP_TRY(hipMalloc(reinterpret_cast<void **>(dst), bytes));
@@ -512,10 +512,10 @@ int upload(DevicePlan *dp, T **dst, const std::vector<T> &src, hipStream_t st)
     return MPS_OK;
 }
 
-template <typename T>
-void release(std::vector<T> &v)
+template <typename T, typename A>
+void release(std::vector<T, A> &v)
 {
-    std::vector<T>().swap(v);
+    std::vector<T, A>().swap(v);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

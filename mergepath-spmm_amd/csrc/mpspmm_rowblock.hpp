@@ -51,7 +51,9 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include <functional>
+#include <new>
 #include <vector>
 
 namespace mps_rb {
@@ -83,6 +85,39 @@ constexpr int kPackedPieceBits = 5;
 constexpr uint32_t kPackedAdvMax = (1u << (2 * kPackedPieceBits)) - 1u;
 constexpr int kPackedRoundWords = 64 * 3;
 
+// A vector whose resize() hands out zeroed memory without writing to it: large blocks come from the system as
+// untouched zero pages, which the builder's threads then touch as they fill them, instead of one thread writing
+// zeros over tens of megabytes first.  (An Entry of zero bytes is {word 0, value 0.f}: the padding.)
+template <typename T>
+struct ZeroPages {
+    using value_type = T;
+    template <typename U>
+    struct rebind {
+        using other = ZeroPages<U>;
+    };
+    ZeroPages() = default;
+    template <typename U>
+    ZeroPages(const ZeroPages<U> &) {}
+    T *allocate(size_t count)
+    {
+        void *p = std::calloc(count ? count : 1, sizeof(T));
+        if (!p) throw std::bad_alloc();
+        return static_cast<T *>(p);
+    }
+    void deallocate(T *p, size_t) { std::free(p); }
+    template <typename U, typename... Args>
+    void construct(U *p, Args &&...args)
+    {
+        if constexpr (sizeof...(Args) > 0) ::new (static_cast<void *>(p)) U(static_cast<Args &&>(args)...);
+    }
+    template <typename U>
+    bool operator==(const ZeroPages<U> &) const { return true; }
+    template <typename U>
+    bool operator!=(const ZeroPages<U> &) const { return false; }
+};
+template <typename T>
+using Zeroed = std::vector<T, ZeroPages<T>>;
+
 struct Layout {
     int n = 0, nnz = 0, K = 16;
     int steps = 0;        // T
@@ -99,10 +134,10 @@ struct Layout {
     std::vector<int> table_used;        // [NB] local tables: rows of the block's last table that its entries refer to (the rest is not loaded)
     std::vector<int> meta;              // [NB][T][16][4] {hot entries, cold entries, first local row, 0}; [..][15] unused
     std::vector<long long> wave_base;   // [NB * 16][2] first round of the wavefront's hot / cold stream; [..][15]: where the block's streams end
-    std::vector<Entry> hot, cold;       // rounds of 64 entries
+    Zeroed<Entry> hot, cold;            // rounds of 64 entries
     std::vector<int> hot_src, cold_src; // original nonzero index per entry slot, -1 = padding (optional)
-    std::vector<uint32_t> hot_packed;   // the hot stream in packed form
-    std::vector<uint32_t> cold_packed;  // the cold stream in packed form; empty if it does not fit (see pack_cold_stream)
+    Zeroed<uint32_t> hot_packed;        // the hot stream in packed form
+    Zeroed<uint32_t> cold_packed;       // the cold stream in packed form; empty if it does not fit (see pack_cold_stream)
     int cold_index_bits = 0;            // of a packed cold entry's 16 bits, those of the column (counted from cold_begin[t])
 };
 

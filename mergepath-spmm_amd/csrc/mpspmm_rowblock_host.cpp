@@ -210,20 +210,41 @@ int plan_columns(const int *rp, const int *ci, int n, int nnz, const BuildParams
 {
     // ---- 3. nonzeros per column; the steps; hot columns by rank, cold columns by id range
     auto d_of = [&](int c) { return deg[(size_t)c]; };
+    // the columns that hold nonzeros, busiest first, equally busy ones by id
     std::vector<int> cand;
-    cand.reserve((size_t)n);
-    for (int c = 0; c < n; ++c)
-        if (d_of(c) > 0) cand.push_back(c);
     auto hotter = [&](int a, int b) {
         const int da = d_of(a), db = d_of(b);
         return da != db ? da > db : a < b;
     };
+    int most = 0;
+    for (int c = 0; c < n; ++c) most = std::max(most, d_of(c));
+    const bool counted = (long long)most <= 4ll * n + 1024;  // one bucket per count: all of them in order, in two passes
+    if (counted) {
+        std::vector<int> first((size_t)most + 2, 0);  // first[d]: where the columns with d nonzeros start
+        for (int c = 0; c < n; ++c)
+            if (d_of(c) > 0) ++first[(size_t)d_of(c)];
+        int at = 0;
+        for (int d = most; d >= 1; --d) {
+            const int here = first[(size_t)d];
+            first[(size_t)d] = at;
+            at += here;
+        }
+        cand.resize((size_t)at);
+        for (int c = 0; c < n; ++c)
+            if (d_of(c) > 0) cand[(size_t)first[(size_t)d_of(c)]++] = c;
+    } else {
+        cand.reserve((size_t)n);
+        for (int c = 0; c < n; ++c)
+            if (d_of(c) > 0) cand.push_back(c);
+    }
     // what every further table would serve, for as many tables as a plan may get
     constexpr int kMostTables = 32;
     long long table_nnz[kMostTables] = {0};
     const size_t top = std::min<size_t>((size_t)kMostTables * H, cand.size());
-    if (top < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)top, cand.end(), hotter);
-    std::sort(cand.begin(), cand.begin() + (long)top, hotter);
+    if (!counted) {
+        if (top < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)top, cand.end(), hotter);
+        std::sort(cand.begin(), cand.begin() + (long)top, hotter);
+    }
     for (size_t k = 0; k < top; ++k) table_nnz[k / (size_t)H] += d_of(cand[k]);
     int T = bp.steps;
     if (T <= 0) T = default_steps(n, nnz, H, L.num_blocks, table_nnz, (int)((top + (size_t)H - 1) / (size_t)H));
@@ -248,18 +269,33 @@ int plan_columns(const int *rp, const int *ci, int n, int nnz, const BuildParams
         // T H columns holds the most of the block's nonzeros.  Worth it where the tables serve most of the
         // nonzeros; a wider band stays with the slab plans.
         if (bp.table_rows <= 0) H = std::min(H, (n + 3) / 4 * 4);
+        // a block's column indices in ascending order: counted where they span few columns (what local tables are
+        // for), sorted otherwise
+        auto columns_in_order = [&](int e0, int e1, std::vector<int> &cols, std::vector<int> &count) {
+            cols.clear();
+            if (e1 == e0) return;
+            const auto ends = std::minmax_element(ci + e0, ci + e1);
+            const int c_min = *ends.first;
+            const long long range = (long long)*ends.second - c_min + 1;
+            if (range <= 4ll * (e1 - e0) + 1024) {
+                count.assign((size_t)range, 0);
+                for (int e = e0; e < e1; ++e) ++count[(size_t)(ci[e] - c_min)];
+                cols.reserve((size_t)(e1 - e0));
+                for (long long c = 0; c < range; ++c) cols.insert(cols.end(), (size_t)count[(size_t)c], c_min + (int)c);
+            } else {
+                cols.assign(ci + e0, ci + e1);
+                std::sort(cols.begin(), cols.end());
+            }
+        };
         std::vector<int> span((size_t)L.num_blocks, 1);
-        parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
-            std::vector<int> cols;
+        parallel_for(L.num_blocks, 8, [&](int64_t b0, int64_t b1) {
+            std::vector<int> cols, count;
             for (int64_t b = b0; b < b1; ++b) {
                 const int e0 = rp[L.block_row[(size_t)b]], e1 = rp[L.block_row[(size_t)b + 1]];
                 if (e1 == e0) continue;
-                cols.assign(ci + e0, ci + e1);
+                columns_in_order(e0, e1, cols, count);
                 const size_t lo = cols.size() / 40, hi = cols.size() - 1 - cols.size() / 40;
-                std::nth_element(cols.begin(), cols.begin() + (long)lo, cols.end());
-                const int c_lo = cols[lo];
-                std::nth_element(cols.begin(), cols.begin() + (long)hi, cols.end());
-                span[(size_t)b] = cols[hi] - c_lo + 1;
+                span[(size_t)b] = cols[hi] - cols[lo] + 1;
             }
         });
         T = bp.steps;
@@ -273,12 +309,11 @@ int plan_columns(const int *rp, const int *ci, int n, int nnz, const BuildParams
         const long long W = (long long)T * H;
         L.table_base.assign((size_t)L.num_blocks, 0);
         std::atomic<long long> covered{0};
-        parallel_for(L.num_blocks, 1, [&](int64_t b0, int64_t b1) {
-            std::vector<int> cols;
+        parallel_for(L.num_blocks, 8, [&](int64_t b0, int64_t b1) {
+            std::vector<int> cols, count;
             for (int64_t b = b0; b < b1; ++b) {
                 const int e0 = rp[L.block_row[(size_t)b]], e1 = rp[L.block_row[(size_t)b + 1]];
-                cols.assign(ci + e0, ci + e1);
-                std::sort(cols.begin(), cols.end());
+                columns_in_order(e0, e1, cols, count);
                 size_t best = 0, best_at = 0;
                 for (size_t lo = 0, hi = 0; lo < cols.size(); ++lo) {
                     while (hi < cols.size() && cols[hi] < cols[lo] + W) ++hi;
@@ -314,8 +349,10 @@ int plan_columns(const int *rp, const int *ci, int n, int nnz, const BuildParams
     L.steps = T;
     L.hot_bits = bits_for(H > 1 ? H - 1 : 1);
     const size_t R = std::min<size_t>((size_t)T * H, cand.size());
-    if (R < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)R, cand.end(), hotter);
-    std::sort(cand.begin(), cand.begin() + (long)R, hotter);
+    if (!counted) {
+        if (R < cand.size()) std::nth_element(cand.begin(), cand.begin() + (long)R, cand.end(), hotter);
+        std::sort(cand.begin(), cand.begin() + (long)R, hotter);
+    }
     cm.step.assign((size_t)n, 0);
     cm.slot.assign((size_t)n, -1);
     L.hot_cols.assign((size_t)T * H, -1);
@@ -375,7 +412,7 @@ static void count_columns(const int *ci, int n, int nnz, std::vector<int> &deg)
 {
     std::vector<std::atomic<int>> cnt((size_t)n);
     for (auto &d : cnt) d.store(0, std::memory_order_relaxed);
-    parallel_for(nnz, 1 << 20, [&](int64_t a, int64_t b) {
+    parallel_for(nnz, 1 << 16, [&](int64_t a, int64_t b) {
         for (int64_t e = a; e < b; ++e) cnt[(size_t)ci[e]].fetch_add(1, std::memory_order_relaxed);
     });
     deg.resize((size_t)n);
@@ -453,12 +490,16 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     }
     L.hot_rounds = hr;
     L.cold_rounds = cr;
-    const Entry empty{0u, 0.f};
-    L.hot.assign((size_t)hr * kRoundEntries, empty);
-    L.cold.assign((size_t)cr * kRoundEntries, empty);
+    // (fresh vectors: what resize() hands out is zeroed memory only when it comes from the allocator)
+    Zeroed<Entry>().swap(L.hot);
+    Zeroed<Entry>().swap(L.cold);
+    L.hot.resize((size_t)hr * kRoundEntries);
+    L.cold.resize((size_t)cr * kRoundEntries);
     if (bp.keep_src) {
-        L.hot_src.assign(L.hot.size(), -1);
-        L.cold_src.assign(L.cold.size(), -1);
+        L.hot_src.resize(L.hot.size());
+        L.cold_src.resize(L.cold.size());
+        for (std::vector<int> *v : {&L.hot_src, &L.cold_src})
+            parallel_for((int64_t)v->size(), 1 << 16, [&](int64_t a, int64_t b) { std::fill(v->begin() + a, v->begin() + b, -1); });
     }
 
     // ---- 6. pass 2: place the entries
@@ -520,7 +561,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                             // round j / 2; inside it lane (g, e) holds entry e of the group's two windows side by side
                             const size_t dst = (size_t)(round_off[w][k] + j / kPair) * kRoundEntries + (size_t)g * kWin * kPair + (size_t)(j % kPair);
                             const int take = left < kWin ? left : kWin;
-                            std::vector<Entry> &out = k ? L.cold : L.hot;
+                            Zeroed<Entry> &out = k ? L.cold : L.hot;
                             for (int e = 0; e < kWin; ++e) {
                                 // padding repeats the window's last nonzero with value 0
                                 const size_t src = p + (size_t)(e < take ? e : take - 1);
@@ -553,6 +594,7 @@ bool pack_hot_stream(Layout &L)
     const size_t rounds = L.hot.size() / kRoundEntries;
     const uint32_t slot_mask = (1u << L.hot_bits) - 1u, piece_mask = (1u << kPackedPieceBits) - 1u;
     std::atomic<bool> fits{true};
+    Zeroed<uint32_t>().swap(L.hot_packed);
     L.hot_packed.resize(rounds * kPackedRoundWords);
     parallel_for((int64_t)rounds, 256, [&](int64_t r0, int64_t r1) {
         for (int64_t r = r0; r < r1; ++r)
@@ -590,7 +632,8 @@ bool pack_cold_stream(Layout &L)
     const uint32_t idx_mask = (1u << L.cold_bits) - 1u, piece_mask = (1u << pb) - 1u;
     const uint32_t adv_max = pb * kWin >= 32 ? 0xffffffffu : (1u << (pb * kWin)) - 1u;
     std::atomic<bool> fits{true};
-    L.cold_packed.assign((size_t)L.cold_rounds * kPackedRoundWords, 0u);
+    Zeroed<uint32_t>().swap(L.cold_packed);
+    L.cold_packed.resize((size_t)L.cold_rounds * kPackedRoundWords);
     parallel_for(NB, 1, [&](int64_t b0, int64_t b1) {
         for (int64_t b = b0; b < b1; ++b)
             for (int w = 0; w < kWaves; ++w) {
@@ -627,7 +670,7 @@ bool pack_cold_stream(Layout &L)
             }
     });
     if (!fits.load()) {
-        std::vector<uint32_t>().swap(L.cold_packed);
+        Zeroed<uint32_t>().swap(L.cold_packed);
         return false;
     }
     L.cold_index_bits = ib;
