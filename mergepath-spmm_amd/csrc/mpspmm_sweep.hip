@@ -415,7 +415,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
         if (e == hipSuccess) e = hipStreamSynchronize(st);
         if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
         if (rp[0] != 0 || rp[(size_t)n] != nnz) return fail(MPS_ERR_INVALID_CSR);
-        std::vector<ListedRow> listed_rows;
+        Bulk<ListedRow> listed_rows;
         rc = plan_panels(rp.data(), n, nnz, K, bp, dp->host, listed_rows);
         if (rc != MPS_OK) return fail(rc);
         // (an X of 4 GiB or more is read through pointers, with nothing to catch the lane that reads past the end of

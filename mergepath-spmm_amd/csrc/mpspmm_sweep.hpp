@@ -127,9 +127,9 @@ struct ListedRow {
 // The builder in two parts.  plan_panels: everything that needs row_ptr alone (panels, rows cut across panels, listed
 // rows, accumulator rows); it fills the small tables of `out` except wave_meta and panel_rounds.  build_streams: the
 // passes over the nonzeros (accumulator rows to wavefronts, entries by column, list scheduling, the stream).
-int plan_panels(const int *row_ptr, int n, int nnz, int K, const BuildParams &bp, Layout &out, std::vector<ListedRow> &listed_rows);
+int plan_panels(const int *row_ptr, int n, int nnz, int K, const BuildParams &bp, Layout &out, Bulk<ListedRow> &listed_rows);
 int build_streams(const int *row_ptr, const int *col_idx, const float *val, const BuildParams &bp, Layout &out,
-                  const std::vector<ListedRow> &listed_rows);
+                  const Bulk<ListedRow> &listed_rows);
 
 // Host arrays in, layout out.  Returns an mps_status (MPS_ERR_UNSUPPORTED for a row of X that is not a multiple of
 // 64 bytes or a matrix whose column ids leave no room for the accumulator row in an entry word).
@@ -153,7 +153,7 @@ struct DeviceStreams {
     size_t slots = 0, bytes = 0;
 };
 int build_streams_on_device(const int *d_row_ptr, const int *d_col_idx, const float *d_val, const BuildParams &bp, Layout &out,
-                            const std::vector<ListedRow> &listed_rows, hipStream_t st, DeviceStreams *ds);
+                            const Bulk<ListedRow> &listed_rows, hipStream_t st, DeviceStreams *ds);
 int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n, int nnz, int K, const BuildParams &bp,
            hipStream_t st, DevicePlan **out);
 void destroy(DevicePlan *dp);

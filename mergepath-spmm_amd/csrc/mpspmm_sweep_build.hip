@@ -241,7 +241,7 @@ __global__ __launch_bounds__(256) void swb_emit_kernel(const unsigned long long 
 }  // namespace
 
 int build_streams_on_device(const int *d_rp, const int *d_ci, const float *d_val, const BuildParams &bp, Layout &out,
-                            const std::vector<ListedRow> &listed_rows, hipStream_t st, DeviceStreams *ds)
+                            const Bulk<ListedRow> &listed_rows, hipStream_t st, DeviceStreams *ds)
 {
     const int NP = out.num_panels, L = out.lanes, gpw = 64 / L, together = out.together;
     const int group_slots = gpw * together, groups_per_round = kRoundInstr / together, words_per_round = gpw * kWin * 4;

@@ -135,7 +135,7 @@ bool deal_largest_first(const std::vector<int> &order, Size size_of, Cost cost_o
 
 }  // namespace
 
-int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Layout &out, std::vector<ListedRow> &listed_rows)
+int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Layout &out, Bulk<ListedRow> &listed_rows)
 {
     if (n < 1 || nnz < 0 || K < 1 || !rp) return MPS_ERR_INVALID_ARG;
     if (bp.elem_bytes != 4 && bp.elem_bytes != 2) return MPS_ERR_INVALID_ARG;
@@ -177,7 +177,7 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
     auto deg = [&](int r) { return (long long)rp[r + 1] - rp[r]; };
 
     // ---- panels: how many, how rows are cut, which row goes where
-    std::vector<Item> items;
+    Bulk<Item> items;  // (filled chunk by chunk on all threads: not zeroed first)
     std::vector<int> item_panel, order;  // order: the items that hold nonzeros, largest first
     std::vector<int> split_of((size_t)n, 0);  // sub-rows of a row (0: not split)
     int NP = 0, piece = 0;
@@ -288,7 +288,14 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
                     out.split_row.push_back(r);
                     out.split_ptr.push_back(out.split_ptr.back() + split_of[(size_t)r]);
                 }
-            for (const Item &it : items) totv += it.pieces;
+            std::atomic<long long> pieces{0};
+            mps_host::parallel_for(chunks, 1, [&](int64_t c0, int64_t c1) {
+                long long mine = 0;
+                for (int64_t c = c0; c < c1; ++c)
+                    for (const Item &it : chunk_items[(size_t)c]) mine += it.pieces;
+                pieces.fetch_add(mine, std::memory_order_relaxed);
+            });
+            totv = pieces.load();
         }
         if (totv > (long long)NP * vcap) continue;
         order = largest_first((int)items.size(), [&](int i) { return items[(size_t)i].nnz; });
@@ -404,7 +411,7 @@ int plan_panels(const int *rp, int n, int nnz, int K, const BuildParams &bp, Lay
 }
 
 int build_streams(const int *rp, const int *ci, const float *val, const BuildParams &bp, Layout &out,
-                  const std::vector<ListedRow> &listed_rows)
+                  const Bulk<ListedRow> &listed_rows)
 {
     if (out.nnz > 0 && (!ci || !val)) return MPS_ERR_INVALID_ARG;
     const int NP = out.num_panels, L = out.lanes, G = out.bank_rows, gpw = 64 / L, together = out.together, piece = out.piece;
@@ -543,7 +550,7 @@ int build_streams(const int *rp, const int *ci, const float *val, const BuildPar
 int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz, int K, const BuildParams &bp, Layout &out)
 {
     if (nnz > 0 && (!ci || !val)) return MPS_ERR_INVALID_ARG;
-    std::vector<ListedRow> listed_rows;
+    Bulk<ListedRow> listed_rows;
     const int rc = plan_panels(rp, n, nnz, K, bp, out, listed_rows);
     return rc != MPS_OK ? rc : build_streams(rp, ci, val, bp, out, listed_rows);
 }
