@@ -216,6 +216,30 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
         const int cs1 = cold_ib - (16 - cold_ib), cs2 = cold_ib - 2 * (16 - cold_ib), cs3 = cold_ib - 3 * (16 - cold_ib);
         asm volatile("" : "+v"(hmask), "+v"(cmask), "+v"(hot_hi), "+v"(cold_hi));
         int4 m = meta_b[wave];
+        // a round of the hot stream: 768 bytes (packed), of the cold stream: 1 KiB
+        constexpr unsigned kHotRoundBytes = kPackedRoundWords * 4u;
+        constexpr unsigned kColdRoundBytes = CPACK ? kHotRoundBytes : 1024u;
+        // A step's streams on their way into L2 before the step is walked: one dword of every 128-byte line (the first
+        // 64 lines of each stream: ten rounds), asked for between two walks, where the L1 has nothing else to ask
+        // for, with plain loads; the walk then finds its rounds a cache away instead of in HBM, and its own loads of
+        // them are the last use.  A wavefront's loads return in order and a line from HBM holds one of the L1's
+        // ~64 request slots four to six times as long as a gather that hits L2: asked for during the walk, the
+        // stream lines held half of the slot time.  Measured on MI355X, 232,965-row power-law matrix, ms per
+        // product: none 0.418; the first 2, 3, 5, 7, 8, 10, 12, 16 rounds of the next step 0.430, 0.421, 0.412,
+        // 0.398, 0.393, 0.389, 0.398, 0.398 (a few rounds cost the wait for them and gain little; all rounds of all
+        // wavefronts are more than an XCD's L2 holds beside the step's rows of X); with the streaming hint on the
+        // requests themselves 0.457; the same ahead of the first step as well: +0.003.
+        auto request_ahead = [&](long long at_h, long long at_c, int nh2, int nc2) {
+            const int lines_h = min(rounds_of(nh2) * (int)(kHotRoundBytes / 128u), 64);
+            const int lines_c = min(rounds_of(nc2) * (int)(kColdRoundBytes / 128u), 64);
+            const __amdgpu_buffer_rsrc_t hp2 = stream_rsrc(hot + (size_t)at_h * kPackedRoundWords);
+            const __amdgpu_buffer_rsrc_t cp2 = CPACK ? stream_rsrc(cold_p + (size_t)at_c * kPackedRoundWords)
+                                                     : stream_rsrc(cold + (size_t)at_c * kRoundEntries);
+            unsigned a0 = 0, a1 = 0;
+            if (lane < lines_h) a0 = __builtin_amdgcn_raw_buffer_load_b32(hp2, lane * 128, 0, 0);
+            if (lane < lines_c) a1 = __builtin_amdgcn_raw_buffer_load_b32(cp2, lane * 128, 0, 0);
+            return a0 ^ a1;
+        };
         __syncthreads();
 
         for (int t = 0; t < T; ++t) {
@@ -302,14 +326,11 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             constexpr std::false_type kCold{};
 
             const bool keep = t >= keep_from;
-            // a round of the hot stream: 768 bytes (packed), of the cold stream: 1 KiB
-            constexpr unsigned kHotRoundBytes = kPackedRoundWords * 4u;
             const __amdgpu_buffer_rsrc_t hp = stream_rsrc(hot + (size_t)cur_h * kPackedRoundWords);
             const unsigned hoff = (unsigned)lane * 12u;
             auto load_hot = [&](int r) { return load_round_packed(hp, hoff + (unsigned)r * kHotRoundBytes, keep); };
             const __amdgpu_buffer_rsrc_t cp = CPACK ? stream_rsrc(cold_p + (size_t)cur_c * kPackedRoundWords)
                                                     : stream_rsrc(cold + (size_t)cur_c * kRoundEntries);
-            constexpr unsigned kColdRoundBytes = CPACK ? kHotRoundBytes : 1024u;
             const unsigned loff = (unsigned)lane * (CPACK ? 12u : 16u);
             auto load_cold = [&](int r) {
                 if constexpr (CPACK) return load_round_packed(cp, loff + (unsigned)r * kColdRoundBytes, keep);
@@ -462,6 +483,9 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
             }
             RB_PRE_LOAD(0) RB_PRE_LOAD(1) RB_PRE_LOAD(2) RB_PRE_LOAD(3) RB_PRE_LOAD(4) RB_PRE_LOAD(5)
             m = m_next;
+            // the next step's streams: on their way like the table
+            unsigned ahead = 0;
+            if (t + 1 < T) ahead = request_ahead(cur_h, cur_c, __builtin_amdgcn_readfirstlane(m.x), __builtin_amdgcn_readfirstlane(m.y));
 
             __syncthreads();  // every gather from this step's table and every add of this step is done
             if (wave == 0) {
@@ -488,6 +512,7 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 RB_PRE_STORE(0) RB_PRE_STORE(1) RB_PRE_STORE(2) RB_PRE_STORE(3) RB_PRE_STORE(4) RB_PRE_STORE(5)
             }
             __syncthreads();
+            asm volatile("" ::"v"(ahead));  // (what keeps the requests: their dwords are of no use)
         }
     }
 #undef RB_PRE_LOAD
@@ -1059,17 +1084,21 @@ int create(const int *d_row_ptr, const int *d_col_idx, const float *d_val, int n
     dp->cold_slots = (size_t)L.cold_rounds * kRoundEntries;
     const bool cold_is_packed = on_device ? dp->cold_packed != nullptr : !L.cold_packed.empty();
     {
-        // The streams of the last steps, as many as fit kStreamKeepBytes, are read with plain loads and so stay in
-        // the 256 MiB last-level cache from one product to the next; all others carry the streaming hint and pass
-        // it by.  A product reads a plan once, front to back: left to itself the cache would hold the end of the
-        // previous pass and lose it again before the next pass gets there.  Measured on MI355X, 232,965-row
-        // power-law matrix, 1.07 GB of streams in 16 steps of 67 MB: 0, 2, 3, 4, 5, 16 steps kept: 0.500, 0.482,
-        // 0.484, 0.493, 0.503, 0.516 ms per product; with both streams packed, 16 steps of 50 MB: 2, 3, 4, 5 steps
-        // kept: 0.435, 0.4285, 0.432, 0.442 ms.
+        // Streams that fit the 256 MiB last-level cache (kStreamKeepBytes of them, from the last step backwards) are
+        // read with plain loads and so stay there from one product to the next; all others carry the streaming hint
+        // and pass it by.  A product reads a plan once, front to back: left to itself the cache would hold the end of
+        // the previous pass and lose it again before the next pass gets there.  Streams of more than twice that size
+        // are not kept at all: every step's lines are asked for ahead of its walk (request_ahead in the kernel), which
+        // serves the walk better than a cache that holds a fifth of them.  Measured on MI355X, ms per product, no
+        // step kept against kStreamKeepBytes kept: 232,965-row power-law matrix with 115 M nonzeros (803 MB of
+        // streams, 3 of 16 steps) 0.385 / 0.390; with 50 M nonzeros (351 MB) 0.2165 / 0.2163; with 20 M (140 MB, all
+        // kept) 0.1218 / 0.1184; R-MAT scale 20 (130 MB, all kept) 0.194 / 0.187.  (Before the lines were asked for
+        // ahead, the 115 M-nonzero matrix ran at 0.435, 0.4285, 0.432, 0.442 ms with 2, 3, 4, 5 steps kept.)
         const size_t hot_bytes = (size_t)L.hot_rounds * kPackedRoundWords * sizeof(uint32_t);
         const size_t cold_bytes = cold_is_packed ? (size_t)L.cold_rounds * kPackedRoundWords * sizeof(uint32_t) : dp->cold_slots * sizeof(Entry);
         const size_t per_step = (hot_bytes + cold_bytes) / (size_t)(L.steps > 0 ? L.steps : 1);
-        const size_t keep = per_step > 0 ? kStreamKeepBytes / per_step : (size_t)L.steps;
+        size_t keep = per_step > 0 ? kStreamKeepBytes / per_step : (size_t)L.steps;
+        if (hot_bytes + cold_bytes > 2 * kStreamKeepBytes) keep = 0;
         dp->keep_from = keep >= (size_t)L.steps ? 0 : L.steps - (int)keep;
     }
     if (!on_device) {
