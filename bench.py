@@ -360,9 +360,10 @@ def main():
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     orc = None if args.no_cpu else entry.load_oracle()
 
-    def run(wl, wname, steps, warmup, plain=False, graph=False, cpu_loop=None, defer_check=False, **overrides):
-        """One workload with one kind of plan: exactly `steps` timed products after `warmup`, then the per-kernel
-        durations, the counter readings on file for that plan shape, and the check against the fp64 row loop."""
+    def prepare(wl, plain=False, **overrides):
+        """The per-matrix preprocessing for one kind of plan, and how long it takes (a second plan of the same kind,
+        built and timed before any product and before the check against the CPU loops, whose OpenMP threads keep
+        spinning for a while after their loop and would share the cores with the builder's)."""
         plan, sched = None, None
         cost = args.cost if args.cost > 0 else sp.default_cost(wl.n, wl.nnz, wl.K, wl.eb)
         if plain:
@@ -370,17 +371,21 @@ def main():
         else:
             plan, cost = make_plan(wl, **overrides)
         torch.cuda.synchronize()
-        info = plan.info if plan is not None else None
-        # preprocessing time (once per matrix, not part of a step): a second plan of the same kind, built and timed
-        # before any product and before the check against the CPU loops, whose OpenMP threads keep spinning for a
-        # while after their loop and would share the cores with the builder's
         t1 = time.perf_counter()
         if plan is not None:
             make_plan(wl, **overrides)[0].close()
         else:
             sp.generate_mp_sched(wl.csr.row_ptr, wl.nnz, cost=cost)
         torch.cuda.synchronize()
-        preprocessing_ms = round((time.perf_counter() - t1) * 1e3, 3)
+        return plan, sched, cost, round((time.perf_counter() - t1) * 1e3, 3)
+
+    def measure(wl, wname, prepared, steps, warmup, graph=False, cpu_loop=None, defer_check=False, busy_ms=0.0):
+        """One workload with one prepared plan: exactly `steps` timed products after `warmup` untimed ones, then the
+        per-kernel durations, the counter readings on file for that plan shape, and the check against the fp64 row
+        loop.  busy_ms: the untimed products go on, ten at a time, until the device has worked that long - a GPU that
+        idled for some tens of milliseconds needs about 30 ms of work before its clocks are back up."""
+        plan, sched, cost, preprocessing_ms = prepared
+        info = plan.info if plan is not None else None
 
         def step(phases=None):
             if plan is not None:
@@ -388,8 +393,14 @@ def main():
             else:
                 sp.spmm_merge_path(wl.csr, wl.d_X, sched, threads_per_wave=args.tpw, out=wl.d_Y, phases=phases)
 
-        for _ in range(warmup):
-            step()
+        warmed = 0
+        t_busy = time.perf_counter()
+        while warmed < warmup or (time.perf_counter() - t_busy) * 1e3 < busy_ms:
+            for _ in range(min(10, warmup - warmed) if warmed < warmup else 10):
+                step()
+                warmed += 1
+            if busy_ms > 0.0:
+                torch.cuda.synchronize()
         timed_step = step
         if graph:
             torch.cuda.synchronize()
@@ -415,6 +426,7 @@ def main():
         traffic, l2_hit, where, gather_hit = measured_counters(desc["plan_signature"], with_requests=True,
                                                                other_lines=lines_read_once(wl, info))
         res = {"ms_per_step": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5), "gflops": round(wl.flops / (ms * 1e6), 2),
+               "steps": steps, "warmup": warmed,
                "kernel_ms": kernel_ms, "main_kernel": main_name,
                "phases": {k.lower(): v for k, v in kernels.items()},  # the kernel each phase launches; null: nothing
                "frac_step": round(wl.b_alg / (ms * 1e6) / PEAK_HBM_GBS, 4),
@@ -424,18 +436,33 @@ def main():
         res.update(desc)
         res["preprocessing_ms"] = preprocessing_ms
         if orc is not None:
-            Y_step = wl.d_Y.float().cpu().numpy()
             if defer_check:
-                res["_Y"] = Y_step  # the caller checks it, once the CPU loops have run
+                res["_Y"] = wl.d_Y.clone()  # the caller checks it later; the device is not kept waiting for a copy to the host
             else:
-                res["check"] = check_product(np, orc, wl, Y_step, cpu_loop)
+                res["check"] = check_product(np, orc, wl, wl.d_Y.float().cpu().numpy(), cpu_loop)
         if plan is not None:
             plan.close()
         return res
 
+    def run(wl, wname, steps, warmup, plain=False, **kw):
+        overrides = {k: kw.pop(k) for k in list(kw) if k not in ("graph", "cpu_loop", "defer_check", "busy_ms")}
+        return measure(wl, wname, prepare(wl, plain=plain, **overrides), steps, warmup, **kw)
+
+    with_configs = not args.no_configs and not custom and args.workload == HEADLINE
+    steps_c, warm_c = min(args.steps, 30), min(args.warmup, 10)
+    kBusyMs = 40.0  # configurations beside the headline: untimed products for at least this long
     # The GPU's run first: the CPU baseline below keeps the host busy for ten seconds, during which an idle GPU drops
     # its clocks, and the products that follow would be timed while they come back up.
-    head = run(w, name, args.steps, args.warmup, plain=args.mode == "plain", graph=args.graph, defer_check=True)
+    # And of the two plans of the headline matrix the merge-path slab plan first (partitioner, LDS-staged windows,
+    # carry-out fix-up: a `configs` entry), the library's own plan straight after it: both are prepared before either is
+    # timed, so that the headline's `--warmup` products find a device that is already at work, as every later product
+    # of a caller's loop does.
+    head_prepared = prepare(w, plain=args.mode == "plain")
+    slab_row = None
+    if with_configs:
+        r = measure(w, name, prepare(w, rowblock="off", sweep="off"), steps_c, warm_c, defer_check=True, busy_ms=kBusyMs)
+        slab_row = dict({"workload": name + "|slab", "n_rows": int(w.n), "nnz": int(w.nnz), "K": K, "dtype": dt}, **r)
+    head = measure(w, name, head_prepared, args.steps, args.warmup, graph=args.graph, defer_check=True)
     cpu = None
     Yc = None
     if orc is not None:
@@ -458,7 +485,9 @@ def main():
                "kind": "port", "sample": "%d full passes over the same workload, %.3f s each" % (passes, cpu_s)}
 
     if orc is not None:
-        head["check"] = check_product(np, orc, w, head.pop("_Y"), Yc)
+        head["check"] = check_product(np, orc, w, head.pop("_Y").float().cpu().numpy(), Yc)
+        if slab_row is not None:
+            slab_row["check"] = check_product(np, orc, w, slab_row.pop("_Y").float().cpu().numpy(), None)
     achieved = w.b_alg / (head["kernel_ms"][head["main_kernel"]] * 1e6)
     out = {
         "metric": "SpMM GFLOP/s (2*nnz*K/t), merge-path CSR x row-major dense",
@@ -499,19 +528,16 @@ def main():
         out["check_vs_cpu_fp32"] = head["check"]
         ok = head["check"]["ok"]
 
-    if not args.no_configs and not custom and args.workload == HEADLINE:
-        # the other configurations of the benchmark, each with the library's own plan and the same timed loop; first
-        # the headline graph once more with the merge-path slab plan (partitioner, LDS-staged windows, carry-out fix-up)
-        rows = []
-        steps_c, warm_c = min(args.steps, 30), min(args.warmup, 10)
-        r = run(w, name, steps_c, warm_c, rowblock="off", sweep="off")
-        rows.append(dict({"workload": name + "|slab", "n_rows": int(w.n), "nnz": int(w.nnz), "K": K, "dtype": dt}, **r))
+    if with_configs:
+        # the other configurations of the benchmark, each with the library's own plan and the same timed loop, after
+        # the headline graph's slab plan from above
+        rows = [slab_row]
         del w
         torch.cuda.empty_cache()
         for cname in OTHER_CONFIGS:
             cspec, cK, cdt = WORKLOADS[cname]
             wl = Workload(pkg, cname, cspec, cK, cdt, args.seed, torch, dev)
-            r = run(wl, cname, steps_c, warm_c)
+            r = run(wl, cname, steps_c, warm_c, busy_ms=kBusyMs)
             rows.append(dict({"workload": cname, "n_rows": int(wl.n), "nnz": int(wl.nnz), "K": cK, "dtype": cdt}, **r))
             del wl
             torch.cuda.empty_cache()
@@ -521,8 +547,11 @@ def main():
                 ok = ok and r["check"]["ok"]
         out["configs"] = rows
         out["configs_note"] = ("frac = algorithmic bytes / whole-step time / 8 TB/s, frac_main_kernel the same over the main "
-                               "kernel's time; %d steps after %d warm-ups each; kernel_ms: a phase that launches nothing has "
-                               "no entry; traffic and l2_hit_rate from the counter runs under profiles/" % (steps_c, warm_c))
+                               "kernel's time; %d steps each, after at least %d untimed ones and %d ms of them (`warmup` per entry: a GPU "
+                               "that idled needs about 30 ms of work before its clocks are back up); the slab plan of the "
+                               "headline matrix is timed before the headline's own warm-up; kernel_ms: a phase that "
+                               "launches nothing has no entry; traffic and l2_hit_rate from the counter runs under profiles/"
+                               % (steps_c, warm_c, int(kBusyMs)))
 
     print(json.dumps(out))
     if not ok:
