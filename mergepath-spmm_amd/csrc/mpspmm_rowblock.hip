@@ -367,7 +367,12 @@ __global__ __launch_bounds__(kThreads) void rb_spmm_kernel(const uint32_t *__res
                 // launched took 40 % longer for the same number of windows (55 against 39 thousand cycles per step
                 // on the 232,965-row power-law matrix), and 15 wavefronts waited for it at the barrier.  The
                 // priority goes round, a pass at each rank: 46 to 49 thousand cycles for all, the step 7 % shorter.
-                switch (((wave >> 2) + pass) & 3) {
+                // (Since the next step's stream lines are asked for after the walk, equal walks are no longer the aim:
+                // a wavefront that is done early has its lines on the way from HBM while the others still gather.
+                // Walks by launch rank, thousands of cycles, and ms per product: rank + pass 38 / 34 / 38 / 45 and
+                // 0.3835; rank - pass 39 / 37 / 38 / 37 and 0.387 - the evenest and not the fastest; rank + pass + 3,
+                // the highest priority to the oldest first, 34 / 42 / 39 / 41 and 0.3807.)
+                switch (((wave >> 2) + pass + 3) & 3) {
                 case 0: __builtin_amdgcn_s_setprio(0); break;
                 case 1: __builtin_amdgcn_s_setprio(1); break;
                 case 2: __builtin_amdgcn_s_setprio(2); break;
