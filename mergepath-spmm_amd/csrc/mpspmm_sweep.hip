@@ -110,6 +110,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     using P = Piece<T>;
     constexpr int GPW = 64 / L;        // lane-groups of a wavefront
     constexpr int RQ = GPW * kWin;     // 16-byte units of a round
+    constexpr int kSync = L == 4 ? 1 : kSyncRounds;  // a workgroup barrier every so many rounds
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int b = blockIdx.x, tile = blockIdx.y;
@@ -203,7 +204,22 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
             // Every few rounds the wavefronts of the workgroup wait for each other (the first time: for the zeroed
             // accumulators): left alone, the oldest wavefront of a SIMD runs ahead of the youngest by a third of the
             // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
-            if ((r & (kSyncRounds - 1)) == 0) __syncthreads();
+            // (64-byte rows: every round - R-MAT scale 20, fp32, K = 16, a barrier every 1 / 2 / 4 / 8 / 16 / 64 rounds:
+            // 0.117 / 0.122 / 0.125 / 0.130 / 0.136 / 0.147 ms per product; 128-byte tiles: every fourth - K = 32
+            // 0.162 / 0.161 / 0.158 / 0.166 / 0.173 / 0.190, K = 128 0.672 / 0.671 / 0.658 / 0.681 / 0.700 / 0.758)
+            if ((r & (kSync - 1)) == 0) __syncthreads();
+            // Between two barriers a SIMD would serve the oldest of its four wavefronts first in every round and the
+            // other three would arrive late together.  The priority goes round instead, a round at each rank, the
+            // youngest first (launch rank - round).  Measured on MI355X, R-MAT scale 20, fp32, ms per product without
+            // / with: K = 16 0.1277 / 0.1257, K = 32 0.1628 / 0.1579, K = 128 0.6857 / 0.6605; R-MAT scale 22, fp16,
+            // K = 64 0.916 / 0.915.  (rank + round: 0.126, 0.164, 0.682, 0.912; a step per two or four rounds, or the
+            // same rotation begun at another rank: between these and slower than none.)
+            switch (((wave >> 2) - r) & 3) {
+            case 0: __builtin_amdgcn_s_setprio(0); break;
+            case 1: __builtin_amdgcn_s_setprio(1); break;
+            case 2: __builtin_amdgcn_s_setprio(2); break;
+            default: __builtin_amdgcn_s_setprio(3); break;
+            }
             const uint4 cn = nx;
             nx = stream_load(min(r + 2, last));
             const unsigned cm = r < last ? cmask : 0u;  // (past the last round: row 0 of X, eight times)
@@ -231,7 +247,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
 #undef SW_FMA
 #undef SW_GATHER
     // the barriers of the rounds that other wavefronts of the panel still have, and the one before the sums are read
-    for (int r = (rounds + kSyncRounds - 1) & ~(kSyncRounds - 1); r < most; r += kSyncRounds) __syncthreads();
+    for (int r = (rounds + kSync - 1) & ~(kSync - 1); r < most; r += kSync) __syncthreads();
     __syncthreads();
 
     // the panel's rows, once: a row's pieces added up in order, rows without nonzeros as zeros
