@@ -592,7 +592,7 @@ __global__ __launch_bounds__(256) void rbb_ranges_kernel(const int *__restrict__
 // the nonzero is written to its place in the packed hot or cold stream (pass 2 of build_layout).
 struct PlaceArgs {
     const float *val;
-    const int *pre, *prevrow, *block_row, *meta, *run_start, *step_windows, *cold_begin;
+    const int *pre, *prevrow, *block_row, *meta, *run_start, *cuts, *cold_begin;
     const long long *round_off;
     uint32_t *hot, *cold;
     int *hot_src, *cold_src, *overflow;
@@ -663,10 +663,10 @@ __global__ __launch_bounds__(256) void rbb_rows_kernel(const int *__restrict__ r
             const int pk = (k ? pre_c : pre_h) + wi;  // windows of this kind before this one in the step
             const long long q = (long long)pre_h + pre_c + (k ? (cnt[gi] + kWin - 1) / kWin : 0) + wi;  // windows before it
             const size_t bt = (size_t)b * T + t;
-            const long long E = pa.step_windows[bt];
-            int w = (int)min(q * kWaves / E, (long long)(kWaves - 1));  // the run of window q: runs start at w E / 16
-            while (w > 0 && q < (long long)w * E / kWaves) --w;
-            while (q >= (long long)(w + 1) * E / kWaves) ++w;
+            const int *cut = pa.cuts + bt * (kWaves + 1);  // the run of window q: cut[w] <= q < cut[w + 1]
+            int w = (int)min(q * kWaves / cut[kWaves], (long long)(kWaves - 1));
+            while (w > 0 && q < cut[w]) --w;
+            while (q >= cut[w + 1]) ++w;
             const size_t run = bt * kWaveSlots + w;
             int g, j;
             deal(pa.meta[run * 4 + k], pk - pa.run_start[run * 2 + k], &g, &j);
@@ -757,15 +757,16 @@ __device__ __forceinline__ int block_max_before(int v, int *scratch)  // -1 wher
 }
 
 // One workgroup per (block, step), one thread per row of the block (pass 1 of build_layout, split_step): the windows
-// of kind k before every row (pre), the last row before it that has any (prevrow), the 16 equal runs (meta:
-// {hot windows, cold windows, first row, 0}; run_start: hot and cold windows of the step before the run), the step's
-// windows in all.
+// of kind k before every row (pre), the last row before it that has any (prevrow), the 16 runs (meta: {hot windows,
+// cold windows, first row, 0}; run_start: hot and cold windows of the step before the run; cuts: all windows of the
+// step before the run, and the step's windows in all as the 17th).
 __global__ __launch_bounds__(1024) void rbb_split_kernel(const int *__restrict__ cnt, const int *__restrict__ block_row, int n,
                                                           int T, int *__restrict__ pre, int *__restrict__ prevrow,
                                                           int *__restrict__ meta, int *__restrict__ run_start,
-                                                          int *__restrict__ step_windows)
+                                                          int *__restrict__ cuts)
 {
-    __shared__ int scratch[17], first_row[kWaves], hstart[kWaves + 1], cstart[kWaves + 1];
+    __shared__ int scratch[17], first_row[kWaves], hstart[kWaves + 1], cstart[kWaves + 1], cut[kWaves + 1];
+    __shared__ unsigned long long best;
     const int b = blockIdx.x / T, t = blockIdx.x % T, lr = threadIdx.x;
     const int r0 = block_row[b], nr = block_row[b + 1] - r0;
     const size_t gi = ((size_t)t * n + (size_t)(r0 + lr)) * 2;
@@ -783,27 +784,40 @@ __global__ __launch_bounds__(1024) void rbb_split_kernel(const int *__restrict__
         prevrow[gi] = ph;
         prevrow[gi + 1] = pc;
     }
-    if (lr < kWaves) {  // runs that find nothing left (a step without windows)
-        first_row[lr] = 0;
-        hstart[lr] = hot_total;
-        cstart[lr] = cold_total;
-    }
-    if (lr == 0) {
-        hstart[kWaves] = hot_total;
-        cstart[kWaves] = cold_total;
+    if (lr <= kWaves) {  // a step without windows: every run begins and ends at 0
+        if (lr < kWaves) first_row[lr] = 0;
+        hstart[lr] = lr < kWaves ? 0 : hot_total;
+        cstart[lr] = lr < kWaves ? 0 : cold_total;
+        cut[lr] = lr < kWaves ? 0 : hot_total + cold_total;
     }
     __syncthreads();
-    const long long E = (long long)hot_total + cold_total, q = (long long)hq + cq;
-    if (h + c > 0)
-        for (int w = 0; w < kWaves; ++w) {
-            const long long S = (long long)w * E / kWaves;
-            if (S < q || S >= q + h + c) continue;
-            const long long d = S - q;
+    // The cuts one after the other, as split_step makes them: every row looks at the places for the cut that lie
+    // among its own windows, the best key wins.
+    const long long E = (long long)hot_total + cold_total, q0 = (long long)hq + cq;
+    const long long slack = E / kWaves / kCutSlack;
+    for (int w = E > 0 ? 0 : kWaves; w < kWaves; ++w) {
+        const long long equal_cut = (long long)w * E / kWaves;
+        const long long lo = w == 0 ? 0 : max((long long)cut[w - 1], equal_cut - slack);
+        const long long hi = w == 0 ? 0 : min(equal_cut + slack, E - 1);
+        const int run_h = w == 0 ? 0 : hstart[w - 1], run_c = w == 0 ? 0 : cstart[w - 1];
+        if (lr == 0) best = ~0ull;
+        __syncthreads();
+        for (long long q = max(lo, q0); q <= min(hi, q0 + h + c - 1); ++q) {
+            const long long d = q - q0;
+            const int hot = d < h ? hq + (int)d : hq + h, cold = d < h ? cq : cq + (int)(d - h);
+            atomicMin(&best, cut_key(hot - run_h, cold - run_c, q, equal_cut));
+        }
+        __syncthreads();
+        const long long q = (long long)(best & 0xffffffffull);
+        if (q >= q0 && q < q0 + h + c) {  // the row that holds the cut
+            const long long d = q - q0;
+            cut[w] = (int)q;
             first_row[w] = lr;
             hstart[w] = d < h ? hq + (int)d : hq + h;
             cstart[w] = d < h ? cq : cq + (int)(d - h);
         }
-    __syncthreads();
+        __syncthreads();
+    }
     const size_t bt = (size_t)b * T + t;
     if (lr < kWaves) {
         int *m = meta + (bt * kWaveSlots + lr) * 4;
@@ -814,7 +828,7 @@ __global__ __launch_bounds__(1024) void rbb_split_kernel(const int *__restrict__
         run_start[(bt * kWaveSlots + lr) * 2] = hstart[lr];
         run_start[(bt * kWaveSlots + lr) * 2 + 1] = cstart[lr];
     }
-    if (lr == 0) step_windows[bt] = (int)E;
+    if (lr <= kWaves) cuts[bt * (kWaves + 1) + lr] = cut[lr];
 }
 
 // Device memory that lives for the length of a build
@@ -898,7 +912,7 @@ int build_on_device(const int *d_rp, const int *d_ci, const float *d_val, int n,
     if (ib > 15) return kNeedHost;
 
     // passes 1 and 2
-    Scratch d_step, d_slot, d_cnt, d_pre, d_prev, d_run_start, d_windows, d_round_off, d_flag;
+    Scratch d_step, d_slot, d_cnt, d_pre, d_prev, d_run_start, d_cuts, d_round_off, d_flag;
     const size_t groups = (size_t)T * (size_t)n * 2, runs = (size_t)NB * T * kWaveSlots;
     RBB_TRY(d_step.get((size_t)n * sizeof(int16_t)));
     RBB_TRY(d_slot.get((size_t)n * sizeof(int16_t)));
@@ -906,7 +920,7 @@ int build_on_device(const int *d_rp, const int *d_ci, const float *d_val, int n,
     RBB_TRY(d_pre.get(groups * sizeof(int)));
     RBB_TRY(d_prev.get(groups * sizeof(int)));
     RBB_TRY(d_run_start.get(runs * 2 * sizeof(int)));
-    RBB_TRY(d_windows.get((size_t)NB * T * sizeof(int)));
+    RBB_TRY(d_cuts.get((size_t)NB * T * (kWaves + 1) * sizeof(int)));
     RBB_TRY(d_round_off.get(runs * 2 * sizeof(long long)));
     RBB_TRY(d_flag.get(sizeof(int)));
     RBB_TRY(hipMemcpyAsync(d_step.p, cm.step.data(), (size_t)n * sizeof(int16_t), hipMemcpyHostToDevice, st));
@@ -920,7 +934,7 @@ int build_on_device(const int *d_rp, const int *d_ci, const float *d_val, int n,
     hipLaunchKernelGGL(rbb_rows_kernel<false>, row_grid, dim3(256), 0, st, d_rp, d_ci, d_step.as<int16_t>(), d_slot.as<int16_t>(), n,
                        T, d_cnt.as<int>(), pa);
     hipLaunchKernelGGL(rbb_split_kernel, dim3((unsigned)(NB * T)), dim3(1024), 0, st, d_cnt.as<int>(), dp->block_row, n, T,
-                       d_pre.as<int>(), d_prev.as<int>(), dp->meta, d_run_start.as<int>(), d_windows.as<int>());
+                       d_pre.as<int>(), d_prev.as<int>(), dp->meta, d_run_start.as<int>(), d_cuts.as<int>());
     L.meta.resize(runs * 4);
     RBB_TRY(hipMemcpyAsync(L.meta.data(), dp->meta, runs * 4 * sizeof(int), hipMemcpyDeviceToHost, st));
     RBB_TRY(hipStreamSynchronize(st));
@@ -969,7 +983,7 @@ int build_on_device(const int *d_rp, const int *d_ci, const float *d_val, int n,
     pa.block_row = dp->block_row;
     pa.meta = dp->meta;
     pa.run_start = d_run_start.as<int>();
-    pa.step_windows = d_windows.as<int>();
+    pa.cuts = d_cuts.as<int>();
     pa.cold_begin = dp->cold_begin;
     pa.round_off = d_round_off.as<long long>();
     pa.hot = dp->hot;

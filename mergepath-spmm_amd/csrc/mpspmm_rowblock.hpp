@@ -217,7 +217,25 @@ inline int bits_for(long long v)
     return b;
 }
 // rounds (two windows per lane-group each) that a wavefront needs for `windows` windows dealt to its 16 lane-groups
-inline int rounds_for(int windows) { return (windows / kGroups + (windows % kGroups != 0) + kPair - 1) / kPair; }
+MPS_RB_HD inline int rounds_for(int windows) { return (windows / kGroups + (windows % kGroups != 0) + kPair - 1) / kPair; }
+
+// Where the runs of a step are cut.  A step's E windows, in row order (a row's hot windows, then its cold ones), go
+// to the 16 wavefronts in runs of about E / 16; a run's hot and cold windows fill rounds of 32, and the last round of
+// either kind is walked and read like a full one however few windows it holds.  So run w begins not at w E / 16 but
+// at the window within kCutSlack of it (a fraction of a run's length, either side) that leaves the least padding in
+// the rounds of run w - 1; among equals the nearest to w E / 16, then the first.  (232,965-row power-law matrix, 16
+// steps: 6.5 % of the entry slots were padding of last rounds and 96 % of the runs had a partly filled round of
+// either kind with the cuts at w E / 16; 1.7 % and half of the runs with these.)  A step of fewer than 16 x
+// kCutSlack windows is cut at w E / 16.
+constexpr int kCutSlack = 8;  // the slack is 1 / kCutSlack of a run
+MPS_RB_HD inline int round_padding(int windows) { return rounds_for(windows) * (kGroups * kPair) - windows; }
+// what decides between two places for a cut: padding, then distance from the equal cut, then the place itself
+MPS_RB_HD inline unsigned long long cut_key(int hot_in_run, int cold_in_run, long long place, long long equal_cut)
+{
+    const long long away = place < equal_cut ? equal_cut - place : place - equal_cut;
+    return ((unsigned long long)(round_padding(hot_in_run) + round_padding(cold_in_run)) << 56) |
+           ((unsigned long long)away << 32) | (unsigned long long)place;
+}
 
 // Host arrays in, layout out.  Returns an mps_status.
 int build_layout(const int *row_ptr, const int *col_idx, const float *val, int n, int nnz, int K,

@@ -43,47 +43,64 @@ inline int windows_of(int entries) { return (entries + kWin - 1) / kWin; }
 struct StepSplit {
     int first_row[kWaves];
     int hstart[kWaves + 1], cstart[kWaves + 1];
+    int cut[kWaves + 1];  // windows of the step (hot and cold, row order) before the run
 };
 
 // cnt_t: [lr * 2 + kind] nonzeros of local row lr in this step (kind 0 hot, 1 cold).  The step's
-// windows in row order (a row's hot windows, then its cold ones) are cut into 16 equal runs.
-void split_step(const int *cnt_t, int nr, StepSplit &sp)
+// windows in row order (a row's hot windows, then its cold ones) are cut into 16 runs (see kCutSlack).
+void split_step(const int *cnt_t, int nr, StepSplit &sp, std::vector<int> &before)
 {
-    long long E = 0;
-    for (int i = 0; i < 2 * nr; ++i) E += windows_of(cnt_t[i]);
-    long long S[kWaves + 1];
-    for (int w = 0; w <= kWaves; ++w) S[w] = (long long)w * E / kWaves;
-    long long q = 0;
-    int hq = 0, cq = 0, wp = 0;
-    for (int lr = 0; lr < nr && wp < kWaves; ++lr) {
-        const int h = windows_of(cnt_t[2 * lr]), c = windows_of(cnt_t[2 * lr + 1]);
-        while (wp < kWaves && S[wp] < q + h + c) {
-            const long long d = S[wp] - q;
-            sp.first_row[wp] = lr;
-            if (d < h) {
-                sp.hstart[wp] = hq + (int)d;
-                sp.cstart[wp] = cq;
-            } else {
-                sp.hstart[wp] = hq + h;
-                sp.cstart[wp] = cq + (int)(d - h);
-            }
-            ++wp;
-        }
-        q += h + c;
-        hq += h;
-        cq += c;
-    }
-    // runs that start at the very end (nothing left for them)
+    // before[lr * 2 + kind]: windows of the kind in the rows before lr
+    before.resize((size_t)2 * nr + 2);
     int hot_total = 0, cold_total = 0;
     for (int lr = 0; lr < nr; ++lr) {
+        before[(size_t)2 * lr] = hot_total;
+        before[(size_t)2 * lr + 1] = cold_total;
         hot_total += windows_of(cnt_t[2 * lr]);
         cold_total += windows_of(cnt_t[2 * lr + 1]);
     }
-    for (; wp < kWaves; ++wp) {
-        sp.first_row[wp] = wp > 0 ? sp.first_row[wp - 1] : 0;
-        sp.hstart[wp] = hot_total;
-        sp.cstart[wp] = cold_total;
+    before[(size_t)2 * nr] = hot_total;
+    before[(size_t)2 * nr + 1] = cold_total;
+    const long long E = (long long)hot_total + cold_total;
+    // the row that holds window q of the step (q < E), and the hot and cold windows in front of q
+    int at = 0;  // (the cuts never go back: the search starts where the last one ended)
+    auto locate = [&](long long q, int *hot, int *cold) {
+        while ((long long)before[(size_t)2 * (at + 1)] + before[(size_t)2 * (at + 1) + 1] <= q) ++at;
+        const int hq = before[(size_t)2 * at], cq = before[(size_t)2 * at + 1], h = before[(size_t)2 * (at + 1)] - hq;
+        const long long d = q - hq - cq;
+        *hot = d < h ? hq + (int)d : hq + h;
+        *cold = d < h ? cq : cq + (int)(d - h);
+        return at;
+    };
+    const long long slack = E / kWaves / kCutSlack;
+    sp.cut[0] = 0;
+    sp.hstart[0] = sp.cstart[0] = 0;
+    sp.first_row[0] = 0;
+    if (E > 0) {
+        int h0, c0;
+        sp.first_row[0] = locate(0, &h0, &c0);
     }
+    for (int w = 1; w < kWaves; ++w) {
+        if (E == 0) {  // nothing to cut
+            sp.cut[w] = sp.hstart[w] = sp.cstart[w] = 0;
+            sp.first_row[w] = 0;
+            continue;
+        }
+        const long long equal_cut = (long long)w * E / kWaves;
+        const long long lo = std::max<long long>(sp.cut[w - 1], equal_cut - slack), hi = std::min(equal_cut + slack, E - 1);
+        unsigned long long best = ~0ull;
+        const int at0 = at;
+        for (long long q = lo; q <= hi; ++q) {
+            int hot, cold;
+            locate(q, &hot, &cold);
+            best = std::min(best, cut_key(hot - sp.hstart[w - 1], cold - sp.cstart[w - 1], q, equal_cut));
+        }
+        at = at0;
+        const long long q = (long long)(best & 0xffffffffull);
+        sp.cut[w] = (int)q;
+        sp.first_row[w] = locate(q, &sp.hstart[w], &sp.cstart[w]);
+    }
+    sp.cut[kWaves] = (int)E;
     sp.hstart[kWaves] = hot_total;
     sp.cstart[kWaves] = cold_total;
 }
@@ -459,14 +476,16 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
     const int NB = L.num_blocks;
     L.meta.assign((size_t)NB * T * kWaveSlots * 4, 0);
     std::vector<long long> rounds((size_t)NB * kWaveSlots * 2, 0);
+    std::vector<int> cuts((size_t)NB * T * (kWaves + 1));  // where the runs of every (block, step) begin
     parallel_for(NB, 1, [&](int64_t b0, int64_t b1) {
-        std::vector<int> cnt;
+        std::vector<int> cnt, before;
         for (int64_t b = b0; b < b1; ++b) {
             const int r0 = L.block_row[(size_t)b], nr = L.block_row[(size_t)b + 1] - r0;
             count_block(rp, ci, cm, (int)b, r0, nr, T, cnt);
             for (int t = 0; t < T; ++t) {
                 StepSplit sp;
-                split_step(cnt.data() + (size_t)t * nr * 2, nr, sp);
+                split_step(cnt.data() + (size_t)t * nr * 2, nr, sp, before);
+                std::copy(sp.cut, sp.cut + kWaves + 1, cuts.begin() + (ptrdiff_t)(((size_t)b * T + t) * (kWaves + 1)));
                 for (int w = 0; w < kWaves; ++w) {
                     int *m = &L.meta[(((size_t)b * T + t) * kWaveSlots + w) * 4];
                     m[0] = sp.hstart[w + 1] - sp.hstart[w];
@@ -535,10 +554,9 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
             for (int t = 0; t < T; ++t) {
                 const int *m0 = &L.meta[((size_t)b * T + t) * kWaveSlots * 4];
                 const int *cnt_t = cnt.data() + (size_t)t * nr * 2;
-                long long E = 0;
-                for (int i = 0; i < 2 * nr; ++i) E += windows_of(cnt_t[i]);
+                const int *cut = &cuts[((size_t)b * T + t) * (kWaves + 1)];
                 int w = 0;
-                long long w_end = E / kWaves;  // first window of run w + 1
+                long long w_end = cut[1];  // first window of run w + 1
                 int placed[2] = {0, 0}, last_row[2] = {0, 0};
                 long long q = 0;           // windows so far
                 size_t p = (size_t)t_begin[(size_t)t];  // sorted nonzeros so far
@@ -548,7 +566,7 @@ int build_layout(const int *rp, const int *ci, const float *val, int n, int nnz,
                         while (left > 0) {
                             while (q >= w_end) {
                                 ++w;
-                                w_end = (long long)(w + 1) * E / kWaves;
+                                w_end = cut[w + 1];
                                 placed[0] = placed[1] = 0;
                             }
                             const int *m = m0 + w * 4;

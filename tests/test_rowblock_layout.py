@@ -190,6 +190,67 @@ def test_layout_walk_reproduces_the_product(pkg, case):
                     r += 1
 
 
+def greedy_cuts(win, slack_div=8):
+    """The runs of one (block, step), restated: win[row, kind] windows in row order (a row's hot ones, then its cold
+    ones); run w begins within a run's length / slack_div of w E / 16, where the rounds of run w - 1 get the least
+    padding; among equals the nearest to w E / 16, then the first."""
+    kind = np.repeat(np.tile([0, 1], win.shape[0]), win.ravel())
+    E = kind.size
+    before = [np.concatenate([[0], np.cumsum(kind == k)]) for k in range(2)]
+    pad = lambda x: rounds_for(int(x)) * 32 - int(x)
+    slack = E // WAVES // slack_div
+    cuts = [0]
+    for w in range(1, WAVES):
+        equal = w * E // WAVES
+        if E == 0:
+            cuts.append(0)
+            continue
+        lo, hi = max(cuts[-1], equal - slack), min(equal + slack, E - 1)
+        cuts.append(min(range(lo, hi + 1), key=lambda q: (pad(before[0][q] - before[0][cuts[-1]]) +
+                                                           pad(before[1][q] - before[1][cuts[-1]]), abs(q - equal), q)))
+    cuts.append(E)
+    return [[int(before[k][cuts[w + 1]] - before[k][cuts[w]]) for k in range(2)] for w in range(WAVES)], cuts, E
+
+
+def test_runs_are_cut_where_their_last_rounds_fill(pkg):
+    C = pkg._cabi
+    rng = np.random.default_rng(77)
+    n, T, H = 1500, 6, 32
+    rp, ci = random_csr(rng, n, 300, p_empty=0.05, hub_rows=((3, 1400), (900, 1200)))
+    val = rng.random(ci.size).astype(np.float32)
+    lay = pkg.spmm.RowBlockLayout(rp, ci, val, K=16, steps=T, table_rows=H, block_rows=0, blocks_per_round=2, keep_sources=False)
+    i = lay.info
+    NB = i.rowblock_blocks
+    brow = lay.array(C.MPS_PLAN_ARRAY_RB_BLOCK_ROW, np.int32)
+    hot_cols = lay.array(C.MPS_PLAN_ARRAY_RB_HOT_COLS, np.int32).reshape(T, H)
+    cold_begin = lay.array(C.MPS_PLAN_ARRAY_RB_COLD_BEGIN, np.int32)
+    meta = lay.array(C.MPS_PLAN_ARRAY_RB_META, np.int32).reshape(NB, T, WSLOTS, 4)
+    col_step, col_hot = np.zeros(n, dtype=np.int64), np.zeros(n, dtype=bool)
+    for t in range(T):
+        col_step[cold_begin[t]:cold_begin[t + 1]] = t
+    for t in range(T):
+        c = hot_cols[t][hot_cols[t] >= 0]
+        col_step[c], col_hot[c] = t, True
+    moved, slots, slots_equal, windows = 0, 0, 0, 0
+    for b in range(NB):
+        r0, r1 = int(brow[b]), int(brow[b + 1])
+        rows = np.repeat(np.arange(r1 - r0), np.diff(rp[r0:r1 + 1]))
+        cols = ci[rp[r0]:rp[r1]]
+        key = (col_step[cols] * (r1 - r0) + rows) * 2 + (~col_hot[cols])
+        win = (np.bincount(key, minlength=T * (r1 - r0) * 2).reshape(T, r1 - r0, 2) + 3) // 4
+        for t in range(T):
+            want, cuts, E = greedy_cuts(win[t])
+            assert meta[b, t, :WAVES, :2].tolist() == want, (b, t)
+            assert all(abs(cuts[w] - w * E // WAVES) <= E // WAVES // 8 for w in range(WAVES + 1))
+            moved += sum(cuts[w] != w * E // WAVES for w in range(WAVES))
+            equal, _, _ = greedy_cuts(win[t], slack_div=10 ** 9)  # no slack: the cuts at w E / 16
+            slots += sum(rounds_for(x) * 32 for run in want for x in run)
+            slots_equal += sum(rounds_for(x) * 32 for run in equal for x in run)
+            windows += E
+    assert moved > NB * T * 8           # most cuts found a better place
+    assert slots - windows < 0.5 * (slots_equal - windows)   # and the last rounds hold less than half the padding
+
+
 def test_hot_columns_are_the_busiest_and_dealt_round_robin(pkg):
     rng = np.random.default_rng(3)
     n = 400
