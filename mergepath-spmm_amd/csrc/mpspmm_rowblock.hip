@@ -802,11 +802,13 @@ __global__ __launch_bounds__(1024) void rbb_split_kernel(const int *__restrict__
         const int run_h = w == 0 ? 0 : hstart[w - 1], run_c = w == 0 ? 0 : cstart[w - 1];
         if (lr == 0) best = ~0ull;
         __syncthreads();
+        unsigned long long mine = ~0ull;
         for (long long q = max(lo, q0); q <= min(hi, q0 + h + c - 1); ++q) {
             const long long d = q - q0;
             const int hot = d < h ? hq + (int)d : hq + h, cold = d < h ? cq : cq + (int)(d - h);
-            atomicMin(&best, cut_key(hot - run_h, cold - run_c, q, equal_cut));
+            mine = min(mine, cut_key(hot - run_h, cold - run_c, q, equal_cut));
         }
+        if (mine != ~0ull) atomicMin(&best, mine);
         __syncthreads();
         const long long q = (long long)(best & 0xffffffffull);
         if (q >= q0 && q < q0 + h + c) {  // the row that holds the cut
