@@ -334,7 +334,8 @@ int mps_spmm_f16_phases(const int *d_row_ptr, const int *d_col_idx, const uint16
  * kernel.  Columns are dealt to `steps` steps: the steps * table_rows columns
  * with the most nonzeros are gathered from a per-step LDS table of rows of X,
  * the others through L2, a contiguous range of column ids per step.  Inside a
- * (block, step) the nonzeros are cut into 16 equal runs (one per wavefront)
+ * (block, step) the nonzeros are cut into 16 runs of about equal length (one
+ * per wavefront; a cut lies where the run before it fills its last rounds)
  * and a wavefront's hot and cold nonzeros are each dealt evenly to its 16
  * lane-groups.  Results are deterministic.  The layout is built with the passes
  * over the nonzeros on the device (row_ptr and the nonzero counts of the

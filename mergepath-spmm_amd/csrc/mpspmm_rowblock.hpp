@@ -23,8 +23,8 @@
 //   * Within (block, step) the nonzeros are grouped into windows of 4 entries
 //     of one row (a row's last hot window and last cold window of the step
 //     are padded: value 0, the last index repeated).  The windows in row order
-//     (a row's hot ones, then its cold ones) are cut into 16 equal runs, one
-//     per wavefront; a wavefront's hot windows are then dealt evenly and in
+//     (a row's hot ones, then its cold ones) are cut into 16 runs of about
+//     equal length (see kCutSlack), one per wavefront; a wavefront's hot windows are then dealt evenly and in
 //     order to its 16 lane-groups, and so are its cold ones.  Every lane-group
 //     therefore walks two short streams (hot: LDS gathers, cold: L2 gathers)
 //     of the same length as its neighbours': no divergence.  A round of a
