@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     constexpr int GPW = 64 / L;        // lane-groups of a wavefront
     constexpr int RQ = GPW * kWin;     // 16-byte units of a round
     constexpr int kSync = L == 4 ? 1 : kSyncRounds;  // a workgroup barrier every so many rounds
-    constexpr bool kPairPrio = L == 8 && sizeof(T) == 2;  // the wavefronts' priorities move on with every pair of entries
+    constexpr bool kPairPrio = L == 8 && sizeof(T) == 2;  // the wavefronts' priorities move on with every entry of a round
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int b = blockIdx.x, tile = blockIdx.y;
@@ -215,9 +215,10 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
             // / with: K = 16 0.1277 / 0.1257, K = 32 0.1628 / 0.1579, K = 128 0.6857 / 0.6605; R-MAT scale 22, fp16,
             // K = 64 0.916 / 0.915.  (rank + round: 0.126, 0.164, 0.682, 0.912; a step per two or four rounds, or the
             // same rotation begun at another rank: between these and slower than none.)
-            // 128-byte tiles: the eight entries of a round are kept in four pairs that the compiler does not mix
-            // (fp32: K = 32 0.1563 -> 0.1546, K = 128 0.6577 -> 0.6526), and for rows of halves the priority moves
-            // on a rank with every pair instead of every round (fp16 K = 64: 0.913 -> 0.870; fp32 loses 1 % by it).
+            // 128-byte tiles: the eight entries of a round are added up and asked for one after the other, in the
+            // order written here - the compiler is told not to mix them (fp32: K = 32 0.1563 -> 0.1526, K = 128
+            // 0.6577 -> 0.6464 ms per product) -, and for rows of halves the priority moves on a rank with every
+            // entry instead of every round (fp16 K = 64: 0.913 -> 0.852; fp32 loses 1 % by that).
 #define SW_PRIO(v)                                        \
     switch ((v) & 3) {                                    \
     case 0: __builtin_amdgcn_s_setprio(0); break;         \
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     } else if constexpr (L == 8) {                                \
         __builtin_amdgcn_sched_barrier(0);                        \
     }
-            const int pr = (wave >> 2) - (kPairPrio ? 4 * r : r);
+            const int pr = (wave >> 2) - (kPairPrio ? 8 * r : r);
             SW_PRIO(pr)
             const uint4 cn = nx;
             nx = stream_load(min(r + 2, last));
@@ -243,15 +244,19 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
                 SW_ADD2(3) SW_GATHER(3, cn.x, 3, cm) SW_GATHER(7, cn.z, 3, cm)
             } else {
                 SW_ADD(0, cu.y, 0) SW_GATHER(0, cn.x, 0, cm)
-                SW_ADD(1, cu.y, 1) SW_GATHER(1, cn.x, 1, cm)
                 SW_NEXT_PAIR(1)
-                SW_ADD(2, cu.y, 2) SW_GATHER(2, cn.x, 2, cm)
-                SW_ADD(3, cu.y, 3) SW_GATHER(3, cn.x, 3, cm)
+                SW_ADD(1, cu.y, 1) SW_GATHER(1, cn.x, 1, cm)
                 SW_NEXT_PAIR(2)
-                SW_ADD(4, cu.w, 0) SW_GATHER(4, cn.z, 0, cm)
-                SW_ADD(5, cu.w, 1) SW_GATHER(5, cn.z, 1, cm)
+                SW_ADD(2, cu.y, 2) SW_GATHER(2, cn.x, 2, cm)
                 SW_NEXT_PAIR(3)
+                SW_ADD(3, cu.y, 3) SW_GATHER(3, cn.x, 3, cm)
+                SW_NEXT_PAIR(4)
+                SW_ADD(4, cu.w, 0) SW_GATHER(4, cn.z, 0, cm)
+                SW_NEXT_PAIR(5)
+                SW_ADD(5, cu.w, 1) SW_GATHER(5, cn.z, 1, cm)
+                SW_NEXT_PAIR(6)
                 SW_ADD(6, cu.w, 2) SW_GATHER(6, cn.z, 2, cm)
+                SW_NEXT_PAIR(7)
                 SW_ADD(7, cu.w, 3) SW_GATHER(7, cn.z, 3, cm)
             }
             cu = cn;
