@@ -25,6 +25,7 @@ struct DevicePlan {
     int *split_row = nullptr, *split_ptr = nullptr;
     float *partial = nullptr;  // [partial rows][K] fp32 sums of the sub-rows of split rows
     size_t lds_bytes = 0, device_bytes = 0, slots = 0;
+    int round_panels = 256;  // panels are made in multiples of this: one round of workgroups
     bool built_on_device = false;
 };
 
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
                                                             const int *__restrict__ panel_ptr, const int *__restrict__ rows,
                                                             const int *__restrict__ piece_ptr, const T *__restrict__ X,
                                                             T *__restrict__ Y, float *__restrict__ partial, int n, int K,
-                                                            int acc_rows, int col_bits, int bank_rows, int stream_keep)
+                                                            int acc_rows, int col_bits, int bank_rows, int stream_keep, int tiles, int round_panels)
 {
     extern __shared__ __align__(16) char smem[];
     f4_t *acc4 = reinterpret_cast<f4_t *>(smem);
@@ -120,7 +121,20 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     constexpr bool kPairPrio = L == 8 && sizeof(T) == 2;  // the wavefronts' priorities move on with every entry of a round
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int b = blockIdx.x, tile = blockIdx.y;
+    // Workgroups in the order of a one-dimensional grid: a round of panels at its first column tile, the same
+    // panels at the next tile, ... then the next round of panels - what a round of panels read of the entry stream
+    // is read again at once for the next tile.  (Tile by tile over all panels instead, as a two-dimensional grid
+    // orders them: R-MAT scale 20, fp32, K = 64 / 128 / 256 2.8 / 4.0 / 3.7 % slower.)
+    // (Kernels for 64-byte tiles keep the two-dimensional grid: their plans of one tile lose 2-4 % by the arithmetic.)
+    int b = blockIdx.x, tile = 0;
+    if constexpr (L == 4) {
+        tile = blockIdx.y;
+        tiles = gridDim.y;
+    } else if (tiles > 1) {
+        const int span = round_panels * tiles, grp = (int)blockIdx.x / span, within = (int)blockIdx.x - grp * span;
+        tile = within / round_panels;
+        b = grp * round_panels + (within - tile * round_panels);
+    }
     const int g = lane / L, c = lane % L, s = lane & 3;
     const int plane_stride = (acc_rows + 1) * L;  // float4 units
     const f4_t zero = {0.f, 0.f, 0.f, 0.f};
@@ -316,7 +330,7 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
             if (col0 < K) store_piece<T, P::kVec>(Y + (size_t)row * K + col0, sum, K - col0);
         } else {
             // read again by the fix-up kernel; a partial row has whole tiles
-            store_acc<P::kVec, false>(partial + (size_t)(row - n) * ((size_t)gridDim.y * (L * P::kVec)) + col0, sum);
+            store_acc<P::kVec, false>(partial + (size_t)(row - n) * ((size_t)tiles * (L * P::kVec)) + col0, sum);
         }
     }
 }
@@ -377,10 +391,13 @@ template <typename T, int L, int TOGETHER, bool FAR>
 int launch_main(const DevicePlan *dp, const T *X, T *Y, hipStream_t st)
 {
     const Layout &Lo = dp->host;
-    hipLaunchKernelGGL((sw_spmm_kernel<T, L, TOGETHER, FAR>), dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles), dim3(kThreads),
+    // (panels come in whole rounds; a layout that does not keep to that is walked tile by tile, one round of all its panels)
+    const int round_panels = dp->round_panels > 0 && Lo.num_panels % dp->round_panels == 0 ? dp->round_panels : Lo.num_panels;
+    const dim3 grid = L == 4 ? dim3((unsigned)Lo.num_panels, (unsigned)Lo.tiles) : dim3((unsigned)(Lo.num_panels * Lo.tiles));
+    hipLaunchKernelGGL((sw_spmm_kernel<T, L, TOGETHER, FAR>), grid, dim3(kThreads),
                        dp->lds_bytes, st, reinterpret_cast<const uint4 *>(dp->stream),
                        reinterpret_cast<const int2 *>(dp->wave_meta), dp->panel_rounds, dp->panel_ptr, dp->rows, dp->piece_ptr, X,
-                       Y, dp->partial, Lo.n, Lo.K, Lo.acc_rows, Lo.col_bits, Lo.bank_rows, dp->slots * 8 <= kStreamKeepBytes ? 1 : 0);
+                       Y, dp->partial, Lo.n, Lo.K, Lo.acc_rows, Lo.col_bits, Lo.bank_rows, dp->slots * 8 <= kStreamKeepBytes ? 1 : 0, Lo.tiles, round_panels);
     MPS_HIP_TRY(hipGetLastError());
     return MPS_OK;
 }
@@ -451,6 +468,7 @@ int create(const int *d_row_ptr, const int *d_col_idx, const void *d_val, int n,
             if (e != hipSuccess) return fail(MPS_ERR_HIP + (int)e);
             bp.num_cus = cus;
         }
+        dp->round_panels = bp.num_cus;
         // half values are widened on the device first (exact): both builders take fp32 values
         struct Dev {
             void *p = nullptr;
