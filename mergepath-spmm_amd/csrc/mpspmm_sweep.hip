@@ -117,7 +117,8 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
     using P = Piece<T>;
     constexpr int GPW = 64 / L;        // lane-groups of a wavefront
     constexpr int RQ = GPW * kWin;     // 16-byte units of a round
-    constexpr int kSync = L == 4 ? 1 : kSyncRounds;  // a workgroup barrier every so many rounds
+    // a workgroup barrier every so many rounds (see below): 1 for 64-byte rows, 2 for 128-byte tiles of fp32, 4 of fp16
+    constexpr int kSync = L == 4 ? 1 : sizeof(T) == 4 ? 2 : kSyncRounds;
     constexpr bool kPairPrio = L == 8 && sizeof(T) == 2;  // the wavefronts' priorities move on with every entry of a round
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -238,7 +239,10 @@ __global__ __launch_bounds__(kThreads) void sw_spmm_kernel(const uint4 *__restri
             // sweep, and the range of X that the chip gathers from at one time no longer fits an L2.
             // (64-byte rows: every round - R-MAT scale 20, fp32, K = 16, a barrier every 1 / 2 / 4 / 8 / 16 / 64 rounds:
             // 0.117 / 0.122 / 0.125 / 0.130 / 0.136 / 0.147 ms per product; 128-byte tiles: every fourth - K = 32
-            // 0.162 / 0.161 / 0.158 / 0.166 / 0.173 / 0.190, K = 128 0.672 / 0.671 / 0.658 / 0.681 / 0.700 / 0.758)
+            // 0.162 / 0.161 / 0.158 / 0.166 / 0.173 / 0.190, K = 128 0.672 / 0.671 / 0.658 / 0.681 / 0.700 / 0.758; with
+            // the entries of a round in strict order, plain stream loads and the rounds of panels taken through their
+            // tiles, every 2 / 4 / 8 rounds: K = 32 0.1343 / 0.1363 / 0.1406, K = 64 0.3020 / 0.3035 / 0.3130, K = 256
+            // 1.214 / 1.215 / 1.257 - every second; fp16, K = 64, every 2 / 4 / 8 / 16: 0.863 / 0.852 / 0.862 / 0.866)
             if ((r & (kSync - 1)) == 0) __syncthreads();
             // Between two barriers a SIMD would serve the oldest of its four wavefronts first in every round and the
             // other three would arrive late together.  The priority goes round instead, a round at each rank, the
